@@ -1,0 +1,170 @@
+/* C-ABI of libmortar_hip.so: the MI355X (gfx950) implementation of the MORTAR sparse-MLP path.
+ *
+ * Every entry point takes plain pointers and sizes.  Device pointers are raw HIP device
+ * addresses, `stream` is a hipStream_t passed as void* (NULL = the null stream).  All entry
+ * points return 0 on success and a negative code on failure; mortar_last_error() returns the
+ * message of the calling thread's last failure.  Nothing here allocates device memory: the
+ * caller owns inputs, outputs and the workspaces named below.
+ *
+ * Reference interfaces replaced (paths relative to the reference checkout):
+ *   stk_dds(lhs, data, offsets, row_indices, column_indices, ..., shape0, shape1, True)
+ *       morph/sparse/stk/backend/custom_ops.py:35-56 (forward use block_sparse.py:956-965)
+ *   _SwiGLUMortar.forward                      morph/model/transformer.py:402-431
+ *   TileRouter.forward steps 5-8               morph/model/routing.py:232-284
+ *   route_flags                                morph/kernels/triton/fused_decode_step.py:1913-1927
+ *   mortar_pack_strips / mortar_gemv           morph/kernels/triton/fused_decode_step.py:1465-1547
+ *   rmsnorm_rows / attention.RMSNorm           fused_decode_step.py:305-321, morph/model/attention.py:133-141
+ *   pack_mortar_ternary                        morph/inference/deploy_quant.py:344-374
+ */
+#ifndef MORTAR_HIP_H
+#define MORTAR_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MORTAR_BLK 16            /* carved block edge (carve(blocking=16)) */
+#define MORTAR_PREFILL_MT 128    /* tokens per prefill workgroup tile */
+#define MORTAR_PREFILL_KCB 14    /* block-columns per prefill K-chunk */
+
+enum {
+    MORTAR_OK = 0,
+    MORTAR_ERR_ARG = -1,       /* bad argument / shape / alignment */
+    MORTAR_ERR_SCALE = -2,     /* scale outside the representable window */
+    MORTAR_ERR_HIP = -3,       /* HIP runtime error (message has hipGetErrorString) */
+    MORTAR_ERR_LIMIT = -4      /* size beyond a stated maximum */
+};
+
+/* One carved matrix W [Rb*16, Cb*16] in device memory.
+ *   codes   [nnz*16] uint32: block j, output row n -> one dword holding its 16 ternary codes in the
+ *           device bit layout produced by mortar_encode_blocks_host
+ *   sdup    [nnz] uint32: per-block scale pattern produced by mortar_encode_blocks_host
+ *   col     [nnz] the reference's mortar_column_indices (int16, unchanged)
+ *   row_ptr [Rb+1] the reference's mortar_offsets (int32, unchanged)                              */
+typedef struct {
+    const uint32_t *codes;
+    const uint32_t *sdup;
+    const int16_t *col;
+    const int32_t *row_ptr;
+    int32_t Rb, Cb, nnz;
+} mortar_bcsr_t;
+
+const char *mortar_last_error(void);
+int mortar_abi_version(void);
+
+/* ---- host-side packing (no GPU needed) ------------------------------------------------------- */
+
+/* Re-encode the reference's flat 2-bit pack (pack_ternary_codes: 4 codes/byte, u=code+1, row-major over
+ * [nnz,16,16]; deploy_quant.py:56-71) into the device layout, and turn fp32 scales (scale_count = 1 for
+ * the reference's per-tensor scale, or nnz for per-block scales) into the per-block pattern.
+ * packed: host [nnz*64] bytes; codes_out host [nnz*16] uint32; sdup_out host [nnz] uint32.
+ * Fails with MORTAR_ERR_SCALE when bf16(scale) is non-finite or its magnitude is outside [2^-100, 2^100]
+ * (0 is allowed and zeroes the block). */
+int mortar_encode_blocks_host(const uint8_t *packed, int64_t nnz, const float *scale, int64_t scale_count,
+                              uint32_t *codes_out, uint32_t *sdup_out);
+
+/* Inverse of the code part (for tests): device-layout dwords -> int8 codes [nnz,16,16]. */
+int mortar_decode_blocks_host(const uint32_t *codes, int64_t nnz, int8_t *codes_out);
+
+/* Prefill K-chunk table: out[r*(nkc+1)+c] = first block of row r whose column >= c*kcb
+ * (nkc = ceil(Cb/kcb)); out host [Rb*(nkc+1)] int32.  Validates the BCSR (sorted, in range). */
+int mortar_chunk_ptr_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
+                          int32_t kcb, int32_t *out);
+
+/* Row-unit schedule for uneven nnz: units sorted by descending block count and dealt so that every
+ * workgroup of `group` units gets a similar total (longest-processing-time first).
+ * rows_per_unit = 1 (plain) or 2 (gate row u and up row u + Rb/2).  order_out host [n_units]. */
+int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_t rows_per_unit, int32_t group,
+                           int32_t *order_out);
+
+/* Decode work list.  Splits every row unit into entries of <= max_blocks blocks inside one K segment of
+ * kseg block-columns.  Each entry is 8 int32: {rowA, pA, cntA, rowB, pB, cntB, slot, seg}; rowB = -1 for
+ * plain units.  Call with entries_out = NULL to get the entry count (return value >= 0), then again with
+ * a buffer.  nslots_out = max partial slots per row; row_slots_out host [Rb] = slots of each row (optional).
+ * Entries are grouped by segment and padded with null entries (rowA = -1) to a multiple of 4 per segment,
+ * because one workgroup serves 4 consecutive entries of one segment. */
+int64_t mortar_decode_worklist_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
+                                    int32_t rows_per_unit, int32_t kseg, int32_t max_blocks,
+                                    int32_t *entries_out, int32_t *nslots_out, int32_t *row_slots_out);
+
+/* ---- prefill (large M), bf16 MFMA, fp32 accumulate -------------------------------------------- */
+
+/* y[M, Rb*16] = x[M, Cb*16] @ W^T (bf16 in, bf16 out).  Replaces stk_dds(..., transpose_b=True).
+ * chunk_ptr: device copy of mortar_chunk_ptr_host(kcb = MORTAR_PREFILL_KCB).
+ * unit_order: device [Rb] from mortar_unit_order_host(rows_per_unit=1, group=mortar_prefill_group(0)) or NULL.
+ * ldx / ldy in elements; x and y 16-byte aligned, ldx % 8 == 0, ldy % 4 == 0. */
+int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int32_t *unit_order,
+                     const uint16_t *x, int64_t M, int64_t ldx, uint16_t *y, int64_t ldy, void *stream);
+
+/* h[M, d_ff] = silu(gate) * up [* gates per cluster], gate_up = W [2*d_ff, d_model] with gate rows
+ * [0, d_ff) and up rows [d_ff, 2*d_ff) (transformer.py:335-336,403-405).  Intermediates are rounded to
+ * bf16 where the reference materialises a bf16 tensor.  gates: device fp32 [M, n_clusters] or NULL;
+ * d_ff % n_clusters == 0.
+ * Routed skipping (optional): tok_cnt/tok_list from mortar_remoe_route with tile = MORTAR_PREFILL_MT; when
+ * given (requires cluster_size % 16 == 0) only active (token, block-row) tiles are computed and written;
+ * inactive entries of h are left untouched and must be masked by the consumer (mortar_spmm_bf16_masked). */
+int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int32_t *unit_order,
+                              const uint16_t *x, int64_t M, int64_t ldx, uint16_t *h, int64_t ldh,
+                              const float *gates, int32_t n_clusters,
+                              const int32_t *tok_cnt, const uint8_t *tok_list, void *stream);
+
+/* As mortar_spmm_bf16, but input element (m, c) is read as 0 when active[m, c / cluster_size] == 0
+ * (active: device uint8 [M, n_clusters]); used for `down` after a routed mortar_gateup_swiglu_bf16. */
+int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int32_t *unit_order,
+                            const uint16_t *x, int64_t M, int64_t ldx, uint16_t *y, int64_t ldy,
+                            const uint8_t *active, int32_t n_clusters, void *stream);
+
+/* Units per prefill workgroup (for mortar_unit_order_host): swiglu = 0 plain, 1 gate/up pairs. */
+int mortar_prefill_group(int swiglu);
+
+/* ---- ReMoE gating --------------------------------------------------------------------------- */
+
+/* TileRouter steps 5-8: kth = k-th largest logit per token; g0 = relu(logit - kth) (threshold only when
+ * k < n); gates = g0 * (k / max(sum g0, 1e-6)); active = gates > 0.  logits/gates fp32 [M, n], active uint8
+ * [M, n] (may be NULL).  n <= 1024. */
+int mortar_remoe_gates(const float *logits, int64_t M, int32_t n, int32_t k, float *gates, uint8_t *active,
+                       void *stream);
+
+/* Wavefront-ballot compaction of active tokens per (token tile, cluster):
+ * tok_cnt[t*n + c] = number of tokens of tile t (tile tokens each, <= 256) with active[m, c] != 0,
+ * tok_list[(t*n + c)*tile + i] = tile-local index of the i-th such token, ascending. */
+int mortar_remoe_route(const uint8_t *active, int64_t M, int32_t n, int32_t tile, int32_t *tok_cnt,
+                       uint8_t *tok_list, void *stream);
+
+/* route_flags: row_act[b, r] (int32 [B, 2*d_ff/16], gate half then up half) and col_act[b, c]
+ * (int32 [B, d_ff/16]) = gate[b, lo] > 0 or gate[b, hi] > 0 with lo = (r*16)/cls, hi = (r*16+15)/cls.
+ * ld* = row strides in elements. */
+int mortar_route_flags(const float *gates, int64_t B, int32_t n_clusters, int64_t ldg, int32_t d_ff,
+                       int32_t *row_act, int64_t ldr, int32_t *col_act, int64_t ldc, void *stream);
+
+/* ---- decode (M <= 64) ------------------------------------------------------------------------ */
+
+/* Generic decode GEMV over a work list (mortar_decode_worklist_host; entries on the device).
+ * x bf16 [B, Cb*16]; B <= 64.
+ *   mode 0: y bf16 [B, Rb*16] = x W^T
+ *   mode 1: W = gate_up; y = h bf16 [B, Rb*8] = silu(g)*u [* gates[b, n/cls]]
+ * nslots = 1: entries write the result directly.  nslots > 1: partial sums go to `part`
+ * (fp32 [nslots, B, Rb*16], caller workspace) and a second kernel combines them in slot order, reading
+ * row_slots (device copy of the work list's row_slots_out).
+ * row_act / col_act (int32, may be NULL): ReMoE flags from mortar_route_flags; a unit all of whose B
+ * streams are inactive is skipped (zeros written); a block whose input column is inactive for all B
+ * streams is skipped. */
+int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_entries, int32_t nslots,
+                     const int32_t *row_slots, int32_t kseg, int32_t mode, const uint16_t *x, int32_t B, int64_t ldx,
+                     uint16_t *y, int64_t ldy, float *part,
+                     const float *gates, int32_t n_clusters, int64_t ldg,
+                     const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc,
+                     void *stream);
+
+/* ---- RMSNorm ---------------------------------------------------------------------------------- */
+
+/* y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) per row; x, y bf16 [M, d]; w bf16 [d] or NULL (= 1). */
+int mortar_rmsnorm_bf16(const uint16_t *x, int64_t M, int32_t d, int64_t ldx, const uint16_t *w, float eps,
+                        uint16_t *y, int64_t ldy, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MORTAR_HIP_H */

@@ -1,0 +1,228 @@
+"""CMSBlockLinear: the carved (MORTAR) linear layer, runtime side.
+
+Mirrors the carve / carved-forward / checkpoint surface of the reference's
+morph/model/layers/block_sparse.py (class and buffer names are kept because other code finds the layer by
+``type(m).__name__ == "CMSBlockLinear"`` and by its ``mortar_*`` attributes).  The training-time scoring and
+pruning machinery of the reference class is not part of this runtime.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from . import ops
+from .deploy_quant import _ternary_quantize, pack_ternary_codes
+from .pack import MortarPack
+
+
+def _stk_transpose(size, data, row_indices, column_indices, offsets):
+    """Transposed-topology metadata (reference: morph/sparse/stk/matrix.py:107-125).  A stable sort fixes the
+    order of blocks inside one block-column, which the reference leaves to the sort backend."""
+    block_columns = size[1] // data.shape[1]
+    gather_indices = torch.sort(column_indices.to(torch.int32), stable=True).indices
+    column_indices_t = row_indices.gather(0, gather_indices)
+    block_offsets_t = gather_indices.int()
+    nnz_per_column = torch.bincount(column_indices.to(torch.int64), minlength=block_columns).int()
+    zero = torch.zeros((1,), dtype=torch.int32, device=data.device)
+    offsets_t = torch.cat([zero, nnz_per_column.cumsum(0, dtype=torch.int32)])
+    return column_indices_t, offsets_t, block_offsets_t
+
+
+class CMSBlockLinear(nn.Module):
+    def __init__(self, in_features: int, out_features: int, tile_size: int = 16, density: float = 1.0,
+                 bias: bool = True, score_ema_alpha: float = 0.95, device=None, dtype=None) -> None:
+        super().__init__()
+        if in_features % tile_size or out_features % tile_size:
+            raise ValueError(f"[{out_features},{in_features}] not divisible by tile_size {tile_size}")
+        self.in_features, self.out_features, self.tile_size = in_features, out_features, tile_size
+        self.R, self.C = out_features // tile_size, in_features // tile_size
+        self.density = float(density)
+        self.K = self.C
+        self.weight = nn.Parameter(torch.empty(out_features, in_features, device=device, dtype=dtype))
+        nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+        self.bias = nn.Parameter(torch.zeros(out_features, device=device, dtype=dtype)) if bias else None
+        self._prune_mask: Tensor | None = None       # [R, C] bool tile mask
+        self._dense_mode, self._mortar, self._mortar_blocking = True, False, 0
+        self._values_ternary_mode, self._values_threshold = False, 0.5
+        self._pack: MortarPack | None = None
+
+    # ------------------------------------------------------------------ masks / carve
+
+    def set_block_mask(self, block_mask: Tensor, blocking: int = 16) -> None:
+        """Install a block-aligned prune mask ([out/blocking, in/blocking] bool) as the [R, C] tile mask."""
+        tpb = blocking // self.tile_size
+        if blocking % self.tile_size:
+            raise ValueError(f"blocking ({blocking}) not divisible by tile_size ({self.tile_size})")
+        self._prune_mask = block_mask.bool().repeat_interleave(tpb, 0).repeat_interleave(tpb, 1)
+
+    def enable_values_ternary(self, threshold: float = 0.5) -> None:
+        self._values_ternary_mode, self._values_threshold = True, float(threshold)
+        if self._mortar:
+            self.mortar_ternary.copy_(torch.tensor([1.0, threshold]))
+        self._pack = None
+
+    def carve(self, blocking: int = 16) -> int:
+        """Dense masked weight -> BCSR storage in the reference's layout (block_sparse.py:810-907):
+        row-major nonzero() order, int16 row/column indices, int32 offsets, data[j, lr, c] =
+        W[row_j*blk+lr, col_j*blk+c], plus the transposed-topology metadata."""
+        assert self._dense_mode, "carve() requires dense mode (pre-carve)"
+        assert not self._mortar, "carve() already applied"
+        if self.out_features % blocking or self.in_features % blocking:
+            raise ValueError(f"carve: [{self.out_features},{self.in_features}] not divisible by blocking {blocking}")
+        B = self.tile_size
+        if blocking % B != 0:
+            raise ValueError(f"carve: blocking ({blocking}) not divisible by tile_size ({B})")
+        with torch.no_grad():
+            tpb = blocking // B
+            Rb, Cb = self.out_features // blocking, self.in_features // blocking
+            w = self.weight.data
+            device = w.device
+            if self._prune_mask is not None:
+                tile_mask = self._prune_mask.to(device)
+                w = w * tile_mask.repeat_interleave(B, 0).repeat_interleave(B, 1).to(w.dtype)
+            else:
+                tile_mask = torch.ones(self.R, self.C, dtype=torch.bool, device=device)
+            m4 = tile_mask.view(Rb, tpb, Cb, tpb)
+            block_mask = m4.any(dim=3).any(dim=1)
+            if not bool(block_mask.any(dim=1).all()):
+                raise RuntimeError("carve: a block-row has zero kept blocks")
+            idx = block_mask.nonzero()
+            row_indices = idx[:, 0].to(torch.int16).contiguous()
+            column_indices = idx[:, 1].to(torch.int16).contiguous()
+            row_nnz = block_mask.sum(dim=1).to(torch.int32)
+            offsets = torch.cat([torch.zeros(1, dtype=torch.int32, device=device),
+                                 row_nnz.cumsum(0, dtype=torch.int32)]).contiguous()
+            blocks = w.reshape(Rb, blocking, Cb, blocking).permute(0, 2, 1, 3)
+            data = blocks[idx[:, 0], idx[:, 1]].contiguous()
+            ct, ot, bt = _stk_transpose((self.out_features, self.in_features), data, row_indices, column_indices, offsets)
+            self._init_mortar_storage(data.clone(), row_indices, column_indices, offsets, ct.contiguous(),
+                                      ot.contiguous(), bt.contiguous(), blocking)
+        nnz = int(self.mortar_data.shape[0])
+        self.density = nnz / (Rb * Cb)
+        return nnz
+
+    def _init_mortar_storage(self, data, row_indices, column_indices, offsets, column_indices_t, offsets_t,
+                             block_offsets_t, blocking: int) -> None:
+        if "weight" in self._parameters:
+            del self._parameters["weight"]
+        self.mortar_data = nn.Parameter(data)
+        for name, t in (("mortar_row_indices", row_indices), ("mortar_column_indices", column_indices),
+                        ("mortar_offsets", offsets), ("mortar_column_indices_t", column_indices_t),
+                        ("mortar_offsets_t", offsets_t), ("mortar_block_offsets_t", block_offsets_t)):
+            self.register_buffer(name, t)
+        self.register_buffer("mortar_ternary", torch.tensor(
+            [1.0 if self._values_ternary_mode else 0.0, self._values_threshold], dtype=torch.float32, device=data.device))
+        self._mortar, self._mortar_blocking, self._dense_mode = True, int(blocking), False
+        self._pack = None
+
+    # ------------------------------------------------------------------ forward
+
+    def get_density(self) -> float:
+        return self.density
+
+    def _mortar_effective_data(self) -> Tensor:
+        """Dense-valued view of the carved weight actually used in forward ([nnz, blk, blk]); the packed
+        form dequantises as bf16(code) * bf16(scale) (deploy_quant.py:367-369)."""
+        if "mortar_packed" in self._buffers:
+            from .deploy_quant import unpack_ternary
+            w = unpack_ternary(self.mortar_packed, self._packed_numel, torch.bfloat16).view(self._packed_shape)
+            s = self.mortar_scale.to(torch.bfloat16)
+            return w * (s.view(-1, 1, 1) if s.dim() else s)
+        d = self.mortar_data
+        if not self._values_ternary_mode:
+            return d
+        scale = d.detach().abs().mean().clamp(min=1e-8)
+        d_norm = d / scale
+        q = torch.sign(d_norm) * (d_norm.abs() > self._values_threshold).to(d.dtype)
+        return d + (scale * q - d).detach()
+
+    def mortar_pack(self) -> MortarPack:
+        """Device weight format for the HIP kernels, built once (topology and values are frozen at deploy)."""
+        if self._pack is not None:
+            return self._pack
+        if not self._mortar:
+            raise RuntimeError("mortar_pack() requires a carved layer")
+        if self._mortar_blocking != 16:
+            raise ValueError(f"the gfx950 MORTAR runtime executes carve(blocking=16); this layer was carved at {self._mortar_blocking}")
+        if "mortar_packed" in self._buffers:
+            packed, scale = self.mortar_packed, self.mortar_scale
+        elif self._values_ternary_mode:
+            q, scale = _ternary_quantize(self.mortar_data.data, self._values_threshold)
+            packed = pack_ternary_codes(q)
+        else:
+            raise RuntimeError("carved layer holds non-ternary values: call pack_mortar_ternary() or "
+                               "enable_values_ternary() first (the MORTAR runtime executes ternary blocks only)")
+        self._pack = MortarPack(packed, scale, self.mortar_column_indices, self.mortar_offsets,
+                                self.out_features, self.in_features, self.mortar_offsets.device)
+        return self._pack
+
+    def _forward_mortar(self, x: Tensor) -> Tensor:
+        """Carved forward y = x @ W_sparse^T (+bias).  Reference: block_sparse.py:921-970 (flatten leading
+        dims, bf16 operands, fp32 accumulate, output in the activation dtype; no M padding is needed)."""
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, self.in_features)
+        xb = x2 if x2.dtype == torch.bfloat16 else x2.to(torch.bfloat16)
+        W = self.mortar_pack()
+        y = ops.gemv(xb, W) if 0 < xb.shape[0] <= 64 else ops.spmm(xb, W)
+        if y.dtype != x.dtype:
+            y = y.to(x.dtype)
+        if self.bias is not None:
+            y = y + self.bias
+        return y.reshape(*lead, self.out_features)
+
+    def forward(self, x: Tensor) -> Tensor:
+        if self._mortar:
+            return self._forward_mortar(x)
+        w = self.weight
+        if self._prune_mask is not None:
+            B = self.tile_size
+            w = w * self._prune_mask.to(w.device).repeat_interleave(B, 0).repeat_interleave(B, 1).to(w.dtype)
+        return F.linear(x, w, self.bias)
+
+    def _apply(self, fn, *a, **k):
+        self._pack = None       # device may change
+        return super()._apply(fn, *a, **k)
+
+    # ------------------------------------------------------------------ checkpoints
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        """Accepts the reference's carved key set (block_sparse.py:983-1036): mortar_data + six index buffers
+        + mortar_ternary, or the packed variant mortar_packed + mortar_scale in place of mortar_data."""
+        dk, pk = prefix + "mortar_data", prefix + "mortar_packed"
+        if (dk in state_dict or pk in state_dict) and not self._mortar:
+            dev = self.weight.device
+            idx = {k: torch.empty_like(state_dict[prefix + k], device=dev) for k in (
+                "mortar_row_indices", "mortar_column_indices", "mortar_offsets", "mortar_column_indices_t",
+                "mortar_offsets_t", "mortar_block_offsets_t")}
+            mt = state_dict.get(prefix + "mortar_ternary")
+            if mt is not None:
+                self._values_ternary_mode = bool(float(mt[0]) > 0)
+                self._values_threshold = float(mt[1])
+            nnz = int(idx["mortar_row_indices"].numel())
+            if dk in state_dict:
+                ck = state_dict[dk]
+                blocking = int(ck.shape[-1])
+                data = torch.empty_like(ck, device=dev)
+            else:
+                blocking = int(round(math.sqrt(state_dict[pk].numel() * 4 / max(nnz, 1))))
+                data = torch.empty(0, device=dev)
+            self._init_mortar_storage(data, idx["mortar_row_indices"], idx["mortar_column_indices"],
+                                      idx["mortar_offsets"], idx["mortar_column_indices_t"], idx["mortar_offsets_t"],
+                                      idx["mortar_block_offsets_t"], blocking)
+            if pk in state_dict and dk not in state_dict:
+                del self._parameters["mortar_data"]
+                self.register_buffer("mortar_packed", torch.empty_like(state_dict[pk], device=dev))
+                self.register_buffer("mortar_scale", torch.empty_like(state_dict[prefix + "mortar_scale"], device=dev))
+                self._packed_shape = (nnz, blocking, blocking)
+                self._packed_numel = nnz * blocking * blocking
+            Rb, Cb = self.out_features // blocking, self.in_features // blocking
+            self.density = nnz / (Rb * Cb)
+        self._pack = None
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
+    def extra_repr(self) -> str:
+        return (f"in_features={self.in_features}, out_features={self.out_features}, tile_size={self.tile_size}, "
+                f"density={self.density:.2f}, mortar={self._mortar}, bias={self.bias is not None}")

@@ -1,0 +1,235 @@
+// Decode (M <= 64) block-sparse ternary GEMV: streams the packed blocks once, bandwidth bound.
+//
+// Replaces the reference's mortar_gemv + combine (morph/kernels/triton/fused_decode_step.py:1341-1547).
+// As there, the schedule is a work list built once per matrix (topology is frozen): every entry is a run
+// of consecutive blocks of ONE row unit, one wavefront per entry, and rows that are split over several
+// entries write fp32 partials that a second kernel sums in slot order (no atomics, deterministic).
+//
+// Per entry the wave streams block pairs (128 B of codes + 2 scales + 2 column ids), unpacks them in
+// registers and contracts them with the staged activations in one 16x16x32 bf16 MFMA per 16 streams: the
+// matrix pipe does the 512 multiply-adds of a block pair in one issue slot, which keeps the vector ALU free
+// for the unpack -- the step that bounds this kernel when done with scalar FMAs.
+#include "mortar_device.h"
+#include "mortar_internal.h"
+
+namespace {
+
+struct GemvParams {
+    const uint32_t *codes;
+    const uint32_t *sdup;
+    const int16_t *col;
+    const int32_t *entries;
+    int n_entries, nslots, kseg, mode, Cb, N;
+    const uint16_t *x;
+    int B;
+    int64_t ldx;
+    uint16_t *y;
+    int64_t ldy;
+    float *part;
+    const float *gates;
+    int n_clusters, cluster_size;
+    int64_t ldg;
+    const int32_t *row_act;
+    int64_t ldr;
+    const int32_t *col_act;
+    int64_t ldc;
+};
+
+constexpr int UN = 4;   // block pairs whose loads are in flight together
+
+template <int MSUB>
+__device__ __forceinline__ void run_blocks(const GemvParams &p, int p0, int cnt, int c0, const uint4 *lx,
+                                           const uint32_t *colflag, int n, int bsel, int hsel,
+                                           f32x4_t (&acc)[MSUB]) {
+    constexpr int LDB = 16 * MSUB + 1;
+    for (int q0 = 0; q0 < cnt; q0 += 2 * UN) {
+        uint32_t w[UN], sd[UN];
+        int c[UN];
+        bool ok[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int q = q0 + 2 * u + bsel;
+            ok[u] = q < cnt;
+            const int64_t j = p0 + (ok[u] ? q : 0);
+            w[u] = p.codes[j * 16 + n];
+            sd[u] = p.sdup[j];
+            c[u] = p.col[j] - c0;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            if (q0 + 2 * u < cnt) {
+                bool on = ok[u];
+                if (colflag) on = on && colflag[c[u]] != 0u;
+                const u32x4_t A = mortar_unpack8(on ? (w[u] << (8 * hsel)) : 0u, sd[u]);
+                const uint32_t xo = (uint32_t)((c[u] * 2 + hsel) * LDB + n);
+#pragma unroll
+                for (int ms = 0; ms < MSUB; ++ms) {
+                    const uint4 b = lx[xo + ms * 16];
+                    const u32x4_t Bv = {b.x, b.y, b.z, b.w};
+                    acc[ms] = mortar_mfma(A, Bv, acc[ms]);
+                }
+            }
+        }
+    }
+}
+
+template <int MSUB>
+__global__ void __launch_bounds__(256) mortar_gemv_kernel(const GemvParams p) {
+    constexpr int LDB = 16 * MSUB + 1;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint4 *lx = reinterpret_cast<uint4 *>(smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
+
+    const int32_t *e0p = p.entries + (int64_t)blockIdx.x * 4 * 8;
+    const int seg = __builtin_amdgcn_readfirstlane(e0p[7]);
+    const int c0 = seg * p.kseg;
+    const int ncb = (p.Cb - c0) < p.kseg ? (p.Cb - c0) : p.kseg;
+    const int nch = 2 * ncb;
+    uint32_t *colflag = reinterpret_cast<uint32_t *>(smem + (size_t)2 * p.kseg * LDB * 16);
+
+    // stage the activations of this K segment: unit (ch, tok) <- x[tok, c0*16 + ch*8 .. +8]
+    for (int tok = 0; tok < p.B; ++tok)
+        for (int ch = tid; ch < nch; ch += 256)
+            lx[ch * LDB + tok] = *reinterpret_cast<const uint4 *>(p.x + (int64_t)tok * p.ldx + (int64_t)c0 * 16 + ch * 8);
+    if (p.col_act) {
+        for (int c = tid; c < ncb; c += 256) {
+            uint32_t f = 0;
+            for (int b = 0; b < p.B; ++b) f |= (uint32_t)(p.col_act[(int64_t)b * p.ldc + c0 + c] != 0);
+            colflag[c] = f;
+        }
+    }
+    __syncthreads();
+
+    const int32_t *ep = e0p + wave * 8;
+    const int rowA = __builtin_amdgcn_readfirstlane(ep[0]);
+    if (rowA < 0) return;
+    const int pA = __builtin_amdgcn_readfirstlane(ep[1]), cntA = __builtin_amdgcn_readfirstlane(ep[2]);
+    const int rowB = __builtin_amdgcn_readfirstlane(ep[3]);
+    const int pB = __builtin_amdgcn_readfirstlane(ep[4]), cntB = __builtin_amdgcn_readfirstlane(ep[5]);
+    const int slot = __builtin_amdgcn_readfirstlane(ep[6]);
+
+    bool unit_on = true;
+    if (p.row_act) {   // skip the unit when no stream has it active
+        int f = 0;
+        if (lane < p.B) f = p.row_act[(int64_t)lane * p.ldr + rowA] != 0;
+        unit_on = __builtin_amdgcn_readfirstlane(__ballot(f) != 0ull);
+    }
+
+    f32x4_t accA[MSUB], accB[MSUB];
+#pragma unroll
+    for (int ms = 0; ms < MSUB; ++ms) accA[ms] = accB[ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (unit_on) {
+        run_blocks<MSUB>(p, pA, cntA, c0, lx, p.col_act ? colflag : nullptr, n, bsel, hsel, accA);
+        if (rowB >= 0) run_blocks<MSUB>(p, pB, cntB, c0, lx, p.col_act ? colflag : nullptr, n, bsel, hsel, accB);
+    }
+
+#pragma unroll
+    for (int ms = 0; ms < MSUB; ++ms) {
+        const int tok = ms * 16 + n;
+        if (tok >= p.B) continue;
+        if (p.nslots > 1) {
+            float *pp = p.part + ((int64_t)slot * p.B + tok) * p.N;
+            *reinterpret_cast<f32x4_t *>(pp + rowA * 16 + 4 * g) = accA[ms];
+            if (rowB >= 0) *reinterpret_cast<f32x4_t *>(pp + rowB * 16 + 4 * g) = accB[ms];
+        } else {
+            uint32_t o[4];
+            const int e0 = rowA * 16 + 4 * g;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                if (p.mode == 0) {
+                    o[v] = bf16_bits_rne(accA[ms][v]);
+                } else {
+                    const float gt = bf16r(accA[ms][v]), up = bf16r(accB[ms][v]);
+                    float h = bf16r(bf16r(silu_f32(gt)) * up);
+                    if (p.gates) h = bf16r(h * bf16r(p.gates[(int64_t)tok * p.ldg + (e0 + v) / p.cluster_size]));
+                    o[v] = bf16_bits_rne(h);
+                }
+            }
+            const u32x2_t pk = {o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
+            *reinterpret_cast<u32x2_t *>(p.y + (int64_t)tok * p.ldy + e0) = pk;
+        }
+    }
+}
+
+// Sums the partials of each output in slot order and applies the epilogue.  row_slots[r] = number of
+// partial slots row r owns (rows of one unit own the same number).
+__global__ void __launch_bounds__(256) mortar_combine_kernel(const GemvParams p, const int32_t *row_slots) {
+    const int nout = p.mode == 0 ? p.N : p.N / 2;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)p.B * nout) return;
+    const int tok = (int)(i / nout), o = (int)(i % nout);
+    const int ns = row_slots[o >> 4];
+    float a = 0.f, b = 0.f;
+    for (int s = 0; s < ns; ++s) {
+        const float *pp = p.part + ((int64_t)s * p.B + tok) * p.N;
+        a += pp[o];
+        if (p.mode == 1) b += pp[nout + o];
+    }
+    float r = a;
+    if (p.mode == 1) {
+        r = bf16r(bf16r(silu_f32(bf16r(a))) * bf16r(b));
+        if (p.gates) r = bf16r(r * bf16r(p.gates[(int64_t)tok * p.ldg + o / p.cluster_size]));
+    }
+    p.y[(int64_t)tok * p.ldy + o] = (uint16_t)bf16_bits_rne(r);
+}
+
+template <int MSUB>
+int launch_gemv(const GemvParams &p, hipStream_t st) {
+    const size_t smem = (size_t)2 * p.kseg * (16 * MSUB + 1) * 16 + (size_t)p.kseg * 4;
+    if (smem > 160 * 1024) return mortar_fail(MORTAR_ERR_LIMIT, "gemv: K segment of %d block-columns needs %zu bytes of LDS", p.kseg, smem);
+    auto kern = mortar_gemv_kernel<MSUB>;
+    static size_t attr_set = 0;
+    if (smem > attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        attr_set = smem;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.n_entries / 4)), dim3(256), smem, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "gemv launch: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}
+
+}  // namespace
+
+extern "C" int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_entries,
+                                int32_t nslots, const int32_t *row_slots, int32_t kseg, int32_t mode,
+                                const uint16_t *x, int32_t B, int64_t ldx, uint16_t *y, int64_t ldy, float *part,
+                                const float *gates, int32_t n_clusters, int64_t ldg,
+                                const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc,
+                                void *stream) {
+    if (!W || !W->codes || !W->sdup || !W->col || !entries || !x || !y)
+        return mortar_fail(MORTAR_ERR_ARG, "gemv: null pointer");
+    if (B <= 0 || B > 64) return mortar_fail(MORTAR_ERR_LIMIT, "gemv: B=%d outside 1..64", B);
+    if (n_entries <= 0 || n_entries % 4 || n_entries > (int64_t)0x7fffffff) return mortar_fail(MORTAR_ERR_ARG, "gemv: entry count must be a positive multiple of 4");
+    if (mode != 0 && mode != 1) return mortar_fail(MORTAR_ERR_ARG, "gemv: mode must be 0 or 1");
+    if (mode == 1 && (W->Rb & 1)) return mortar_fail(MORTAR_ERR_ARG, "gemv: gate_up needs an even number of block-rows");
+    if (nslots < 1 || (nslots > 1 && (!part || !row_slots))) return mortar_fail(MORTAR_ERR_ARG, "gemv: nslots > 1 needs the partial workspace and row_slots");
+    if (kseg <= 0) return mortar_fail(MORTAR_ERR_ARG, "gemv: kseg must be positive");
+    const int64_t nout = mode == 0 ? (int64_t)W->Rb * 16 : (int64_t)W->Rb * 8;
+    if (ldx < (int64_t)W->Cb * 16 || ldx % 8 || ldy < nout || ldy % 4 ||
+        (reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(y) & 7))
+        return mortar_fail(MORTAR_ERR_ARG, "gemv: bad leading dimension or alignment");
+    GemvParams p{};
+    p.codes = W->codes; p.sdup = W->sdup; p.col = W->col; p.entries = entries; p.n_entries = (int)n_entries;
+    p.nslots = nslots; p.kseg = kseg; p.mode = mode; p.Cb = W->Cb; p.N = W->Rb * 16;
+    p.x = x; p.B = B; p.ldx = ldx; p.y = y; p.ldy = ldy; p.part = part;
+    p.n_clusters = 1; p.cluster_size = 1 << 30;
+    if (gates) {
+        if (mode != 1 || n_clusters <= 0 || nout % n_clusters) return mortar_fail(MORTAR_ERR_ARG, "gemv: gates need mode 1 and d_ff %% n_clusters == 0");
+        p.gates = gates; p.n_clusters = n_clusters; p.cluster_size = (int)(nout / n_clusters); p.ldg = ldg;
+    }
+    p.row_act = row_act; p.ldr = ldr; p.col_act = col_act; p.ldc = ldc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int rc = B <= 16 ? launch_gemv<1>(p, st) : (B <= 32 ? launch_gemv<2>(p, st) : launch_gemv<4>(p, st));
+    if (rc) return rc;
+    if (nslots > 1) {
+        const int64_t total = (int64_t)B * nout;
+        hipLaunchKernelGGL(mortar_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, p, row_slots);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "combine launch: %s", hipGetErrorString(e));
+    }
+    return MORTAR_OK;
+}

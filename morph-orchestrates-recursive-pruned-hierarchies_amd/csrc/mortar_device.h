@@ -1,0 +1,54 @@
+// Device helpers shared by the gfx950 kernels: ternary block unpack, MFMA wrappers, bf16 rounding.
+#ifndef MORTAR_DEVICE_H
+#define MORTAR_DEVICE_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+// Lane decomposition used by every MFMA kernel here (v_mfma_f32_16x16x32_bf16):
+//   n = lane & 15   row of the A operand (output feature inside the block-row) / column of B (token)
+//   g = lane >> 4   K group: the lane holds K slots 8g .. 8g+7
+// One MFMA contracts two 16x16 blocks: bsel = g >> 1 picks the block, hsel = g & 1 its column half.
+// The accumulator lane holds D[4g + v][n], v = 0..3: four consecutive output features of token n.
+
+// 8 ternary codes -> 8 bf16 weights (+-bf16(scale) or 0) in four dwords.
+// `t` is the row dword already shifted left by 8*hsel; the pair (2i, 2i+1) of this column half then sits
+// in the top two bits of the half-words of (t << 2i): bit 15/31 = negative, bit 14/30 = non-zero.  Read as
+// 16-bit floats those half-words are -2, 0 or +2; `sd` holds the block scale's bf16 pattern minus one
+// 16-bit-float exponent step in both halves, so one packed half multiply returns exactly +-scale or 0 in bf16
+// bits (a power-of-two product is exact; the host rejects scales whose pattern would leave the normal range).
+__device__ __forceinline__ u32x4_t mortar_unpack8(uint32_t t, uint32_t sd) {
+    const f16x2_t s = __builtin_bit_cast(f16x2_t, sd);
+    u32x4_t r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t f = (t << (2 * i)) & 0xC000C000u;
+        r[i] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, f));
+    }
+    return r;
+}
+
+__device__ __forceinline__ f32x4_t mortar_mfma(u32x4_t a, u32x4_t b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ uint32_t bf16_bits_rne(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ float bf16_to_f32(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
+__device__ __forceinline__ float bf16r(float f) { return bf16_to_f32(bf16_bits_rne(f)); }
+
+// silu in fp32 from a bf16-rounded input; the result is rounded to bf16 by the caller.
+__device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
+
+#endif

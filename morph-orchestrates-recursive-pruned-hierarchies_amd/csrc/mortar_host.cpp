@@ -1,0 +1,243 @@
+// Host-side packing and scheduling for the MORTAR device format (no GPU calls in this file).
+//
+// The reference keeps carved weights as mortar_packed (flat 2-bit codes, u = code + 1) plus a scale
+// (morph/inference/deploy_quant.py:344-374) and re-packs them once for its decode engine
+// (mortar_pack_strips, morph/kernels/triton/fused_decode_step.py:1465-1499).  This file is the
+// equivalent one-time re-pack for the gfx950 kernels.
+#include "mortar_internal.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <numeric>
+#include <vector>
+
+static thread_local char g_err[512] = "";
+
+int mortar_fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+extern "C" const char *mortar_last_error(void) { return g_err; }
+extern "C" int mortar_abi_version(void) { return 1; }
+
+static inline uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// Bit position (in 2-bit slots) of column c inside a row dword: the even columns of each pair sit in the
+// low half-word and the odd columns in the high half-word, so that (dword << 2*(c/2)) & 0xC000C000
+// isolates the pair (c&~1, c|1) in the two top bit pairs of the half-words.
+static inline int slot_of_col(int c) { return ((c & 1) ? 15 : 7) - (c >> 1); }
+
+extern "C" int mortar_encode_blocks_host(const uint8_t *packed, int64_t nnz, const float *scale,
+                                         int64_t scale_count, uint32_t *codes_out, uint32_t *sdup_out) {
+    if (!packed || !scale || !codes_out || !sdup_out || nnz < 0)
+        return mortar_fail(MORTAR_ERR_ARG, "encode_blocks: null pointer or negative nnz");
+    if (scale_count != 1 && scale_count != nnz)
+        return mortar_fail(MORTAR_ERR_ARG, "encode_blocks: scale_count must be 1 or nnz (got %lld, nnz %lld)",
+                           (long long)scale_count, (long long)nnz);
+    for (int64_t j = 0; j < nnz; ++j) {
+        const uint16_t s = f32_to_bf16_bits(scale[scale_count == 1 ? 0 : j]);
+        const int e8 = (s >> 7) & 0xff;
+        uint32_t sd = 0;
+        if ((s & 0x7fff) != 0) {
+            if (e8 < 27 || e8 > 227)
+                return mortar_fail(MORTAR_ERR_SCALE,
+                                   "encode_blocks: scale of block %lld (%g) outside [2^-100, 2^100]",
+                                   (long long)j, (double)scale[scale_count == 1 ? 0 : j]);
+            const uint32_t adj = (uint32_t)s - 0x0400u;   // half the value when read as a 16-bit float
+            sd = adj | (adj << 16);
+        }
+        sdup_out[j] = sd;
+        for (int n = 0; n < 16; ++n) {
+            uint32_t flat;
+            memcpy(&flat, packed + j * 64 + n * 4, 4);    // 16 codes of row n, 2 bits each, col c at bits 2c
+            uint32_t w = 0;
+            for (int c = 0; c < 16; ++c) {
+                const uint32_t u = (flat >> (2 * c)) & 3u;      // 0:-1  1:0  2:+1  (3 never produced)
+                if (u == 3u)
+                    return mortar_fail(MORTAR_ERR_ARG, "encode_blocks: invalid 2-bit code 3 in block %lld",
+                                       (long long)j);
+                const uint32_t enc = sd == 0 ? 0u : (u == 0u ? 3u : (u == 2u ? 1u : 0u));  // bit1 sign, bit0 nonzero
+                w |= enc << (2 * slot_of_col(c));
+            }
+            codes_out[j * 16 + n] = w;
+        }
+    }
+    return MORTAR_OK;
+}
+
+extern "C" int mortar_decode_blocks_host(const uint32_t *codes, int64_t nnz, int8_t *codes_out) {
+    if (!codes || !codes_out) return mortar_fail(MORTAR_ERR_ARG, "decode_blocks: null pointer");
+    for (int64_t j = 0; j < nnz; ++j)
+        for (int n = 0; n < 16; ++n) {
+            const uint32_t w = codes[j * 16 + n];
+            for (int c = 0; c < 16; ++c) {
+                const uint32_t enc = (w >> (2 * slot_of_col(c))) & 3u;
+                codes_out[j * 256 + n * 16 + c] = enc == 1u ? 1 : (enc == 3u ? -1 : 0);
+            }
+        }
+    return MORTAR_OK;
+}
+
+int mortar_check_bcsr_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb) {
+    if (!row_ptr || !col || Rb <= 0 || Cb <= 0) return mortar_fail(MORTAR_ERR_ARG, "bcsr: null pointer or empty shape");
+    if (row_ptr[0] != 0) return mortar_fail(MORTAR_ERR_ARG, "bcsr: offsets[0] != 0");
+    for (int r = 0; r < Rb; ++r) {
+        if (row_ptr[r + 1] < row_ptr[r]) return mortar_fail(MORTAR_ERR_ARG, "bcsr: offsets decrease at row %d", r);
+        for (int p = row_ptr[r]; p < row_ptr[r + 1]; ++p) {
+            if (col[p] < 0 || col[p] >= Cb)
+                return mortar_fail(MORTAR_ERR_ARG, "bcsr: column index %d out of range at block %d", (int)col[p], p);
+            if (p > row_ptr[r] && col[p] <= col[p - 1])
+                return mortar_fail(MORTAR_ERR_ARG, "bcsr: columns of row %d not strictly ascending", r);
+        }
+    }
+    return MORTAR_OK;
+}
+
+extern "C" int mortar_chunk_ptr_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
+                                     int32_t kcb, int32_t *out) {
+    if (!out || kcb <= 0) return mortar_fail(MORTAR_ERR_ARG, "chunk_ptr: bad argument");
+    int rc = mortar_check_bcsr_host(row_ptr, col, Rb, Cb);
+    if (rc) return rc;
+    const int nkc = (Cb + kcb - 1) / kcb;
+    for (int r = 0; r < Rb; ++r) {
+        int p = row_ptr[r];
+        const int e = row_ptr[r + 1];
+        for (int c = 0; c <= nkc; ++c) {
+            while (p < e && col[p] < c * kcb) ++p;
+            out[(int64_t)r * (nkc + 1) + c] = (c == nkc) ? e : p;
+        }
+    }
+    return MORTAR_OK;
+}
+
+extern "C" int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_t rows_per_unit,
+                                      int32_t group, int32_t *order_out) {
+    if (!row_ptr || !order_out || Rb <= 0 || group <= 0 || (rows_per_unit != 1 && rows_per_unit != 2) ||
+        Rb % rows_per_unit)
+        return mortar_fail(MORTAR_ERR_ARG, "unit_order: bad argument");
+    const int nu = Rb / rows_per_unit;
+    std::vector<int64_t> cost(nu);
+    bool uniform = true;
+    for (int u = 0; u < nu; ++u) {
+        cost[u] = row_ptr[u + 1] - row_ptr[u];
+        if (rows_per_unit == 2) cost[u] += row_ptr[u + nu + 1] - row_ptr[u + nu];
+        if (cost[u] != cost[0]) uniform = false;
+    }
+    if (uniform) {   // natural order keeps neighbouring output columns in one wave
+        std::iota(order_out, order_out + nu, 0);
+        return MORTAR_OK;
+    }
+    std::vector<int> idx(nu);
+    std::iota(idx.begin(), idx.end(), 0);
+    std::stable_sort(idx.begin(), idx.end(), [&](int a, int b) { return cost[a] > cost[b]; });
+    const int ng = (nu + group - 1) / group;
+    std::vector<int64_t> load(ng, 0);
+    std::vector<std::vector<int>> members(ng);
+    std::vector<int> cap(ng, group);
+    cap[ng - 1] = nu - (ng - 1) * group;
+    for (int u : idx) {
+        int best = -1;
+        for (int g = 0; g < ng; ++g)
+            if ((int)members[g].size() < cap[g] && (best < 0 || load[g] < load[best])) best = g;
+        members[best].push_back(u);
+        load[best] += cost[u];
+    }
+    // inside a group the waves take consecutive runs; deal the sorted members across the runs
+    const int nw = 4, rw = std::max(1, group / nw);
+    for (int g = 0; g < ng; ++g) {
+        const int n = (int)members[g].size();
+        std::vector<int> placed(group, -1);
+        int k = 0;
+        for (int rnd = 0; rnd < rw && k < n; ++rnd)
+            for (int w = 0; w < nw && k < n; ++w) {
+                const int ww = (rnd & 1) ? nw - 1 - w : w;     // snake
+                placed[ww * rw + rnd] = members[g][k++];
+            }
+        int o = g * group;
+        for (int i = 0; i < group; ++i)
+            if (placed[i] >= 0) order_out[o++] = placed[i];
+    }
+    return MORTAR_OK;
+}
+
+extern "C" int64_t mortar_decode_worklist_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb,
+                                               int32_t Cb, int32_t rows_per_unit, int32_t kseg,
+                                               int32_t max_blocks, int32_t *entries_out, int32_t *nslots_out,
+                                               int32_t *row_slots_out) {
+    if (kseg <= 0 || max_blocks <= 0 || (rows_per_unit != 1 && rows_per_unit != 2) || Rb % rows_per_unit)
+        return mortar_fail(MORTAR_ERR_ARG, "decode_worklist: bad argument");
+    int rc = mortar_check_bcsr_host(row_ptr, col, Rb, Cb);
+    if (rc) return rc;
+    const int nu = Rb / rows_per_unit;
+    const int nseg = (Cb + kseg - 1) / kseg;
+    struct Ent { int32_t v[8]; };
+    std::vector<std::vector<Ent>> per_seg(nseg);
+    std::vector<int> slot_of_unit(nu, 0);
+    int nslots = 1;
+    // range of row r inside segment s
+    auto seg_range = [&](int r, int s, int &a, int &b) {
+        a = row_ptr[r];
+        const int e = row_ptr[r + 1];
+        while (a < e && col[a] < s * kseg) ++a;
+        b = a;
+        while (b < e && col[b] < (s + 1) * kseg) ++b;
+    };
+    for (int s = 0; s < nseg; ++s)
+        for (int u = 0; u < nu; ++u) {
+            int a0, b0, a1 = 0, b1 = 0;
+            seg_range(u, s, a0, b0);
+            if (rows_per_unit == 2) seg_range(u + nu, s, a1, b1);
+            const int n0 = b0 - a0, n1 = b1 - a1;
+            const int nch = std::max((n0 + max_blocks - 1) / max_blocks, (n1 + max_blocks - 1) / max_blocks);
+            for (int i = 0; i < nch; ++i) {
+                Ent e;
+                const int c0 = std::max(0, std::min(max_blocks, n0 - i * max_blocks));
+                const int c1 = std::max(0, std::min(max_blocks, n1 - i * max_blocks));
+                e.v[0] = u; e.v[1] = c0 > 0 ? a0 + i * max_blocks : a0; e.v[2] = c0;
+                e.v[3] = rows_per_unit == 2 ? u + nu : -1; e.v[4] = c1 > 0 ? a1 + i * max_blocks : a1; e.v[5] = c1;
+                e.v[6] = slot_of_unit[u]++; e.v[7] = s;
+                per_seg[s].push_back(e);
+            }
+        }
+    for (int u = 0; u < nu; ++u) nslots = std::max(nslots, slot_of_unit[u]);
+    // a unit with no block at all (cannot happen after carve, which keeps >= 1 block per row) still needs
+    // one entry so its output is written
+    for (int u = 0; u < nu; ++u)
+        if (slot_of_unit[u] == 0) {
+            Ent e = {{u, row_ptr[u], 0, rows_per_unit == 2 ? u + nu : -1,
+                      rows_per_unit == 2 ? row_ptr[u + nu] : 0, 0, 0, 0}};
+            per_seg[0].push_back(e);
+        }
+    int64_t total = 0;
+    for (int s = 0; s < nseg; ++s) total += ((int64_t)per_seg[s].size() + 3) / 4 * 4;   // workgroup = 4 entries
+    if (nslots_out) *nslots_out = nslots;
+    if (row_slots_out)
+        for (int u = 0; u < nu; ++u) {
+            row_slots_out[u] = std::max(1, slot_of_unit[u]);
+            if (rows_per_unit == 2) row_slots_out[u + nu] = row_slots_out[u];
+        }
+    if (!entries_out) return total;
+    int64_t o = 0;
+    for (int s = 0; s < nseg; ++s) {
+        for (const Ent &e : per_seg[s]) { memcpy(entries_out + o * 8, e.v, 32); ++o; }
+        while (o % 4) {
+            const int32_t nul[8] = {-1, 0, 0, -1, 0, 0, 0, s};
+            memcpy(entries_out + o * 8, nul, 32);
+            ++o;
+        }
+    }
+    return total;
+}

@@ -1,0 +1,71 @@
+"""Decode-side callers of the carved MLP: the reference engine's MLP subset
+(morph/inference/engine.py:307-332,367-431,936-994) and its kernel entry points
+(mortar_pack_strips / mortar_gemv, morph/kernels/triton/fused_decode_step.py:1465-1547)."""
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from . import ops
+from .pack import MortarPack
+
+
+def mortar_pack_strips(cms) -> MortarPack:
+    """One-time engine pack of a pack_mortar_ternary'd CMSBlockLinear.  The reference returns the tuple
+    (strips, col_idx, offsets, scale, out_features, ent, nspl_max, cnts); here the device format and the
+    work lists live in one MortarPack (``.codes``, ``.col``, ``.row_ptr``, ``.sdup``, ``.out_features``,
+    ``.worklist(...)``)."""
+    return cms.mortar_pack()
+
+
+def mortar_gemv(x: Tensor, pack: MortarPack, swiglu_x: bool = False, swiglu_out: bool = False,
+                row_act: Tensor | None = None, col_act: Tensor | None = None, gates: Tensor | None = None,
+                cluster_size: int = 0) -> Tensor:
+    """x [B, I] row-contiguous -> [B, O], or [B, O/2] = silu(g)*u with swiglu_out (the gate_up call).
+    Same keywords as the reference; activations are bf16 on this path (fp32 input is rounded to bf16 and the
+    result returned as fp32, the reference engine's dtype)."""
+    if swiglu_x:
+        raise NotImplementedError("swiglu_x (SwiGLU on load) is superseded by swiglu_out on the gate_up call")
+    if gates is not None and cluster_size and (pack.out_features // 2) // gates.shape[-1] != cluster_size:
+        raise ValueError("cluster_size does not match d_ff / n_clusters")
+    xb = x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16)
+    y = ops.gemv(xb, pack, swiglu_out=swiglu_out, gates=gates, row_act=row_act, col_act=col_act)
+    return y if x.dtype == torch.bfloat16 else y.to(x.dtype)
+
+
+class MortarDecodeMLP:
+    """The engine's ``_mlp_fn`` MORTAR branch for one block: rmsnorm -> [router gates -> gather flags] ->
+    gate_up GEMV with fused SwiGLU/gates -> down GEMV.  Packs are built once at construction."""
+
+    def __init__(self, mlp, norm_weight: Tensor | None = None, eps: float = 1e-6, iter_idx: int = 0):
+        self.mlp = mlp
+        self.Mgu = mortar_pack_strips(mlp.gate_up._cms)
+        self.Mdown = mortar_pack_strips(mlp.down._cms)
+        self.norm_weight, self.eps, self.iter_idx = norm_weight, eps, iter_idx
+        self.d_ff = mlp.d_ff
+
+    @torch.no_grad()
+    def __call__(self, x: Tensor, gates: Tensor | None = None) -> Tensor:
+        B = x.shape[0]
+        xn = ops.rmsnorm(x.reshape(B, -1).to(torch.bfloat16), self.norm_weight, self.eps)
+        rt = getattr(self.mlp, "router", None)
+        if gates is None and rt is not None:
+            gates = rt(xn, iter_idx=self.iter_idx)[0].reshape(B, -1).float().contiguous()
+        if gates is not None:
+            ract, cact = ops.route_flags(gates, self.d_ff)
+            h = ops.gemv(xn, self.Mgu, swiglu_out=True, gates=gates, row_act=ract)
+            return ops.gemv(h, self.Mdown, col_act=cact).view(B, 1, -1)
+        h = ops.gemv(xn, self.Mgu, swiglu_out=True)
+        return ops.gemv(h, self.Mdown).view(B, 1, -1)
+
+
+@torch.no_grad()
+def looped_core_forward(mlps, x: Tensor, n_iters: int, norm_weights=None, eps: float = 1e-6) -> Tensor:
+    """Core-loop call pattern (morph/model/transformer.py:685-728,1146-1169) reduced to the MLP path:
+    n_iters passes over the shared blocks, the same weights every pass, iter_idx = t forwarded to each MLP,
+    activations RMS-normalised before every MLP (mhc.py:249-250)."""
+    for t in range(n_iters):
+        for i, m in enumerate(mlps):
+            w = norm_weights[i] if norm_weights is not None else None
+            x = m(ops.rmsnorm(x, w, eps), iter_idx=t)
+    return x

@@ -1,0 +1,133 @@
+"""SwiGLU MLP host for the carved path: _SwiGLUMortar / _KwargSequential / _make_swiglu.
+
+Interface mirror of morph/model/transformer.py:259-431.  Once gate_up and down are carved and ternary, the
+forward is two HIP launches: gate_up with the SwiGLU (and the per-cluster router gates) fused into its
+epilogue, then down.  Before carving the layers run their dense forward.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from . import ops
+from .pack import PREFILL_MT
+from .sparsity import MortarLinear
+
+DECODE_MAX_ROWS = 64       # flattened rows up to which the decode GEMV kernels serve the MLP
+
+
+class _KwargSequential(nn.Sequential):
+    """nn.Sequential that forwards **kwargs (iter_idx) to its first child; children keep indices "0"/"1"."""
+
+    def forward(self, x, **kwargs):
+        it = iter(self)
+        x = next(it)(x, **kwargs)
+        for m in it:
+            x = m(x)
+        return x
+
+    def enable_routing(self, *args, **kwargs):
+        return self[0].enable_routing(*args, **kwargs)
+
+    @property
+    def router(self):
+        return getattr(self[0], "router", None)
+
+    @property
+    def d_ff(self):
+        return self[0].d_ff
+
+
+def _make_swiglu(d_model: int, d_ff: int, dropout: float) -> nn.Module:
+    mlp: nn.Module = _SwiGLUMortar(d_model, d_ff)
+    if dropout > 0:
+        return _KwargSequential(mlp, nn.Dropout(dropout))
+    return mlp
+
+
+class _SwiGLUMortar(nn.Module):
+    def __init__(self, d_model: int, d_ff: int):
+        super().__init__()
+        self.gate_up = MortarLinear(d_model, d_ff * 2, bias=False, initial_density=1.0)
+        self.down = MortarLinear(d_ff, d_model, bias=False, initial_density=1.0)
+        self.d_model, self.d_ff = d_model, d_ff
+        self.router: nn.Module | None = None
+        self._last_aux_loss: Tensor | None = None
+        self._aux_detach_input = True
+        self.route_skip = True       # skip inactive (token, block-row) tiles when the cluster size allows
+
+    def enable_routing(self, n_clusters: int = 16, activation_ratio: float = 0.5, aux_loss_coeff: float = 1e-2,
+                       n_iters: int = 1, n_sub_keys: int = 0, detach_input: bool = True) -> None:
+        """Attach an iteration-aware TileRouter over the d_ff hidden neuron bank (transformer.py:344-400)."""
+        self._aux_detach_input = bool(detach_input)
+        from .routing import TileRouter
+        try:
+            dev = next(self.down.parameters()).device
+        except StopIteration:
+            dev = next(self.down.buffers()).device
+        self.router = TileRouter(n_tile_groups=n_clusters, d_model=self.d_model, activation_ratio=activation_ratio,
+                                 n_sub_keys=n_sub_keys, aux_loss_coeff=aux_loss_coeff, n_iters=n_iters).to(dev)
+        self.n_clusters = n_clusters
+        base, rem = self.d_ff // n_clusters, self.d_ff % n_clusters
+        sizes = torch.tensor([base + (1 if c < rem else 0) for c in range(n_clusters)])
+        self.register_buffer("hidden_to_cluster", torch.repeat_interleave(torch.arange(n_clusters), sizes).to(dev))
+
+    def _carved(self) -> bool:
+        return self.gate_up._cms._mortar and self.down._cms._mortar
+
+    def forward(self, x: Tensor, iter_idx: int = 0, gates: Tensor | None = None) -> Tensor:
+        """x [..., d_model] -> [..., d_model].  ``gates`` overrides the router output (fp32 [N, n_clusters]);
+        it exists so that a caller which already evaluated the router (or holds seeded logits) can feed it."""
+        if not self._carved():
+            gu = self.gate_up(x)
+            gate, up = gu.chunk(2, dim=-1)
+            h = F.silu(gate) * up
+            if self.router is not None or gates is not None:
+                if gates is None:
+                    gates, aux = self.router(x.detach() if self._aux_detach_input else x, iter_idx=iter_idx)
+                    self._last_aux_loss = aux
+                g = gates.to(h.dtype).reshape(*h.shape[:-1], -1)
+                ncl = g.shape[-1]
+                if self.d_ff % ncl == 0:
+                    h = (h.unflatten(-1, (ncl, self.d_ff // ncl)) * g.unsqueeze(-1)).flatten(-2)
+                else:
+                    h = h * g[..., self.hidden_to_cluster]
+            return self.down(h)
+
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, self.d_model)
+        xb = x2 if x2.dtype == torch.bfloat16 else x2.to(torch.bfloat16)
+        Wgu, Wdn = self.gate_up._cms.mortar_pack(), self.down._cms.mortar_pack()
+        active = None
+        if gates is None and self.router is not None:
+            rx = x2.detach() if self._aux_detach_input else x2
+            g3, aux = self.router(rx, iter_idx=iter_idx)
+            self._last_aux_loss = aux
+            gates = g3.reshape(-1, g3.shape[-1]).float().contiguous()
+            active = self.router.last_active
+        elif gates is not None:
+            gates = gates.reshape(-1, gates.shape[-1]).float().contiguous()
+        if gates is not None and self.d_ff % gates.shape[-1]:
+            raise ValueError("the carved MLP needs equal-size clusters (d_ff % n_clusters == 0)")
+        N = xb.shape[0]
+        if 0 < N <= DECODE_MAX_ROWS:
+            ract = cact = None
+            if gates is not None:
+                ract, cact = ops.route_flags(gates, self.d_ff)
+            h = ops.gemv(xb, Wgu, swiglu_out=True, gates=gates, row_act=ract)
+            y = ops.gemv(h, Wdn, col_act=cact)
+        else:
+            cs = self.d_ff // gates.shape[-1] if gates is not None else 0
+            if gates is not None and self.route_skip and cs % 16 == 0:
+                if active is None:
+                    active = (gates > 0).to(torch.uint8)
+                route = ops.remoe_route(active, PREFILL_MT)
+                h = ops.gateup_swiglu(xb, Wgu, gates=gates, route=route)
+                y = ops.spmm(h, Wdn, active=active)
+            else:
+                h = ops.gateup_swiglu(xb, Wgu, gates=gates)
+                y = ops.spmm(h, Wdn)
+        if y.dtype != x.dtype:
+            y = y.to(x.dtype)
+        return y.reshape(*lead, self.d_model)

@@ -1,0 +1,205 @@
+"""Operator-level entry points: the reference's sparse-backend and decode-kernel call signatures, served by
+the HIP library.  Every function requires tensors on a ROCm device; there is no CPU path."""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from .pack import BLK, PREFILL_MT, MortarPack
+
+
+def _stream(t: Tensor):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _need_gpu(t: Tensor, what: str):
+    if not t.is_cuda:
+        raise RuntimeError(f"{what}: tensor must live on a ROCm device (the MORTAR runtime has no CPU path)")
+
+
+def _bf16_2d(x: Tensor, what: str) -> Tensor:
+    _need_gpu(x, what)
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"{what}: expected bfloat16, got {x.dtype}")
+    if x.dim() != 2:
+        raise ValueError(f"{what}: expected a 2-D tensor")
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    return x
+
+
+def _p(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+# ----------------------------------------------------------------------------- prefill
+
+
+def spmm(x: Tensor, W: MortarPack, out: Tensor | None = None, active: Tensor | None = None) -> Tensor:
+    """y[M, out] = x[M, in] @ W^T, bf16 -> bf16, fp32 accumulate.  ``active`` (uint8 [M, n_clusters]) zeroes
+    the input elements of inactive clusters on load."""
+    x = _bf16_2d(x, "spmm")
+    M = x.shape[0]
+    if x.shape[1] != W.in_features:
+        raise ValueError(f"spmm: x has {x.shape[1]} features, matrix expects {W.in_features}")
+    y = out if out is not None else torch.empty((M, W.out_features), dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return y
+    L = _lib.lib()
+    order = W.unit_order(1)
+    if active is None:
+        rc = L.mortar_spmm_bf16(C.byref(W.struct), _p(W.chunk_ptr), _p(order), _p(x), M, x.stride(0), _p(y),
+                                y.stride(0), _stream(x))
+    else:
+        if active.dtype != torch.uint8 or not active.is_contiguous():
+            raise TypeError("spmm: active must be a contiguous uint8 tensor")
+        rc = L.mortar_spmm_bf16_masked(C.byref(W.struct), _p(W.chunk_ptr), _p(order), _p(x), M, x.stride(0), _p(y),
+                                       y.stride(0), _p(active), active.shape[1], _stream(x))
+    _lib.check(rc, "mortar_spmm_bf16")
+    return y
+
+
+def gateup_swiglu(x: Tensor, W: MortarPack, gates: Tensor | None = None, route: tuple | None = None,
+                  out: Tensor | None = None) -> Tensor:
+    """h[M, d_ff] = silu(gate) * up [* gates per cluster] with gate_up = W [2*d_ff, d_model].
+    route = (tok_cnt, tok_list) from remoe_route switches on active-tile skipping."""
+    x = _bf16_2d(x, "gateup_swiglu")
+    M = x.shape[0]
+    d_ff = W.out_features // 2
+    if x.shape[1] != W.in_features:
+        raise ValueError(f"gateup_swiglu: x has {x.shape[1]} features, matrix expects {W.in_features}")
+    h = out if out is not None else torch.empty((M, d_ff), dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return h
+    ncl = 0
+    if gates is not None:
+        if gates.dtype != torch.float32 or gates.dim() != 2 or not gates.is_contiguous() or gates.shape[0] != M:
+            raise TypeError("gateup_swiglu: gates must be a contiguous float32 [M, n_clusters] tensor")
+        ncl = gates.shape[1]
+    cnt, lst = route if route is not None else (None, None)
+    rc = _lib.lib().mortar_gateup_swiglu_bf16(C.byref(W.struct), _p(W.chunk_ptr), _p(W.unit_order(2)), _p(x), M,
+                                              x.stride(0), _p(h), h.stride(0), _p(gates), ncl, _p(cnt), _p(lst),
+                                              _stream(x))
+    _lib.check(rc, "mortar_gateup_swiglu_bf16")
+    return h
+
+
+# ----------------------------------------------------------------------------- ReMoE
+
+
+def remoe_gates(logits: Tensor, k: int) -> tuple[Tensor, Tensor]:
+    """(gates fp32 [M, n], active uint8 [M, n]) from fp32 logits: TileRouter.forward steps 5-8."""
+    _need_gpu(logits, "remoe_gates")
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise TypeError("remoe_gates: logits must be float32 [M, n]")
+    logits = logits.contiguous()
+    M, n = logits.shape
+    gates = torch.empty_like(logits)
+    active = torch.empty((M, n), dtype=torch.uint8, device=logits.device)
+    if M:
+        _lib.check(_lib.lib().mortar_remoe_gates(_p(logits), M, n, int(k), _p(gates), _p(active), _stream(logits)),
+                   "mortar_remoe_gates")
+    return gates, active
+
+
+def remoe_route(active: Tensor, tile: int = PREFILL_MT) -> tuple[Tensor, Tensor]:
+    """Per (token tile, cluster): count and ascending list of the tile-local indices of active tokens."""
+    _need_gpu(active, "remoe_route")
+    if active.dtype != torch.uint8 or active.dim() != 2 or not active.is_contiguous():
+        raise TypeError("remoe_route: active must be a contiguous uint8 [M, n] tensor")
+    M, n = active.shape
+    nt = -(-M // tile)
+    cnt = torch.empty((nt, n), dtype=torch.int32, device=active.device)
+    lst = torch.empty((nt, n, tile), dtype=torch.uint8, device=active.device)
+    _lib.check(_lib.lib().mortar_remoe_route(_p(active), M, n, tile, _p(cnt), _p(lst), _stream(active)),
+               "mortar_remoe_route")
+    return cnt, lst
+
+
+def route_flags(gates: Tensor, d_ff: int, row_act: Tensor | None = None, col_act: Tensor | None = None):
+    """Decode gather flags (reference route_flags with blk = 16): row_act int32 [B, 2*d_ff/16],
+    col_act int32 [B, d_ff/16]; out buffers may be sliced views of a wider scratch."""
+    _need_gpu(gates, "route_flags")
+    if gates.dtype != torch.float32 or gates.dim() != 2 or gates.stride(1) != 1:
+        raise TypeError("route_flags: gates must be float32 [B, n_clusters] with unit inner stride")
+    B, ncl = gates.shape
+    nc = d_ff // BLK
+    if row_act is None:
+        row_act = torch.empty((B, 2 * nc), dtype=torch.int32, device=gates.device)
+    if col_act is None:
+        col_act = torch.empty((B, nc), dtype=torch.int32, device=gates.device)
+    _lib.check(_lib.lib().mortar_route_flags(_p(gates), B, ncl, gates.stride(0), d_ff, _p(row_act), row_act.stride(0),
+                                             _p(col_act), col_act.stride(0), _stream(gates)), "mortar_route_flags")
+    return row_act, col_act
+
+
+# ----------------------------------------------------------------------------- decode
+
+
+def _kseg_for(W: MortarPack, B: int) -> int:
+    """Block-columns per K segment so that the staged activations fit in 64 KiB of LDS."""
+    mt = 16 if B <= 16 else (32 if B <= 32 else 64)
+    units = (64 * 1024) // ((mt + 1) * 16)        # 16-byte units = column halves
+    return max(2, min(W.Cb, units // 2))
+
+
+def gemv(x: Tensor, W: MortarPack, swiglu_out: bool = False, gates: Tensor | None = None,
+         row_act: Tensor | None = None, col_act: Tensor | None = None, max_blocks: int | None = None,
+         out: Tensor | None = None) -> Tensor:
+    """Decode GEMV for B <= 64 streams: y = x W^T (bf16), or with swiglu_out the fused silu(g)*u[*gates]."""
+    x = _bf16_2d(x, "gemv")
+    B = x.shape[0]
+    if not 1 <= B <= 64:
+        raise ValueError(f"gemv: batch {B} outside 1..64 (use the prefill path)")
+    if x.shape[1] != W.in_features:
+        raise ValueError(f"gemv: x has {x.shape[1]} features, matrix expects {W.in_features}")
+    rpu = 2 if swiglu_out else 1
+    kseg = _kseg_for(W, B)
+    if max_blocks is None:
+        max_blocks = 1 << 20                       # whole row (per segment) in one entry
+    ent, nslots, row_slots, _ = W.worklist(rpu, kseg, max_blocks)
+    nout = W.out_features // 2 if swiglu_out else W.out_features
+    y = out if out is not None else torch.empty((B, nout), dtype=torch.bfloat16, device=x.device)
+    part = None
+    if nslots > 1:
+        part = torch.empty((nslots, B, W.out_features), dtype=torch.float32, device=x.device)
+    ncl, ldg = 0, 0
+    if gates is not None:
+        if gates.dtype != torch.float32 or gates.stride(1) != 1:
+            raise TypeError("gemv: gates must be float32 with unit inner stride")
+        ncl, ldg = gates.shape[1], gates.stride(0)
+    for f in (row_act, col_act):
+        if f is not None and (f.dtype != torch.int32 or f.stride(1) != 1):
+            raise TypeError("gemv: row_act / col_act must be int32 with unit inner stride")
+    rc = _lib.lib().mortar_gemv_bf16(
+        C.byref(W.struct), _p(ent), ent.shape[0], nslots, _p(row_slots), kseg, 1 if swiglu_out else 0,
+        _p(x), B, x.stride(0), _p(y), y.stride(0), _p(part), _p(gates), ncl, ldg,
+        _p(row_act), row_act.stride(0) if row_act is not None else 0,
+        _p(col_act), col_act.stride(0) if col_act is not None else 0, _stream(x))
+    _lib.check(rc, "mortar_gemv_bf16")
+    return y
+
+
+# ----------------------------------------------------------------------------- RMSNorm
+
+
+def rmsnorm(x: Tensor, weight: Tensor | None = None, eps: float = 1e-6) -> Tensor:
+    """bf16 RMSNorm over the last dim (attention.RMSNorm semantics: normalise in fp32, cast, scale)."""
+    _need_gpu(x, "rmsnorm")
+    shp = x.shape
+    x2 = x.reshape(-1, shp[-1])
+    if x2.dtype != torch.bfloat16:
+        raise TypeError("rmsnorm: expected bfloat16")
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    w = None
+    if weight is not None:
+        w = weight.to(torch.bfloat16).contiguous()
+    y = torch.empty_like(x2, memory_format=torch.contiguous_format)
+    if x2.shape[0]:
+        _lib.check(_lib.lib().mortar_rmsnorm_bf16(_p(x2), x2.shape[0], shp[-1], x2.stride(0), _p(w), float(eps), _p(y),
+                                                  y.stride(0), _stream(x)), "mortar_rmsnorm_bf16")
+    return y.reshape(shp)

@@ -1,0 +1,135 @@
+"""Device-side weight format of one carved matrix, built once from the reference's carve output.
+
+Counterpart of the reference's one-time engine re-pack (mortar_pack_strips,
+morph/kernels/triton/fused_decode_step.py:1465-1499): the ternary codes keep their BCSR order, the
+reference's ``mortar_column_indices`` (int16) and ``mortar_offsets`` (int32) are uploaded unchanged, and
+only the bit layout inside each block-row dword and the scale pattern are device specific.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import _lib
+
+BLK = 16
+PREFILL_KCB = 14
+PREFILL_MT = 128
+
+
+def _np(a, dtype):
+    if isinstance(a, torch.Tensor):
+        a = a.detach().cpu().numpy()
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def _vp(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def encode_blocks(packed, nnz: int, scale) -> tuple[np.ndarray, np.ndarray]:
+    """Reference flat 2-bit pack + scale(s) -> (device code dwords [nnz*16] uint32, scale patterns [nnz] uint32)."""
+    packed = _np(packed, np.uint8).reshape(-1)
+    if packed.size < nnz * 64:
+        raise ValueError(f"packed codes hold {packed.size} bytes, need {nnz * 64}")
+    scale = _np(scale, np.float32).reshape(-1)
+    codes = np.empty(nnz * 16, dtype=np.uint32)
+    sdup = np.empty(nnz, dtype=np.uint32)
+    _lib.check(_lib.lib().mortar_encode_blocks_host(_vp(packed), nnz, _vp(scale), scale.size, _vp(codes), _vp(sdup)),
+               "mortar_encode_blocks_host")
+    return codes, sdup
+
+
+def decode_blocks(codes: np.ndarray) -> np.ndarray:
+    codes = _np(codes, np.uint32).reshape(-1)
+    nnz = codes.size // 16
+    out = np.empty((nnz, 16, 16), dtype=np.int8)
+    _lib.check(_lib.lib().mortar_decode_blocks_host(_vp(codes), nnz, _vp(out)), "mortar_decode_blocks_host")
+    return out
+
+
+def chunk_ptr(offsets, col, Rb: int, Cb: int, kcb: int = PREFILL_KCB) -> np.ndarray:
+    offsets, col = _np(offsets, np.int32), _np(col, np.int16)
+    nkc = -(-Cb // kcb)
+    out = np.empty((Rb, nkc + 1), dtype=np.int32)
+    _lib.check(_lib.lib().mortar_chunk_ptr_host(_vp(offsets), _vp(col), Rb, Cb, kcb, _vp(out)), "mortar_chunk_ptr_host")
+    return out
+
+
+def unit_order(offsets, Rb: int, rows_per_unit: int) -> np.ndarray:
+    offsets = _np(offsets, np.int32)
+    group = _lib.lib().mortar_prefill_group(1 if rows_per_unit == 2 else 0)
+    out = np.empty(Rb // rows_per_unit, dtype=np.int32)
+    _lib.check(_lib.lib().mortar_unit_order_host(_vp(offsets), Rb, rows_per_unit, group, _vp(out)), "mortar_unit_order_host")
+    return out
+
+
+def decode_worklist(offsets, col, Rb: int, Cb: int, rows_per_unit: int, kseg: int, max_blocks: int):
+    """-> (entries [E, 8] int32, nslots, row_slots [Rb] int32).  See mortar_decode_worklist_host."""
+    offsets, col = _np(offsets, np.int32), _np(col, np.int16)
+    L = _lib.lib()
+    ns = C.c_int32(0)
+    n = _lib.check(L.mortar_decode_worklist_host(_vp(offsets), _vp(col), Rb, Cb, rows_per_unit, kseg, max_blocks,
+                                                 None, C.byref(ns), None), "mortar_decode_worklist_host")
+    ent = np.empty((n, 8), dtype=np.int32)
+    row_slots = np.empty(Rb, dtype=np.int32)
+    _lib.check(L.mortar_decode_worklist_host(_vp(offsets), _vp(col), Rb, Cb, rows_per_unit, kseg, max_blocks,
+                                             _vp(ent), C.byref(ns), _vp(row_slots)), "mortar_decode_worklist_host")
+    return ent, int(ns.value), row_slots
+
+
+class MortarPack:
+    """One carved matrix W [out, in] resident on a device, plus its cached schedules.
+
+    Built from the reference's buffers: ``packed`` = mortar_packed (flat 2-bit codes over [nnz,16,16]),
+    ``scale`` = mortar_scale (scalar) or a per-block fp32 vector, ``col`` = mortar_column_indices,
+    ``offsets`` = mortar_offsets.
+    """
+
+    def __init__(self, packed, scale, col, offsets, out_features: int, in_features: int, device):
+        if out_features % BLK or in_features % BLK:
+            raise ValueError(f"[{out_features},{in_features}] not divisible by blocking {BLK}")
+        self.out_features, self.in_features = int(out_features), int(in_features)
+        self.Rb, self.Cb = out_features // BLK, in_features // BLK
+        self.h_offsets = _np(offsets, np.int32).reshape(-1)
+        self.h_col = _np(col, np.int16).reshape(-1)
+        if self.h_offsets.size != self.Rb + 1:
+            raise ValueError(f"offsets has {self.h_offsets.size} entries, expected {self.Rb + 1}")
+        self.nnz = int(self.h_offsets[-1])
+        if self.h_col.size != self.nnz:
+            raise ValueError(f"column_indices has {self.h_col.size} entries, offsets say {self.nnz}")
+        if (np.diff(self.h_offsets) <= 0).any():
+            raise RuntimeError("carved matrix has a block-row with zero kept blocks")
+        self.device = torch.device(device)
+        codes, sdup = encode_blocks(packed, self.nnz, scale)
+        self.h_chunk_ptr = chunk_ptr(self.h_offsets, self.h_col, self.Rb, self.Cb)      # also validates the BCSR
+        dev = self.device
+        self.codes = torch.from_numpy(codes.view(np.int32)).to(dev)
+        self.sdup = torch.from_numpy(sdup.view(np.int32)).to(dev)
+        self.col = torch.from_numpy(self.h_col).to(dev)
+        self.row_ptr = torch.from_numpy(self.h_offsets).to(dev)
+        self.chunk_ptr = torch.from_numpy(self.h_chunk_ptr).to(dev)
+        self._orders: dict[int, torch.Tensor] = {}
+        self._worklists: dict[tuple, tuple] = {}
+        self.struct = _lib.BcsrStruct(self.codes.data_ptr(), self.sdup.data_ptr(), self.col.data_ptr(),
+                                      self.row_ptr.data_ptr(), self.Rb, self.Cb, self.nnz)
+
+    def unit_order(self, rows_per_unit: int) -> torch.Tensor:
+        if rows_per_unit not in self._orders:
+            o = unit_order(self.h_offsets, self.Rb, rows_per_unit)
+            self._orders[rows_per_unit] = torch.from_numpy(o).to(self.device)
+        return self._orders[rows_per_unit]
+
+    def worklist(self, rows_per_unit: int, kseg: int, max_blocks: int):
+        key = (rows_per_unit, kseg, max_blocks)
+        if key not in self._worklists:
+            ent, ns, rs = decode_worklist(self.h_offsets, self.h_col, self.Rb, self.Cb, rows_per_unit, kseg, max_blocks)
+            self._worklists[key] = (torch.from_numpy(ent).to(self.device), ns, torch.from_numpy(rs).to(self.device), ent)
+        return self._worklists[key]
+
+    @property
+    def weight_bytes(self) -> int:
+        """Algorithmic weight-side bytes: 64 B codes + 4 B scale + 2 B column id per block + 4 B per row pointer."""
+        return self.nnz * 70 + 4 * (self.Rb + 1)

@@ -1,0 +1,297 @@
+"""GPU parity: the HIP path, called through the C-ABI, against the CPU oracle on the same seeded inputs.
+Indexing and tile selection are compared bit-exactly; bf16 outputs to max relative error 1e-2."""
+import numpy as np
+import pytest
+import torch
+
+import mortar_amd
+from mortar_amd import ops, synth
+from oracle import mortar_oracle as O
+from util import assert_close_bf16, oracle_spmm, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+# ---------------------------------------------------------------------------------------------- prefill SpMM
+
+def test_c0_single_spmm(dev):
+    """BASELINE config 0: x 64x768, W 768->2048, 25 % uniform, ternary p=(.3,.4,.3), scale U(.01,.1)."""
+    m = synth.synth_matrix(2048, 768, 0.25, seed=100)
+    x = synth.synth_x(64, 768, seed=101)
+    W = synth.to_pack(m, dev)
+    for fn in (ops.spmm, ops.gemv):
+        y = to_np(fn(to_dev(x, dev), W))
+        assert_close_bf16(y, oracle_spmm(x, m), fn.__name__)
+
+
+@pytest.mark.parametrize("M", [1, 15, 16, 17, 100, 128, 129, 300])
+def test_spmm_ragged_m(dev, M):
+    m = synth.synth_matrix(16 * 10, 16 * 20, 0.3, seed=M)
+    x = synth.synth_x(M, 320, seed=M + 1)
+    y = to_np(ops.spmm(to_dev(x, dev), synth.to_pack(m, dev)))
+    assert_close_bf16(y, oracle_spmm(x, m), f"M={M}")
+
+
+@pytest.mark.parametrize("shape,density,zipf", [((16, 16), 1.0, None), ((16 * 3, 16 * 29), 0.1, None),
+                                                 ((16 * 37, 16 * 15), 1.0, None), ((16 * 40, 16 * 60), 0.25, 1.2),
+                                                 ((16 * 5, 16 * 352), 0.25, 1.2)])
+def test_spmm_shapes(dev, shape, density, zipf):
+    m = synth.synth_matrix(shape[0], shape[1], density, seed=7, zipf_s=zipf)
+    x = synth.synth_x(200, shape[1], seed=8)
+    y = to_np(ops.spmm(to_dev(x, dev), synth.to_pack(m, dev)))
+    assert_close_bf16(y, oracle_spmm(x, m), str(shape))
+
+
+def test_spmm_exact_cases(dev):
+    # identity blocks, power-of-two scales: the result is an exact scaled block permutation of x
+    perm = np.array([2, 0, 3, 1], np.int16)
+    m = dict(codes=np.tile(np.eye(16, dtype=np.int8), (4, 1, 1)), scales=np.array([0.5, 0.25, 2.0, 1.0], np.float32),
+             col_idx=perm, row_idx=np.arange(4, dtype=np.int16), offsets=np.arange(5, dtype=np.int32), shape=(64, 64))
+    x = synth.synth_x(40, 64, 3)
+    y = to_np(ops.spmm(to_dev(x, dev), synth.to_pack(m, dev)))
+    for r in range(4):
+        assert np.array_equal(y[:, 16 * r:16 * r + 16], m["scales"][r] * x[:, 16 * perm[r]:16 * perm[r] + 16])
+    # negative identity and every single (n, c) position of a block: catches any unpack bit-position slip
+    for n, c, sgn in [(n, c, s) for n in (0, 5, 15) for c in range(16) for s in (1, -1)]:
+        codes = np.zeros((1, 16, 16), np.int8); codes[0, n, c] = sgn
+        m1 = dict(codes=codes, scales=np.array([1.0], np.float32), col_idx=np.zeros(1, np.int16),
+                  row_idx=np.zeros(1, np.int16), offsets=np.array([0, 1], np.int32), shape=(16, 16))
+        xx = synth.synth_x(16, 16, 5)
+        yy = to_np(ops.spmm(to_dev(xx, dev), synth.to_pack(m1, dev)))
+        want = np.zeros((16, 16), np.float32); want[:, n] = sgn * xx[:, c]
+        assert np.array_equal(yy, want), (n, c, sgn)
+
+
+def test_spmm_noncontiguous_input_and_errors(dev):
+    m = synth.synth_matrix(64, 128, 0.5, 1)
+    W = synth.to_pack(m, dev)
+    x = synth.synth_x(50, 256, 2)
+    xt = to_dev(x, dev)[:, ::2]                                   # strided view -> made contiguous by the wrapper
+    assert_close_bf16(to_np(ops.spmm(xt, W)), oracle_spmm(np.ascontiguousarray(x[:, ::2]), m))
+    with pytest.raises(ValueError):
+        ops.spmm(to_dev(x, dev), W)                               # wrong feature count
+    with pytest.raises(TypeError):
+        ops.spmm(to_dev(x[:, :128], dev).float(), W)
+
+
+def test_stk_dds_operator_signature(dev):
+    m = synth.synth_matrix(128, 96, 0.5, 11)
+    data = torch.from_numpy(O.effective_blocks(m["codes"], m["scales"])).to(torch.bfloat16).to(dev)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    z16, z32 = torch.zeros(1, dtype=torch.int16, device=dev), torch.zeros(1, dtype=torch.int32, device=dev)
+    x = synth.synth_x(70, 96, 12)
+    y = mortar_amd.stk_dds(to_dev(x, dev), data, t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32,
+                           96, 128, True)
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (70, 128)
+    assert_close_bf16(to_np(y), oracle_spmm(x, m))
+    with pytest.raises(ValueError, match="int16"):
+        mortar_amd.stk_dds(to_dev(x, dev), data, t(m["offsets"]), t(m["row_idx"]).int(), t(m["col_idx"]), z32, z16, z32, 96, 128, True)
+    with pytest.raises(ValueError, match="ternary"):
+        mortar_amd.stk_dds(to_dev(x, dev), torch.randn_like(data), t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32, 96, 128, True)
+
+
+# ---------------------------------------------------------------------------------------------- SwiGLU MLP
+
+@pytest.mark.parametrize("M", [64, 200])
+def test_mlp_base_config_slice(dev, M):
+    """BASELINE config 1 shapes (d_model 768, d_ff 2048) on a token slice the oracle finishes quickly."""
+    spec = synth.synth_mlp(768, 2048, 0.25, seed=20)
+    x = synth.synth_x(M, 768, 21)
+    ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
+    Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    h = ops.gateup_swiglu(to_dev(x, dev), Wgu)
+    assert_close_bf16(to_np(h), ref["h"], "h", ulps=4)
+    y = ops.spmm(h, Wdn)
+    assert_close_bf16(to_np(y), ref["y"], "y", ulps=8)
+    mlp = synth.mlp_module(spec, dev)
+    y2 = mlp(to_dev(x, dev).reshape(2, M // 2, 768))
+    assert tuple(y2.shape) == (2, M // 2, 768) and y2.dtype == torch.bfloat16
+    assert torch.equal(y2.reshape(M, 768), y) or M <= 64          # same kernels for M > 64
+    assert_close_bf16(to_np(y2).reshape(M, 768), ref["y"], "module", ulps=8)
+
+
+def test_mlp_with_gates_and_skip(dev):
+    """ReMoE-routed MLP: cluster size 16 (one block-row per cluster), k-th threshold gating, tile skipping."""
+    d_model, d_ff, M, ncl, k = 256, 16 * 40, 300, 40, 10
+    spec = synth.synth_mlp(d_model, d_ff, 0.3, seed=30)
+    x = synth.synth_x(M, d_model, 31)
+    logits = synth.synth_logits(M, ncl, 32)
+    g_ref, act_ref = O.remoe_gates(logits, k)
+    ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=g_ref)
+    gates, active = ops.remoe_gates(torch.from_numpy(logits).to(dev), k)
+    assert np.array_equal(active.cpu().numpy().astype(bool), act_ref)           # tile selection bit-exact
+    np.testing.assert_allclose(gates.cpu().numpy(), g_ref, rtol=2e-6, atol=0)
+    Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    xd = to_dev(x, dev)
+    h_dense = ops.gateup_swiglu(xd, Wgu, gates=gates)
+    assert_close_bf16(to_np(h_dense), ref["h"], "h gated", ulps=4)
+    cnt, lst = ops.remoe_route(active)
+    h_skip = torch.full_like(h_dense, float("nan"))                             # untouched entries stay NaN
+    ops.gateup_swiglu(xd, Wgu, gates=gates, route=(cnt, lst), out=h_skip)
+    hs, hd = to_np(h_skip), to_np(h_dense)
+    on = np.repeat(act_ref, 16, axis=1)
+    assert np.array_equal(hs[on], hd[on]) and np.isnan(hs[~on]).all()           # exactly the active tiles written
+    y = ops.spmm(h_skip, Wdn, active=active)
+    assert_close_bf16(to_np(y), ref["y"], "y routed", ulps=8)
+    mlp = synth.mlp_module(spec, dev)
+    y2 = mlp(xd, gates=gates)
+    assert torch.equal(y2, y)
+
+
+def test_remoe_route_lists_exact(dev):
+    rng = np.random.default_rng(40)
+    act = (rng.random((333, 70)) < 0.25).astype(np.uint8)
+    act[:128, 3] = 0; act[128:256, 5] = 1
+    cnt, lst = ops.remoe_route(torch.from_numpy(act).to(dev), 128)
+    cnt, lst = cnt.cpu().numpy(), lst.cpu().numpy()
+    for t in range(3):
+        for c in range(70):
+            want = np.nonzero(act[t * 128:(t + 1) * 128, c])[0]
+            assert cnt[t, c] == len(want) and np.array_equal(lst[t, c, :len(want)], want)
+
+
+def test_remoe_gates_ties_and_edges(dev):
+    rng = np.random.default_rng(41)
+    for n, k in ((8, 3), (16, 8), (352, 88), (100, 100), (65, 1), (1024, 256)):
+        lg = rng.integers(-3, 4, size=(257, n)).astype(np.float32)
+        lg[0] = 1.0; lg[1, 0] = -0.0; lg[1, 1] = 0.0
+        g_ref, a_ref = O.remoe_gates(lg, k)
+        g, a = ops.remoe_gates(torch.from_numpy(lg).to(dev), k)
+        assert np.array_equal(a.cpu().numpy().astype(bool), a_ref), (n, k)
+        np.testing.assert_allclose(g.cpu().numpy(), g_ref, rtol=3e-6, atol=0)
+    lg = synth.synth_logits(4096, 352, 42)                                      # BASELINE config 3 router
+    g_ref, a_ref = O.remoe_gates(lg, 88)
+    g, a = ops.remoe_gates(torch.from_numpy(lg).to(dev), 88)
+    assert np.array_equal(a.cpu().numpy().astype(bool), a_ref) and (a_ref.sum(1) == 87).all()
+    with pytest.raises(ValueError):
+        ops.remoe_gates(torch.zeros(2, 2000, device=dev), 5)
+
+
+def test_route_flags_exact(dev):
+    for ncl, d_ff in ((352, 5632), (16, 2048), (256, 2048), (44, 5632)):
+        lg = synth.synth_logits(5, ncl, ncl)
+        gates, _ = O.remoe_gates(lg, max(1, ncl // 4))
+        r_ref, c_ref = O.route_flags(gates, d_ff)
+        scratch = torch.zeros(5, 1024, dtype=torch.int32, device=dev)           # sliced scratch, as the engine does
+        r, c = ops.route_flags(torch.from_numpy(gates).to(dev), d_ff, row_act=scratch[:, :2 * d_ff // 16])
+        assert np.array_equal(r.cpu().numpy(), r_ref) and np.array_equal(c.cpu().numpy(), c_ref)
+
+
+# ---------------------------------------------------------------------------------------------- decode
+
+@pytest.mark.parametrize("B", [1, 4, 16, 17, 64])
+def test_decode_mlp_cloud_width(dev, B):
+    """BASELINE config 2: d_model 2048, d_ff 5632, batch of single-token rows."""
+    spec = synth.synth_mlp(2048, 5632, 0.25, seed=50)
+    x = synth.synth_x(B, 2048, 51 + B)
+    ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
+    Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    h = ops.gemv(to_dev(x, dev), Wgu, swiglu_out=True)
+    assert_close_bf16(to_np(h), ref["h"], "h", ulps=4)
+    y = ops.gemv(h, Wdn)
+    assert_close_bf16(to_np(y), ref["y"], "y", ulps=8)
+    gu = ops.gemv(to_dev(x, dev), Wgu)                                           # plain mode on gate_up
+    assert_close_bf16(to_np(gu), ref["gu"], "gu")
+
+
+@pytest.mark.parametrize("max_blocks", [3, 8])
+def test_decode_split_rows_partials(dev, max_blocks):
+    spec = synth.synth_mlp(512, 16 * 90, 0.3, seed=60, zipf_s=1.2)
+    x = synth.synth_x(5, 512, 61)
+    ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
+    Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    h = ops.gemv(to_dev(x, dev), Wgu, swiglu_out=True, max_blocks=max_blocks)
+    assert_close_bf16(to_np(h), ref["h"], "h", ulps=4)
+    y = ops.gemv(h, Wdn, max_blocks=max_blocks)
+    assert_close_bf16(to_np(y), ref["y"], "y", ulps=8)
+    h1 = ops.gemv(to_dev(x, dev), Wgu, swiglu_out=True)
+    assert_close_bf16(to_np(h), to_np(h1), "split vs whole", ulps=2)
+
+
+@pytest.mark.parametrize("B", [1, 3])
+def test_decode_routed(dev, B):
+    d_model, d_ff, ncl, k = 512, 16 * 64, 64, 16
+    spec = synth.synth_mlp(d_model, d_ff, 0.3, seed=70)
+    x = synth.synth_x(B, d_model, 71)
+    g_ref, _ = O.remoe_gates(synth.synth_logits(B, ncl, 72), k)
+    ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=g_ref)
+    gates = torch.from_numpy(g_ref).to(dev)
+    mlp = synth.mlp_module(spec, dev)
+    y = mlp(to_dev(x, dev), gates=gates)
+    assert_close_bf16(to_np(y), ref["y"], "routed decode", ulps=8)
+    dec = mortar_amd.MortarDecodeMLP(mlp)
+    xr = O.rmsnorm(x)
+    ref2 = O.swiglu_mlp(xr, spec["gate_up"], spec["down"], gates=g_ref)
+    y2 = dec(to_dev(x, dev).reshape(B, 1, d_model), gates=gates)
+    assert tuple(y2.shape) == (B, 1, d_model)
+    assert_close_bf16(to_np(y2).reshape(B, d_model), ref2["y"], "engine mlp_fn", ulps=8)
+
+
+def test_mortar_gemv_reference_signature(dev):
+    spec = synth.synth_mlp(256, 512, 0.5, seed=80)
+    mlp = synth.mlp_module(spec, dev)
+    pk = mortar_amd.mortar_pack_strips(mlp.gate_up._cms)
+    x = synth.synth_x(2, 256, 81)
+    h = mortar_amd.mortar_gemv(torch.from_numpy(x).to(dev), pk, swiglu_out=True)      # fp32 in -> fp32 out
+    assert h.dtype == torch.float32
+    ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
+    assert_close_bf16(h.cpu().numpy(), ref["h"], "h", ulps=4)
+    with pytest.raises(NotImplementedError):
+        mortar_amd.mortar_gemv(torch.from_numpy(x).to(dev), pk, swiglu_x=True)
+
+
+def test_rmsnorm(dev):
+    x = synth.synth_x(37, 2048, 90) * 3
+    w = synth.synth_x(1, 2048, 91)[0]
+    y = ops.rmsnorm(to_dev(x, dev), to_dev(w, dev))
+    assert_close_bf16(to_np(y), O.rmsnorm(x, w), "rmsnorm", ulps=2)
+    y = ops.rmsnorm(to_dev(x, dev).reshape(37, 1, 2048))
+    assert_close_bf16(to_np(y).reshape(37, 2048), O.rmsnorm(x), "rmsnorm unit weight", ulps=2)
+
+
+def test_looped_core_stack_small(dev):
+    """BASELINE config 4 call pattern at reduced size: shared blocks x iterations, RMS-normalised input, Zipf rows."""
+    d_model, d_ff, M = 256, 16 * 44, 150
+    specs = [synth.synth_mlp(d_model, d_ff, 0.25, seed=200 + i, zipf_s=1.2) for i in range(2)]
+    x = synth.synth_x(M, d_model, 210)
+    ref = x
+    for t in range(3):
+        for s in specs:
+            ref = O.swiglu_mlp(O.rmsnorm(ref), s["gate_up"], s["down"])["y"]
+    mlps = [synth.mlp_module(s, dev) for s in specs]
+    y = mortar_amd.looped_core_forward(mlps, to_dev(x, dev), 3)
+    assert_close_bf16(to_np(y), ref, "looped stack", ulps=64, max_rel=2e-2)
+
+
+# ---------------------------------------------------------------------------------------------- full size, by properties
+
+def test_full_size_properties(dev):
+    """BASELINE config 3 shapes (d_model 2048, d_ff 5632, 4096 tokens): size-independent checks.
+    (1) rows sampled from the prefill output equal the oracle on those rows; (2) prefill and decode kernels
+    agree on the same rows; (3) linearity in a power-of-two scale is exact."""
+    spec = synth.synth_mlp(2048, 5632, 0.25, seed=300)
+    Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    x = synth.synth_x(4096, 2048, 301)
+    xd = to_dev(x, dev)
+    h = ops.gateup_swiglu(xd, Wgu)
+    y = ops.spmm(h, Wdn)
+    rows = np.array([0, 1, 127, 128, 2047, 4095, 1234, 3071])
+    ref = O.swiglu_mlp(x[rows], spec["gate_up"], spec["down"])
+    assert_close_bf16(to_np(h)[rows], ref["h"], "h rows", ulps=4)
+    assert_close_bf16(to_np(y)[rows], ref["y"], "y rows", ulps=8)
+    hd = ops.gemv(xd[rows], Wgu, swiglu_out=True)
+    assert_close_bf16(to_np(hd), to_np(h)[rows], "decode vs prefill h", ulps=2)
+    gu = ops.spmm(xd, Wgu)
+    gu4 = ops.spmm(xd * 4, Wgu)
+    assert torch.equal(gu4.float(), gu.float() * 4)
+    # routed, full size: selection bit-exact and sampled rows against the oracle
+    lg = synth.synth_logits(4096, 352, 302)
+    g_ref, a_ref = O.remoe_gates(lg, 88)
+    gates, active = ops.remoe_gates(torch.from_numpy(lg).to(dev), 88)
+    assert np.array_equal(active.cpu().numpy().astype(bool), a_ref)
+    cnt, lst = ops.remoe_route(active)
+    assert int(cnt.sum()) == int(a_ref.sum())
+    hr = ops.gateup_swiglu(xd, Wgu, gates=gates, route=(cnt, lst))
+    yr = ops.spmm(hr, Wdn, active=active)
+    refr = O.swiglu_mlp(x[rows], spec["gate_up"], spec["down"], gates=g_ref[rows])
+    assert_close_bf16(to_np(yr)[rows], refr["y"], "routed y rows", ulps=8)

@@ -1,0 +1,213 @@
+"""CPU tests of the host logic: C-ABI exports, device-format encoding, schedules, module state (no GPU compute)."""
+import ctypes
+import itertools
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import mortar_amd
+from mortar_amd import _lib, pack as P, synth
+from oracle import mortar_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    hdr = open(os.path.join(ROOT, "include", "mortar_hip.h")).read()
+    code = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)                       # declarations only, not comments
+    declared = set(re.findall(r"\b(mortar_[a-z0-9_]+)\s*\(", code))
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in mortar_hip.h but not exported"
+    assert declared == set(_lib.EXPORTS)
+    assert _lib.lib().mortar_abi_version() == 1
+
+
+def test_encode_round_trip_and_bit_layout():
+    rng = np.random.default_rng(0)
+    codes = rng.integers(-1, 2, (9, 16, 16)).astype(np.int8)
+    scale = rng.uniform(0.01, 0.1, 9).astype(np.float32)
+    dw, sdup = P.encode_blocks(O.pack_ternary_codes(codes), 9, scale)
+    assert np.array_equal(P.decode_blocks(dw), codes)
+    # the pair (2i, 2i+1) of column half h is isolated by (w << 8h << 2i) & 0xC000C000: bit 15/31 sign, 14/30 non-zero
+    for j, n, h, i in itertools.product((0, 8), (0, 7, 15), (0, 1), range(4)):
+        w = int(dw[j * 16 + n])
+        f = ((w << (8 * h + 2 * i)) & 0xFFFFFFFF) & 0xC000C000
+        for half, c in ((0, 8 * h + 2 * i), (1, 8 * h + 2 * i + 1)):
+            bits = (f >> (16 * half + 14)) & 3
+            assert {0: 0, 1: 1, 3: -1}[bits] == codes[j, n, c]
+    # scale pattern: bf16 bits minus one 16-bit-float exponent step, in both halves
+    s16 = O.bf16_bits(scale).astype(np.uint32) - 0x400
+    assert np.array_equal(sdup, s16 | (s16 << 16))
+    # multiplying the pattern (as 16-bit floats) by +-2 gives +-bf16(scale) bit-exactly
+    half = (sdup & 0xFFFF).astype(np.uint16).view(np.float16)
+    for sign in (2.0, -2.0):
+        prod = (half.astype(np.float32) * np.float32(sign)).astype(np.float16).view(np.uint16)
+        want = O.bf16_bits(scale) | (0x8000 if sign < 0 else 0)
+        assert np.array_equal(prod, want)
+
+
+def test_encode_scalar_scale_and_errors():
+    codes = np.ones((2, 16, 16), np.int8)
+    dw, sdup = P.encode_blocks(O.pack_ternary_codes(codes), 2, np.float32(0.05))
+    assert sdup[0] == sdup[1]
+    with pytest.raises(ValueError, match="outside"):
+        P.encode_blocks(O.pack_ternary_codes(codes), 2, np.float32(1e38))
+    with pytest.raises(ValueError, match="outside"):
+        P.encode_blocks(O.pack_ternary_codes(codes), 2, np.float32(float("inf")))
+    with pytest.raises(ValueError, match="scale_count"):
+        P.encode_blocks(O.pack_ternary_codes(codes), 2, np.ones(3, np.float32))
+    bad = O.pack_ternary_codes(codes).copy(); bad[5] = 0xFF
+    with pytest.raises(ValueError, match="invalid 2-bit code"):
+        P.encode_blocks(bad, 2, np.float32(1.0))
+    dw0, sd0 = P.encode_blocks(O.pack_ternary_codes(codes), 2, np.float32(0.0))     # zero scale zeroes the block
+    assert not dw0.any() and not sd0.any()
+
+
+def test_chunk_ptr_partitions_rows():
+    m = synth.synth_matrix(16 * 9, 16 * 50, 0.3, 3, zipf_s=1.2)
+    cp = P.chunk_ptr(m["offsets"], m["col_idx"], 9, 50, 14)
+    assert cp.shape == (9, 5)
+    for r in range(9):
+        assert cp[r, 0] == m["offsets"][r] and cp[r, -1] == m["offsets"][r + 1]
+        for c in range(4):
+            cols = m["col_idx"][cp[r, c]:cp[r, c + 1]]
+            assert ((cols >= c * 14) & (cols < (c + 1) * 14)).all()
+    bad = m["col_idx"].copy(); bad[1] = bad[0]
+    with pytest.raises(ValueError, match="ascending"):
+        P.chunk_ptr(m["offsets"], bad, 9, 50, 14)
+
+
+def test_unit_order_is_balanced_permutation():
+    m = synth.synth_matrix(16 * 64, 16 * 40, 0.25, 4, zipf_s=1.2)
+    for rpu in (1, 2):
+        o = P.unit_order(m["offsets"], 64, rpu)
+        nu = 64 // rpu
+        assert sorted(o.tolist()) == list(range(nu))
+        cost = np.diff(m["offsets"])
+        if rpu == 2:
+            cost = cost[:nu] + cost[nu:]
+        group = _lib.lib().mortar_prefill_group(rpu == 2)
+        loads = [cost[o[g:g + group]].sum() for g in range(0, nu, group)]
+        naive = [cost[g:g + group].sum() for g in range(0, nu, group)]
+        assert max(loads) <= max(naive)
+    u = synth.synth_matrix(16 * 8, 16 * 8, 0.25, 5)
+    assert P.unit_order(u["offsets"], 8, 1).tolist() == list(range(8))             # uniform rows keep natural order
+
+
+@pytest.mark.parametrize("rpu,kseg,mb", [(1, 1000, 1 << 20), (2, 1000, 1 << 20), (1, 7, 3), (2, 16, 4)])
+def test_decode_worklist_covers_every_block_once(rpu, kseg, mb):
+    m = synth.synth_matrix(16 * 12, 16 * 40, 0.3, 6, zipf_s=1.2)
+    ent, nslots, row_slots = P.decode_worklist(m["offsets"], m["col_idx"], 12, 40, rpu, kseg, mb)
+    assert ent.shape[0] % 4 == 0
+    seen = np.zeros(m["offsets"][-1], int)
+    slots = {}
+    for g in range(0, len(ent), 4):
+        assert len({e[7] for e in ent[g:g + 4]}) == 1                                  # one segment per workgroup
+    for e in ent:
+        if e[0] < 0:
+            continue
+        for row, p, c in ((e[0], e[1], e[2]), (e[3], e[4], e[5])):
+            if row < 0:
+                continue
+            assert c <= mb and m["offsets"][row] <= p and p + c <= m["offsets"][row + 1]
+            cols = m["col_idx"][p:p + c]
+            assert ((cols >= e[7] * kseg) & (cols < (e[7] + 1) * kseg)).all()
+            seen[p:p + c] += 1
+        slots.setdefault(e[0], []).append(e[6])
+        if rpu == 2:
+            assert e[3] == e[0] + 6
+    assert (seen == 1).all()
+    for u, s in slots.items():
+        assert sorted(s) == list(range(len(s))) and row_slots[u] == len(s)
+    assert nslots == max(len(s) for s in slots.values())
+
+
+def test_module_carve_matches_oracle_layout():
+    torch.manual_seed(0)
+    lin = mortar_amd.MortarLinear(16 * 6, 16 * 5, bias=False)
+    rng = np.random.default_rng(7)
+    mask = rng.random((5, 6)) < 0.5
+    mask[np.arange(5), rng.integers(0, 6, 5)] = True
+    w = lin._cms.weight.detach().numpy().copy()
+    lin._cms.set_block_mask(torch.from_numpy(mask), 16)
+    nnz = lin.carve(16)
+    c = O.carve(w, mask, 16)
+    assert nnz == mask.sum() and lin.is_compact
+    sd = lin.state_dict()
+    for k in ("mortar_data", "mortar_row_indices", "mortar_column_indices", "mortar_offsets",
+              "mortar_column_indices_t", "mortar_offsets_t", "mortar_block_offsets_t"):
+        assert np.array_equal(sd["_cms." + k].numpy(), c[k]), k
+        assert sd["_cms." + k].numpy().dtype == c[k].dtype
+    assert "_cms.mortar_ternary" in sd
+    with pytest.raises(AssertionError):
+        lin.carve(16)
+
+
+def test_pack_mortar_ternary_and_state_dict_round_trip():
+    torch.manual_seed(1)
+    lin = mortar_amd.MortarLinear(64, 48, bias=False)
+    info = mortar_amd.shrink_mlp_to_mortar_ternary(lin, 0.5, 16, generator=torch.Generator().manual_seed(3))
+    cms = lin._cms
+    assert type(cms).__name__ == "CMSBlockLinear" and cms._mortar and cms._packed_shape == (info["nnz"], 16, 16)
+    assert cms.mortar_packed.dtype == torch.uint8 and cms.mortar_packed.numel() == info["nnz"] * 64
+    eff = cms._mortar_effective_data().float()
+    mags = eff.abs()[eff != 0].unique()
+    assert len(mags) == 1 and torch.isclose(mags[0], cms.mortar_scale.to(torch.bfloat16).float())
+    # oracle quantiser agrees
+    lin2 = mortar_amd.MortarLinear(64, 48, bias=False)
+    lin2.load_state_dict(lin.state_dict())
+    assert lin2._cms._mortar and torch.equal(lin2._cms.mortar_packed, cms.mortar_packed)
+    assert lin2._cms._packed_shape == cms._packed_shape
+    # per-block variant
+    lin3 = mortar_amd.MortarLinear(64, 48, bias=False)
+    mortar_amd.shrink_mlp_to_mortar_ternary(lin3, 0.5, 16, per_block=True)
+    assert lin3._cms.mortar_scale.shape == (lin3._cms._packed_shape[0],)
+
+
+def test_quantize_mirror_matches_oracle():
+    from mortar_amd.deploy_quant import _ternary_quantize, _ternary_quantize_per_block
+    w = torch.randn(7, 16, 16, generator=torch.Generator().manual_seed(2))
+    q, s = _ternary_quantize(w)
+    qo, so = O.ternary_quantize(w.numpy())
+    assert np.array_equal(q.numpy(), qo) and np.isclose(float(s), so, rtol=1e-6)
+    q, s = _ternary_quantize_per_block(w)
+    qo, so = O.ternary_quantize_per_block(w.numpy())
+    assert np.array_equal(q.numpy(), qo) and np.allclose(s.numpy(), so, rtol=1e-6)
+    assert np.array_equal(mortar_amd.pack_ternary_codes(q).numpy(), O.pack_ternary_codes(qo))
+    assert np.array_equal(synth.flat_pack(qo), O.pack_ternary_codes(qo))
+
+
+def test_product_fails_loudly_without_gpu_or_library(monkeypatch):
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    m = synth.synth_matrix(32, 64, 0.5, 0)
+    W = synth.to_pack(m, "cpu")
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mortar_amd.ops.spmm(x, W)
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libmortar_hip.so")
+    with pytest.raises(RuntimeError, match="has not been built"):
+        _lib.lib()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "morph-orchestrates-recursive-pruned-hierarchies_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".cpp", ".h")):
+                assert "oracle" not in open(os.path.join(dirpath, f)).read().lower(), f
+
+
+def test_synth_generators_are_deterministic_and_shaped():
+    a, b = synth.synth_matrix(2048, 768, 0.25, 1), synth.synth_matrix(2048, 768, 0.25, 1)
+    assert all(np.array_equal(a[k], b[k]) for k in ("codes", "scales", "col_idx", "offsets"))
+    assert a["offsets"][-1] == 1536 and (np.diff(a["offsets"]) == 12).all()
+    frac = [(a["codes"] == v).mean() for v in (-1, 0, 1)]
+    assert np.allclose(frac, [0.3, 0.4, 0.3], atol=0.01)
+    z = synth.synth_matrix(16 * 128, 16 * 352, 0.25, 2, zipf_s=1.2)
+    cnt = np.diff(z["offsets"])
+    assert cnt.min() >= round(0.05 * 352) and cnt.max() <= round(0.60 * 352)
+    assert abs(cnt.mean() / 352 - 0.25) < 0.02 and cnt.std() > 10

@@ -1,0 +1,286 @@
+"""Pins the CPU oracle WITHOUT the reference: closed forms, brute force, library routines, invariants.
+Each check is chosen so that a plausible mistake (dropped term, wrong index, transposed operand) fails."""
+import itertools
+
+import numpy as np
+import pytest
+
+from oracle import c_oracle
+from oracle import mortar_oracle as O
+
+
+def rand_case(Rb, Cb, density, seed, blk=16):
+    rng = np.random.default_rng(seed)
+    mask = rng.random((Rb, Cb)) < density
+    mask[np.arange(Rb), rng.integers(0, Cb, Rb)] = True
+    w = rng.standard_normal((Rb * blk, Cb * blk)).astype(np.float32)
+    return w, mask
+
+
+# ---- carve -------------------------------------------------------------------------------------------
+
+def test_carve_layout_closed_form():
+    w, mask = rand_case(5, 7, 0.4, 0)
+    c = O.carve(w, mask, 16)
+    # row-major nonzero order, int16/int32 dtypes, offsets = exclusive cumsum (block_sparse.py:874-883)
+    rows, cols = np.nonzero(mask)
+    assert c["mortar_row_indices"].dtype == np.int16 and c["mortar_column_indices"].dtype == np.int16
+    assert c["mortar_offsets"].dtype == np.int32
+    assert np.array_equal(c["mortar_row_indices"], rows) and np.array_equal(c["mortar_column_indices"], cols)
+    assert np.array_equal(c["mortar_offsets"], np.concatenate([[0], np.cumsum(mask.sum(1))]))
+    # element order inside a block: data[j, lr, c] = W[row*blk+lr, col*blk+c] -- checked element by element
+    for j in (0, len(rows) // 2, len(rows) - 1):
+        for lr, cc in ((0, 0), (3, 11), (15, 15), (7, 2)):
+            assert c["mortar_data"][j, lr, cc] == w[rows[j] * 16 + lr, cols[j] * 16 + cc]
+
+
+def test_carve_scatter_round_trip():
+    w, mask = rand_case(6, 9, 0.3, 1)
+    c = O.carve(w, mask, 16)
+    dense = O.to_dense(c["mortar_data"], c["mortar_row_indices"], c["mortar_column_indices"], w.shape, 16)
+    expect = w * np.kron(mask, np.ones((16, 16), dtype=np.float32))
+    assert np.array_equal(dense, expect)
+
+
+def test_carve_errors():
+    w, mask = rand_case(4, 4, 0.5, 2)
+    mask[2, :] = False
+    with pytest.raises(RuntimeError):
+        O.carve(w, mask, 16)
+    with pytest.raises(ValueError):
+        O.carve(w[:-1], mask, 16)
+
+
+def test_transpose_meta_invariants():
+    w, mask = rand_case(6, 5, 0.5, 3)
+    c = O.carve(w, mask, 16)
+    ct, ot, bt = c["mortar_column_indices_t"], c["mortar_offsets_t"], c["mortar_block_offsets_t"]
+    assert np.array_equal(ot, np.concatenate([[0], np.cumsum(mask.sum(0))]))
+    assert sorted(bt.tolist()) == list(range(mask.sum()))                      # a permutation of the blocks
+    for col in range(5):
+        js = bt[ot[col]:ot[col + 1]]
+        assert (c["mortar_column_indices"][js] == col).all()
+        assert np.array_equal(ct[ot[col]:ot[col + 1]], c["mortar_row_indices"][js])
+
+
+# ---- ternary / pack ----------------------------------------------------------------------------------
+
+def test_ternary_quantize_rule():
+    w = np.array([0.0, 0.49, 0.5, 0.51, -0.5, -0.51, 2.0, -3.0], dtype=np.float32)
+    w = w * np.float32(1.0) / np.abs(w).mean() * np.float32(1.0)            # mean|w| == 1 -> thresholds are |w| > 0.5
+    q, s = O.ternary_quantize(w)
+    wn = w / s
+    assert np.array_equal(q, (np.sign(wn) * (np.abs(wn) > 0.5)).astype(np.int8))
+    assert q[2 if abs(wn[2]) <= 0.5 else 0] == 0                             # strict >
+    # invariant of tests/test_lifecycle_tst_qat.py:100-105: every non-zero effective weight has one magnitude
+    eff = q.astype(np.float32) * s
+    assert len(np.unique(np.abs(eff[eff != 0]))) == 1
+    assert O.ternary_quantize(np.zeros(8, np.float32))[1] == np.float32(1e-8)  # clamp
+
+
+def test_ternary_per_block_is_per_tensor_on_each_block():
+    rng = np.random.default_rng(4)
+    w = rng.standard_normal((5, 16, 16)).astype(np.float32)
+    q, s = O.ternary_quantize_per_block(w)
+    for j in range(5):
+        qj, sj = O.ternary_quantize(w[j])
+        assert np.array_equal(q[j], qj) and np.isclose(s[j], sj, rtol=1e-6)
+
+
+def test_pack_exhaustive_bytes():
+    # all 256 byte values: decode by definition (2 bits each, little-endian, minus one)
+    for b in range(256):
+        codes = O.unpack_ternary(np.array([b], dtype=np.uint8), 4)
+        assert codes.tolist() == [((b >> (2 * i)) & 3) - 1 for i in range(4)]
+    # all 81 valid quadruples round-trip, and the byte is u0 + 4*u1 + 16*u2 + 64*u3
+    for quad in itertools.product((-1, 0, 1), repeat=4):
+        p = O.pack_ternary_codes(np.array(quad, dtype=np.int8))
+        assert p.tolist() == [sum((c + 1) << (2 * i) for i, c in enumerate(quad))]
+        assert O.unpack_ternary(p, 4).tolist() == list(quad)
+    # padding to a multiple of four with stored value 0
+    assert O.pack_ternary_codes(np.array([1, 1, 1, 1, 1], np.int8)).tolist() == [0xAA, 0x02]
+
+
+def test_pack_strips_layout():
+    rng = np.random.default_rng(5)
+    codes = rng.integers(-1, 2, size=(3, 16, 16)).astype(np.int8)
+    s = O.pack_strips(codes)
+    assert s.shape == (3, 16, 4)
+    for j, lr, b in ((0, 0, 0), (1, 5, 3), (2, 15, 2)):
+        got = [((int(s[j, lr, b]) >> (2 * k)) & 3) - 1 for k in range(4)]
+        assert got == [codes[j, lr, b + 4 * k] for k in range(4)]            # columns {b, 4+b, 8+b, 12+b}
+
+
+def test_work_list_partitions_rows():
+    offsets = np.array([0, 3, 3 + 9, 12 + 4, 16 + 1], dtype=np.int32)
+    ent, nmax, cnts = O.work_list(offsets, cb=4)
+    assert cnts.tolist() == [1, 3, 1, 1] and nmax == 3
+    for r in range(4):
+        e = ent[:, ent[0] == r]
+        assert e[2].tolist() == list(range(cnts[r]))
+        assert e[1].tolist() == [offsets[r] + 4 * s for s in range(cnts[r])]
+
+
+# ---- SpMM ---------------------------------------------------------------------------------------------
+
+def make_mat(Rb, Cb, density, seed):
+    rng = np.random.default_rng(seed)
+    mask = rng.random((Rb, Cb)) < density
+    mask[np.arange(Rb), rng.integers(0, Cb, Rb)] = True
+    rows, cols = np.nonzero(mask)
+    nnz = len(rows)
+    return dict(codes=rng.integers(-1, 2, (nnz, 16, 16)).astype(np.int8),
+                scales=rng.uniform(0.01, 0.1, nnz).astype(np.float32),
+                col_idx=cols.astype(np.int16), row_idx=rows.astype(np.int16),
+                offsets=np.concatenate([[0], np.cumsum(mask.sum(1))]).astype(np.int32), shape=(Rb * 16, Cb * 16))
+
+
+def xbf(M, K, seed):
+    return O.bf16_round(np.random.default_rng(seed).standard_normal((M, K)).astype(np.float32))
+
+
+def test_spmm_equals_dense_scatter_matmul():
+    m = make_mat(7, 9, 0.35, 10)
+    x = xbf(13, 9 * 16, 11)
+    y = O.bcsr_spmm(x, m["codes"], m["scales"], m["col_idx"], m["offsets"], round_out=False)
+    W = O.to_dense(m["codes"].astype(np.float64) * O.bf16_round(m["scales"]).astype(np.float64)[:, None, None],
+                   m["row_idx"], m["col_idx"], m["shape"])
+    ref = x.astype(np.float64) @ W.T                                          # library routine, W not transposed twice
+    assert np.allclose(y, ref, rtol=1e-6, atol=1e-6)
+    # a transposed block (data[j,c,n] instead of data[j,n,c]) must NOT pass
+    bad = O.bcsr_spmm(x, m["codes"].transpose(0, 2, 1), m["scales"], m["col_idx"], m["offsets"], round_out=False)
+    assert not np.allclose(bad, ref, rtol=1e-3, atol=1e-3)
+
+
+def test_spmm_special_cases():
+    rng = np.random.default_rng(12)
+    # density 1, scale 1 == dense GEMM with the ternary matrix
+    Rb, Cb = 3, 4
+    codes = rng.integers(-1, 2, (Rb * Cb, 16, 16)).astype(np.int8)
+    col = np.tile(np.arange(Cb), Rb).astype(np.int16)
+    row = np.repeat(np.arange(Rb), Cb).astype(np.int16)
+    off = (np.arange(Rb + 1) * Cb).astype(np.int32)
+    x = xbf(5, Cb * 16, 13)
+    W = O.to_dense(codes.astype(np.float32), row, col, (Rb * 16, Cb * 16))
+    y = O.bcsr_spmm(x, codes, np.float32(1.0), col, off, round_out=False)
+    assert np.allclose(y, x @ W.T, atol=1e-5)
+    # identity blocks on a block permutation: output block r == scale_r * input block perm[r]
+    perm = np.array([2, 0, 3, 1])
+    eye = np.tile(np.eye(16, dtype=np.int8), (4, 1, 1))
+    s = np.array([0.5, 0.25, 2.0, 1.0], np.float32)
+    y = O.bcsr_spmm(x, eye, s, perm.astype(np.int16), np.arange(5, dtype=np.int32), round_out=False)
+    for r in range(4):
+        assert np.allclose(y[:, r * 16:(r + 1) * 16], s[r] * x[:, perm[r] * 16:(perm[r] + 1) * 16])
+    # all-zero codes -> zeros ; scale rounded to bf16 (0.1 is not bf16-representable)
+    assert not O.bcsr_spmm(x, np.zeros_like(eye), s, perm.astype(np.int16), np.arange(5, dtype=np.int32)).any()
+    y01 = O.bcsr_spmm(x, eye[:1], np.float32(0.1), np.array([0], np.int16), np.array([0, 1], np.int32), round_out=False)
+    assert np.allclose(y01, O.bf16_round(np.float32(0.1)) * x[:, :16], rtol=1e-7)
+    assert not np.allclose(y01, np.float32(0.1) * x[:, :16], rtol=1e-5)
+
+
+def test_c_oracle_matches_numpy_oracle():
+    m = make_mat(8, 12, 0.3, 20)
+    x = xbf(9, 12 * 16, 21)
+    ynp = O.bcsr_spmm(x, m["codes"], m["scales"], m["col_idx"], m["offsets"])
+    yc = O.bf16_from_bits(c_oracle.bcsr_spmm_bf16(O.bf16_bits(x), m["codes"], m["scales"], m["col_idx"], m["offsets"]))
+    # fp32 vs float64 accumulation may flip a bf16 rounding: allow 1 ulp on < 1 % of entries
+    diff = np.abs(ynp - yc)
+    assert (diff <= np.abs(ynp) * 2 ** -7 + 1e-6).all()
+    assert (diff > 0).mean() < 0.01
+
+
+def test_swiglu_mlp_against_dense():
+    gu, dn = make_mat(2 * 6, 4, 0.5, 30), make_mat(4, 6, 0.5, 31)
+    x = xbf(11, 64, 32)
+    r = O.swiglu_mlp(x, gu, dn)
+    Wg = O.to_dense(O.effective_blocks(gu["codes"], gu["scales"]), gu["row_idx"], gu["col_idx"], gu["shape"])
+    g_u = O.bf16_round((x.astype(np.float64) @ Wg.astype(np.float64).T).astype(np.float32))
+    g, u = g_u[:, :96], g_u[:, 96:]
+    sig = 1.0 / (1.0 + np.exp(-g.astype(np.float64)))
+    h = O.bf16_round(O.bf16_round((g * sig).astype(np.float32)) * u)
+    assert np.array_equal(r["h"], h)
+    Wd = O.to_dense(O.effective_blocks(dn["codes"], dn["scales"]), dn["row_idx"], dn["col_idx"], dn["shape"])
+    y = O.bf16_round((h.astype(np.float64) @ Wd.astype(np.float64).T).astype(np.float32))
+    assert np.array_equal(r["y"], y)
+    # gates: per-cluster multiply; gate 0 kills the cluster, gate 1 leaves it
+    gates = np.zeros((11, 6), np.float32); gates[:, 1] = 1.0
+    rg = O.swiglu_mlp(x, gu, dn, gates=gates)
+    assert not rg["h"][:, :16].any() and np.array_equal(rg["h"][:, 16:32], h[:, 16:32]) and not rg["h"][:, 32:].any()
+    gc, hc, yc = c_oracle.mlp_bf16(O.bf16_bits(x), gu, dn, 96, gates=gates)
+    assert np.abs(O.bf16_from_bits(yc) - rg["y"]).max() <= np.abs(rg["y"]).max() * 2 ** -6
+
+
+def test_decode_gemv_form_equals_spmm_unrounded():
+    m = make_mat(5, 8, 0.4, 40)
+    # decode applies fp32 scales exactly; make them bf16-representable so both forms agree
+    m["scales"] = O.bf16_round(m["scales"])
+    x = xbf(3, 128, 41)
+    a = O.mortar_gemv(x, m["codes"], m["scales"], m["col_idx"], m["offsets"])
+    b = O.bcsr_spmm(x, m["codes"], m["scales"], m["col_idx"], m["offsets"], round_out=False)
+    assert np.allclose(a, b, rtol=1e-6, atol=1e-6)
+
+
+# ---- ReMoE ---------------------------------------------------------------------------------------------
+
+def brute_remoe(logits, k):
+    out = []
+    for row in logits:
+        n = len(row)
+        if k < n:
+            # k-th largest VALUE by counting: smallest v in row with #(row > v) < k
+            cands = [v for v in row if (row > v).sum() < k <= (row >= v).sum()]
+            kth = cands[0]
+            out.append(row > kth)
+        else:
+            out.append(row > 0)
+    return np.array(out)
+
+
+def test_remoe_brute_force_incl_ties():
+    rng = np.random.default_rng(50)
+    for n, k in ((8, 3), (16, 8), (6, 1), (5, 5), (7, 6)):
+        lg = rng.integers(-3, 4, size=(200, n)).astype(np.float32)            # many ties
+        lg[0, :] = 1.0                                                        # all equal -> nothing strictly above
+        gates, act = O.remoe_gates(lg, k)
+        assert np.array_equal(act, brute_remoe(lg, k))
+        gc, ac = c_oracle.remoe_gates(lg, k)
+        assert np.array_equal(ac, act) and np.allclose(gc, gates, rtol=1e-6)
+        if k < n:
+            assert (act.sum(1) <= k - 1).all() and not act[0].any()           # the k-th itself is inactive
+        assert (gates >= 0).all()
+        on = act.any(1)
+        assert np.allclose(gates[on].sum(1), k, rtol=1e-5)                     # normalised to sum k
+        assert (gates[~on] == 0).all()
+
+
+def test_remoe_distinct_logits_count():
+    lg = np.random.default_rng(51).standard_normal((64, 352)).astype(np.float32)
+    gates, act = O.remoe_gates(lg, 88)
+    assert (act.sum(1) == 87).all()
+    top = np.argsort(-lg, axis=1)[:, :87]
+    assert all(set(np.nonzero(act[i])[0]) == set(top[i]) for i in range(64))
+
+
+def test_route_flags_closed_form():
+    gates = np.zeros((2, 4), np.float32); gates[0, 1] = 0.5; gates[1, 3] = 2.0   # d_ff 128, 4 clusters of 32
+    ract, cact = O.route_flags(gates, 128, 16)
+    assert cact.tolist() == [[0, 0, 1, 1, 0, 0, 0, 0], [0, 0, 0, 0, 0, 0, 1, 1]]
+    assert ract.tolist() == [c + c for c in cact.tolist()]
+    g2 = np.zeros((1, 16), np.float32); g2[0, 3] = 1.0                           # clusters of 8: a block spans two
+    assert O.route_flags(g2, 128, 16)[1].tolist() == [[0, 1, 0, 0, 0, 0, 0, 0]]
+
+
+def test_rmsnorm_closed_form():
+    x = xbf(4, 64, 60)
+    y = O.rmsnorm(x, None, 1e-6, bf16_out=False)
+    assert np.allclose((y.astype(np.float64) ** 2).mean(1), 1.0, atol=1e-4)
+    assert np.allclose(y, x / np.sqrt((x.astype(np.float64) ** 2).mean(1, keepdims=True) + 1e-6), rtol=1e-5)
+    w = np.full(64, 2.0, np.float32)
+    assert np.allclose(O.rmsnorm(x, w, bf16_out=False), 2 * y)
+
+
+def test_bf16_round_matches_torch():
+    import torch
+    a = np.random.default_rng(70).standard_normal(10000).astype(np.float32) * 1e3
+    a[:4] = [0.1, 1.00390625, 1.005859375, -1.00390625]                           # ties-to-even cases
+    assert np.array_equal(O.bf16_round(a), torch.from_numpy(a).to(torch.bfloat16).float().numpy())
