@@ -1,0 +1,178 @@
+"""Benchmark of the MORTAR sparse-MLP path on one MI355X.
+
+Step = one pass of the carved SwiGLU MLP (gate_up with fused SwiGLU, then down) over one batch of synthetic
+tokens.  Workload at N=1: d_model 2048, d_ff 5632, 16x16 BCSR at 25 % block density, ternary codes with one
+fp32 scale per block, 4096-token prefill (the shapes of BASELINE.json configs 2/3).  The same run also times
+the decode GEMVs (batch 1/4/16/64), the ReMoE-routed prefill, and a bounded CPU baseline on the host cores.
+
+Prints ONE JSON line.  `value` = prefill tokens/s with inputs resident in HBM.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+D_MODEL, D_FF, DENSITY, TOKENS = 2048, 5632, 0.25, 4096
+N_CLUSTERS, TOP_K = 352, 88
+PEAK_BF16_TFLOPS, PEAK_HBM_GBS = 2500.0, 8000.0
+
+
+def event_time_ms(fn, iters: int, warmup: int = 2) -> float:
+    """Average duration of fn() measured with HIP events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
+def cpu_baseline(spec, sample_tokens: int) -> dict:
+    """The C restatement of the path (oracle, 'port') on the host cores over a bounded token sample."""
+    import numpy as np
+    from oracle import c_oracle, mortar_oracle as O
+    from mortar_amd import synth
+    x = O.bf16_bits(synth.synth_x(sample_tokens, D_MODEL, seed=999))
+    c_oracle.mlp_bf16(x[:8], spec["gate_up"], spec["down"], D_FF)            # warm caches / thread pool
+    t0 = time.perf_counter()
+    c_oracle.mlp_bf16(x, spec["gate_up"], spec["down"], D_FF)
+    dt = time.perf_counter() - t0
+    return {"value": sample_tokens / dt, "unit": "tokens/s", "cores": c_oracle.num_threads(), "kind": "port",
+            "sample": f"{sample_tokens} tokens of the same d{D_MODEL}/ff{D_FF} MLP, blockwise C BCSR (OpenMP), {dt:.2f} s"}
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="prefill only (for profiling one kernel)")
+    ap.add_argument("--cpu-tokens", type=int, default=2048)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the path shards by tokens with replicated weights; "
+                 "no multi-GPU code is part of it). Use --gpus 1.")
+
+    import torch
+    import mortar_amd
+    from mortar_amd import ops, synth
+
+    dev = torch.device("cuda:0")
+    spec = synth.synth_mlp(D_MODEL, D_FF, DENSITY, seed=0)
+    Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    x = torch.from_numpy(synth.synth_x(TOKENS, D_MODEL, seed=1)).to(torch.bfloat16).to(dev)
+    h = torch.empty((TOKENS, D_FF), dtype=torch.bfloat16, device=dev)
+    y = torch.empty((TOKENS, D_MODEL), dtype=torch.bfloat16, device=dev)
+
+    def step():
+        ops.gateup_swiglu(x, Wgu, out=h)
+        ops.spmm(h, Wdn, out=y)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    flops_gu = 2.0 * TOKENS * 256 * Wgu.nnz
+    flops_dn = 2.0 * TOKENS * 256 * Wdn.nnz
+    it = max(10, args.steps)
+    ms_gu = event_time_ms(lambda: ops.gateup_swiglu(x, Wgu, out=h), it)
+    ms_dn = event_time_ms(lambda: ops.spmm(h, Wdn, out=y), it)
+    out = {
+        "metric": "sparse-MLP prefill tokens/s @ d_model=2048, d_ff=5632, 25% block density, 4096 tokens",
+        "value": TOKENS / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "carved SwiGLU MLP prefill, d_model 2048 / d_ff 5632, 16x16 BCSR 25 % uniform, "
+                               "ternary + per-block scale, 4096 tokens bf16 (BASELINE configs 2/3 shapes)",
+                   "tokens": TOKENS, "nnz_blocks": [Wgu.nnz, Wdn.nnz]},
+        "effective_tflops": (flops_gu + flops_dn) / (ms * 1e-3) / 1e12,
+        "roofline": {"bound": "mfma", "kernel": "mortar_spmm_kernel<gate_up+swiglu>",
+                     "achieved": flops_gu / (ms_gu * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops_gu / (ms_gu * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
+                     "ms": ms_gu},
+        "roofline_down": {"bound": "mfma", "kernel": "mortar_spmm_kernel<plain>",
+                          "achieved": flops_dn / (ms_dn * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                          "frac": flops_dn / (ms_dn * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "ms": ms_dn},
+    }
+
+    if not args.no_extras:
+        # ---- decode: one MLP per call (2 launches), weights warm in cache --------------------------------
+        dec = {}
+        wbytes = Wgu.weight_bytes + Wdn.weight_bytes
+        for B in (1, 4, 16, 64):
+            xb = x[:B].contiguous()
+            hb = torch.empty((B, D_FF), dtype=torch.bfloat16, device=dev)
+            yb = torch.empty((B, D_MODEL), dtype=torch.bfloat16, device=dev)
+
+            def dstep():
+                ops.gemv(xb, Wgu, swiglu_out=True, out=hb)
+                ops.gemv(hb, Wdn, out=yb)
+            t = event_time_ms(dstep, 200, 20)
+            abytes = B * (2 * D_MODEL + 2 * D_FF) * 2
+            dec[f"b{B}"] = {"us_per_mlp": t * 1e3, "tokens_per_s": B / (t * 1e-3),
+                            "algorithmic_GBps": (wbytes + abytes) / (t * 1e-3) / 1e9}
+        out["decode_warm"] = dec
+        # ---- decode, cold: stream distinct weight sets so that the Infinity Cache cannot hold them --------
+        n_sets = 160                                                 # 160 x 2.37 MB = 379 MB > 256 MB
+        packs = []
+        for i in range(n_sets):
+            packs.append((Wgu, Wdn) if i == 0 else (Wgu.clone_weights(), Wdn.clone_weights()))
+        cold = {}
+        for B in (1, 16):
+            xb = x[:B].contiguous()
+            hb = torch.empty((B, D_FF), dtype=torch.bfloat16, device=dev)
+            yb = torch.empty((B, D_MODEL), dtype=torch.bfloat16, device=dev)
+
+            def sweep():
+                for g, d in packs:
+                    ops.gemv(xb, g, swiglu_out=True, out=hb)
+                    ops.gemv(hb, d, out=yb)
+            t = event_time_ms(sweep, 5, 1) / n_sets
+            abytes = B * (2 * D_MODEL + 2 * D_FF) * 2
+            gbps = (wbytes + abytes) / (t * 1e-3) / 1e9
+            cold[f"b{B}"] = {"us_per_mlp": t * 1e3, "tokens_per_s": B / (t * 1e-3), "algorithmic_GBps": gbps,
+                             "frac_hbm": gbps / PEAK_HBM_GBS}
+        out["decode_cold"] = cold
+        out["roofline_decode"] = {"bound": "hbm", "kernel": "mortar_gemv_kernel (per-MLP launches, cold weights)",
+                                  "achieved": cold["b1"]["algorithmic_GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                  "frac": cold["b1"]["frac_hbm"], "traffic": None}
+        # ---- ReMoE-routed prefill (BASELINE config 3) ----------------------------------------------------
+        logits = torch.from_numpy(synth.synth_logits(TOKENS, N_CLUSTERS, seed=2)).to(dev)
+
+        def routed():
+            gates, active = ops.remoe_gates(logits, TOP_K)
+            route = ops.remoe_route(active)
+            ops.gateup_swiglu(x, Wgu, gates=gates, route=route, out=h)
+            ops.spmm(h, Wdn, active=active, out=y)
+        t = event_time_ms(routed, it)
+        n_act = int(ops.remoe_gates(logits, TOP_K)[1].sum())
+        out["routed_prefill"] = {"ms": t, "tokens_per_s": TOKENS / (t * 1e-3),
+                                 "active_fraction": n_act / (TOKENS * N_CLUSTERS)}
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(spec, args.cpu_tokens)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -133,3 +133,15 @@ class MortarPack:
     def weight_bytes(self) -> int:
         """Algorithmic weight-side bytes: 64 B codes + 4 B scale + 2 B column id per block + 4 B per row pointer."""
         return self.nnz * 70 + 4 * (self.Rb + 1)
+
+    def clone_weights(self) -> "MortarPack":
+        """A second resident copy (own device buffers and schedules) of the same matrix."""
+        import copy
+        c = copy.copy(self)
+        for name in ("codes", "sdup", "col", "row_ptr", "chunk_ptr"):
+            setattr(c, name, getattr(self, name).clone())
+        c._orders = {k: v.clone() for k, v in self._orders.items()}
+        c._worklists = {k: (v[0].clone(), v[1], v[2].clone(), v[3]) for k, v in self._worklists.items()}
+        c.struct = _lib.BcsrStruct(c.codes.data_ptr(), c.sdup.data_ptr(), c.col.data_ptr(), c.row_ptr.data_ptr(),
+                                   c.Rb, c.Cb, c.nnz)
+        return c
