@@ -39,16 +39,19 @@ __device__ __forceinline__ f32x4_t mortar_mfma(u32x4_t a, u32x4_t b, f32x4_t c) 
                                                    __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
-__device__ __forceinline__ uint32_t bf16_bits_rne(float f) {
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+// fp32 -> bf16 (round to nearest even) through the hardware conversion (v_cvt_pk_bf16_f32).
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bf16_pack2(float lo, float hi) {
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+__device__ __forceinline__ uint32_t bf16_bits_rne(float f) { return bf16_pack2(f, 0.f) & 0xffffu; }
 __device__ __forceinline__ float bf16_to_f32(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
-__device__ __forceinline__ float bf16r(float f) { return bf16_to_f32(bf16_bits_rne(f)); }
+__device__ __forceinline__ float bf16r(float f) { return __builtin_bit_cast(float, bf16_pack2(0.f, f) & 0xffff0000u); }
 
-// silu in fp32 from a bf16-rounded input; the result is rounded to bf16 by the caller.
-__device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
+// silu in fp32 from a bf16-rounded input; the result is rounded to bf16 by the caller, which absorbs the
+// 1-ulp error of the hardware exp and reciprocal.
+__device__ __forceinline__ float silu_f32(float g) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)); }
 
 #endif

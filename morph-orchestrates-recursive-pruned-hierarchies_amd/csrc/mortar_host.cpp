@@ -156,7 +156,7 @@ extern "C" int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_
         load[best] += cost[u];
     }
     // inside a group the waves take consecutive runs; deal the sorted members across the runs
-    const int nw = 4, rw = std::max(1, group / nw);
+    const int nw = 4, rw = std::max(1, group / nw);   // 4 wavefronts per prefill workgroup
     for (int g = 0; g < ng; ++g) {
         const int n = (int)members[g].size();
         std::vector<int> placed(group, -1);

@@ -18,7 +18,7 @@
 namespace {
 
 constexpr int KCB = MORTAR_PREFILL_KCB;
-constexpr int NW = 4;
+constexpr int NW = 4;   // wavefronts per workgroup (one per SIMD, 512 registers each)
 
 struct SpmmParams {
     const uint32_t *codes;
@@ -41,18 +41,20 @@ struct SpmmParams {
 };
 
 template <int MSUB, int RW, int NACC, bool ROUTED, bool MASKED>
-__global__ void __launch_bounds__(256, 2) mortar_spmm_kernel(const SpmmParams p) {
-    constexpr int MT = 16 * MSUB, LDM = MT + 1, NA = RW * NACC;
-    constexpr int XUNITS = 2 * KCB * LDM;
-    constexpr int WDW = NA * KCB * 18;   // per wave: codes [NA*KCB*16] + scale [NA*KCB] + x offset [NA*KCB]
+__global__ void __launch_bounds__(NW * 64, 1) mortar_spmm_kernel(const SpmmParams p) {
+    constexpr int MT = 16 * MSUB, LDM = MT + 1, NA = RW * NACC, NT = NW * 64;
+    constexpr int XUNITS = 2 * KCB * LDM;                 // one activation buffer, in 16-byte units
+    constexpr int WBLK = NA * KCB + 4;                    // block slots in a wave's staging list (+ pads)
+    constexpr int WDW = WBLK * 18;                        // codes [WBLK*16] + scale [WBLK] + x offset [WBLK]
+    constexpr int NIT = (2 * KCB * MT + NT - 1) / NT;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    uint4 *lx = reinterpret_cast<uint4 *>(smem);
+    uint4 *lxbuf = reinterpret_cast<uint4 *>(smem);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
-    uint32_t *lwc = reinterpret_cast<uint32_t *>(smem + XUNITS * 16) + wave * WDW;
-    uint32_t *lws = lwc + NA * KCB * 16;
-    uint32_t *lwl = lws + NA * KCB;
+    uint32_t *lwc = reinterpret_cast<uint32_t *>(smem + 2 * XUNITS * 16) + wave * WDW;
+    uint32_t *lws = lwc + WBLK * 16;
+    uint32_t *lwl = lws + WBLK;
 
     // Workgroup -> (token tile, unit group).  Consecutive workgroup ids land on consecutive XCDs; with the
     // XCD map every workgroup that reads one token tile runs on the same XCD and shares its L2.
@@ -110,105 +112,185 @@ __global__ void __launch_bounds__(256, 2) mortar_spmm_kernel(const SpmmParams p)
 #pragma unroll
         for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int kc = 0; kc < p.nkc; ++kc) {
+    // Per-wave copy of the chunk pointer rows of its NA block-rows (read once; the table is then consulted
+    // from LDS so that no global round trip sits between the loads of a chunk).
+    int32_t *lcp = reinterpret_cast<int32_t *>(smem + 2 * XUNITS * 16 + NW * WDW * 4) + wave * NA * (p.nkc + 1);
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+        for (int c = lane; c <= p.nkc; c += 64)
+            lcp[a * (p.nkc + 1) + c] = rows[a] >= 0 ? p.chunk_ptr[(int64_t)rows[a] * (p.nkc + 1) + c] : 0;
+
+    // Registers that carry chunk kc+1 from global memory to LDS while chunk kc is being multiplied.
+    // Staging map: thread t < 2*KCB*8 owns column-half ch = t % (2*KCB) of rows r0 + 8*it, r0 = t / (2*KCB).
+    constexpr int RG = 8, NITX = MT / RG;
+    const bool stager = tid < 2 * KCB * RG;
+    const int ch = tid % (2 * KCB), r0 = tid / (2 * KCB);
+    const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;          // last valid token row of the tile
+    const bool full_tile = rlast == MT - 1;
+    const uint32_t ldxB = (uint32_t)p.ldx * 2u;
+    const char *xtile = reinterpret_cast<const char *>(p.x) + (int64_t)m0 * ldxB;
+    uint4 xv[NITX];
+    uint32_t xm[MASKED ? NITX : 1];
+    uint32_t wv[NA][4], wsd[NA];
+    int wcl[NA], nbn[NA], np[NA], nxt[NA], c0n = 0;
+
+    // All global loads of one chunk.  Addresses are clamped into the tensor instead of predicated: rows past
+    // M and columns past in_features receive copies of valid data that no block or output ever refers to.
+    auto load_chunk = [&](int kc) {
         const int c0 = kc * KCB;
-        __syncthreads();
-        // ---- issue every global load of this chunk first (token tile + this wave's blocks), with clamped
-        //      addresses so that no load sits behind a branch, then write LDS -----------------------------
-        int nb[NA];
-        uint32_t wv[NA][4], wsd[NA];
-        int wcl[NA];
+        c0n = c0;
+        if (stager) {
+            int cu = c0 * 2 + ch;
+            cu = cu < 2 * p.Cb ? cu : 2 * p.Cb - 1;
+            int clus = 0;
+            if (MASKED) clus = (cu * 8) / p.cluster_size;
+            if (full_tile) {
+                const uint32_t voff = (uint32_t)r0 * ldxB + (uint32_t)cu * 16u;
 #pragma unroll
-        for (int a = 0; a < NA; ++a) {
-            nb[a] = 0;
-            const int r = rows[a];
-            if (r >= 0 && (!ROUTED || cnt[a / NACC] > 0)) {
-                const int32_t *cp = p.chunk_ptr + (int64_t)r * (p.nkc + 1) + kc;
-                const int P0 = __builtin_amdgcn_readfirstlane(cp[0]);
-                const int P1 = __builtin_amdgcn_readfirstlane(cp[1]);
-                nb[a] = P1 - P0;
-                const int last = nb[a] > 0 ? nb[a] * 16 - 1 : 0;
-                const int64_t base = nb[a] > 0 ? (int64_t)P0 : 0;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int i = lane + 64 * k;
-                    wv[a][k] = p.codes[base * 16 + (i < last ? i : last)];
+                for (int it = 0; it < NITX; ++it) {
+                    xv[it] = *reinterpret_cast<const uint4 *>(xtile + (int64_t)(RG * it) * ldxB + voff);
+                    if (MASKED) xm[it] = p.active[(int64_t)(m0 + r0 + RG * it) * p.n_clusters + clus];
                 }
-                const int j = lane < nb[a] ? lane : 0;
-                wsd[a] = p.sdup[base + j];
-                wcl[a] = p.col[base + j];
-            }
-        }
-        // token tile in two batches of loads (bounds the registers held across the loads)
-        constexpr int NIT = (2 * KCB * MT + 255) / 256, NH = (NIT + 1) / 2;
+            } else {
 #pragma unroll
-        for (int hb = 0; hb < NIT; hb += NH) {
-            uint4 xv[NH];
-            bool xok[NH];
-#pragma unroll
-            for (int it = 0; it < NH; ++it) {
-                const int i = (hb + it) * 256 + tid;
-                const int ch = i % (2 * KCB), row = i / (2 * KCB);
-                const int cb = c0 + (ch >> 1), tok = m0 + row;
-                xok[it] = (hb + it < NIT) && (i < 2 * KCB * MT) && tok < p.M && cb < p.Cb;
-                const int tokc = tok < p.M ? tok : p.M - 1;
-                const int e0 = (cb < p.Cb ? cb : p.Cb - 1) * 16 + (ch & 1) * 8;
-                xv[it] = *reinterpret_cast<const uint4 *>(p.x + (int64_t)tokc * p.ldx + e0);
-                if (MASKED) xok[it] = xok[it] && p.active[(int64_t)tokc * p.n_clusters + e0 / p.cluster_size] != 0;
-            }
-#pragma unroll
-            for (int it = 0; it < NH; ++it) {
-                const int i = (hb + it) * 256 + tid;
-                if ((hb + it < NIT) && i < 2 * KCB * MT) {
-                    const int ch = i % (2 * KCB), row = i / (2 * KCB);
-                    lx[ch * LDM + row] = xok[it] ? xv[it] : make_uint4(0u, 0u, 0u, 0u);
+                for (int it = 0; it < NITX; ++it) {
+                    int r = r0 + RG * it;
+                    r = r < rlast ? r : rlast;
+                    xv[it] = *reinterpret_cast<const uint4 *>(xtile + (uint32_t)r * ldxB + (uint32_t)cu * 16u);
+                    if (MASKED) xm[it] = p.active[(int64_t)(m0 + r) * p.n_clusters + clus];
                 }
             }
         }
+        int P0v = 0, P1v = 0;
+        if (lane < NA) {
+            P0v = lcp[lane * (p.nkc + 1) + kc];
+            P1v = lcp[lane * (p.nkc + 1) + kc + 1];
+        }
 #pragma unroll
         for (int a = 0; a < NA; ++a) {
-            if (nb[a] > 0) {
+            const int P0 = __builtin_amdgcn_readlane(P0v, a);
+            int nb = __builtin_amdgcn_readlane(P1v, a) - P0;
+            if (ROUTED && cnt[a / NACC] == 0) nb = 0;
+            nbn[a] = nb;
+            if (nb > 0) {
+                const int last = nb * 16 - 1;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const int i = lane + 64 * k;
-                    if (i < nb[a] * 16) lwc[a * KCB * 16 + i] = wv[a][k];
+                    if (k == 0 || nb * 16 > 64 * k) wv[a][k] = p.codes[(int64_t)P0 * 16 + (i < last ? i : last)];
                 }
-                if (lane < nb[a]) {
-                    lws[a * KCB + lane] = wsd[a];
-                    lwl[a * KCB + lane] = (uint32_t)((wcl[a] - c0) * 2 * LDM);
+                const int j = lane < nb ? lane : 0;
+                wsd[a] = p.sdup[P0 + j];
+                wcl[a] = p.col[P0 + j];        // chunk base is subtracted at store time: no ALU use here,
+                                               // so no wait for this load sits between the loads of a chunk
+            }
+        }
+    };
+    // Registers -> LDS: activation buffer `buf` (shared) and this wave's own block list.  The rows' blocks are
+    // laid back to back, each row padded to a whole pair with an all-zero block, and the list ends with two
+    // zero blocks so that the software pipeline below may read one pair past the end.
+    auto store_chunk = [&](int buf) {
+        uint4 *lx = lxbuf + buf * XUNITS;
+        if (stager) {
+#pragma unroll
+            for (int it = 0; it < NITX; ++it) {
+                uint4 v = xv[it];
+                if (MASKED && xm[it] == 0u) v = make_uint4(0u, 0u, 0u, 0u);
+                lx[ch * LDM + r0 + RG * it] = v;
+            }
+        }
+        int o = 0;
+#pragma unroll
+        for (int a = 0; a < NA; ++a) {
+            const int nb = nbn[a];
+            np[a] = (nb + 1) >> 1;
+            if (nb > 0) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int i = lane + 64 * k;
+                    if (i < nb * 16) lwc[o * 16 + i] = wv[a][k];
                 }
-                if (nb[a] & 1) {   // pad to a whole pair with an all-zero block
-                    if (lane < 16) lwc[(a * KCB + nb[a]) * 16 + lane] = 0u;
+                if (lane < nb) {
+                    lws[o + lane] = wsd[a];
+                    lwl[o + lane] = (uint32_t)((wcl[a] - c0n) * 2 * LDM);
+                }
+                if (nb & 1) {
+                    if (lane < 16) lwc[(o + nb) * 16 + lane] = 0u;
                     if (lane == 0) {
-                        lws[a * KCB + nb[a]] = 0u;
-                        lwl[a * KCB + nb[a]] = 0u;
+                        lws[o + nb] = 0u;
+                        lwl[o + nb] = 0u;
                     }
                 }
             }
+            o += 2 * np[a];
         }
-        __syncthreads();
-        // ---- MFMA over the chunk -----------------------------------------------------------------
+        if (lane < 32) lwc[o * 16 + lane] = 0u;
+        if (lane < 2) {
+            lws[o + lane] = 0u;
+            lwl[o + lane] = 0u;
+        }
+        // row unit of the next non-empty row after a (routed mode: whose token list the look-ahead uses)
+        int nx = RW - 1;
+#pragma unroll
+        for (int a = NA - 1; a >= 0; --a) {
+            nxt[a] = nx;
+            if (np[a] > 0) nx = a / NACC;
+        }
+    };
+
+    load_chunk(0);
+    store_chunk(0);
+    __syncthreads();
+    for (int kc = 0; kc < p.nkc; ++kc) {
+        const bool more = kc + 1 < p.nkc;
+        if (more) load_chunk(kc + 1);
+        const uint4 *lx = lxbuf + (kc & 1) * XUNITS;
+        // ---- MFMA over the chunk: one software pipeline across all rows of the wave --------------------
+        // stage 1 reads a pair's codes/scale/offset, stage 2 unpacks it and issues its activation reads,
+        // stage 3 multiplies; three consecutive pairs are in flight.
+        int first_rw = 0;
+        if (ROUTED) {
+            first_rw = RW - 1;
+#pragma unroll
+            for (int a = NA - 1; a >= 0; --a)
+                if (np[a] > 0) first_rw = a / NACC;
+        }
+        int cur = bsel;                                   // block index (this lane's half of the pair)
+        uint32_t w1 = lwc[cur * 16 + n], sd1 = lws[cur], xo1 = lwl[cur] + hsel * LDM;
+        u32x4_t A = mortar_unpack8(w1 << (8 * hsel), sd1);
+        uint4 B[MSUB];
+#pragma unroll
+        for (int ms = 0; ms < MSUB; ++ms) B[ms] = lx[xo1 + tk[ROUTED ? first_rw : 0][ms]];
+        cur += 2;
+        w1 = lwc[cur * 16 + n]; sd1 = lws[cur]; xo1 = lwl[cur] + hsel * LDM;
 #pragma unroll
         for (int a = 0; a < NA; ++a) {
             const int rw = a / NACC;
-            const int np = (nb[a] + 1) >> 1;
             const int nsub = ROUTED ? (cnt[rw] + 15) >> 4 : MSUB;
-            for (int q = 0; q < np; ++q) {
-                const int blk = a * KCB + 2 * q + bsel;
-                const uint32_t w = lwc[blk * 16 + n];
-                const uint32_t sd = lws[blk];
-                const uint32_t xo = lwl[blk] + hsel * LDM;
-                const u32x4_t A = mortar_unpack8(w << (8 * hsel), sd);
+            for (int q = 0; q < np[a]; ++q) {
+                // stage 1 for the pair after the next one
+                cur += 2;
+                const uint32_t w0 = lwc[cur * 16 + n], sd0 = lws[cur], xo0 = lwl[cur] + hsel * LDM;
+                // stage 2 (unpack) of the next pair
+                const u32x4_t An = mortar_unpack8(w1 << (8 * hsel), sd1);
+                // the next pair belongs to this row, except after the row's last pair
+                const int rn = (ROUTED && q + 1 == np[a]) ? nxt[a] : rw;
+                // stage 3: multiply, and refill each activation register for the next pair as soon as its
+                // MFMA has been issued
 #pragma unroll
                 for (int ms = 0; ms < MSUB; ++ms) {
                     if (!ROUTED || ms < nsub) {
-                        const uint4 b = lx[xo + tk[rw][ms]];
-                        const u32x4_t B = {b.x, b.y, b.z, b.w};
-                        acc[a][ms] = mortar_mfma(A, B, acc[a][ms]);
+                        const u32x4_t Bv = {B[ms].x, B[ms].y, B[ms].z, B[ms].w};
+                        acc[a][ms] = mortar_mfma(A, Bv, acc[a][ms]);
                     }
+                    B[ms] = lx[xo1 + (ROUTED ? tk[rn][ms] : tk[0][ms])];
                 }
+                A = An;
+                w1 = w0; sd1 = sd0; xo1 = xo0;
             }
         }
+        if (more) store_chunk((kc + 1) & 1);
+        __syncthreads();
     }
 
     // ---- epilogue: lane holds D[4g+v][token n] ------------------------------------------------------
@@ -221,44 +303,45 @@ __global__ void __launch_bounds__(256, 2) mortar_spmm_kernel(const SpmmParams p)
             if (ROUTED && li >= cnt[rw]) continue;
             const int tok = m0 + (int)tk[rw][ms];
             if (tok >= p.M) continue;
-            uint32_t o[4];
+            float o[4];
             if (NACC == 1) {
 #pragma unroll
-                for (int v = 0; v < 4; ++v) o[v] = bf16_bits_rne(acc[rw][ms][v]);
+                for (int v = 0; v < 4; ++v) o[v] = acc[rw][ms][v];
             } else {
                 const int e0 = outb[rw] * 16 + 4 * g;
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const float gt = bf16r(acc[rw * 2][ms][v]);
                     const float up = bf16r(acc[rw * 2 + 1][ms][v]);
-                    float h = bf16r(bf16r(silu_f32(gt)) * up);
+                    float h = bf16r(silu_f32(gt)) * up;
                     if (p.gates) {
                         const float gv = p.gates[(int64_t)tok * p.n_clusters + (e0 + v) / p.cluster_size];
-                        h = bf16r(h * bf16r(gv));
+                        h = bf16r(h) * bf16r(gv);
                     }
-                    o[v] = bf16_bits_rne(h);
+                    o[v] = h;
                 }
             }
-            u32x2_t pk = {o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
+            const u32x2_t pk = {bf16_pack2(o[0], o[1]), bf16_pack2(o[2], o[3])};
             *reinterpret_cast<u32x2_t *>(p.y + (int64_t)tok * p.ldy + outb[rw] * 16 + 4 * g) = pk;
         }
     }
 }
 
 template <int MSUB, int RW, int NACC>
-constexpr int smem_bytes() {
-    return 2 * KCB * (16 * MSUB + 1) * 16 + NW * RW * NACC * KCB * 18 * 4;
+constexpr int smem_fixed_bytes() {
+    return 2 * 2 * KCB * (16 * MSUB + 1) * 16 + NW * (RW * NACC * KCB + 4) * 18 * 4;
 }
 
 template <int MSUB, int RW, int NACC, bool ROUTED, bool MASKED>
 int launch(SpmmParams &p, hipStream_t st) {
     constexpr int MT = 16 * MSUB;
-    constexpr int smem = smem_bytes<MSUB, RW, NACC>();
+    const int smem = smem_fixed_bytes<MSUB, RW, NACC>() + NW * RW * NACC * (p.nkc + 1) * 4;
+    if (smem > 160 * 1024) return mortar_fail(MORTAR_ERR_LIMIT, "prefill: in_features too large for the LDS chunk table (%d bytes)", smem);
     static bool attr_done = false;
     auto kern = mortar_spmm_kernel<MSUB, RW, NACC, ROUTED, MASKED>;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
         attr_done = true;
     }
@@ -268,7 +351,7 @@ int launch(SpmmParams &p, hipStream_t st) {
     const int mt_slots = p.xcd_map ? (p.n_mtiles + 7) / 8 * 8 : p.n_mtiles;
     const int64_t grid = (int64_t)mt_slots * p.n_groups;
     if (grid <= 0 || grid > 0x7fffffff) return mortar_fail(MORTAR_ERR_LIMIT, "prefill grid %lld out of range", (long long)grid);
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), smem, st, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), smem, st, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "prefill launch: %s", hipGetErrorString(e));
     return MORTAR_OK;
@@ -298,7 +381,7 @@ void fill(SpmmParams &p, const mortar_bcsr_t *W, const int32_t *chunk_ptr, const
 
 }  // namespace
 
-extern "C" int mortar_prefill_group(int swiglu) { return swiglu ? NW * 2 : NW * 4; }
+extern "C" int mortar_prefill_group(int swiglu) { return swiglu ? NW * 4 : NW * 8; }
 
 extern "C" int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int32_t *unit_order,
                                 const uint16_t *x, int64_t M, int64_t ldx, uint16_t *y, int64_t ldy,
@@ -308,7 +391,10 @@ extern "C" int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr
     SpmmParams p;
     fill(p, W, chunk_ptr, unit_order, x, M, ldx, y, ldy);
     p.n_units = W->Rb;
-    return launch<8, 4, 1, false, false>(p, static_cast<hipStream_t>(stream));
+    // few block-rows (e.g. `down`): halve the rows per workgroup so that the grid still covers every CU
+    const int64_t wgs4 = ((M + 127) / 128) * ((W->Rb + NW * 8 - 1) / (NW * 8));
+    if (wgs4 < 2 * 256) return launch<8, 4, 1, false, false>(p, static_cast<hipStream_t>(stream));
+    return launch<8, 8, 1, false, false>(p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *chunk_ptr,
@@ -323,7 +409,9 @@ extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *ch
     fill(p, W, chunk_ptr, unit_order, x, M, ldx, y, ldy);
     p.n_units = W->Rb;
     p.active = active; p.n_clusters = n_clusters; p.cluster_size = (W->Cb * 16) / n_clusters;
-    return launch<8, 4, 1, false, true>(p, static_cast<hipStream_t>(stream));
+    const int64_t wgs4 = ((M + 127) / 128) * ((W->Rb + NW * 8 - 1) / (NW * 8));
+    if (wgs4 < 2 * 256) return launch<8, 4, 1, false, true>(p, static_cast<hipStream_t>(stream));
+    return launch<8, 8, 1, false, true>(p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr,
@@ -345,7 +433,7 @@ extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *
         if (!tok_cnt || !tok_list || !gates) return mortar_fail(MORTAR_ERR_ARG, "gateup: routed mode needs gates, tok_cnt and tok_list");
         if (p.cluster_size % 16) return mortar_fail(MORTAR_ERR_ARG, "gateup: routed mode needs cluster_size %% 16 == 0");
         p.tok_cnt = tok_cnt; p.tok_list = tok_list;
-        return launch<8, 2, 2, true, false>(p, static_cast<hipStream_t>(stream));
+        return launch<8, 4, 2, true, false>(p, static_cast<hipStream_t>(stream));
     }
-    return launch<8, 2, 2, false, false>(p, static_cast<hipStream_t>(stream));
+    return launch<8, 4, 2, false, false>(p, static_cast<hipStream_t>(stream));
 }
