@@ -159,7 +159,7 @@ def main() -> None:
 
         def routed():
             gates, active = ops.remoe_gates(logits, TOP_K)
-            route = ops.remoe_route(active)
+            route = ops.remoe_route(active, ops.prefill_tile(Wgu))
             ops.gateup_swiglu(x, Wgu, gates=gates, route=route, out=h)
             ops.spmm(h, Wdn, active=active, out=y)
         t = event_time_ms(routed, it)

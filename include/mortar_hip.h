@@ -102,7 +102,7 @@ int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int
  * [0, d_ff) and up rows [d_ff, 2*d_ff) (transformer.py:335-336,403-405).  Intermediates are rounded to
  * bf16 where the reference materialises a bf16 tensor.  gates: device fp32 [M, n_clusters] or NULL;
  * d_ff % n_clusters == 0.
- * Routed skipping (optional): tok_cnt/tok_list from mortar_remoe_route with tile = MORTAR_PREFILL_MT; when
+ * Routed skipping (optional): tok_cnt/tok_list from mortar_remoe_route with tile = mortar_prefill_tile(Cb); when
  * given (requires cluster_size % 16 == 0) only active (token, block-row) tiles are computed and written;
  * inactive entries of h are left untouched and must be masked by the consumer (mortar_spmm_bf16_masked). */
 int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int32_t *unit_order,
@@ -116,6 +116,10 @@ int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *chunk_ptr, co
                             const uint16_t *x, int64_t M, int64_t ldx, uint16_t *y, int64_t ldy,
                             const uint8_t *active, int32_t n_clusters, void *stream);
 
+/* Token tile the prefill kernels use for a matrix with Cb block-columns: the tile size that
+ * mortar_remoe_route must be called with for routed mortar_gateup_swiglu_bf16 on that matrix. */
+int mortar_prefill_tile(int32_t Cb);
+
 /* Units per prefill workgroup (for mortar_unit_order_host): swiglu = 0 plain, 1 gate/up pairs. */
 int mortar_prefill_group(int swiglu);
 
@@ -128,7 +132,7 @@ int mortar_remoe_gates(const float *logits, int64_t M, int32_t n, int32_t k, flo
                        void *stream);
 
 /* Wavefront-ballot compaction of active tokens per (token tile, cluster):
- * tok_cnt[t*n + c] = number of tokens of tile t (tile tokens each, <= 256) with active[m, c] != 0,
+ * tok_cnt[t*n + c] = number of tokens of tile t (tile tokens each, a multiple of 16, <= 256) with active[m, c] != 0,
  * tok_list[(t*n + c)*tile + i] = tile-local index of the i-th such token, ascending. */
 int mortar_remoe_route(const uint8_t *active, int64_t M, int32_t n, int32_t tile, int32_t *tok_cnt,
                        uint8_t *tok_list, void *stream);

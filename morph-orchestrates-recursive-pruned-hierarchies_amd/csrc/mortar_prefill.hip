@@ -25,6 +25,7 @@ struct SpmmParams {
     const uint32_t *sdup;
     const int16_t *col;
     const int32_t *chunk_ptr;
+    const int32_t *row_ptr;
     const int32_t *unit_order;
     int n_units, nkc, Cb;
     const uint16_t *x;
@@ -38,6 +39,7 @@ struct SpmmParams {
     const uint8_t *tok_list;  // routed: [n_mtiles, n_clusters, MT]
     int n_clusters, cluster_size;
     int xcd_map, n_mtiles, n_groups;
+    int n_split;              // resident kernel: workgroups that share one token tile
 };
 
 template <int MSUB, int RW, int NACC, bool ROUTED, bool MASKED>
@@ -357,6 +359,188 @@ int launch(SpmmParams &p, hipStream_t st) {
     return MORTAR_OK;
 }
 
+
+// ---------------------------------------------------------------------------------------------------------
+// Resident-activation variant, used when a token tile of ALL K columns fits in LDS (in_features <= 2480 at
+// 32 tokens).  The workgroup (16 wavefronts) stages x[MT, K] once, then every wave walks whole row units on
+// its own: it streams the unit's block pairs straight from global memory in batches (a row's blocks are
+// contiguous), unpacks them in registers and multiplies against the resident tile.  There is no K chunking,
+// no barrier after the first one and no per-chunk staging; latency is hidden by the four waves per SIMD.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int RES_WAVES = 16;
+constexpr int RES_BATCH = 8;     // block pairs loaded per batch
+
+template <int MSUB, int NACC, bool ROUTED>
+__global__ void __launch_bounds__(RES_WAVES * 64) mortar_resident_kernel(const SpmmParams p) {
+    constexpr int MT = 16 * MSUB, LDM = MT + 1;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint4 *lx = reinterpret_cast<uint4 *>(smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
+    const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
+    const int m0 = mt * MT;
+
+    // ---- stage the token tile: unit (ch, row) <- x[m0 + row, ch*8 .. ch*8+8]; rows past M repeat the last row
+    {
+        const int nch = 2 * p.Cb;
+        const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;
+        const char *xt = reinterpret_cast<const char *>(p.x) + (int64_t)m0 * p.ldx * 2;
+        for (int i0 = 0; i0 < nch * MT; i0 += RES_WAVES * 64 * 4) {
+            uint4 v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                int i = i0 + k * RES_WAVES * 64 + tid;
+                i = i < nch * MT ? i : nch * MT - 1;
+                const int ch = i % nch;
+                int row = i / nch;
+                row = row < rlast ? row : rlast;
+                v[k] = *reinterpret_cast<const uint4 *>(xt + (int64_t)row * p.ldx * 2 + ch * 16);
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int i = i0 + k * RES_WAVES * 64 + tid;
+                if (i < nch * MT) lx[(i % nch) * LDM + i / nch] = v[k];
+            }
+        }
+    }
+    __syncthreads();
+
+    const int per = (p.n_units + p.n_split - 1) / p.n_split;
+    const int u_end = (sp + 1) * per < p.n_units ? (sp + 1) * per : p.n_units;
+    for (int pos = sp * per + wave; pos < u_end; pos += RES_WAVES) {
+        int unit = p.unit_order ? p.unit_order[pos] : pos;
+        unit = __builtin_amdgcn_readfirstlane(unit);
+        int cnt = MT;
+        uint32_t tk[MSUB];
+#pragma unroll
+        for (int ms = 0; ms < MSUB; ++ms) tk[ms] = ms * 16 + n;
+        if (ROUTED) {
+            const int cl = (unit * 16) / p.cluster_size;
+            const int64_t e = (int64_t)mt * p.n_clusters + cl;
+            cnt = __builtin_amdgcn_readfirstlane(p.tok_cnt[e]);
+            if (cnt == 0) continue;
+#pragma unroll
+            for (int ms = 0; ms < MSUB; ++ms) {
+                const int i = ms * 16 + n;
+                tk[ms] = i < cnt ? p.tok_list[e * MT + i] : 0;
+            }
+        }
+        const int nsub = ROUTED ? (cnt + 15) >> 4 : MSUB;
+        f32x4_t acc[NACC][MSUB];
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+        for (int a = 0; a < NACC; ++a) {
+            const int row = unit + a * p.n_units;
+            const int p0 = __builtin_amdgcn_readfirstlane(p.row_ptr[row]);
+            const int p1 = __builtin_amdgcn_readfirstlane(p.row_ptr[row + 1]);
+            for (int q0 = p0; q0 < p1; q0 += 2 * RES_BATCH) {
+                uint32_t w[RES_BATCH], sd[RES_BATCH];
+                int c[RES_BATCH];
+#pragma unroll
+                for (int u = 0; u < RES_BATCH; ++u) {
+                    const int j = q0 + 2 * u + bsel;
+                    const int jc = j < p1 ? j : p1 - 1;
+                    w[u] = p.codes[(int64_t)jc * 16 + n];
+                    sd[u] = p.sdup[jc];
+                    c[u] = p.col[jc];
+                }
+#pragma unroll
+                for (int u = 0; u < RES_BATCH; ++u) {
+                    if (q0 + 2 * u < p1) {
+                        const bool ok = q0 + 2 * u + bsel < p1;
+                        const u32x4_t A = mortar_unpack8(ok ? (w[u] << (8 * hsel)) : 0u, sd[u]);
+                        const uint32_t xo = (uint32_t)((c[u] * 2 + hsel) * LDM);
+#pragma unroll
+                        for (int ms = 0; ms < MSUB; ++ms) {
+                            if (!ROUTED || ms < nsub) {
+                                const uint4 b = lx[xo + tk[ms]];
+                                const u32x4_t Bv = {b.x, b.y, b.z, b.w};
+                                acc[a][ms] = mortar_mfma(A, Bv, acc[a][ms]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+
+        // epilogue: lane holds D[4g+v][token]
+#pragma unroll
+        for (int ms = 0; ms < MSUB; ++ms) {
+            const int li = ms * 16 + n;
+            if (ROUTED && li >= cnt) continue;
+            const int tok = m0 + (int)tk[ms];
+            if (tok >= p.M) continue;
+            float o[4];
+            if (NACC == 1) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) o[v] = acc[0][ms][v];
+            } else {
+                const int e0 = unit * 16 + 4 * g;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float gt = bf16r(acc[0][ms][v]);
+                    const float up = bf16r(acc[NACC - 1][ms][v]);
+                    float h = bf16r(silu_f32(gt)) * up;
+                    if (p.gates) {
+                        const float gv = p.gates[(int64_t)tok * p.n_clusters + (e0 + v) / p.cluster_size];
+                        h = bf16r(h) * bf16r(gv);
+                    }
+                    o[v] = h;
+                }
+            }
+            const u32x2_t pk = {bf16_pack2(o[0], o[1]), bf16_pack2(o[2], o[3])};
+            *reinterpret_cast<u32x2_t *>(p.y + (int64_t)tok * p.ldy + unit * 16 + 4 * g) = pk;
+        }
+    }
+}
+
+// Token tile of the resident kernel for a matrix with Cb block-columns (0 = does not fit).
+int resident_msub(int Cb) {
+    for (int msub : {6, 4, 2})
+        if ((int64_t)2 * Cb * (16 * msub + 1) * 16 <= 156 * 1024) return msub;
+    return 0;
+}
+
+template <int MSUB, int NACC, bool ROUTED>
+int launch_resident(SpmmParams &p, hipStream_t st) {
+    constexpr int MT = 16 * MSUB;
+    const int smem = 2 * p.Cb * (MT + 1) * 16;
+    static bool attr_done = false;
+    auto kern = mortar_resident_kernel<MSUB, NACC, ROUTED>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        attr_done = true;
+    }
+    p.n_mtiles = (p.M + MT - 1) / MT;
+    // enough workgroups to cover the 256 CUs, but at least RES_WAVES units per workgroup
+    int split = (2 * 256 + p.n_mtiles - 1) / p.n_mtiles;
+    const int max_split = (p.n_units + RES_WAVES - 1) / RES_WAVES;
+    split = split < 1 ? 1 : (split > max_split ? max_split : split);
+    p.n_split = split;
+    const int64_t grid = (int64_t)p.n_mtiles * split;
+    if (grid <= 0 || grid > 0x7fffffff) return mortar_fail(MORTAR_ERR_LIMIT, "prefill grid %lld out of range", (long long)grid);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(RES_WAVES * 64), smem, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "prefill launch: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}
+
+template <int NACC, bool ROUTED>
+int launch_resident_any(SpmmParams &p, hipStream_t st) {
+    switch (resident_msub(p.Cb)) {
+        case 6: return launch_resident<6, NACC, ROUTED>(p, st);
+        case 4: return launch_resident<4, NACC, ROUTED>(p, st);
+        default: return launch_resident<2, NACC, ROUTED>(p, st);
+    }
+}
+
 int check_common(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const uint16_t *x, int64_t M, int64_t ldx,
                  const uint16_t *y, int64_t ldy, int64_t out_cols) {
     if (!W || !W->codes || !W->sdup || !W->col || !W->row_ptr || !chunk_ptr || !x || !y)
@@ -373,13 +557,19 @@ int check_common(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const uint16_
 void fill(SpmmParams &p, const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int32_t *unit_order,
           const uint16_t *x, int64_t M, int64_t ldx, uint16_t *y, int64_t ldy) {
     p = SpmmParams{};
-    p.codes = W->codes; p.sdup = W->sdup; p.col = W->col; p.chunk_ptr = chunk_ptr; p.unit_order = unit_order;
+    p.codes = W->codes; p.sdup = W->sdup; p.col = W->col; p.chunk_ptr = chunk_ptr; p.row_ptr = W->row_ptr;
+    p.unit_order = unit_order;
     p.nkc = (W->Cb + KCB - 1) / KCB; p.Cb = W->Cb;
     p.x = x; p.ldx = ldx; p.M = (int)M; p.y = y; p.ldy = ldy;
     p.n_clusters = 1; p.cluster_size = 1 << 30;
 }
 
 }  // namespace
+
+extern "C" int mortar_prefill_tile(int32_t Cb) {
+    const int msub = resident_msub(Cb);
+    return msub ? 16 * msub : MORTAR_PREFILL_MT;
+}
 
 extern "C" int mortar_prefill_group(int swiglu) { return swiglu ? NW * 4 : NW * 8; }
 
@@ -391,6 +581,7 @@ extern "C" int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr
     SpmmParams p;
     fill(p, W, chunk_ptr, unit_order, x, M, ldx, y, ldy);
     p.n_units = W->Rb;
+    if (resident_msub(W->Cb)) return launch_resident_any<1, false>(p, static_cast<hipStream_t>(stream));
     // few block-rows (e.g. `down`): halve the rows per workgroup so that the grid still covers every CU
     const int64_t wgs4 = ((M + 127) / 128) * ((W->Rb + NW * 8 - 1) / (NW * 8));
     if (wgs4 < 2 * 256) return launch<8, 4, 1, false, false>(p, static_cast<hipStream_t>(stream));
@@ -433,7 +624,9 @@ extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *
         if (!tok_cnt || !tok_list || !gates) return mortar_fail(MORTAR_ERR_ARG, "gateup: routed mode needs gates, tok_cnt and tok_list");
         if (p.cluster_size % 16) return mortar_fail(MORTAR_ERR_ARG, "gateup: routed mode needs cluster_size %% 16 == 0");
         p.tok_cnt = tok_cnt; p.tok_list = tok_list;
+        if (resident_msub(W->Cb)) return launch_resident_any<2, true>(p, static_cast<hipStream_t>(stream));
         return launch<8, 4, 2, true, false>(p, static_cast<hipStream_t>(stream));
     }
+    if (resident_msub(W->Cb)) return launch_resident_any<2, false>(p, static_cast<hipStream_t>(stream));
     return launch<8, 4, 2, false, false>(p, static_cast<hipStream_t>(stream));
 }

@@ -122,7 +122,7 @@ class _SwiGLUMortar(nn.Module):
             if gates is not None and self.route_skip and cs % 16 == 0:
                 if active is None:
                     active = (gates > 0).to(torch.uint8)
-                route = ops.remoe_route(active, PREFILL_MT)
+                route = ops.remoe_route(active, ops.prefill_tile(Wgu))
                 h = ops.gateup_swiglu(xb, Wgu, gates=gates, route=route)
                 y = ops.spmm(h, Wdn, active=active)
             else:

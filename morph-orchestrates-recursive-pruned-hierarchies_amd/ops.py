@@ -105,6 +105,11 @@ def remoe_gates(logits: Tensor, k: int) -> tuple[Tensor, Tensor]:
     return gates, active
 
 
+def prefill_tile(W: MortarPack) -> int:
+    """Token tile of the prefill kernels for this matrix (the tile remoe_route must use for it)."""
+    return int(_lib.lib().mortar_prefill_tile(W.Cb))
+
+
 def remoe_route(active: Tensor, tile: int = PREFILL_MT) -> tuple[Tensor, Tensor]:
     """Per (token tile, cluster): count and ascending list of the tile-local indices of active tokens."""
     _need_gpu(active, "remoe_route")
