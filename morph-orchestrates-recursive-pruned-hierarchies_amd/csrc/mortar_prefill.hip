@@ -380,6 +380,7 @@ __global__ void __launch_bounds__(RES_WAVES * 64) mortar_resident_kernel(const S
     const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
     const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
     const int m0 = mt * MT;
+    const uint32_t lane_xo = (uint32_t)(hsel * LDM + (ROUTED ? 0 : n));
 
     // ---- stage the token tile: unit (ch, row) <- x[m0 + row, ch*8 .. ch*8+8]; rows past M repeat the last row
     {
@@ -438,7 +439,50 @@ __global__ void __launch_bounds__(RES_WAVES * 64) mortar_resident_kernel(const S
             const int row = unit + a * p.n_units;
             const int p0 = __builtin_amdgcn_readfirstlane(p.row_ptr[row]);
             const int p1 = __builtin_amdgcn_readfirstlane(p.row_ptr[row + 1]);
-            for (int q0 = p0; q0 < p1; q0 += 2 * RES_BATCH) {
+            // Full batches: every offset is the batch base plus a compile-time constant, so the loads need no
+            // per-pair address arithmetic and no predication.
+            int q0 = p0;
+            for (; q0 + 2 * RES_BATCH <= p1; q0 += 2 * RES_BATCH) {
+                const uint32_t jb = (uint32_t)(q0 + bsel);
+                const uint32_t *cw = p.codes + (size_t)jb * 16 + n;
+                const uint32_t *cs = p.sdup + jb;
+                const int16_t *cc = p.col + jb;
+                uint32_t w[RES_BATCH], sd[RES_BATCH];
+                int c[RES_BATCH];
+#pragma unroll
+                for (int u = 0; u < RES_BATCH; ++u) {
+                    w[u] = cw[u * 32];
+                    sd[u] = cs[u * 2];
+                    c[u] = cc[u * 2];
+                }
+                // activation operands are fetched one pair ahead of the MFMAs that use them
+                uint4 Bc[MSUB], Bn[MSUB];
+                {
+                    const uint32_t xo = (uint32_t)c[0] * (2 * LDM) + lane_xo;
+#pragma unroll
+                    for (int ms = 0; ms < MSUB; ++ms) Bc[ms] = lx[xo + (ROUTED ? tk[ms] : ms * 16)];
+                }
+#pragma unroll
+                for (int u = 0; u < RES_BATCH; ++u) {
+                    const u32x4_t A = mortar_unpack8(w[u] << (8 * hsel), sd[u]);
+                    if (u + 1 < RES_BATCH) {
+                        const uint32_t xo = (uint32_t)c[u + 1] * (2 * LDM) + lane_xo;
+#pragma unroll
+                        for (int ms = 0; ms < MSUB; ++ms) Bn[ms] = lx[xo + (ROUTED ? tk[ms] : ms * 16)];
+                    }
+#pragma unroll
+                    for (int ms = 0; ms < MSUB; ++ms) {
+                        if (!ROUTED || ms < nsub) {
+                            const u32x4_t Bv = {Bc[ms].x, Bc[ms].y, Bc[ms].z, Bc[ms].w};
+                            acc[a][ms] = mortar_mfma(A, Bv, acc[a][ms]);
+                        }
+                    }
+#pragma unroll
+                    for (int ms = 0; ms < MSUB; ++ms) Bc[ms] = Bn[ms];
+                }
+            }
+            // Row tail (fewer than a full batch of pairs): clamped loads, odd last pair padded with zero codes.
+            if (q0 < p1) {
                 uint32_t w[RES_BATCH], sd[RES_BATCH];
                 int c[RES_BATCH];
 #pragma unroll
@@ -454,11 +498,11 @@ __global__ void __launch_bounds__(RES_WAVES * 64) mortar_resident_kernel(const S
                     if (q0 + 2 * u < p1) {
                         const bool ok = q0 + 2 * u + bsel < p1;
                         const u32x4_t A = mortar_unpack8(ok ? (w[u] << (8 * hsel)) : 0u, sd[u]);
-                        const uint32_t xo = (uint32_t)((c[u] * 2 + hsel) * LDM);
+                        const uint32_t xo = (uint32_t)c[u] * (2 * LDM) + lane_xo;
 #pragma unroll
                         for (int ms = 0; ms < MSUB; ++ms) {
                             if (!ROUTED || ms < nsub) {
-                                const uint4 b = lx[xo + tk[ms]];
+                                const uint4 b = lx[xo + (ROUTED ? tk[ms] : ms * 16)];
                                 const u32x4_t Bv = {b.x, b.y, b.z, b.w};
                                 acc[a][ms] = mortar_mfma(A, Bv, acc[a][ms]);
                             }
