@@ -42,12 +42,22 @@ enum {
  *           device bit layout produced by mortar_encode_blocks_host
  *   sdup    [nnz] uint32: per-block scale pattern produced by mortar_encode_blocks_host
  *   col     [nnz] the reference's mortar_column_indices (int16, unchanged)
- *   row_ptr [Rb+1] the reference's mortar_offsets (int32, unchanged)                              */
+ *   row_ptr [Rb+1] the reference's mortar_offsets (int32, unchanged)
+ * Octet stream (second copy for the prefill kernels, from mortar_octet_layout_host): every row is cut into
+ * groups of 8 blocks (the last one padded with all-zero blocks) so that one 16-byte load per lane fetches
+ * the lane's code dwords of four consecutive block pairs:
+ *   row_desc [Rb*4] int32 per row: {first group, end group, number of blocks, 0}
+ *   codes_o [ngroups*2*16*4] uint32: ((group*2 + s)*16 + n)*4 + t = row n of block 8*g + 2*t + s of the row
+ *   sd_o    [ngroups*2*4] uint32 and col_o [ngroups*2*4] int32: (group*2 + s)*4 + t, same block             */
 typedef struct {
     const uint32_t *codes;
     const uint32_t *sdup;
     const int16_t *col;
     const int32_t *row_ptr;
+    const int32_t *row_desc;
+    const uint32_t *codes_o;
+    const uint32_t *sd_o;
+    const int32_t *col_o;
     int32_t Rb, Cb, nnz;
 } mortar_bcsr_t;
 
@@ -72,6 +82,14 @@ int mortar_decode_blocks_host(const uint32_t *codes, int64_t nnz, int8_t *codes_
  * (nkc = ceil(Cb/kcb)); out host [Rb*(nkc+1)] int32.  Validates the BCSR (sorted, in range). */
 int mortar_chunk_ptr_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
                           int32_t kcb, int32_t *out);
+
+/* Octet stream of one matrix (see mortar_bcsr_t).  row_desc_out host [Rb*4] is always written; the return
+ * value is the number of groups.  With codes_o_out == NULL only row_desc_out is filled (size query);
+ * otherwise codes_o_out [ngroups*128], sd_o_out [ngroups*8], col_o_out [ngroups*8] are filled from the
+ * encoded codes / sdup and the column indices. */
+int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, const uint32_t *codes, const uint32_t *sdup,
+                                 const int16_t *col, int32_t *row_desc_out, uint32_t *codes_o_out,
+                                 uint32_t *sd_o_out, int32_t *col_o_out);
 
 /* Row-unit schedule for uneven nnz: units sorted by descending block count and dealt so that every
  * workgroup of `group` units gets a similar total (longest-processing-time first).

@@ -134,20 +134,15 @@ __global__ void __launch_bounds__(256) mortar_gemv_kernel(const GemvParams p) {
             *reinterpret_cast<f32x4_t *>(pp + rowA * 16 + 4 * g) = accA[ms];
             if (rowB >= 0) *reinterpret_cast<f32x4_t *>(pp + rowB * 16 + 4 * g) = accB[ms];
         } else {
-            uint32_t o[4];
             const int e0 = rowA * 16 + 4 * g;
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                if (p.mode == 0) {
-                    o[v] = bf16_bits_rne(accA[ms][v]);
-                } else {
-                    const float gt = bf16r(accA[ms][v]), up = bf16r(accB[ms][v]);
-                    float h = bf16r(bf16r(silu_f32(gt)) * up);
-                    if (p.gates) h = bf16r(h * bf16r(p.gates[(int64_t)tok * p.ldg + (e0 + v) / p.cluster_size]));
-                    o[v] = bf16_bits_rne(h);
-                }
+            u32x2_t pk;
+            if (p.mode == 0) {
+                pk = u32x2_t{bf16_pack2(accA[ms][0], accA[ms][1]), bf16_pack2(accA[ms][2], accA[ms][3])};
+            } else {
+                float gv = 0.f;
+                if (p.gates) gv = p.gates[(int64_t)tok * p.ldg + e0 / p.cluster_size];
+                pk = swiglu_pack4(accA[ms], accB[ms], p.gates != nullptr, gv);
             }
-            const u32x2_t pk = {o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
             *reinterpret_cast<u32x2_t *>(p.y + (int64_t)tok * p.ldy + e0) = pk;
         }
     }
@@ -218,7 +213,8 @@ extern "C" int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, 
     p.x = x; p.B = B; p.ldx = ldx; p.y = y; p.ldy = ldy; p.part = part;
     p.n_clusters = 1; p.cluster_size = 1 << 30;
     if (gates) {
-        if (mode != 1 || n_clusters <= 0 || nout % n_clusters) return mortar_fail(MORTAR_ERR_ARG, "gemv: gates need mode 1 and d_ff %% n_clusters == 0");
+        if (mode != 1 || n_clusters <= 0 || nout % n_clusters || (nout / n_clusters) % 4)
+            return mortar_fail(MORTAR_ERR_ARG, "gemv: gates need mode 1 and d_ff / n_clusters a whole multiple of 4");
         p.gates = gates; p.n_clusters = n_clusters; p.cluster_size = (int)(nout / n_clusters); p.ldg = ldg;
     }
     p.row_act = row_act; p.ldr = ldr; p.col_act = col_act; p.ldc = ldc;

@@ -123,6 +123,41 @@ extern "C" int mortar_chunk_ptr_host(const int32_t *row_ptr, const int16_t *col,
     return MORTAR_OK;
 }
 
+extern "C" int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, const uint32_t *codes,
+                                            const uint32_t *sdup, const int16_t *col, int32_t *row_desc_out,
+                                            uint32_t *codes_o_out, uint32_t *sd_o_out, int32_t *col_o_out) {
+    if (!row_ptr || !row_desc_out || Rb <= 0) return mortar_fail(MORTAR_ERR_ARG, "octet_layout: bad argument");
+    int64_t ng = 0;
+    for (int r = 0; r < Rb; ++r) {
+        const int nb = row_ptr[r + 1] - row_ptr[r];
+        row_desc_out[4 * r] = (int32_t)ng;
+        ng += (nb + 7) / 8;
+        row_desc_out[4 * r + 1] = (int32_t)ng;
+        row_desc_out[4 * r + 2] = nb;
+        row_desc_out[4 * r + 3] = 0;
+        if (ng > 0x7fffffff / 128) return mortar_fail(MORTAR_ERR_LIMIT, "octet_layout: too many blocks");
+    }
+    if (!codes_o_out) return ng;
+    if (!codes || !sdup || !col || !sd_o_out || !col_o_out) return mortar_fail(MORTAR_ERR_ARG, "octet_layout: null pointer");
+    for (int r = 0; r < Rb; ++r) {
+        const int nb = row_ptr[r + 1] - row_ptr[r];
+        for (int gl = 0; gl * 8 < nb; ++gl) {
+            const int64_t gidx = row_desc_out[4 * r] + gl;
+            for (int s2 = 0; s2 < 2; ++s2)
+                for (int t = 0; t < 4; ++t) {
+                    const int b = 8 * gl + 2 * t + s2;
+                    const bool ok = b < nb;
+                    const int64_t j = (int64_t)row_ptr[r] + b;
+                    sd_o_out[(gidx * 2 + s2) * 4 + t] = ok ? sdup[j] : 0u;
+                    col_o_out[(gidx * 2 + s2) * 4 + t] = ok ? (int32_t)col[j] : 0;
+                    for (int n = 0; n < 16; ++n)
+                        codes_o_out[((gidx * 2 + s2) * 16 + n) * 4 + t] = ok ? codes[j * 16 + n] : 0u;
+                }
+        }
+    }
+    return ng;
+}
+
 extern "C" int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_t rows_per_unit,
                                       int32_t group, int32_t *order_out) {
     if (!row_ptr || !order_out || Rb <= 0 || group <= 0 || (rows_per_unit != 1 && rows_per_unit != 2) ||

@@ -26,6 +26,10 @@ struct SpmmParams {
     const int16_t *col;
     const int32_t *chunk_ptr;
     const int32_t *row_ptr;
+    const u32x4_t *row_desc;  // octet stream (resident kernel)
+    const u32x4_t *codes_o;
+    const u32x4_t *sd_o;
+    const u32x4_t *col_o;
     const int32_t *unit_order;
     int n_units, nkc, Cb;
     const uint16_t *x;
@@ -296,6 +300,7 @@ __global__ void __launch_bounds__(NW * 64, 1) mortar_spmm_kernel(const SpmmParam
     }
 
     // ---- epilogue: lane holds D[4g+v][token n] ------------------------------------------------------
+    const bool has_gates = p.gates != nullptr;
 #pragma unroll
     for (int rw = 0; rw < RW; ++rw) {
         if (outb[rw] < 0) continue;
@@ -305,25 +310,14 @@ __global__ void __launch_bounds__(NW * 64, 1) mortar_spmm_kernel(const SpmmParam
             if (ROUTED && li >= cnt[rw]) continue;
             const int tok = m0 + (int)tk[rw][ms];
             if (tok >= p.M) continue;
-            float o[4];
+            u32x2_t pk;
             if (NACC == 1) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v) o[v] = acc[rw][ms][v];
+                pk = u32x2_t{bf16_pack2(acc[rw][ms][0], acc[rw][ms][1]), bf16_pack2(acc[rw][ms][2], acc[rw][ms][3])};
             } else {
-                const int e0 = outb[rw] * 16 + 4 * g;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float gt = bf16r(acc[rw * 2][ms][v]);
-                    const float up = bf16r(acc[rw * 2 + 1][ms][v]);
-                    float h = bf16r(silu_f32(gt)) * up;
-                    if (p.gates) {
-                        const float gv = p.gates[(int64_t)tok * p.n_clusters + (e0 + v) / p.cluster_size];
-                        h = bf16r(h) * bf16r(gv);
-                    }
-                    o[v] = h;
-                }
+                float gv = 0.f;
+                if (has_gates) gv = p.gates[(int64_t)tok * p.n_clusters + (outb[rw] * 16 + 4 * g) / p.cluster_size];
+                pk = swiglu_pack4(acc[rw * NACC][ms], acc[rw * NACC + NACC - 1][ms], has_gates, gv);
             }
-            const u32x2_t pk = {bf16_pack2(o[0], o[1]), bf16_pack2(o[2], o[3])};
             *reinterpret_cast<u32x2_t *>(p.y + (int64_t)tok * p.ldy + outb[rw] * 16 + 4 * g) = pk;
         }
     }
@@ -367,12 +361,13 @@ int launch(SpmmParams &p, hipStream_t st) {
 // contiguous), unpacks them in registers and multiplies against the resident tile.  There is no K chunking,
 // no barrier after the first one and no per-chunk staging; latency is hidden by the four waves per SIMD.
 // ---------------------------------------------------------------------------------------------------------
-constexpr int RES_WAVES = 16;
-constexpr int RES_BATCH = 8;     // block pairs loaded per batch
+constexpr int RES_GROUPS = 4;    // octets (4 block pairs each) loaded per batch
+// wavefronts per workgroup: 16 (4 per SIMD, 128 registers) for the 32-token tile, 8 for larger tiles
+constexpr int res_waves(int msub) { return msub <= 2 ? 16 : 8; }
 
 template <int MSUB, int NACC, bool ROUTED>
-__global__ void __launch_bounds__(RES_WAVES * 64) mortar_resident_kernel(const SpmmParams p) {
-    constexpr int MT = 16 * MSUB, LDM = MT + 1;
+__global__ void __launch_bounds__(res_waves(MSUB) * 64) mortar_resident_kernel(const SpmmParams p) {
+    constexpr int MT = 16 * MSUB, LDM = MT + 1, RES_WAVES = res_waves(MSUB);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint4 *lx = reinterpret_cast<uint4 *>(smem);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -381,6 +376,7 @@ __global__ void __launch_bounds__(RES_WAVES * 64) mortar_resident_kernel(const S
     const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
     const int m0 = mt * MT;
     const uint32_t lane_xo = (uint32_t)(hsel * LDM + (ROUTED ? 0 : n));
+    const bool has_gates = p.gates != nullptr;
 
     // ---- stage the token tile: unit (ch, row) <- x[m0 + row, ch*8 .. ch*8+8]; rows past M repeat the last row
     {
@@ -409,24 +405,50 @@ __global__ void __launch_bounds__(RES_WAVES * 64) mortar_resident_kernel(const S
 
     const int per = (p.n_units + p.n_split - 1) / p.n_split;
     const int u_end = (sp + 1) * per < p.n_units ? (sp + 1) * per : p.n_units;
-    for (int pos = sp * per + wave; pos < u_end; pos += RES_WAVES) {
-        int unit = p.unit_order ? p.unit_order[pos] : pos;
-        unit = __builtin_amdgcn_readfirstlane(unit);
+    // Unit ids are fetched two units ahead and row descriptors one unit ahead, so that no dependent global
+    // round trip (order -> descriptor -> blocks) is exposed between two units of a wave.
+    auto unit_of = [&](int pos_) { return (p.unit_order && pos_ < u_end) ? p.unit_order[pos_] : pos_; };
+    auto desc_of = [&](int unit_, int a_) {
+        const int r = unit_ + a_ * p.n_units;
+        return p.row_desc[r < NACC * p.n_units ? r : 0];
+    };
+    int pos = sp * per + wave;
+    int unit_v = unit_of(pos), unit_v1 = unit_of(pos + RES_WAVES);
+    u32x4_t dcur[NACC], dnxt[NACC];
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) dcur[a] = desc_of(unit_v, a);
+    for (; pos < u_end; pos += RES_WAVES) {
+        const int unit = __builtin_amdgcn_readfirstlane(unit_v);
+        const int unit_v2 = unit_of(pos + 2 * RES_WAVES);
+#pragma unroll
+        for (int a = 0; a < NACC; ++a) dnxt[a] = desc_of(unit_v1 < p.n_units ? unit_v1 : 0, a);
         int cnt = MT;
         uint32_t tk[MSUB];
 #pragma unroll
         for (int ms = 0; ms < MSUB; ++ms) tk[ms] = ms * 16 + n;
+        bool skip = false;
         if (ROUTED) {
             const int cl = (unit * 16) / p.cluster_size;
             const int64_t e = (int64_t)mt * p.n_clusters + cl;
             cnt = __builtin_amdgcn_readfirstlane(p.tok_cnt[e]);
-            if (cnt == 0) continue;
+            skip = cnt == 0;
 #pragma unroll
             for (int ms = 0; ms < MSUB; ++ms) {
                 const int i = ms * 16 + n;
                 tk[ms] = i < cnt ? p.tok_list[e * MT + i] : 0;
             }
         }
+        int rg0[NACC], rg1[NACC], rnb[NACC];
+#pragma unroll
+        for (int a = 0; a < NACC; ++a) {
+            rg0[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][0]);
+            rg1[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][1]);
+            rnb[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][2]);
+            dcur[a] = dnxt[a];
+        }
+        unit_v = unit_v1;
+        unit_v1 = unit_v2;
+        if (skip) continue;
         const int nsub = ROUTED ? (cnt + 15) >> 4 : MSUB;
         f32x4_t acc[NACC][MSUB];
 #pragma unroll
@@ -436,74 +458,42 @@ __global__ void __launch_bounds__(RES_WAVES * 64) mortar_resident_kernel(const S
 
 #pragma unroll
         for (int a = 0; a < NACC; ++a) {
-            const int row = unit + a * p.n_units;
-            const int p0 = __builtin_amdgcn_readfirstlane(p.row_ptr[row]);
-            const int p1 = __builtin_amdgcn_readfirstlane(p.row_ptr[row + 1]);
-            // Full batches: every offset is the batch base plus a compile-time constant, so the loads need no
-            // per-pair address arithmetic and no predication.
-            int q0 = p0;
-            for (; q0 + 2 * RES_BATCH <= p1; q0 += 2 * RES_BATCH) {
-                const uint32_t jb = (uint32_t)(q0 + bsel);
-                const uint32_t *cw = p.codes + (size_t)jb * 16 + n;
-                const uint32_t *cs = p.sdup + jb;
-                const int16_t *cc = p.col + jb;
-                uint32_t w[RES_BATCH], sd[RES_BATCH];
-                int c[RES_BATCH];
+            const int g0 = rg0[a], g1 = rg1[a], nb = rnb[a];
+            // One batch = RES_GROUPS octets (8 blocks = 4 pairs each).  Per octet a lane needs three 16-byte
+            // loads: its code dwords, scale patterns and block-columns of the four pairs.
+            for (int gq = g0; gq < g1; gq += RES_GROUPS) {
+                u32x4_t cw[RES_GROUPS], sd[RES_GROUPS], cc[RES_GROUPS];
 #pragma unroll
-                for (int u = 0; u < RES_BATCH; ++u) {
-                    w[u] = cw[u * 32];
-                    sd[u] = cs[u * 2];
-                    c[u] = cc[u * 2];
+                for (int k = 0; k < RES_GROUPS; ++k) {
+                    const uint32_t gi = (uint32_t)(gq + k < g1 ? gq + k : g1 - 1) * 2u + (uint32_t)bsel;
+                    cw[k] = p.codes_o[gi * 16u + n];
+                    sd[k] = p.sd_o[gi];
+                    cc[k] = p.col_o[gi];
                 }
-                // activation operands are fetched one pair ahead of the MFMAs that use them
-                uint4 Bc[MSUB], Bn[MSUB];
-                {
-                    const uint32_t xo = (uint32_t)c[0] * (2 * LDM) + lane_xo;
+                const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;      // block pairs left in the row from this batch on
+                // activation operands are fetched two pairs ahead of the MFMAs that use them
+                constexpr int NP = 4 * RES_GROUPS;
+                uint4 Bq[3][MSUB];
 #pragma unroll
-                    for (int ms = 0; ms < MSUB; ++ms) Bc[ms] = lx[xo + (ROUTED ? tk[ms] : ms * 16)];
+                for (int d = 0; d < 2; ++d) {
+                    const uint32_t xo = cc[d >> 2][d & 3] * (2 * LDM) + lane_xo;
+#pragma unroll
+                    for (int ms = 0; ms < MSUB; ++ms) Bq[d][ms] = lx[xo + (ROUTED ? tk[ms] : ms * 16)];
                 }
 #pragma unroll
-                for (int u = 0; u < RES_BATCH; ++u) {
-                    const u32x4_t A = mortar_unpack8(w[u] << (8 * hsel), sd[u]);
-                    if (u + 1 < RES_BATCH) {
-                        const uint32_t xo = (uint32_t)c[u + 1] * (2 * LDM) + lane_xo;
+                for (int u = 0; u < NP; ++u) {
+                    if (u < pairs) {
+                        const u32x4_t A = mortar_unpack8(cw[u >> 2][u & 3] << (8 * hsel), sd[u >> 2][u & 3]);
+                        if (u + 2 < NP) {
+                            const uint32_t xo = cc[(u + 2) >> 2][(u + 2) & 3] * (2 * LDM) + lane_xo;
 #pragma unroll
-                        for (int ms = 0; ms < MSUB; ++ms) Bn[ms] = lx[xo + (ROUTED ? tk[ms] : ms * 16)];
-                    }
-#pragma unroll
-                    for (int ms = 0; ms < MSUB; ++ms) {
-                        if (!ROUTED || ms < nsub) {
-                            const u32x4_t Bv = {Bc[ms].x, Bc[ms].y, Bc[ms].z, Bc[ms].w};
-                            acc[a][ms] = mortar_mfma(A, Bv, acc[a][ms]);
+                            for (int ms = 0; ms < MSUB; ++ms) Bq[(u + 2) % 3][ms] = lx[xo + (ROUTED ? tk[ms] : ms * 16)];
                         }
-                    }
-#pragma unroll
-                    for (int ms = 0; ms < MSUB; ++ms) Bc[ms] = Bn[ms];
-                }
-            }
-            // Row tail (fewer than a full batch of pairs): clamped loads, odd last pair padded with zero codes.
-            if (q0 < p1) {
-                uint32_t w[RES_BATCH], sd[RES_BATCH];
-                int c[RES_BATCH];
-#pragma unroll
-                for (int u = 0; u < RES_BATCH; ++u) {
-                    const int j = q0 + 2 * u + bsel;
-                    const int jc = j < p1 ? j : p1 - 1;
-                    w[u] = p.codes[(int64_t)jc * 16 + n];
-                    sd[u] = p.sdup[jc];
-                    c[u] = p.col[jc];
-                }
-#pragma unroll
-                for (int u = 0; u < RES_BATCH; ++u) {
-                    if (q0 + 2 * u < p1) {
-                        const bool ok = q0 + 2 * u + bsel < p1;
-                        const u32x4_t A = mortar_unpack8(ok ? (w[u] << (8 * hsel)) : 0u, sd[u]);
-                        const uint32_t xo = (uint32_t)c[u] * (2 * LDM) + lane_xo;
 #pragma unroll
                         for (int ms = 0; ms < MSUB; ++ms) {
                             if (!ROUTED || ms < nsub) {
-                                const uint4 b = lx[xo + (ROUTED ? tk[ms] : ms * 16)];
-                                const u32x4_t Bv = {b.x, b.y, b.z, b.w};
+                                const uint4 bq = Bq[u % 3][ms];
+                                const u32x4_t Bv = {bq.x, bq.y, bq.z, bq.w};
                                 acc[a][ms] = mortar_mfma(A, Bv, acc[a][ms]);
                             }
                         }
@@ -519,25 +509,14 @@ __global__ void __launch_bounds__(RES_WAVES * 64) mortar_resident_kernel(const S
             if (ROUTED && li >= cnt) continue;
             const int tok = m0 + (int)tk[ms];
             if (tok >= p.M) continue;
-            float o[4];
+            u32x2_t pk;
             if (NACC == 1) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v) o[v] = acc[0][ms][v];
+                pk = u32x2_t{bf16_pack2(acc[0][ms][0], acc[0][ms][1]), bf16_pack2(acc[0][ms][2], acc[0][ms][3])};
             } else {
-                const int e0 = unit * 16 + 4 * g;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float gt = bf16r(acc[0][ms][v]);
-                    const float up = bf16r(acc[NACC - 1][ms][v]);
-                    float h = bf16r(silu_f32(gt)) * up;
-                    if (p.gates) {
-                        const float gv = p.gates[(int64_t)tok * p.n_clusters + (e0 + v) / p.cluster_size];
-                        h = bf16r(h) * bf16r(gv);
-                    }
-                    o[v] = h;
-                }
+                float gv = 0.f;
+                if (has_gates) gv = p.gates[(int64_t)tok * p.n_clusters + (unit * 16 + 4 * g) / p.cluster_size];
+                pk = swiglu_pack4(acc[0][ms], acc[NACC - 1][ms], has_gates, gv);
             }
-            const u32x2_t pk = {bf16_pack2(o[0], o[1]), bf16_pack2(o[2], o[3])};
             *reinterpret_cast<u32x2_t *>(p.y + (int64_t)tok * p.ldy + unit * 16 + 4 * g) = pk;
         }
     }
@@ -552,7 +531,7 @@ int resident_msub(int Cb) {
 
 template <int MSUB, int NACC, bool ROUTED>
 int launch_resident(SpmmParams &p, hipStream_t st) {
-    constexpr int MT = 16 * MSUB;
+    constexpr int MT = 16 * MSUB, RES_WAVES = res_waves(MSUB);
     const int smem = 2 * p.Cb * (MT + 1) * 16;
     static bool attr_done = false;
     auto kern = mortar_resident_kernel<MSUB, NACC, ROUTED>;
@@ -587,7 +566,7 @@ int launch_resident_any(SpmmParams &p, hipStream_t st) {
 
 int check_common(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const uint16_t *x, int64_t M, int64_t ldx,
                  const uint16_t *y, int64_t ldy, int64_t out_cols) {
-    if (!W || !W->codes || !W->sdup || !W->col || !W->row_ptr || !chunk_ptr || !x || !y)
+    if (!W || !W->codes || !W->sdup || !W->col || !W->row_ptr || !W->row_desc || !W->codes_o || !W->sd_o || !W->col_o || !chunk_ptr || !x || !y)
         return mortar_fail(MORTAR_ERR_ARG, "prefill: null pointer");
     if (W->Rb <= 0 || W->Cb <= 0 || W->nnz <= 0) return mortar_fail(MORTAR_ERR_ARG, "prefill: empty matrix");
     if (M <= 0 || M > (1 << 30)) return mortar_fail(MORTAR_ERR_ARG, "prefill: M=%lld out of range", (long long)M);
@@ -602,6 +581,10 @@ void fill(SpmmParams &p, const mortar_bcsr_t *W, const int32_t *chunk_ptr, const
           const uint16_t *x, int64_t M, int64_t ldx, uint16_t *y, int64_t ldy) {
     p = SpmmParams{};
     p.codes = W->codes; p.sdup = W->sdup; p.col = W->col; p.chunk_ptr = chunk_ptr; p.row_ptr = W->row_ptr;
+    p.row_desc = reinterpret_cast<const u32x4_t *>(W->row_desc);
+    p.codes_o = reinterpret_cast<const u32x4_t *>(W->codes_o);
+    p.sd_o = reinterpret_cast<const u32x4_t *>(W->sd_o);
+    p.col_o = reinterpret_cast<const u32x4_t *>(W->col_o);
     p.unit_order = unit_order;
     p.nkc = (W->Cb + KCB - 1) / KCB; p.Cb = W->Cb;
     p.x = x; p.ldx = ldx; p.M = (int)M; p.y = y; p.ldy = ldy;
@@ -661,7 +644,8 @@ extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *
     fill(p, W, chunk_ptr, unit_order, x, M, ldx, h, ldh);
     p.n_units = W->Rb / 2;
     if (gates) {
-        if (n_clusters <= 0 || d_ff % n_clusters) return mortar_fail(MORTAR_ERR_ARG, "gateup: d_ff %% n_clusters != 0");
+        if (n_clusters <= 0 || d_ff % n_clusters || (d_ff / n_clusters) % 4)
+            return mortar_fail(MORTAR_ERR_ARG, "gateup: d_ff / n_clusters must be a whole multiple of 4");
         p.gates = gates; p.n_clusters = n_clusters; p.cluster_size = (int)(d_ff / n_clusters);
     }
     if (tok_cnt || tok_list) {

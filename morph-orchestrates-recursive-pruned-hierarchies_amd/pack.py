@@ -58,6 +58,22 @@ def chunk_ptr(offsets, col, Rb: int, Cb: int, kcb: int = PREFILL_KCB) -> np.ndar
     return out
 
 
+def octet_layout(offsets, Rb: int, codes: np.ndarray, sdup: np.ndarray, col):
+    """-> (row_desc [Rb*4] int32, codes_o uint32, sd_o uint32, col_o int32): see mortar_octet_layout_host."""
+    offsets, col = _np(offsets, np.int32), _np(col, np.int16)
+    codes, sdup = _np(codes, np.uint32), _np(sdup, np.uint32)
+    L = _lib.lib()
+    grp = np.empty(Rb * 4, dtype=np.int32)
+    ng = _lib.check(L.mortar_octet_layout_host(_vp(offsets), Rb, None, None, None, _vp(grp), None, None, None),
+                    "mortar_octet_layout_host")
+    codes_o = np.empty(ng * 128, dtype=np.uint32)
+    sd_o = np.empty(ng * 8, dtype=np.uint32)
+    col_o = np.empty(ng * 8, dtype=np.int32)
+    _lib.check(L.mortar_octet_layout_host(_vp(offsets), Rb, _vp(codes), _vp(sdup), _vp(col), _vp(grp), _vp(codes_o),
+                                          _vp(sd_o), _vp(col_o)), "mortar_octet_layout_host")
+    return grp, codes_o, sd_o, col_o
+
+
 def unit_order(offsets, Rb: int, rows_per_unit: int) -> np.ndarray:
     offsets = _np(offsets, np.int32)
     group = _lib.lib().mortar_prefill_group(1 if rows_per_unit == 2 else 0)
@@ -111,10 +127,19 @@ class MortarPack:
         self.col = torch.from_numpy(self.h_col).to(dev)
         self.row_ptr = torch.from_numpy(self.h_offsets).to(dev)
         self.chunk_ptr = torch.from_numpy(self.h_chunk_ptr).to(dev)
+        grp, codes_o, sd_o, col_o = octet_layout(self.h_offsets, self.Rb, codes, sdup, self.h_col)
+        self.row_desc = torch.from_numpy(grp).to(dev)
+        self.codes_o = torch.from_numpy(codes_o.view(np.int32)).to(dev)
+        self.sd_o = torch.from_numpy(sd_o.view(np.int32)).to(dev)
+        self.col_o = torch.from_numpy(col_o).to(dev)
         self._orders: dict[int, torch.Tensor] = {}
         self._worklists: dict[tuple, tuple] = {}
-        self.struct = _lib.BcsrStruct(self.codes.data_ptr(), self.sdup.data_ptr(), self.col.data_ptr(),
-                                      self.row_ptr.data_ptr(), self.Rb, self.Cb, self.nnz)
+        self.struct = self._make_struct()
+
+    def _make_struct(self):
+        return _lib.BcsrStruct(self.codes.data_ptr(), self.sdup.data_ptr(), self.col.data_ptr(),
+                               self.row_ptr.data_ptr(), self.row_desc.data_ptr(), self.codes_o.data_ptr(),
+                               self.sd_o.data_ptr(), self.col_o.data_ptr(), self.Rb, self.Cb, self.nnz)
 
     def unit_order(self, rows_per_unit: int) -> torch.Tensor:
         if rows_per_unit not in self._orders:
@@ -138,10 +163,9 @@ class MortarPack:
         """A second resident copy (own device buffers and schedules) of the same matrix."""
         import copy
         c = copy.copy(self)
-        for name in ("codes", "sdup", "col", "row_ptr", "chunk_ptr"):
+        for name in ("codes", "sdup", "col", "row_ptr", "chunk_ptr", "row_desc", "codes_o", "sd_o", "col_o"):
             setattr(c, name, getattr(self, name).clone())
         c._orders = {k: v.clone() for k, v in self._orders.items()}
         c._worklists = {k: (v[0].clone(), v[1], v[2].clone(), v[3]) for k, v in self._worklists.items()}
-        c.struct = _lib.BcsrStruct(c.codes.data_ptr(), c.sdup.data_ptr(), c.col.data_ptr(), c.row_ptr.data_ptr(),
-                                   c.Rb, c.Cb, c.nnz)
+        c.struct = c._make_struct()
         return c
