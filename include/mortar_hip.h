@@ -43,10 +43,12 @@ enum {
  *   sdup    [nnz] uint32: per-block scale pattern produced by mortar_encode_blocks_host
  *   col     [nnz] the reference's mortar_column_indices (int16, unchanged)
  *   row_ptr [Rb+1] the reference's mortar_offsets (int32, unchanged)
- * Octet stream (second copy for the prefill kernels, from mortar_octet_layout_host): every row is cut into
- * groups of 8 blocks (the last one padded with all-zero blocks) so that one 16-byte load per lane fetches
- * the lane's code dwords of four consecutive block pairs:
- *   row_desc [Rb*4] int32 per row: {first group, end group, number of blocks, 0}
+ * Octet stream (second copy for the prefill kernels, from mortar_octet_layout_host): the block-columns are cut
+ * into nseg = ceil(Cb / seg_cb) K segments, and every (segment, row) run of blocks into groups of 8 blocks
+ * (the last one padded with all-zero blocks) so that one 16-byte load per lane fetches the lane's code dwords
+ * of four consecutive block pairs:
+ *   row_desc [nseg*Rb*4] int32 per (segment, row): {first group, end group, number of blocks, 0}
+ *   col_o holds block-columns relative to the segment start
  *   codes_o [ngroups*2*16*4] uint32: ((group*2 + s)*16 + n)*4 + t = row n of block 8*g + 2*t + s of the row
  *   sd_o    [ngroups*2*4] uint32 and col_o [ngroups*2*4] int32: (group*2 + s)*4 + t, same block             */
 typedef struct {
@@ -59,6 +61,7 @@ typedef struct {
     const uint32_t *sd_o;
     const int32_t *col_o;
     int32_t Rb, Cb, nnz;
+    int32_t seg_cb;   /* block-columns per K segment of the octet stream (>= Cb: one segment) */
 } mortar_bcsr_t;
 
 const char *mortar_last_error(void);
@@ -87,9 +90,14 @@ int mortar_chunk_ptr_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb
  * value is the number of groups.  With codes_o_out == NULL only row_desc_out is filled (size query);
  * otherwise codes_o_out [ngroups*128], sd_o_out [ngroups*8], col_o_out [ngroups*8] are filled from the
  * encoded codes / sdup and the column indices. */
-int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, const uint32_t *codes, const uint32_t *sdup,
-                                 const int16_t *col, int32_t *row_desc_out, uint32_t *codes_o_out,
-                                 uint32_t *sd_o_out, int32_t *col_o_out);
+int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, int32_t Cb, int32_t seg_cb,
+                                 const uint32_t *codes, const uint32_t *sdup, const int16_t *col,
+                                 int32_t *row_desc_out, uint32_t *codes_o_out, uint32_t *sd_o_out,
+                                 int32_t *col_o_out);
+
+/* Largest K segment (in block-columns) whose 32-token activation tile fits in LDS; a matrix with
+ * Cb <= this runs the single-segment prefill kernel.  Use seg_cb = ceil(Cb / ceil(Cb / max)). */
+int mortar_prefill_max_seg_cb(void);
 
 /* Row-unit schedule for uneven nnz: units sorted by descending block count and dealt so that every
  * workgroup of `group` units gets a similar total (longest-processing-time first).

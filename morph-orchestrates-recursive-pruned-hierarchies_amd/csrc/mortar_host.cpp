@@ -123,33 +123,47 @@ extern "C" int mortar_chunk_ptr_host(const int32_t *row_ptr, const int16_t *col,
     return MORTAR_OK;
 }
 
-extern "C" int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, const uint32_t *codes,
-                                            const uint32_t *sdup, const int16_t *col, int32_t *row_desc_out,
-                                            uint32_t *codes_o_out, uint32_t *sd_o_out, int32_t *col_o_out) {
-    if (!row_ptr || !row_desc_out || Rb <= 0) return mortar_fail(MORTAR_ERR_ARG, "octet_layout: bad argument");
-    int64_t ng = 0;
+extern "C" int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, int32_t Cb, int32_t seg_cb,
+                                            const uint32_t *codes, const uint32_t *sdup, const int16_t *col,
+                                            int32_t *row_desc_out, uint32_t *codes_o_out, uint32_t *sd_o_out,
+                                            int32_t *col_o_out) {
+    if (!row_ptr || !col || !row_desc_out || Rb <= 0 || Cb <= 0 || seg_cb <= 0)
+        return mortar_fail(MORTAR_ERR_ARG, "octet_layout: bad argument");
+    const int nseg = (Cb + seg_cb - 1) / seg_cb;
+    // block range of (segment, row): columns are ascending inside a row
+    std::vector<int32_t> lo((size_t)nseg * Rb), hi((size_t)nseg * Rb);
     for (int r = 0; r < Rb; ++r) {
-        const int nb = row_ptr[r + 1] - row_ptr[r];
-        row_desc_out[4 * r] = (int32_t)ng;
+        int p = row_ptr[r];
+        for (int sg = 0; sg < nseg; ++sg) {
+            lo[(size_t)sg * Rb + r] = p;
+            while (p < row_ptr[r + 1] && col[p] < (sg + 1) * seg_cb) ++p;
+            hi[(size_t)sg * Rb + r] = p;
+        }
+    }
+    int64_t ng = 0;
+    for (int64_t v = 0; v < (int64_t)nseg * Rb; ++v) {
+        const int nb = hi[v] - lo[v];
+        row_desc_out[4 * v] = (int32_t)ng;
         ng += (nb + 7) / 8;
-        row_desc_out[4 * r + 1] = (int32_t)ng;
-        row_desc_out[4 * r + 2] = nb;
-        row_desc_out[4 * r + 3] = 0;
+        row_desc_out[4 * v + 1] = (int32_t)ng;
+        row_desc_out[4 * v + 2] = nb;
+        row_desc_out[4 * v + 3] = 0;
         if (ng > 0x7fffffff / 128) return mortar_fail(MORTAR_ERR_LIMIT, "octet_layout: too many blocks");
     }
     if (!codes_o_out) return ng;
-    if (!codes || !sdup || !col || !sd_o_out || !col_o_out) return mortar_fail(MORTAR_ERR_ARG, "octet_layout: null pointer");
-    for (int r = 0; r < Rb; ++r) {
-        const int nb = row_ptr[r + 1] - row_ptr[r];
+    if (!codes || !sdup || !sd_o_out || !col_o_out) return mortar_fail(MORTAR_ERR_ARG, "octet_layout: null pointer");
+    for (int64_t v = 0; v < (int64_t)nseg * Rb; ++v) {
+        const int nb = hi[v] - lo[v];
+        const int c0 = (int)(v / Rb) * seg_cb;
         for (int gl = 0; gl * 8 < nb; ++gl) {
-            const int64_t gidx = row_desc_out[4 * r] + gl;
+            const int64_t gidx = row_desc_out[4 * v] + gl;
             for (int s2 = 0; s2 < 2; ++s2)
                 for (int t = 0; t < 4; ++t) {
                     const int b = 8 * gl + 2 * t + s2;
                     const bool ok = b < nb;
-                    const int64_t j = (int64_t)row_ptr[r] + b;
+                    const int64_t j = (int64_t)lo[v] + b;
                     sd_o_out[(gidx * 2 + s2) * 4 + t] = ok ? sdup[j] : 0u;
-                    col_o_out[(gidx * 2 + s2) * 4 + t] = ok ? (int32_t)col[j] : 0;
+                    col_o_out[(gidx * 2 + s2) * 4 + t] = ok ? (int32_t)col[j] - c0 : 0;
                     for (int n = 0; n < 16; ++n)
                         codes_o_out[((gidx * 2 + s2) * 16 + n) * 4 + t] = ok ? codes[j * 16 + n] : 0u;
                 }

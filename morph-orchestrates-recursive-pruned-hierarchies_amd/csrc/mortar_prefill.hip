@@ -44,6 +44,7 @@ struct SpmmParams {
     int n_clusters, cluster_size;
     int xcd_map, n_mtiles, n_groups;
     int n_split;              // resident kernel: workgroups that share one token tile
+    int seg_cb, nseg, Rb;     // segmented kernel: K segments of the octet stream
 };
 
 template <int MSUB, int RW, int NACC, bool ROUTED, bool MASKED>
@@ -564,11 +565,177 @@ int launch_resident_any(SpmmParams &p, hipStream_t st) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Segmented variant for matrices whose K does not fit in LDS at once (e.g. `down`, K = d_ff).  Same inner
+// loop as the resident kernel, but the workgroup walks the K segments of the octet stream: per segment it
+// stages x[32, 16*seg_cb] (one barrier pair), and every wave multiplies the segment's blocks of its own
+// UPW row units, whose accumulators stay in registers across all segments.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int SEG_WAVES = 16, SEG_UPW = 4;
+
+template <int NACC, bool MASKED>
+__global__ void __launch_bounds__(SEG_WAVES * 64) mortar_segmented_kernel(const SpmmParams p) {
+    constexpr int MSUB = 2, MT = 16 * MSUB, LDM = MT + 1;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint4 *lx = reinterpret_cast<uint4 *>(smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
+    const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
+    const int m0 = mt * MT;
+    const uint32_t lane_xo = (uint32_t)(hsel * LDM + n);
+    const bool has_gates = p.gates != nullptr;
+    const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;
+    const char *xt = reinterpret_cast<const char *>(p.x) + (int64_t)m0 * p.ldx * 2;
+
+    // this wave's units: positions u0 + wave + SEG_WAVES*k of the schedule
+    const int per = SEG_WAVES * SEG_UPW;
+    int units[SEG_UPW];
+#pragma unroll
+    for (int k = 0; k < SEG_UPW; ++k) {
+        const int pos = sp * per + wave + SEG_WAVES * k;
+        int u = -1;
+        if (pos < p.n_units) u = p.unit_order ? p.unit_order[pos] : pos;
+        units[k] = __builtin_amdgcn_readfirstlane(u);
+    }
+    f32x4_t acc[SEG_UPW][NACC][MSUB];
+#pragma unroll
+    for (int k = 0; k < SEG_UPW; ++k)
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int ms = 0; ms < MSUB; ++ms) acc[k][a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int sg = 0; sg < p.nseg; ++sg) {
+        const int c0 = sg * p.seg_cb;
+        const int ncb = p.Cb - c0 < p.seg_cb ? p.Cb - c0 : p.seg_cb;
+        const int nch = 2 * ncb;
+        // row descriptors of this segment (loaded before the barrier so that their latency is hidden)
+        u32x4_t desc[SEG_UPW][NACC];
+#pragma unroll
+        for (int k = 0; k < SEG_UPW; ++k)
+#pragma unroll
+            for (int a = 0; a < NACC; ++a)
+                desc[k][a] = p.row_desc[(int64_t)sg * p.Rb + (units[k] < 0 ? 0 : units[k] + a * p.n_units)];
+        if (sg > 0) __syncthreads();
+        for (int i0 = 0; i0 < nch * MT; i0 += SEG_WAVES * 64 * 4) {
+            uint4 v[4];
+            bool on[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                int i = i0 + k * SEG_WAVES * 64 + tid;
+                i = i < nch * MT ? i : nch * MT - 1;
+                const int ch = i % nch;
+                int row = i / nch;
+                row = row < rlast ? row : rlast;
+                v[k] = *reinterpret_cast<const uint4 *>(xt + (int64_t)row * p.ldx * 2 + (int64_t)c0 * 32 + ch * 16);
+                on[k] = true;
+                if (MASKED) on[k] = p.active[(int64_t)(m0 + row) * p.n_clusters + (c0 * 16 + ch * 8) / p.cluster_size] != 0;
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int i = i0 + k * SEG_WAVES * 64 + tid;
+                if (i < nch * MT) lx[(i % nch) * LDM + i / nch] = on[k] ? v[k] : make_uint4(0u, 0u, 0u, 0u);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < SEG_UPW; ++k) {
+            if (units[k] < 0) continue;
+#pragma unroll
+            for (int a = 0; a < NACC; ++a) {
+                const int g0 = __builtin_amdgcn_readfirstlane((int)desc[k][a][0]);
+                const int g1 = __builtin_amdgcn_readfirstlane((int)desc[k][a][1]);
+                const int nb = __builtin_amdgcn_readfirstlane((int)desc[k][a][2]);
+                for (int gq = g0; gq < g1; gq += RES_GROUPS) {
+                    u32x4_t cw[RES_GROUPS], sd[RES_GROUPS], cc[RES_GROUPS];
+#pragma unroll
+                    for (int q = 0; q < RES_GROUPS; ++q) {
+                        const uint32_t gi = (uint32_t)(gq + q < g1 ? gq + q : g1 - 1) * 2u + (uint32_t)bsel;
+                        cw[q] = p.codes_o[gi * 16u + n];
+                        sd[q] = p.sd_o[gi];
+                        cc[q] = p.col_o[gi];
+                    }
+                    const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;
+                    constexpr int NP = 4 * RES_GROUPS;
+                    uint4 Bq[3][MSUB];
+#pragma unroll
+                    for (int d = 0; d < 2; ++d) {
+                        const uint32_t xo = cc[d >> 2][d & 3] * (2 * LDM) + lane_xo;
+#pragma unroll
+                        for (int ms = 0; ms < MSUB; ++ms) Bq[d][ms] = lx[xo + ms * 16];
+                    }
+#pragma unroll
+                    for (int u = 0; u < NP; ++u) {
+                        if (u < pairs) {
+                            const u32x4_t A = mortar_unpack8(cw[u >> 2][u & 3] << (8 * hsel), sd[u >> 2][u & 3]);
+                            if (u + 2 < NP) {
+                                const uint32_t xo = cc[(u + 2) >> 2][(u + 2) & 3] * (2 * LDM) + lane_xo;
+#pragma unroll
+                                for (int ms = 0; ms < MSUB; ++ms) Bq[(u + 2) % 3][ms] = lx[xo + ms * 16];
+                            }
+#pragma unroll
+                            for (int ms = 0; ms < MSUB; ++ms) {
+                                const uint4 bq = Bq[u % 3][ms];
+                                const u32x4_t Bv = {bq.x, bq.y, bq.z, bq.w};
+                                acc[k][a][ms] = mortar_mfma(A, Bv, acc[k][a][ms]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int k = 0; k < SEG_UPW; ++k) {
+        if (units[k] < 0) continue;
+#pragma unroll
+        for (int ms = 0; ms < MSUB; ++ms) {
+            const int tok = m0 + ms * 16 + n;
+            if (tok >= p.M) continue;
+            u32x2_t pk;
+            if (NACC == 1) {
+                pk = u32x2_t{bf16_pack2(acc[k][0][ms][0], acc[k][0][ms][1]), bf16_pack2(acc[k][0][ms][2], acc[k][0][ms][3])};
+            } else {
+                float gv = 0.f;
+                if (has_gates) gv = p.gates[(int64_t)tok * p.n_clusters + (units[k] * 16 + 4 * g) / p.cluster_size];
+                pk = swiglu_pack4(acc[k][0][ms], acc[k][NACC - 1][ms], has_gates, gv);
+            }
+            *reinterpret_cast<u32x2_t *>(p.y + (int64_t)tok * p.ldy + units[k] * 16 + 4 * g) = pk;
+        }
+    }
+}
+
+template <int NACC, bool MASKED>
+int launch_segmented(SpmmParams &p, hipStream_t st) {
+    constexpr int MT = 32;
+    const int smem = 2 * p.seg_cb * (MT + 1) * 16;
+    static bool attr_done = false;
+    auto kern = mortar_segmented_kernel<NACC, MASKED>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        attr_done = true;
+    }
+    p.n_mtiles = (p.M + MT - 1) / MT;
+    p.n_split = (p.n_units + SEG_WAVES * SEG_UPW - 1) / (SEG_WAVES * SEG_UPW);
+    const int64_t grid = (int64_t)p.n_mtiles * p.n_split;
+    if (grid <= 0 || grid > 0x7fffffff) return mortar_fail(MORTAR_ERR_LIMIT, "prefill grid %lld out of range", (long long)grid);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(SEG_WAVES * 64), smem, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "prefill launch: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}
+
 int check_common(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const uint16_t *x, int64_t M, int64_t ldx,
                  const uint16_t *y, int64_t ldy, int64_t out_cols) {
     if (!W || !W->codes || !W->sdup || !W->col || !W->row_ptr || !W->row_desc || !W->codes_o || !W->sd_o || !W->col_o || !chunk_ptr || !x || !y)
         return mortar_fail(MORTAR_ERR_ARG, "prefill: null pointer");
     if (W->Rb <= 0 || W->Cb <= 0 || W->nnz <= 0) return mortar_fail(MORTAR_ERR_ARG, "prefill: empty matrix");
+    if (W->seg_cb <= 0 || (int64_t)2 * (W->seg_cb < W->Cb ? W->seg_cb : W->Cb) * 33 * 16 > 156 * 1024)
+        return mortar_fail(MORTAR_ERR_ARG, "prefill: seg_cb=%d does not fit LDS (max %d)", W->seg_cb, 156 * 1024 / (2 * 33 * 16));
     if (M <= 0 || M > (1 << 30)) return mortar_fail(MORTAR_ERR_ARG, "prefill: M=%lld out of range", (long long)M);
     if (ldx < (int64_t)W->Cb * 16 || ldx % 8) return mortar_fail(MORTAR_ERR_ARG, "prefill: ldx=%lld must be >= in_features and a multiple of 8", (long long)ldx);
     if (ldy < out_cols || ldy % 4) return mortar_fail(MORTAR_ERR_ARG, "prefill: ldy=%lld must be >= out_features and a multiple of 4", (long long)ldy);
@@ -585,6 +752,7 @@ void fill(SpmmParams &p, const mortar_bcsr_t *W, const int32_t *chunk_ptr, const
     p.codes_o = reinterpret_cast<const u32x4_t *>(W->codes_o);
     p.sd_o = reinterpret_cast<const u32x4_t *>(W->sd_o);
     p.col_o = reinterpret_cast<const u32x4_t *>(W->col_o);
+    p.seg_cb = W->seg_cb < W->Cb ? W->seg_cb : W->Cb; p.nseg = (W->Cb + p.seg_cb - 1) / p.seg_cb; p.Rb = W->Rb;
     p.unit_order = unit_order;
     p.nkc = (W->Cb + KCB - 1) / KCB; p.Cb = W->Cb;
     p.x = x; p.ldx = ldx; p.M = (int)M; p.y = y; p.ldy = ldy;
@@ -592,6 +760,8 @@ void fill(SpmmParams &p, const mortar_bcsr_t *W, const int32_t *chunk_ptr, const
 }
 
 }  // namespace
+
+extern "C" int mortar_prefill_max_seg_cb(void) { return 156 * 1024 / (2 * 33 * 16); }
 
 extern "C" int mortar_prefill_tile(int32_t Cb) {
     const int msub = resident_msub(Cb);
@@ -608,7 +778,8 @@ extern "C" int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr
     SpmmParams p;
     fill(p, W, chunk_ptr, unit_order, x, M, ldx, y, ldy);
     p.n_units = W->Rb;
-    if (resident_msub(W->Cb)) return launch_resident_any<1, false>(p, static_cast<hipStream_t>(stream));
+    if (p.nseg == 1) return launch_resident_any<1, false>(p, static_cast<hipStream_t>(stream));
+    return launch_segmented<1, false>(p, static_cast<hipStream_t>(stream));
     // few block-rows (e.g. `down`): halve the rows per workgroup so that the grid still covers every CU
     const int64_t wgs4 = ((M + 127) / 128) * ((W->Rb + NW * 8 - 1) / (NW * 8));
     if (wgs4 < 2 * 256) return launch<8, 4, 1, false, false>(p, static_cast<hipStream_t>(stream));
@@ -627,6 +798,7 @@ extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *ch
     fill(p, W, chunk_ptr, unit_order, x, M, ldx, y, ldy);
     p.n_units = W->Rb;
     p.active = active; p.n_clusters = n_clusters; p.cluster_size = (W->Cb * 16) / n_clusters;
+    return launch_segmented<1, true>(p, static_cast<hipStream_t>(stream));
     const int64_t wgs4 = ((M + 127) / 128) * ((W->Rb + NW * 8 - 1) / (NW * 8));
     if (wgs4 < 2 * 256) return launch<8, 4, 1, false, true>(p, static_cast<hipStream_t>(stream));
     return launch<8, 8, 1, false, true>(p, static_cast<hipStream_t>(stream));
@@ -652,9 +824,9 @@ extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *
         if (!tok_cnt || !tok_list || !gates) return mortar_fail(MORTAR_ERR_ARG, "gateup: routed mode needs gates, tok_cnt and tok_list");
         if (p.cluster_size % 16) return mortar_fail(MORTAR_ERR_ARG, "gateup: routed mode needs cluster_size %% 16 == 0");
         p.tok_cnt = tok_cnt; p.tok_list = tok_list;
-        if (resident_msub(W->Cb)) return launch_resident_any<2, true>(p, static_cast<hipStream_t>(stream));
+        if (p.nseg == 1) return launch_resident_any<2, true>(p, static_cast<hipStream_t>(stream));
         return launch<8, 4, 2, true, false>(p, static_cast<hipStream_t>(stream));
     }
-    if (resident_msub(W->Cb)) return launch_resident_any<2, false>(p, static_cast<hipStream_t>(stream));
-    return launch<8, 4, 2, false, false>(p, static_cast<hipStream_t>(stream));
+    if (p.nseg == 1) return launch_resident_any<2, false>(p, static_cast<hipStream_t>(stream));
+    return launch_segmented<2, false>(p, static_cast<hipStream_t>(stream));
 }

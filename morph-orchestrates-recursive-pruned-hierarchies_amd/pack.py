@@ -58,19 +58,20 @@ def chunk_ptr(offsets, col, Rb: int, Cb: int, kcb: int = PREFILL_KCB) -> np.ndar
     return out
 
 
-def octet_layout(offsets, Rb: int, codes: np.ndarray, sdup: np.ndarray, col):
-    """-> (row_desc [Rb*4] int32, codes_o uint32, sd_o uint32, col_o int32): see mortar_octet_layout_host."""
+def octet_layout(offsets, Rb: int, Cb: int, seg_cb: int, codes: np.ndarray, sdup: np.ndarray, col):
+    """-> (row_desc [nseg*Rb*4] int32, codes_o uint32, sd_o uint32, col_o int32): see mortar_octet_layout_host."""
     offsets, col = _np(offsets, np.int32), _np(col, np.int16)
     codes, sdup = _np(codes, np.uint32), _np(sdup, np.uint32)
     L = _lib.lib()
-    grp = np.empty(Rb * 4, dtype=np.int32)
-    ng = _lib.check(L.mortar_octet_layout_host(_vp(offsets), Rb, None, None, None, _vp(grp), None, None, None),
+    nseg = -(-Cb // seg_cb)
+    grp = np.empty(nseg * Rb * 4, dtype=np.int32)
+    ng = _lib.check(L.mortar_octet_layout_host(_vp(offsets), Rb, Cb, seg_cb, None, None, _vp(col), _vp(grp), None, None, None),
                     "mortar_octet_layout_host")
     codes_o = np.empty(ng * 128, dtype=np.uint32)
     sd_o = np.empty(ng * 8, dtype=np.uint32)
     col_o = np.empty(ng * 8, dtype=np.int32)
-    _lib.check(L.mortar_octet_layout_host(_vp(offsets), Rb, _vp(codes), _vp(sdup), _vp(col), _vp(grp), _vp(codes_o),
-                                          _vp(sd_o), _vp(col_o)), "mortar_octet_layout_host")
+    _lib.check(L.mortar_octet_layout_host(_vp(offsets), Rb, Cb, seg_cb, _vp(codes), _vp(sdup), _vp(col), _vp(grp),
+                                          _vp(codes_o), _vp(sd_o), _vp(col_o)), "mortar_octet_layout_host")
     return grp, codes_o, sd_o, col_o
 
 
@@ -127,7 +128,10 @@ class MortarPack:
         self.col = torch.from_numpy(self.h_col).to(dev)
         self.row_ptr = torch.from_numpy(self.h_offsets).to(dev)
         self.chunk_ptr = torch.from_numpy(self.h_chunk_ptr).to(dev)
-        grp, codes_o, sd_o, col_o = octet_layout(self.h_offsets, self.Rb, codes, sdup, self.h_col)
+        max_seg = int(_lib.lib().mortar_prefill_max_seg_cb())
+        nseg = -(-self.Cb // max_seg)
+        self.seg_cb = -(-self.Cb // nseg)
+        grp, codes_o, sd_o, col_o = octet_layout(self.h_offsets, self.Rb, self.Cb, self.seg_cb, codes, sdup, self.h_col)
         self.row_desc = torch.from_numpy(grp).to(dev)
         self.codes_o = torch.from_numpy(codes_o.view(np.int32)).to(dev)
         self.sd_o = torch.from_numpy(sd_o.view(np.int32)).to(dev)
@@ -139,7 +143,7 @@ class MortarPack:
     def _make_struct(self):
         return _lib.BcsrStruct(self.codes.data_ptr(), self.sdup.data_ptr(), self.col.data_ptr(),
                                self.row_ptr.data_ptr(), self.row_desc.data_ptr(), self.codes_o.data_ptr(),
-                               self.sd_o.data_ptr(), self.col_o.data_ptr(), self.Rb, self.Cb, self.nnz)
+                               self.sd_o.data_ptr(), self.col_o.data_ptr(), self.Rb, self.Cb, self.nnz, self.seg_cb)
 
     def unit_order(self, rows_per_unit: int) -> torch.Tensor:
         if rows_per_unit not in self._orders:
