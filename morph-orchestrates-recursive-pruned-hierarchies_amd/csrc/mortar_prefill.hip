@@ -4,14 +4,14 @@
 // custom_ops.py:35-56) and, in gate_up mode, fuses the SwiGLU of _SwiGLUMortar.forward
 // (morph/model/transformer.py:402-431) into the epilogue.
 //
-// Work decomposition.  A workgroup (4 wavefronts) owns a tile of MT = 16*MSUB tokens and NW*RW row units
-// (a unit is one 16-row block-row, or a gate/up pair of block-rows).  It walks K in chunks of KCB
-// block-columns.  Per chunk the token tile x[MT, 16*KCB] is staged in LDS as 16-byte units
-// [column-half][token] (token stride padded by one unit so both the staging writes and the MFMA operand
-// reads are bank-conflict free), and every wave stages the packed blocks of its own rows that fall into the
-// chunk (found through the chunk pointer table).  Accumulators stay in registers across all chunks, so each
-// output element is written exactly once.  Per MFMA the weights of two blocks are unpacked in registers once
-// and reused for the MSUB token sub-tiles; the activation operand is one 16-byte LDS read per lane.
+// Three kernels share the inner step (unpack the ternary codes of two blocks in registers, read the
+// activation operand from LDS, one 16x16x32 MFMA per 16 tokens):
+//   mortar_resident_kernel   in_features fits LDS for a 32..96-token tile: stage x once, every wave then walks
+//                            whole row units on its own from the octet weight stream (no K loop, no barriers)
+//   mortar_segmented_kernel  wide K (e.g. `down`): the same, with K cut into LDS-sized segments and the
+//                            accumulators of a wave's few row units kept in registers across segments
+//   mortar_spmm_kernel       K-chunked kernel with 128-token tiles and one wave per SIMD; serves the routed
+//                            gate_up of matrices that are too wide for the resident kernel
 #include "mortar_device.h"
 #include "mortar_internal.h"
 
@@ -780,10 +780,6 @@ extern "C" int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr
     p.n_units = W->Rb;
     if (p.nseg == 1) return launch_resident_any<1, false>(p, static_cast<hipStream_t>(stream));
     return launch_segmented<1, false>(p, static_cast<hipStream_t>(stream));
-    // few block-rows (e.g. `down`): halve the rows per workgroup so that the grid still covers every CU
-    const int64_t wgs4 = ((M + 127) / 128) * ((W->Rb + NW * 8 - 1) / (NW * 8));
-    if (wgs4 < 2 * 256) return launch<8, 4, 1, false, false>(p, static_cast<hipStream_t>(stream));
-    return launch<8, 8, 1, false, false>(p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *chunk_ptr,
@@ -799,9 +795,6 @@ extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *ch
     p.n_units = W->Rb;
     p.active = active; p.n_clusters = n_clusters; p.cluster_size = (W->Cb * 16) / n_clusters;
     return launch_segmented<1, true>(p, static_cast<hipStream_t>(stream));
-    const int64_t wgs4 = ((M + 127) / 128) * ((W->Rb + NW * 8 - 1) / (NW * 8));
-    if (wgs4 < 2 * 256) return launch<8, 4, 1, false, true>(p, static_cast<hipStream_t>(stream));
-    return launch<8, 8, 1, false, true>(p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr,
