@@ -128,7 +128,7 @@ int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int
  * [0, d_ff) and up rows [d_ff, 2*d_ff) (transformer.py:335-336,403-405).  Intermediates are rounded to
  * bf16 where the reference materialises a bf16 tensor.  gates: device fp32 [M, n_clusters] or NULL;
  * d_ff % n_clusters == 0.
- * Routed skipping (optional): tok_cnt/tok_list from mortar_remoe_route with tile = mortar_prefill_tile(Cb); when
+ * Routed skipping (optional): tok_cnt/tok_list from mortar_remoe_route with tile = mortar_prefill_tile(Cb, M); when
  * given (requires cluster_size % 16 == 0) only active (token, block-row) tiles are computed and written;
  * inactive entries of h are left untouched and must be masked by the consumer (mortar_spmm_bf16_masked). */
 int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int32_t *unit_order,
@@ -142,9 +142,10 @@ int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *chunk_ptr, co
                             const uint16_t *x, int64_t M, int64_t ldx, uint16_t *y, int64_t ldy,
                             const uint8_t *active, int32_t n_clusters, void *stream);
 
-/* Token tile the prefill kernels use for a matrix with Cb block-columns: the tile size that
- * mortar_remoe_route must be called with for routed mortar_gateup_swiglu_bf16 on that matrix. */
-int mortar_prefill_tile(int32_t Cb);
+/* Token tile the gate_up kernels use for M rows against a matrix with Cb block-columns: the tile size that
+ * mortar_remoe_route must be called with for routed mortar_gateup_swiglu_bf16 on that (matrix, M).
+ * 4 or 16 for decode-sized M (<= 16), otherwise a multiple of 16 that depends on Cb only. */
+int mortar_prefill_tile(int32_t Cb, int64_t M);
 
 /* Units per prefill workgroup (for mortar_unit_order_host): swiglu = 0 plain, 1 gate/up pairs. */
 int mortar_prefill_group(int swiglu);
@@ -158,7 +159,7 @@ int mortar_remoe_gates(const float *logits, int64_t M, int32_t n, int32_t k, flo
                        void *stream);
 
 /* Wavefront-ballot compaction of active tokens per (token tile, cluster):
- * tok_cnt[t*n + c] = number of tokens of tile t (tile tokens each, a multiple of 16, <= 256) with active[m, c] != 0,
+ * tok_cnt[t*n + c] = number of tokens of tile t (tile tokens each: 4 or a multiple of 16, <= 256) with active[m, c] != 0,
  * tok_list[(t*n + c)*tile + i] = tile-local index of the i-th such token, ascending. */
 int mortar_remoe_route(const uint8_t *active, int64_t M, int32_t n, int32_t tile, int32_t *tok_cnt,
                        uint8_t *tok_list, void *stream);
@@ -170,6 +171,27 @@ int mortar_route_flags(const float *gates, int64_t B, int32_t n_clusters, int64_
                        int32_t *row_act, int64_t ldr, int32_t *col_act, int64_t ldc, void *stream);
 
 /* ---- decode (M <= 64) ------------------------------------------------------------------------ */
+
+/* mortar_spmm_bf16 / mortar_gateup_swiglu_bf16 / mortar_spmm_bf16_masked serve decode batches directly: for
+ * M <= 16 they run small-tile variants (4- or 16-token tile, small workgroups) that read every weight block
+ * once per launch.  That path replaces mortar_gemv of fused_decode_step.py:1701-1842 for the MLP pair.
+ *
+ * Layer-batched form for M <= 16: ONE launch runs the same operation on n_layers independent
+ * (matrix, input, output) triples of identical shape (Rb, Cb, seg_cb).  No counterpart in the reference,
+ * whose decode megakernel walks its layers inside one persistent program (fused_decode_step.py:2104-2300);
+ * this is the launch-level equivalent for callers that hold many weight sets (a stack of layers whose
+ * inputs are known, several models, bandwidth measurement).
+ *   mortar_stack_table_bytes  bytes of device memory the parameter table needs
+ *   mortar_stack_prepare      validates the layers, writes the table (synchronous host-to-device copy);
+ *                             W: host array [n_layers] of descriptors with device pointers, x / y: host arrays
+ *                             of device pointers; swiglu = 0: y_l = x_l W_l^T, 1: y_l = silu(g) * u of gate_up W_l
+ *   mortar_stack_run          launches the prepared table (any number of times); W0 = &W[0], same swiglu,
+ *                             n_layers and M as prepared */
+int64_t mortar_stack_table_bytes(int32_t n_layers);
+int mortar_stack_prepare(int32_t swiglu, int32_t n_layers, const mortar_bcsr_t *W, const uint16_t *const *x,
+                         uint16_t *const *y, int64_t M, int64_t ldx, int64_t ldy, void *table_dev, void *stream);
+int mortar_stack_run(int32_t swiglu, int32_t n_layers, const mortar_bcsr_t *W0, int64_t M, const void *table_dev,
+                     void *stream);
 
 /* Generic decode GEMV over a work list (mortar_decode_worklist_host; entries on the device).
  * x bf16 [B, Cb*16]; B <= 64.

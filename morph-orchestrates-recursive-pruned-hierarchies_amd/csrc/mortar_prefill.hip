@@ -12,40 +12,14 @@
 //                            accumulators of a wave's few row units kept in registers across segments
 //   mortar_spmm_kernel       K-chunked kernel with 128-token tiles and one wave per SIMD; serves the routed
 //                            gate_up of matrices that are too wide for the resident kernel
-#include "mortar_device.h"
-#include "mortar_internal.h"
+#include "mortar_spmm_core.h"
+
+#include <vector>
 
 namespace {
 
 constexpr int KCB = MORTAR_PREFILL_KCB;
 constexpr int NW = 4;   // wavefronts per workgroup (one per SIMD, 512 registers each)
-
-struct SpmmParams {
-    const uint32_t *codes;
-    const uint32_t *sdup;
-    const int16_t *col;
-    const int32_t *chunk_ptr;
-    const int32_t *row_ptr;
-    const u32x4_t *row_desc;  // octet stream (resident kernel)
-    const u32x4_t *codes_o;
-    const u32x4_t *sd_o;
-    const u32x4_t *col_o;
-    const int32_t *unit_order;
-    int n_units, nkc, Cb;
-    const uint16_t *x;
-    int64_t ldx;
-    int M;
-    uint16_t *y;
-    int64_t ldy;
-    const float *gates;       // [M, n_clusters] fp32 or null
-    const uint8_t *active;    // [M, n_clusters] input mask or null
-    const int32_t *tok_cnt;   // routed: [n_mtiles, n_clusters]
-    const uint8_t *tok_list;  // routed: [n_mtiles, n_clusters, MT]
-    int n_clusters, cluster_size;
-    int xcd_map, n_mtiles, n_groups;
-    int n_split;              // resident kernel: workgroups that share one token tile
-    int seg_cb, nseg, Rb;     // segmented kernel: K segments of the octet stream
-};
 
 template <int MSUB, int RW, int NACC, bool ROUTED, bool MASKED>
 __global__ void __launch_bounds__(NW * 64, 1) mortar_spmm_kernel(const SpmmParams p) {
@@ -355,380 +329,6 @@ int launch(SpmmParams &p, hipStream_t st) {
 }
 
 
-// ---------------------------------------------------------------------------------------------------------
-// Resident-activation variant, used when a token tile of ALL K columns fits in LDS (in_features <= 2480 at
-// 32 tokens).  The workgroup (16 wavefronts) stages x[MT, K] once, then every wave walks whole row units on
-// its own: it streams the unit's block pairs straight from global memory in batches (a row's blocks are
-// contiguous), unpacks them in registers and multiplies against the resident tile.  There is no K chunking,
-// no barrier after the first one and no per-chunk staging; latency is hidden by the four waves per SIMD.
-// ---------------------------------------------------------------------------------------------------------
-constexpr int RES_GROUPS = 4;    // octets (4 block pairs each) loaded per batch
-// wavefronts per workgroup: 16 (4 per SIMD, 128 registers) for the 32-token tile, 8 for larger tiles
-constexpr int res_waves(int msub) { return msub <= 2 ? 16 : 8; }
-
-template <int MSUB, int NACC, bool ROUTED>
-__global__ void __launch_bounds__(res_waves(MSUB) * 64) mortar_resident_kernel(const SpmmParams p) {
-    constexpr int MT = 16 * MSUB, LDM = MT + 1, RES_WAVES = res_waves(MSUB);
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    uint4 *lx = reinterpret_cast<uint4 *>(smem);
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
-    const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
-    const int m0 = mt * MT;
-    const uint32_t lane_xo = (uint32_t)(hsel * LDM + (ROUTED ? 0 : n));
-    const bool has_gates = p.gates != nullptr;
-
-    // ---- stage the token tile: unit (ch, row) <- x[m0 + row, ch*8 .. ch*8+8]; rows past M repeat the last row
-    {
-        const int nch = 2 * p.Cb;
-        const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;
-        const char *xt = reinterpret_cast<const char *>(p.x) + (int64_t)m0 * p.ldx * 2;
-        for (int i0 = 0; i0 < nch * MT; i0 += RES_WAVES * 64 * 4) {
-            uint4 v[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                int i = i0 + k * RES_WAVES * 64 + tid;
-                i = i < nch * MT ? i : nch * MT - 1;
-                const int ch = i % nch;
-                int row = i / nch;
-                row = row < rlast ? row : rlast;
-                v[k] = *reinterpret_cast<const uint4 *>(xt + (int64_t)row * p.ldx * 2 + ch * 16);
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int i = i0 + k * RES_WAVES * 64 + tid;
-                if (i < nch * MT) lx[(i % nch) * LDM + i / nch] = v[k];
-            }
-        }
-    }
-    __syncthreads();
-
-    const int per = (p.n_units + p.n_split - 1) / p.n_split;
-    const int u_end = (sp + 1) * per < p.n_units ? (sp + 1) * per : p.n_units;
-    // Unit ids are fetched two units ahead and row descriptors one unit ahead, so that no dependent global
-    // round trip (order -> descriptor -> blocks) is exposed between two units of a wave.
-    auto unit_of = [&](int pos_) { return (p.unit_order && pos_ < u_end) ? p.unit_order[pos_] : pos_; };
-    auto desc_of = [&](int unit_, int a_) {
-        const int r = unit_ + a_ * p.n_units;
-        return p.row_desc[r < NACC * p.n_units ? r : 0];
-    };
-    int pos = sp * per + wave;
-    int unit_v = unit_of(pos), unit_v1 = unit_of(pos + RES_WAVES);
-    u32x4_t dcur[NACC], dnxt[NACC];
-#pragma unroll
-    for (int a = 0; a < NACC; ++a) dcur[a] = desc_of(unit_v, a);
-    for (; pos < u_end; pos += RES_WAVES) {
-        const int unit = __builtin_amdgcn_readfirstlane(unit_v);
-        const int unit_v2 = unit_of(pos + 2 * RES_WAVES);
-#pragma unroll
-        for (int a = 0; a < NACC; ++a) dnxt[a] = desc_of(unit_v1 < p.n_units ? unit_v1 : 0, a);
-        int cnt = MT;
-        uint32_t tk[MSUB];
-#pragma unroll
-        for (int ms = 0; ms < MSUB; ++ms) tk[ms] = ms * 16 + n;
-        bool skip = false;
-        if (ROUTED) {
-            const int cl = (unit * 16) / p.cluster_size;
-            const int64_t e = (int64_t)mt * p.n_clusters + cl;
-            cnt = __builtin_amdgcn_readfirstlane(p.tok_cnt[e]);
-            skip = cnt == 0;
-#pragma unroll
-            for (int ms = 0; ms < MSUB; ++ms) {
-                const int i = ms * 16 + n;
-                tk[ms] = i < cnt ? p.tok_list[e * MT + i] : 0;
-            }
-        }
-        int rg0[NACC], rg1[NACC], rnb[NACC];
-#pragma unroll
-        for (int a = 0; a < NACC; ++a) {
-            rg0[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][0]);
-            rg1[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][1]);
-            rnb[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][2]);
-            dcur[a] = dnxt[a];
-        }
-        unit_v = unit_v1;
-        unit_v1 = unit_v2;
-        if (skip) continue;
-        const int nsub = ROUTED ? (cnt + 15) >> 4 : MSUB;
-        f32x4_t acc[NACC][MSUB];
-#pragma unroll
-        for (int a = 0; a < NACC; ++a)
-#pragma unroll
-            for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-#pragma unroll
-        for (int a = 0; a < NACC; ++a) {
-            const int g0 = rg0[a], g1 = rg1[a], nb = rnb[a];
-            // One batch = RES_GROUPS octets (8 blocks = 4 pairs each).  Per octet a lane needs three 16-byte
-            // loads: its code dwords, scale patterns and block-columns of the four pairs.
-            for (int gq = g0; gq < g1; gq += RES_GROUPS) {
-                u32x4_t cw[RES_GROUPS], sd[RES_GROUPS], cc[RES_GROUPS];
-#pragma unroll
-                for (int k = 0; k < RES_GROUPS; ++k) {
-                    const uint32_t gi = (uint32_t)(gq + k < g1 ? gq + k : g1 - 1) * 2u + (uint32_t)bsel;
-                    cw[k] = p.codes_o[gi * 16u + n];
-                    sd[k] = p.sd_o[gi];
-                    cc[k] = p.col_o[gi];
-                }
-                const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;      // block pairs left in the row from this batch on
-                // activation operands are fetched two pairs ahead of the MFMAs that use them
-                constexpr int NP = 4 * RES_GROUPS;
-                uint4 Bq[3][MSUB];
-#pragma unroll
-                for (int d = 0; d < 2; ++d) {
-                    const uint32_t xo = cc[d >> 2][d & 3] * (2 * LDM) + lane_xo;
-#pragma unroll
-                    for (int ms = 0; ms < MSUB; ++ms) Bq[d][ms] = lx[xo + (ROUTED ? tk[ms] : ms * 16)];
-                }
-#pragma unroll
-                for (int u = 0; u < NP; ++u) {
-                    if (u < pairs) {
-                        const u32x4_t A = mortar_unpack8(cw[u >> 2][u & 3] << (8 * hsel), sd[u >> 2][u & 3]);
-                        if (u + 2 < NP) {
-                            const uint32_t xo = cc[(u + 2) >> 2][(u + 2) & 3] * (2 * LDM) + lane_xo;
-#pragma unroll
-                            for (int ms = 0; ms < MSUB; ++ms) Bq[(u + 2) % 3][ms] = lx[xo + (ROUTED ? tk[ms] : ms * 16)];
-                        }
-#pragma unroll
-                        for (int ms = 0; ms < MSUB; ++ms) {
-                            if (!ROUTED || ms < nsub) {
-                                const uint4 bq = Bq[u % 3][ms];
-                                const u32x4_t Bv = {bq.x, bq.y, bq.z, bq.w};
-                                acc[a][ms] = mortar_mfma(A, Bv, acc[a][ms]);
-                            }
-                        }
-                    }
-                }
-            }
-        }
-
-        // epilogue: lane holds D[4g+v][token]
-#pragma unroll
-        for (int ms = 0; ms < MSUB; ++ms) {
-            const int li = ms * 16 + n;
-            if (ROUTED && li >= cnt) continue;
-            const int tok = m0 + (int)tk[ms];
-            if (tok >= p.M) continue;
-            u32x2_t pk;
-            if (NACC == 1) {
-                pk = u32x2_t{bf16_pack2(acc[0][ms][0], acc[0][ms][1]), bf16_pack2(acc[0][ms][2], acc[0][ms][3])};
-            } else {
-                float gv = 0.f;
-                if (has_gates) gv = p.gates[(int64_t)tok * p.n_clusters + (unit * 16 + 4 * g) / p.cluster_size];
-                pk = swiglu_pack4(acc[0][ms], acc[NACC - 1][ms], has_gates, gv);
-            }
-            *reinterpret_cast<u32x2_t *>(p.y + (int64_t)tok * p.ldy + unit * 16 + 4 * g) = pk;
-        }
-    }
-}
-
-// Token tile of the resident kernel for a matrix with Cb block-columns (0 = does not fit).
-int resident_msub(int Cb) {
-    for (int msub : {6, 4, 2})
-        if ((int64_t)2 * Cb * (16 * msub + 1) * 16 <= 156 * 1024) return msub;
-    return 0;
-}
-
-template <int MSUB, int NACC, bool ROUTED>
-int launch_resident(SpmmParams &p, hipStream_t st) {
-    constexpr int MT = 16 * MSUB, RES_WAVES = res_waves(MSUB);
-    const int smem = 2 * p.Cb * (MT + 1) * 16;
-    static bool attr_done = false;
-    auto kern = mortar_resident_kernel<MSUB, NACC, ROUTED>;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-        attr_done = true;
-    }
-    p.n_mtiles = (p.M + MT - 1) / MT;
-    // enough workgroups to cover the 256 CUs, but at least RES_WAVES units per workgroup
-    int split = (2 * 256 + p.n_mtiles - 1) / p.n_mtiles;
-    const int max_split = (p.n_units + RES_WAVES - 1) / RES_WAVES;
-    split = split < 1 ? 1 : (split > max_split ? max_split : split);
-    p.n_split = split;
-    const int64_t grid = (int64_t)p.n_mtiles * split;
-    if (grid <= 0 || grid > 0x7fffffff) return mortar_fail(MORTAR_ERR_LIMIT, "prefill grid %lld out of range", (long long)grid);
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(RES_WAVES * 64), smem, st, p);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "prefill launch: %s", hipGetErrorString(e));
-    return MORTAR_OK;
-}
-
-template <int NACC, bool ROUTED>
-int launch_resident_any(SpmmParams &p, hipStream_t st) {
-    switch (resident_msub(p.Cb)) {
-        case 6: return launch_resident<6, NACC, ROUTED>(p, st);
-        case 4: return launch_resident<4, NACC, ROUTED>(p, st);
-        default: return launch_resident<2, NACC, ROUTED>(p, st);
-    }
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// Segmented variant for matrices whose K does not fit in LDS at once (e.g. `down`, K = d_ff).  Same inner
-// loop as the resident kernel, but the workgroup walks the K segments of the octet stream: per segment it
-// stages x[32, 16*seg_cb] (one barrier pair), and every wave multiplies the segment's blocks of its own
-// UPW row units, whose accumulators stay in registers across all segments.
-// ---------------------------------------------------------------------------------------------------------
-constexpr int SEG_WAVES = 16, SEG_UPW = 4;
-
-template <int NACC, bool MASKED>
-__global__ void __launch_bounds__(SEG_WAVES * 64) mortar_segmented_kernel(const SpmmParams p) {
-    constexpr int MSUB = 2, MT = 16 * MSUB, LDM = MT + 1;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    uint4 *lx = reinterpret_cast<uint4 *>(smem);
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
-    const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
-    const int m0 = mt * MT;
-    const uint32_t lane_xo = (uint32_t)(hsel * LDM + n);
-    const bool has_gates = p.gates != nullptr;
-    const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;
-    const char *xt = reinterpret_cast<const char *>(p.x) + (int64_t)m0 * p.ldx * 2;
-
-    // this wave's units: positions u0 + wave + SEG_WAVES*k of the schedule
-    const int per = SEG_WAVES * SEG_UPW;
-    int units[SEG_UPW];
-#pragma unroll
-    for (int k = 0; k < SEG_UPW; ++k) {
-        const int pos = sp * per + wave + SEG_WAVES * k;
-        int u = -1;
-        if (pos < p.n_units) u = p.unit_order ? p.unit_order[pos] : pos;
-        units[k] = __builtin_amdgcn_readfirstlane(u);
-    }
-    f32x4_t acc[SEG_UPW][NACC][MSUB];
-#pragma unroll
-    for (int k = 0; k < SEG_UPW; ++k)
-#pragma unroll
-        for (int a = 0; a < NACC; ++a)
-#pragma unroll
-            for (int ms = 0; ms < MSUB; ++ms) acc[k][a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-    for (int sg = 0; sg < p.nseg; ++sg) {
-        const int c0 = sg * p.seg_cb;
-        const int ncb = p.Cb - c0 < p.seg_cb ? p.Cb - c0 : p.seg_cb;
-        const int nch = 2 * ncb;
-        // row descriptors of this segment (loaded before the barrier so that their latency is hidden)
-        u32x4_t desc[SEG_UPW][NACC];
-#pragma unroll
-        for (int k = 0; k < SEG_UPW; ++k)
-#pragma unroll
-            for (int a = 0; a < NACC; ++a)
-                desc[k][a] = p.row_desc[(int64_t)sg * p.Rb + (units[k] < 0 ? 0 : units[k] + a * p.n_units)];
-        if (sg > 0) __syncthreads();
-        for (int i0 = 0; i0 < nch * MT; i0 += SEG_WAVES * 64 * 4) {
-            uint4 v[4];
-            bool on[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                int i = i0 + k * SEG_WAVES * 64 + tid;
-                i = i < nch * MT ? i : nch * MT - 1;
-                const int ch = i % nch;
-                int row = i / nch;
-                row = row < rlast ? row : rlast;
-                v[k] = *reinterpret_cast<const uint4 *>(xt + (int64_t)row * p.ldx * 2 + (int64_t)c0 * 32 + ch * 16);
-                on[k] = true;
-                if (MASKED) on[k] = p.active[(int64_t)(m0 + row) * p.n_clusters + (c0 * 16 + ch * 8) / p.cluster_size] != 0;
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int i = i0 + k * SEG_WAVES * 64 + tid;
-                if (i < nch * MT) lx[(i % nch) * LDM + i / nch] = on[k] ? v[k] : make_uint4(0u, 0u, 0u, 0u);
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < SEG_UPW; ++k) {
-            if (units[k] < 0) continue;
-#pragma unroll
-            for (int a = 0; a < NACC; ++a) {
-                const int g0 = __builtin_amdgcn_readfirstlane((int)desc[k][a][0]);
-                const int g1 = __builtin_amdgcn_readfirstlane((int)desc[k][a][1]);
-                const int nb = __builtin_amdgcn_readfirstlane((int)desc[k][a][2]);
-                for (int gq = g0; gq < g1; gq += RES_GROUPS) {
-                    u32x4_t cw[RES_GROUPS], sd[RES_GROUPS], cc[RES_GROUPS];
-#pragma unroll
-                    for (int q = 0; q < RES_GROUPS; ++q) {
-                        const uint32_t gi = (uint32_t)(gq + q < g1 ? gq + q : g1 - 1) * 2u + (uint32_t)bsel;
-                        cw[q] = p.codes_o[gi * 16u + n];
-                        sd[q] = p.sd_o[gi];
-                        cc[q] = p.col_o[gi];
-                    }
-                    const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;
-                    constexpr int NP = 4 * RES_GROUPS;
-                    uint4 Bq[3][MSUB];
-#pragma unroll
-                    for (int d = 0; d < 2; ++d) {
-                        const uint32_t xo = cc[d >> 2][d & 3] * (2 * LDM) + lane_xo;
-#pragma unroll
-                        for (int ms = 0; ms < MSUB; ++ms) Bq[d][ms] = lx[xo + ms * 16];
-                    }
-#pragma unroll
-                    for (int u = 0; u < NP; ++u) {
-                        if (u < pairs) {
-                            const u32x4_t A = mortar_unpack8(cw[u >> 2][u & 3] << (8 * hsel), sd[u >> 2][u & 3]);
-                            if (u + 2 < NP) {
-                                const uint32_t xo = cc[(u + 2) >> 2][(u + 2) & 3] * (2 * LDM) + lane_xo;
-#pragma unroll
-                                for (int ms = 0; ms < MSUB; ++ms) Bq[(u + 2) % 3][ms] = lx[xo + ms * 16];
-                            }
-#pragma unroll
-                            for (int ms = 0; ms < MSUB; ++ms) {
-                                const uint4 bq = Bq[u % 3][ms];
-                                const u32x4_t Bv = {bq.x, bq.y, bq.z, bq.w};
-                                acc[k][a][ms] = mortar_mfma(A, Bv, acc[k][a][ms]);
-                            }
-                        }
-                    }
-                }
-            }
-        }
-    }
-
-#pragma unroll
-    for (int k = 0; k < SEG_UPW; ++k) {
-        if (units[k] < 0) continue;
-#pragma unroll
-        for (int ms = 0; ms < MSUB; ++ms) {
-            const int tok = m0 + ms * 16 + n;
-            if (tok >= p.M) continue;
-            u32x2_t pk;
-            if (NACC == 1) {
-                pk = u32x2_t{bf16_pack2(acc[k][0][ms][0], acc[k][0][ms][1]), bf16_pack2(acc[k][0][ms][2], acc[k][0][ms][3])};
-            } else {
-                float gv = 0.f;
-                if (has_gates) gv = p.gates[(int64_t)tok * p.n_clusters + (units[k] * 16 + 4 * g) / p.cluster_size];
-                pk = swiglu_pack4(acc[k][0][ms], acc[k][NACC - 1][ms], has_gates, gv);
-            }
-            *reinterpret_cast<u32x2_t *>(p.y + (int64_t)tok * p.ldy + units[k] * 16 + 4 * g) = pk;
-        }
-    }
-}
-
-template <int NACC, bool MASKED>
-int launch_segmented(SpmmParams &p, hipStream_t st) {
-    constexpr int MT = 32;
-    const int smem = 2 * p.seg_cb * (MT + 1) * 16;
-    static bool attr_done = false;
-    auto kern = mortar_segmented_kernel<NACC, MASKED>;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-        attr_done = true;
-    }
-    p.n_mtiles = (p.M + MT - 1) / MT;
-    p.n_split = (p.n_units + SEG_WAVES * SEG_UPW - 1) / (SEG_WAVES * SEG_UPW);
-    const int64_t grid = (int64_t)p.n_mtiles * p.n_split;
-    if (grid <= 0 || grid > 0x7fffffff) return mortar_fail(MORTAR_ERR_LIMIT, "prefill grid %lld out of range", (long long)grid);
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(SEG_WAVES * 64), smem, st, p);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "prefill launch: %s", hipGetErrorString(e));
-    return MORTAR_OK;
-}
-
 int check_common(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const uint16_t *x, int64_t M, int64_t ldx,
                  const uint16_t *y, int64_t ldy, int64_t out_cols) {
     if (!W || !W->codes || !W->sdup || !W->col || !W->row_ptr || !W->row_desc || !W->codes_o || !W->sd_o || !W->col_o || !chunk_ptr || !x || !y)
@@ -759,13 +359,57 @@ void fill(SpmmParams &p, const mortar_bcsr_t *W, const int32_t *chunk_ptr, const
     p.n_clusters = 1; p.cluster_size = 1 << 30;
 }
 
+// Token tile of the resident prefill kernel for a matrix with Cb block-columns (0 = does not fit).
+int resident_mt(int Cb) {
+    for (int mt : {96, 64, 32})
+        if (tile_bytes(mt, Cb) <= LDS_BUDGET) return mt;
+    return 0;
+}
+
+// prefill tiles: 16 wavefronts (4 per SIMD, 128 registers) for the 32-token tile, 8 for larger tiles
+template <int NACC, bool ROUTED>
+int launch_resident_any(SpmmParams &p, hipStream_t st) {
+    switch (resident_mt(p.Cb)) {
+        case 96: return mortar_launch_resident<96, NACC, ROUTED, 8>(p, nullptr, 1, st);
+        case 64: return mortar_launch_resident<64, NACC, ROUTED, 8>(p, nullptr, 1, st);
+        default: return mortar_launch_resident<32, NACC, ROUTED, 16>(p, nullptr, 1, st);
+    }
+}
+
+constexpr int SEG_WAVES = 16, SEG_UPW = 4;
+
+// kind: 0 spmm, 1 gate_up + SwiGLU, 2 routed gate_up + SwiGLU, 3 spmm with an input mask
+int dispatch(int kind, SpmmParams &p, hipStream_t st) {
+    if (p.M <= 16) {
+        const int rc = mortar_smallm_launch(kind, p, nullptr, 1, st);
+        if (rc >= 0) return rc;
+    }
+    switch (kind) {
+        case 0:
+            if (p.nseg == 1) return launch_resident_any<1, false>(p, st);
+            return mortar_launch_segmented<32, 1, false, SEG_WAVES, SEG_UPW>(p, nullptr, 1, st);
+        case 1:
+            if (p.nseg == 1) return launch_resident_any<2, false>(p, st);
+            return mortar_launch_segmented<32, 2, false, SEG_WAVES, SEG_UPW>(p, nullptr, 1, st);
+        case 2:
+            if (p.nseg == 1) return launch_resident_any<2, true>(p, st);
+            return launch<8, 4, 2, true, false>(p, st);
+        default:
+            return mortar_launch_segmented<32, 1, true, SEG_WAVES, SEG_UPW>(p, nullptr, 1, st);
+    }
+}
+
 }  // namespace
 
-extern "C" int mortar_prefill_max_seg_cb(void) { return 156 * 1024 / (2 * 33 * 16); }
+extern "C" int mortar_prefill_max_seg_cb(void) { return (LDS_BUDGET / 16 - LDS_PAD) / (2 * 33); }
 
-extern "C" int mortar_prefill_tile(int32_t Cb) {
-    const int msub = resident_msub(Cb);
-    return msub ? 16 * msub : MORTAR_PREFILL_MT;
+extern "C" int mortar_prefill_tile(int32_t Cb, int64_t M) {
+    if (M > 0 && M <= 16) {
+        const int t = mortar_smallm_tile(Cb, Cb, M, 2);
+        if (t > 0) return t;
+    }
+    const int mt = resident_mt(Cb);
+    return mt ? mt : MORTAR_PREFILL_MT;
 }
 
 extern "C" int mortar_prefill_group(int swiglu) { return swiglu ? NW * 4 : NW * 8; }
@@ -778,8 +422,7 @@ extern "C" int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr
     SpmmParams p;
     fill(p, W, chunk_ptr, unit_order, x, M, ldx, y, ldy);
     p.n_units = W->Rb;
-    if (p.nseg == 1) return launch_resident_any<1, false>(p, static_cast<hipStream_t>(stream));
-    return launch_segmented<1, false>(p, static_cast<hipStream_t>(stream));
+    return dispatch(0, p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *chunk_ptr,
@@ -794,7 +437,7 @@ extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *ch
     fill(p, W, chunk_ptr, unit_order, x, M, ldx, y, ldy);
     p.n_units = W->Rb;
     p.active = active; p.n_clusters = n_clusters; p.cluster_size = (W->Cb * 16) / n_clusters;
-    return launch_segmented<1, true>(p, static_cast<hipStream_t>(stream));
+    return dispatch(3, p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr,
@@ -817,9 +460,54 @@ extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *
         if (!tok_cnt || !tok_list || !gates) return mortar_fail(MORTAR_ERR_ARG, "gateup: routed mode needs gates, tok_cnt and tok_list");
         if (p.cluster_size % 16) return mortar_fail(MORTAR_ERR_ARG, "gateup: routed mode needs cluster_size %% 16 == 0");
         p.tok_cnt = tok_cnt; p.tok_list = tok_list;
-        if (p.nseg == 1) return launch_resident_any<2, true>(p, static_cast<hipStream_t>(stream));
-        return launch<8, 4, 2, true, false>(p, static_cast<hipStream_t>(stream));
+        return dispatch(2, p, static_cast<hipStream_t>(stream));
     }
-    if (p.nseg == 1) return launch_resident_any<2, false>(p, static_cast<hipStream_t>(stream));
-    return launch_segmented<2, false>(p, static_cast<hipStream_t>(stream));
+    return dispatch(1, p, static_cast<hipStream_t>(stream));
+}
+
+// ---- layer-batched small-M launches ---------------------------------------------------------------------
+
+extern "C" int64_t mortar_stack_table_bytes(int32_t n_layers) {
+    return n_layers > 0 ? (int64_t)n_layers * (int64_t)sizeof(SpmmParams) : 0;
+}
+
+extern "C" int mortar_stack_prepare(int32_t swiglu, int32_t n_layers, const mortar_bcsr_t *W,
+                                    const uint16_t *const *x, uint16_t *const *y, int64_t M, int64_t ldx,
+                                    int64_t ldy, void *table_dev, void *stream) {
+    if (n_layers <= 0 || n_layers > 65535 || !W || !x || !y || !table_dev)
+        return mortar_fail(MORTAR_ERR_ARG, "stack_prepare: bad arguments");
+    if (M > 16) return mortar_fail(MORTAR_ERR_LIMIT, "stack_prepare: layer-batched launches serve M <= 16 (got %lld)", (long long)M);
+    static const int32_t dummy_chunk = 0;
+    std::vector<SpmmParams> tab((size_t)n_layers);
+    for (int l = 0; l < n_layers; ++l) {
+        if (W[l].Rb != W[0].Rb || W[l].Cb != W[0].Cb || W[l].seg_cb != W[0].seg_cb)
+            return mortar_fail(MORTAR_ERR_ARG, "stack_prepare: layer %d differs in shape from layer 0", l);
+        if (swiglu && (W[l].Rb & 1)) return mortar_fail(MORTAR_ERR_ARG, "stack_prepare: odd number of block-rows");
+        const int64_t out_cols = swiglu ? (int64_t)W[l].Rb * 8 : (int64_t)W[l].Rb * 16;
+        int rc = check_common(&W[l], &dummy_chunk, x[l], M, ldx, y[l], ldy, out_cols);
+        if (rc) return rc;
+        SpmmParams &p = tab[(size_t)l];
+        fill(p, &W[l], nullptr, nullptr, x[l], M, ldx, y[l], ldy);
+        p.n_units = swiglu ? W[l].Rb / 2 : W[l].Rb;
+        rc = mortar_smallm_shape(swiglu ? 1 : 0, p, n_layers);
+        if (rc) return rc;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = hipMemcpyAsync(table_dev, tab.data(), tab.size() * sizeof(SpmmParams), hipMemcpyHostToDevice, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "stack_prepare: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}
+
+extern "C" int mortar_stack_run(int32_t swiglu, int32_t n_layers, const mortar_bcsr_t *W0, int64_t M,
+                                const void *table_dev, void *stream) {
+    if (n_layers <= 0 || n_layers > 65535 || !W0 || !table_dev || M <= 0 || M > 16)
+        return mortar_fail(MORTAR_ERR_ARG, "stack_run: bad arguments");
+    SpmmParams p;
+    fill(p, W0, nullptr, nullptr, nullptr, M, 0, nullptr, 0);
+    p.n_units = swiglu ? W0->Rb / 2 : W0->Rb;
+    const int rc = mortar_smallm_launch(swiglu ? 1 : 0, p, static_cast<const SpmmParams *>(table_dev), n_layers,
+                                        static_cast<hipStream_t>(stream));
+    if (rc < 0) return mortar_fail(MORTAR_ERR_LIMIT, "stack_run: shape has no small-M kernel");
+    return rc;
 }

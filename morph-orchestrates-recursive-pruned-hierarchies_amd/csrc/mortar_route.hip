@@ -174,7 +174,7 @@ extern "C" int mortar_remoe_route(const uint8_t *active, int64_t M, int32_t n, i
                                   uint8_t *tok_list, void *stream) {
     if (!active || !tok_cnt || !tok_list) return mortar_fail(MORTAR_ERR_ARG, "remoe_route: null pointer");
     if (M <= 0 || n <= 0) return mortar_fail(MORTAR_ERR_ARG, "remoe_route: M and n must be positive");
-    if (tile <= 0 || tile > 256 || tile % 16) return mortar_fail(MORTAR_ERR_LIMIT, "remoe_route: tile must be a multiple of 16, at most 256");
+    if (tile <= 0 || tile > 256 || (tile % 16 && tile != 4)) return mortar_fail(MORTAR_ERR_LIMIT, "remoe_route: tile must be 4 or a multiple of 16, at most 256");
     const unsigned nt = (unsigned)((M + tile - 1) / tile);
     hipLaunchKernelGGL(remoe_route_kernel, dim3(nt, (unsigned)((n + 63) / 64)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), active, M, n, tile, tok_cnt, tok_list);

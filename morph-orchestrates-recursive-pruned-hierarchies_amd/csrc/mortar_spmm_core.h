@@ -1,0 +1,481 @@
+// Octet-stream SpMM kernels shared by the prefill (large M) and decode (M <= 16) entry points.
+//
+// Both kernels keep a token tile of the activations in LDS and let every wavefront walk whole row units of
+// the octet weight stream: unpack the ternary codes of two blocks in registers, read the activation operand
+// from LDS, one 16x16x32 bf16 MFMA per 16 tokens.  They differ in how much of K the LDS tile holds:
+//   mortar_resident_kernel   all of in_features (no K loop, one barrier); the K segments of the stream are
+//                            walked back to back against the one resident tile
+//   mortar_segmented_kernel  one K segment at a time (a barrier pair per segment); a wave owns UPW row units
+//                            whose accumulators stay in registers across the segments
+// A launch can carry several independent problems of one shape ("layers"): blockIdx.y then selects an entry
+// of a parameter table in device memory.
+#ifndef MORTAR_SPMM_CORE_H
+#define MORTAR_SPMM_CORE_H
+
+#include "mortar_device.h"
+#include "mortar_internal.h"
+
+struct SpmmParams {
+    const uint32_t *codes;
+    const uint32_t *sdup;
+    const int16_t *col;
+    const int32_t *chunk_ptr;
+    const int32_t *row_ptr;
+    const u32x4_t *row_desc;  // octet stream: {first octet, end octet, blocks, 0} per (segment, block-row)
+    const u32x4_t *codes_o;
+    const u32x4_t *sd_o;
+    const u32x4_t *col_o;
+    const int32_t *unit_order;
+    int n_units, nkc, Cb;
+    const uint16_t *x;
+    int64_t ldx;
+    int M;
+    uint16_t *y;
+    int64_t ldy;
+    const float *gates;       // [M, n_clusters] fp32 or null
+    const uint8_t *active;    // [M, n_clusters] input mask or null
+    const int32_t *tok_cnt;   // routed: [n_mtiles, n_clusters]
+    const uint8_t *tok_list;  // routed: [n_mtiles, n_clusters, MT]
+    int n_clusters, cluster_size;
+    int xcd_map, n_mtiles, n_groups;
+    int n_split;              // workgroups that share one token tile
+    int seg_cb, nseg, Rb;     // K segments of the octet stream
+};
+
+// Device-side view of the launch parameters: the pointers carry the global address space in their type, so
+// that every access compiles to global_load / global_store (a pointer read from a parameter table in memory
+// would otherwise be generic and cost flat instructions).
+#define MORTAR_GLOBAL __attribute__((address_space(1)))
+struct SpmmView {
+    const MORTAR_GLOBAL u32x4_t *row_desc, *codes_o;
+    const MORTAR_GLOBAL uint32_t *sd_dw, *cc_dw;      // scale patterns / block-columns of the octet stream as dwords
+    const MORTAR_GLOBAL int32_t *unit_order;
+    const MORTAR_GLOBAL char *x;
+    MORTAR_GLOBAL uint16_t *y;
+    const MORTAR_GLOBAL float *gates;
+    const MORTAR_GLOBAL uint8_t *active;
+    const MORTAR_GLOBAL int32_t *tok_cnt;
+    const MORTAR_GLOBAL uint8_t *tok_list;
+    int64_t ldx, ldy;
+    int n_units, Cb, M, n_clusters, cluster_size, n_split, seg_cb, nseg, Rb;
+};
+static_assert(sizeof(SpmmParams) % 16 == 0, "table entries are copied in 16-byte words");
+// Entry i of a parameter table in device memory (uniform address: scalar loads).
+__device__ __forceinline__ SpmmParams mortar_table_entry(const SpmmParams *table, unsigned i) {
+    constexpr unsigned NW16 = sizeof(SpmmParams) / 16;
+    union { SpmmParams p; u32x4_t w[NW16]; } u;
+    const MORTAR_GLOBAL u32x4_t *src = (const MORTAR_GLOBAL u32x4_t *)table + (size_t)i * NW16;
+#pragma unroll
+    for (unsigned k = 0; k < NW16; ++k) u.w[k] = src[k];
+    return u.p;
+}
+__device__ __forceinline__ SpmmView mortar_view(const SpmmParams &q) {
+    SpmmView v;
+    v.row_desc = (const MORTAR_GLOBAL u32x4_t *)q.row_desc; v.codes_o = (const MORTAR_GLOBAL u32x4_t *)q.codes_o;
+    v.sd_dw = (const MORTAR_GLOBAL uint32_t *)q.sd_o; v.cc_dw = (const MORTAR_GLOBAL uint32_t *)q.col_o;
+    v.unit_order = (const MORTAR_GLOBAL int32_t *)q.unit_order;
+    v.x = (const MORTAR_GLOBAL char *)q.x; v.y = (MORTAR_GLOBAL uint16_t *)q.y;
+    v.gates = (const MORTAR_GLOBAL float *)q.gates; v.active = (const MORTAR_GLOBAL uint8_t *)q.active;
+    v.tok_cnt = (const MORTAR_GLOBAL int32_t *)q.tok_cnt; v.tok_list = (const MORTAR_GLOBAL uint8_t *)q.tok_list;
+    v.ldx = q.ldx; v.ldy = q.ldy; v.n_units = q.n_units; v.Cb = q.Cb; v.M = q.M; v.n_clusters = q.n_clusters;
+    v.cluster_size = q.cluster_size; v.n_split = q.n_split; v.seg_cb = q.seg_cb; v.nseg = q.nseg; v.Rb = q.Rb;
+    return v;
+}
+
+constexpr int RES_GROUPS = 4;            // octets (4 block pairs each) loaded per batch
+constexpr int LDS_BUDGET = 156 * 1024;   // bytes of LDS a token tile may take
+constexpr int LDS_PAD = 16;              // 16-byte units past the tile that idle lanes of a narrow tile may read
+
+// LDS bytes of a token tile of MT tokens and ncb block-columns (token stride MT + 1 keeps reads conflict-free).
+constexpr int tile_bytes(int mt, int ncb) { return (2 * ncb * (mt + 1) + LDS_PAD) * 16; }
+
+// Lane k of every 16-lane row broadcast to the whole row (DPP row_newbcast); K must fold to a constant.
+template <int K>
+__device__ __forceinline__ uint32_t mortar_row_bcast_k(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x150 + K, 0xf, 0xf, true);
+}
+__device__ __forceinline__ uint32_t mortar_row_bcast(uint32_t v, int k) {
+    switch (k) {
+        case 0: return mortar_row_bcast_k<0>(v);   case 1: return mortar_row_bcast_k<1>(v);
+        case 2: return mortar_row_bcast_k<2>(v);   case 3: return mortar_row_bcast_k<3>(v);
+        case 4: return mortar_row_bcast_k<4>(v);   case 5: return mortar_row_bcast_k<5>(v);
+        case 6: return mortar_row_bcast_k<6>(v);   case 7: return mortar_row_bcast_k<7>(v);
+        case 8: return mortar_row_bcast_k<8>(v);   case 9: return mortar_row_bcast_k<9>(v);
+        case 10: return mortar_row_bcast_k<10>(v); case 11: return mortar_row_bcast_k<11>(v);
+        case 12: return mortar_row_bcast_k<12>(v); case 13: return mortar_row_bcast_k<13>(v);
+        case 14: return mortar_row_bcast_k<14>(v); default: return mortar_row_bcast_k<15>(v);
+    }
+}
+
+// The batch loop of one row part: blocks [g0, g1) of the octet stream against the tile at `lx`.
+// `xo_base` is the lane's unit offset inside a block-column (column half, token) plus the segment's origin.
+template <int MSUB, int LDM, bool ROUTED>
+__device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *lx, int g0, int g1, int nb,
+                                                uint32_t xo_base, const uint32_t (&tk)[MSUB], int nsub,
+                                                int n, int bsel, int hsel, f32x4_t (&acc)[MSUB]) {
+    // One batch = RES_GROUPS octets (8 blocks = 4 pairs each) = 16 block pairs.  A lane loads its code dwords
+    // of the 16 pairs (one 16-byte load per octet) and, as lane k of its 16-lane row, the scale pattern and
+    // block-column of pair k (one dword each); pair u's metadata then reaches the row by a DPP broadcast.
+    const unsigned char *lb = reinterpret_cast<const unsigned char *>(lx);
+    for (int gq = g0; gq < g1; gq += RES_GROUPS) {
+        u32x4_t cw[RES_GROUPS];
+#pragma unroll
+        for (int k = 0; k < RES_GROUPS; ++k) {
+            const uint32_t gi = (uint32_t)(gq + k < g1 ? gq + k : g1 - 1) * 2u + (uint32_t)bsel;
+            cw[k] = p.codes_o[gi * 16u + n];
+        }
+        const int go = gq + (n >> 2);
+        const uint32_t mi = ((uint32_t)(go < g1 ? go : g1 - 1) * 2u + (uint32_t)bsel) * 4u + (uint32_t)(n & 3);
+        const uint32_t sdv = p.sd_dw[mi];
+        const uint32_t ccs = p.cc_dw[mi] * (uint32_t)(2 * LDM * 16);   // byte offset of the block-column in the tile
+        const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;      // block pairs left in the row from this batch on
+        // activation operands are fetched two pairs ahead of the MFMAs that use them
+        constexpr int NP = 4 * RES_GROUPS;
+        uint4 Bq[3][MSUB];
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+            const uint32_t xo = mortar_row_bcast(ccs, d) + xo_base * 16u;
+#pragma unroll
+            for (int ms = 0; ms < MSUB; ++ms) Bq[d][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 16u : ms * 256u));
+        }
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+            if (u < pairs) {
+                const u32x4_t A = mortar_unpack8(cw[u >> 2][u & 3] << (8 * hsel), mortar_row_bcast(sdv, u));
+                if (u + 2 < NP) {
+                    const uint32_t xo = mortar_row_bcast(ccs, u + 2) + xo_base * 16u;
+#pragma unroll
+                    for (int ms = 0; ms < MSUB; ++ms)
+                        Bq[(u + 2) % 3][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 16u : ms * 256u));
+                }
+#pragma unroll
+                for (int ms = 0; ms < MSUB; ++ms) {
+                    if (!ROUTED || ms < nsub) {
+                        const uint4 bq = Bq[u % 3][ms];
+                        const u32x4_t Bv = {bq.x, bq.y, bq.z, bq.w};
+                        acc[ms] = mortar_mfma(A, Bv, acc[ms]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Stages x[m0 .. m0+MT, 16*c0 .. 16*(c0+ncb)] into the tile: unit (ch, row) <- 8 values of column half ch.
+// A wavefront takes whole rows (row = wave, wave + WAVES, ...), its lanes consecutive 16-byte units of the row,
+// so that addresses need no division: uniform row base + lane offset.  Rows past M repeat the last row.
+// With MASKED, units of (token, input cluster) pairs that are off are zeroed.
+template <int MT, int WAVES, bool MASKED>
+__device__ __forceinline__ void mortar_stage_tile(const SpmmView &p, uint4 *lx, int m0, int c0, int ncb, int tid) {
+    constexpr int LDM = MT + 1, RU = 2, CU = 4;     // rows x 64-unit chunks in flight per lane
+    const int nch = 2 * ncb;
+    const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const MORTAR_GLOBAL char *xt = p.x + (int64_t)m0 * p.ldx * 2 + (int64_t)c0 * 32;
+    for (int r0 = wave; r0 < MT; r0 += WAVES * RU) {
+        for (int ch0 = 0; ch0 < nch; ch0 += 64 * CU) {
+            u32x4_t v[RU][CU];
+#pragma unroll
+            for (int a = 0; a < RU; ++a) {
+                int row = r0 + a * WAVES;
+                row = row < rlast ? row : rlast;
+                const MORTAR_GLOBAL char *xr = xt + (int64_t)row * p.ldx * 2;
+#pragma unroll
+                for (int b = 0; b < CU; ++b) {
+                    int ch = ch0 + b * 64 + lane;
+                    ch = ch < nch ? ch : nch - 1;
+                    v[a][b] = *(const MORTAR_GLOBAL u32x4_t *)(xr + (uint32_t)ch * 16u);
+                    if (MASKED && p.active[(int64_t)(m0 + row) * p.n_clusters + (c0 * 16 + ch * 8) / p.cluster_size] == 0)
+                        v[a][b] = u32x4_t{0u, 0u, 0u, 0u};
+                }
+            }
+#pragma unroll
+            for (int a = 0; a < RU; ++a) {
+                const int row = r0 + a * WAVES;
+#pragma unroll
+                for (int b = 0; b < CU; ++b) {
+                    const int ch = ch0 + b * 64 + lane;
+                    if (row < MT && ch < nch) reinterpret_cast<u32x4_t *>(lx)[ch * LDM + row] = v[a][b];
+                }
+            }
+        }
+    }
+}
+
+// Epilogue of one row unit for the 16 tokens of sub-tile `ms`: the lane holds D[4g+v][token].
+template <int NACC>
+__device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, int tok, int g, bool has_gates,
+                                                  const f32x4_t &a0, const f32x4_t &a1) {
+    u32x2_t pk;
+    if (NACC == 1) {
+        pk = u32x2_t{bf16_pack2(a0[0], a0[1]), bf16_pack2(a0[2], a0[3])};
+    } else {
+        float gv = 0.f;
+        if (has_gates) gv = p.gates[(int64_t)tok * p.n_clusters + (unit * 16 + 4 * g) / p.cluster_size];
+        pk = swiglu_pack4(a0, a1, has_gates, gv);
+    }
+    *(MORTAR_GLOBAL u32x2_t *)(p.y + (int64_t)tok * p.ldy + unit * 16 + 4 * g) = pk;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Resident kernel.  The workgroup stages x[MT, K] once; then every wave walks whole row units on its own,
+// streaming the unit's block pairs straight from global memory in batches (a row's blocks are contiguous).
+// No barrier after the first one; latency is hidden by the waves that share a SIMD.
+// ---------------------------------------------------------------------------------------------------------
+template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE>
+__global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmParams p0, const SpmmParams *table) {
+    constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1;
+    const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint4 *lx = reinterpret_cast<uint4 *>(smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
+    const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
+    const int m0 = mt * MT;
+    const uint32_t lane_xo = (uint32_t)(hsel * LDM + (ROUTED ? 0 : n));
+    const bool has_gates = p.gates != nullptr;
+
+    mortar_stage_tile<MT, WAVES, false>(p, lx, m0, 0, p.Cb, tid);
+    __syncthreads();
+
+    const int per = (p.n_units + p.n_split - 1) / p.n_split;
+    const int u_end = (sp + 1) * per < p.n_units ? (sp + 1) * per : p.n_units;
+    // Unit ids are fetched two units ahead and row descriptors one row part ahead, so that no dependent global
+    // round trip (order -> descriptor -> blocks) is exposed between two units of a wave.
+    auto unit_of = [&](int pos_) { return (p.unit_order && pos_ < u_end) ? p.unit_order[pos_] : pos_; };
+    auto desc_of = [&](int unit_, int a_, int sg_) {
+        const int r = unit_ + a_ * p.n_units;
+        return p.row_desc[sg_ * p.Rb + (r < p.Rb ? r : 0)];
+    };
+    int pos = sp * per + wave;
+    int unit_v = unit_of(pos), unit_v1 = unit_of(pos + WAVES);
+    u32x4_t dcur[NACC], dnxt[NACC];
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) dcur[a] = desc_of(unit_v, a, 0);
+    for (; pos < u_end; pos += WAVES) {
+        const int unit = __builtin_amdgcn_readfirstlane(unit_v);
+        const int unit_v2 = unit_of(pos + 2 * WAVES);
+        const int unit_n = unit_v1 < p.n_units ? unit_v1 : 0;
+        int cnt = MT;
+        uint32_t tk[MSUB];
+#pragma unroll
+        for (int ms = 0; ms < MSUB; ++ms) tk[ms] = ms * 16 + n;
+        bool skip = false;
+        if (ROUTED) {
+            const int cl = (unit * 16) / p.cluster_size;
+            const int64_t e = (int64_t)mt * p.n_clusters + cl;
+            cnt = __builtin_amdgcn_readfirstlane(p.tok_cnt[e]);
+            skip = cnt == 0;
+#pragma unroll
+            for (int ms = 0; ms < MSUB; ++ms) {
+                const int i = ms * 16 + n;
+                tk[ms] = i < cnt ? p.tok_list[e * MT + i] : 0;
+            }
+        }
+        const int nsub = ROUTED ? (cnt + 15) >> 4 : MSUB;
+        f32x4_t acc[NACC][MSUB];
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+        for (int sg = 0; sg < p.nseg; ++sg) {
+            const bool last = sg + 1 == p.nseg;
+            int rg0[NACC], rg1[NACC], rnb[NACC];
+#pragma unroll
+            for (int a = 0; a < NACC; ++a) {
+                dnxt[a] = desc_of(last ? unit_n : unit, a, last ? 0 : sg + 1);
+                rg0[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][0]);
+                rg1[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][1]);
+                rnb[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][2]);
+                dcur[a] = dnxt[a];
+            }
+            if (skip) continue;
+            const uint32_t xo_base = lane_xo + (uint32_t)(sg * p.seg_cb) * (2 * LDM);
+#pragma unroll
+            for (int a = 0; a < NACC; ++a)
+                mortar_row_part<MSUB, LDM, ROUTED>(p, lx, rg0[a], rg1[a], rnb[a], xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+        }
+        unit_v = unit_v1;
+        unit_v1 = unit_v2;
+        if (skip) continue;
+
+#pragma unroll
+        for (int ms = 0; ms < MSUB; ++ms) {
+            const int li = ms * 16 + n;
+            if (li >= (ROUTED ? cnt : MT)) continue;
+            const int tok = m0 + (int)tk[ms];
+            if (tok >= p.M) continue;
+            mortar_store_unit<NACC>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Segmented kernel for matrices whose K does not fit in LDS at once (e.g. `down`, K = d_ff).  The workgroup
+// walks the K segments of the octet stream: per segment it stages x[MT, 16*seg_cb] (one barrier pair), and
+// every wave multiplies the segment's blocks of its own UPW row units.
+// ---------------------------------------------------------------------------------------------------------
+template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE>
+__global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const SpmmParams p0, const SpmmParams *table) {
+    constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1;
+    const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint4 *lx = reinterpret_cast<uint4 *>(smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
+    const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
+    const int m0 = mt * MT;
+    const uint32_t lane_xo = (uint32_t)(hsel * LDM + n);
+    const bool has_gates = p.gates != nullptr;
+
+    // this wave's units: positions sp*per + wave + WAVES*k of the schedule
+    constexpr int per = WAVES * UPW;
+    int units[UPW];
+#pragma unroll
+    for (int k = 0; k < UPW; ++k) {
+        const int pos = sp * per + wave + WAVES * k;
+        int u = -1;
+        if (pos < p.n_units) u = p.unit_order ? p.unit_order[pos] : pos;
+        units[k] = __builtin_amdgcn_readfirstlane(u);
+    }
+    f32x4_t acc[UPW][NACC][MSUB];
+    uint32_t tk[MSUB];
+#pragma unroll
+    for (int ms = 0; ms < MSUB; ++ms) tk[ms] = ms * 16;
+#pragma unroll
+    for (int k = 0; k < UPW; ++k)
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int ms = 0; ms < MSUB; ++ms) acc[k][a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int sg = 0; sg < p.nseg; ++sg) {
+        const int c0 = sg * p.seg_cb;
+        const int ncb = p.Cb - c0 < p.seg_cb ? p.Cb - c0 : p.seg_cb;
+        // row descriptors of this segment (loaded before the barrier so that their latency is hidden)
+        u32x4_t desc[UPW][NACC];
+#pragma unroll
+        for (int k = 0; k < UPW; ++k)
+#pragma unroll
+            for (int a = 0; a < NACC; ++a)
+                desc[k][a] = p.row_desc[(int64_t)sg * p.Rb + (units[k] < 0 ? 0 : units[k] + a * p.n_units)];
+        if (sg > 0) __syncthreads();
+        mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, c0, ncb, tid);
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < UPW; ++k) {
+            if (units[k] < 0) continue;
+#pragma unroll
+            for (int a = 0; a < NACC; ++a) {
+                const int g0 = __builtin_amdgcn_readfirstlane((int)desc[k][a][0]);
+                const int g1 = __builtin_amdgcn_readfirstlane((int)desc[k][a][1]);
+                const int nb = __builtin_amdgcn_readfirstlane((int)desc[k][a][2]);
+                mortar_row_part<MSUB, LDM, false>(p, lx, g0, g1, nb, lane_xo, tk, MSUB, n, bsel, hsel, acc[k][a]);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int k = 0; k < UPW; ++k) {
+        if (units[k] < 0) continue;
+#pragma unroll
+        for (int ms = 0; ms < MSUB; ++ms) {
+            const int li = ms * 16 + n;
+            if (li >= MT) continue;
+            const int tok = m0 + li;
+            if (tok >= p.M) continue;
+            mortar_store_unit<NACC>(p, units[k], tok, g, has_gates, acc[k][0][ms], acc[k][NACC - 1][ms]);
+        }
+    }
+}
+
+// ---- launchers -------------------------------------------------------------------------------------------
+// `layers` > 1 launches the table variant: `table` points at `layers` SpmmParams in device memory whose
+// n_mtiles / n_split fields were filled from the same shape as `p`.
+
+template <typename K>
+inline int mortar_allow_big_lds(K kern, bool &done) {
+    if (!done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        done = true;
+    }
+    return MORTAR_OK;
+}
+
+inline int mortar_launch_check(int64_t grid, int layers) {
+    if (grid <= 0 || grid > 0x7fffffff || layers <= 0 || layers > 65535)
+        return mortar_fail(MORTAR_ERR_LIMIT, "spmm grid %lld x %d out of range", (long long)grid, layers);
+    return MORTAR_OK;
+}
+
+// Fills the launch-shape fields of `p` for the resident kernel and returns the grid width.
+template <int MT, int WAVES>
+inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
+    p.n_mtiles = (p.M + MT - 1) / MT;
+    // Prefill tiles: enough workgroups to cover the 256 CUs twice (every workgroup stages a whole tile, so few
+    // large ones).  Decode tiles stage little: many small workgroups (about 12 per CU, at least `upw` units
+    // per wave) so that the hardware dispatcher evens out the load.
+    constexpr int upw = MT <= 4 ? 2 : (MT <= 16 ? 4 : 1);
+    const int target = MT <= 16 ? 256 * 12 : 256 * 2;
+    int split = (target + layers * p.n_mtiles - 1) / (layers * p.n_mtiles);
+    const int max_split = (p.n_units + WAVES * upw - 1) / (WAVES * upw);
+    split = split < 1 ? 1 : (split > max_split ? max_split : split);
+    p.n_split = split;
+    return (int64_t)p.n_mtiles * split;
+}
+
+template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE = false>
+int mortar_launch_resident(SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
+    if (TABLE != (table != nullptr)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: parameter table mismatch");
+    const int smem = tile_bytes(MT, p.Cb);
+    if (smem > LDS_BUDGET + LDS_PAD * 16) return mortar_fail(MORTAR_ERR_LIMIT, "resident tile of %d bytes does not fit LDS", smem);
+    static bool attr_done = false;
+    auto kern = mortar_resident_kernel<MT, NACC, ROUTED, WAVES, TABLE>;
+    int rc = mortar_allow_big_lds(kern, attr_done);
+    if (rc) return rc;
+    const int64_t grid = mortar_resident_shape<MT, WAVES>(p, layers);
+    if ((rc = mortar_launch_check(grid, layers))) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)layers), dim3(WAVES * 64), smem, st, p, table);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "spmm launch: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}
+
+template <int MT, int WAVES, int UPW>
+inline int64_t mortar_segmented_shape(SpmmParams &p) {
+    p.n_mtiles = (p.M + MT - 1) / MT;
+    p.n_split = (p.n_units + WAVES * UPW - 1) / (WAVES * UPW);
+    return (int64_t)p.n_mtiles * p.n_split;
+}
+
+template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE = false>
+int mortar_launch_segmented(SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
+    if (TABLE != (table != nullptr)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: parameter table mismatch");
+    const int smem = tile_bytes(MT, p.seg_cb);
+    if (smem > LDS_BUDGET + LDS_PAD * 16) return mortar_fail(MORTAR_ERR_LIMIT, "segment tile of %d bytes does not fit LDS", smem);
+    static bool attr_done = false;
+    auto kern = mortar_segmented_kernel<MT, NACC, MASKED, WAVES, UPW, TABLE>;
+    int rc = mortar_allow_big_lds(kern, attr_done);
+    if (rc) return rc;
+    const int64_t grid = mortar_segmented_shape<MT, WAVES, UPW>(p);
+    if ((rc = mortar_launch_check(grid, layers))) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)layers), dim3(WAVES * 64), smem, st, p, table);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "spmm launch: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}
+
+// Small-M (decode) dispatch, compiled in its own translation unit.  kind: 0 spmm, 1 gate_up + SwiGLU,
+// 2 gate_up + SwiGLU routed, 3 spmm with an input mask.  Returns -1 when the shape has no small-M variant.
+__attribute__((visibility("hidden"))) int mortar_smallm_launch(int kind, SpmmParams &p, const SpmmParams *table,
+                                                               int layers, hipStream_t st);
+__attribute__((visibility("hidden"))) int mortar_smallm_tile(int Cb, int seg_cb, int64_t M, int kind);
+// Fills the launch-shape fields (n_mtiles, n_split) of a table entry exactly as mortar_smallm_launch would.
+__attribute__((visibility("hidden"))) int mortar_smallm_shape(int kind, SpmmParams &p, int layers);
+
+#endif

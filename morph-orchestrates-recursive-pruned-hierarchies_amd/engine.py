@@ -51,12 +51,16 @@ class MortarDecodeMLP:
         rt = getattr(self.mlp, "router", None)
         if gates is None and rt is not None:
             gates = rt(xn, iter_idx=self.iter_idx)[0].reshape(B, -1).float().contiguous()
-        if gates is not None:
-            ract, cact = ops.route_flags(gates, self.d_ff)
-            h = ops.gemv(xn, self.Mgu, swiglu_out=True, gates=gates, row_act=ract)
-            return ops.gemv(h, self.Mdown, col_act=cact).view(B, 1, -1)
-        h = ops.gemv(xn, self.Mgu, swiglu_out=True)
-        return ops.gemv(h, self.Mdown).view(B, 1, -1)
+        if gates is not None and (self.d_ff // gates.shape[-1]) % 16 == 0:
+            # gather-skip: only (stream, block-row) tiles of active clusters are computed; `down` reads the
+            # hidden activations of inactive clusters as zero
+            gates = gates.contiguous()
+            active = (gates > 0).to(torch.uint8)
+            route = ops.remoe_route(active, ops.prefill_tile(self.Mgu, B))
+            h = ops.gateup_swiglu(xn, self.Mgu, gates=gates, route=route)
+            return ops.spmm(h, self.Mdown, active=active).view(B, 1, -1)
+        h = ops.gateup_swiglu(xn, self.Mgu, gates=gates.contiguous() if gates is not None else None)
+        return ops.spmm(h, self.Mdown).view(B, 1, -1)
 
 
 @torch.no_grad()

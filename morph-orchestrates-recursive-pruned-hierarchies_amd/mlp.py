@@ -14,7 +14,6 @@ from . import ops
 from .pack import PREFILL_MT
 from .sparsity import MortarLinear
 
-DECODE_MAX_ROWS = 64       # flattened rows up to which the decode GEMV kernels serve the MLP
 
 
 class _KwargSequential(nn.Sequential):
@@ -111,23 +110,17 @@ class _SwiGLUMortar(nn.Module):
         if gates is not None and self.d_ff % gates.shape[-1]:
             raise ValueError("the carved MLP needs equal-size clusters (d_ff % n_clusters == 0)")
         N = xb.shape[0]
-        if 0 < N <= DECODE_MAX_ROWS:
-            ract = cact = None
-            if gates is not None:
-                ract, cact = ops.route_flags(gates, self.d_ff)
-            h = ops.gemv(xb, Wgu, swiglu_out=True, gates=gates, row_act=ract)
-            y = ops.gemv(h, Wdn, col_act=cact)
+        # one path for prefill and decode: the library picks 4- or 16-token tiles for decode-sized N
+        cs = self.d_ff // gates.shape[-1] if gates is not None else 0
+        if gates is not None and self.route_skip and cs % 16 == 0 and N > 0:
+            if active is None:
+                active = (gates > 0).to(torch.uint8)
+            route = ops.remoe_route(active, ops.prefill_tile(Wgu, N))
+            h = ops.gateup_swiglu(xb, Wgu, gates=gates, route=route)
+            y = ops.spmm(h, Wdn, active=active)
         else:
-            cs = self.d_ff // gates.shape[-1] if gates is not None else 0
-            if gates is not None and self.route_skip and cs % 16 == 0:
-                if active is None:
-                    active = (gates > 0).to(torch.uint8)
-                route = ops.remoe_route(active, ops.prefill_tile(Wgu))
-                h = ops.gateup_swiglu(xb, Wgu, gates=gates, route=route)
-                y = ops.spmm(h, Wdn, active=active)
-            else:
-                h = ops.gateup_swiglu(xb, Wgu, gates=gates)
-                y = ops.spmm(h, Wdn)
+            h = ops.gateup_swiglu(xb, Wgu, gates=gates)
+            y = ops.spmm(h, Wdn)
         if y.dtype != x.dtype:
             y = y.to(x.dtype)
         return y.reshape(*lead, self.d_model)

@@ -105,9 +105,9 @@ def remoe_gates(logits: Tensor, k: int) -> tuple[Tensor, Tensor]:
     return gates, active
 
 
-def prefill_tile(W: MortarPack) -> int:
-    """Token tile of the prefill kernels for this matrix (the tile remoe_route must use for it)."""
-    return int(_lib.lib().mortar_prefill_tile(W.Cb))
+def prefill_tile(W: MortarPack, M: int = 0) -> int:
+    """Token tile of the gate_up kernels for M rows against this matrix (the tile remoe_route must use)."""
+    return int(_lib.lib().mortar_prefill_tile(W.Cb, int(M)))
 
 
 def remoe_route(active: Tensor, tile: int = PREFILL_MT) -> tuple[Tensor, Tensor]:
@@ -154,13 +154,19 @@ def _kseg_for(W: MortarPack, B: int) -> int:
 def gemv(x: Tensor, W: MortarPack, swiglu_out: bool = False, gates: Tensor | None = None,
          row_act: Tensor | None = None, col_act: Tensor | None = None, max_blocks: int | None = None,
          out: Tensor | None = None) -> Tensor:
-    """Decode GEMV for B <= 64 streams: y = x W^T (bf16), or with swiglu_out the fused silu(g)*u[*gates]."""
+    """Decode GEMV for B <= 64 streams: y = x W^T (bf16), or with swiglu_out the fused silu(g)*u[*gates].
+    Without gather flags the batch goes to the small-tile SpMM kernels (one pass over the weights); with
+    row_act / col_act (or an explicit max_blocks split) it runs the work-list kernel that honours them."""
     x = _bf16_2d(x, "gemv")
     B = x.shape[0]
     if not 1 <= B <= 64:
         raise ValueError(f"gemv: batch {B} outside 1..64 (use the prefill path)")
     if x.shape[1] != W.in_features:
         raise ValueError(f"gemv: x has {x.shape[1]} features, matrix expects {W.in_features}")
+    if row_act is None and col_act is None and max_blocks is None:
+        if swiglu_out:
+            return gateup_swiglu(x, W, gates=gates.contiguous() if gates is not None else None, out=out)
+        return spmm(x, W, out=out)
     rpu = 2 if swiglu_out else 1
     kseg = _kseg_for(W, B)
     if max_blocks is None:
@@ -186,6 +192,37 @@ def gemv(x: Tensor, W: MortarPack, swiglu_out: bool = False, gates: Tensor | Non
         _p(col_act), col_act.stride(0) if col_act is not None else 0, _stream(x))
     _lib.check(rc, "mortar_gemv_bf16")
     return y
+
+
+class LayerStack:
+    """n layers of one shape (same Rb, Cb, K segments) whose small-M products run in ONE launch:
+    y_l = x_l W_l^T, or with swiglu the fused silu(g)*u of gate_up W_l.  The inputs and outputs are fixed at
+    construction (their device addresses go into a parameter table); run() may be called any number of times."""
+
+    def __init__(self, packs: list[MortarPack], xs: list[Tensor], ys: list[Tensor], swiglu: bool = False):
+        n = len(packs)
+        if n == 0 or len(xs) != n or len(ys) != n:
+            raise ValueError("LayerStack: need one input and one output per layer")
+        xs = [_bf16_2d(x, "LayerStack") for x in xs]
+        M = xs[0].shape[0]
+        for x, y in zip(xs, ys):
+            if x.shape != xs[0].shape or x.stride(0) != xs[0].stride(0) or y.stride(0) != ys[0].stride(0):
+                raise ValueError("LayerStack: inputs / outputs must share shape and row stride")
+            if y.dtype != torch.bfloat16 or not y.is_cuda:
+                raise TypeError("LayerStack: outputs must be bfloat16 device tensors")
+        L = _lib.lib()
+        self.packs, self.xs, self.ys, self.swiglu, self.M, self.n = packs, xs, ys, int(bool(swiglu)), M, n
+        self._structs = (_lib.BcsrStruct * n)(*[p.struct for p in packs])
+        xp = (C.c_void_p * n)(*[x.data_ptr() for x in xs])
+        yp = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
+        self.table = torch.empty(int(L.mortar_stack_table_bytes(n)), dtype=torch.uint8, device=xs[0].device)
+        _lib.check(L.mortar_stack_prepare(self.swiglu, n, self._structs, xp, yp, M, xs[0].stride(0), ys[0].stride(0),
+                                          _p(self.table), _stream(xs[0])), "mortar_stack_prepare")
+
+    def run(self) -> list[Tensor]:
+        _lib.check(_lib.lib().mortar_stack_run(self.swiglu, self.n, self._structs, self.M, _p(self.table),
+                                               _stream(self.xs[0])), "mortar_stack_run")
+        return self.ys
 
 
 # ----------------------------------------------------------------------------- RMSNorm

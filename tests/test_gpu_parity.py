@@ -125,7 +125,7 @@ def test_mlp_with_gates_and_skip(dev):
     xd = to_dev(x, dev)
     h_dense = ops.gateup_swiglu(xd, Wgu, gates=gates)
     assert_close_bf16(to_np(h_dense), ref["h"], "h gated", ulps=4)
-    cnt, lst = ops.remoe_route(active, ops.prefill_tile(Wgu))
+    cnt, lst = ops.remoe_route(active, ops.prefill_tile(Wgu, M))
     h_skip = torch.full_like(h_dense, float("nan"))                             # untouched entries stay NaN
     ops.gateup_swiglu(xd, Wgu, gates=gates, route=(cnt, lst), out=h_skip)
     hs, hd = to_np(h_skip), to_np(h_dense)
@@ -192,6 +192,82 @@ def test_decode_mlp_cloud_width(dev, B):
     assert_close_bf16(to_np(y), ref["y"], "y", ulps=8)
     gu = ops.gemv(to_dev(x, dev), Wgu)                                           # plain mode on gate_up
     assert_close_bf16(to_np(gu), ref["gu"], "gu")
+
+
+@pytest.mark.parametrize("B", [1, 2, 4, 5, 16])
+@pytest.mark.parametrize("dims", [(256, 16 * 44), (512, 16 * 400)])
+def test_decode_small_tiles(dev, B, dims):
+    """Decode batches through the SpMM entry points: 4- and 16-token tiles, K that fits LDS whole (resident)
+    and K cut into segments (d_ff = 6400 > one segment), Zipf rows, per-cluster gates."""
+    d_model, d_ff = dims
+    spec = synth.synth_mlp(d_model, d_ff, 0.3, seed=400 + B, zipf_s=1.2)
+    x = synth.synth_x(B, d_model, 410 + B)
+    ncl = d_ff // 16
+    g_ref, _ = O.remoe_gates(synth.synth_logits(B, ncl, 420 + B), max(1, ncl // 3))
+    Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    xd = to_dev(x, dev)
+    for gates in (None, g_ref):
+        ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=gates)
+        gd = torch.from_numpy(gates).to(dev) if gates is not None else None
+        h = ops.gateup_swiglu(xd, Wgu, gates=gd)
+        assert_close_bf16(to_np(h), ref["h"], "h", ulps=4)
+        y = ops.spmm(h, Wdn)
+        assert_close_bf16(to_np(y), ref["y"], "y", ulps=8)
+        if gates is not None:                                                        # gather-skip form
+            active = (gd > 0).to(torch.uint8)
+            tile = ops.prefill_tile(Wgu, B)
+            assert tile == (4 if B <= 4 else 16)
+            route = ops.remoe_route(active, tile)
+            hs = torch.full_like(h, float("nan"))
+            ops.gateup_swiglu(xd, Wgu, gates=gd, route=route, out=hs)
+            on = np.repeat(to_np(active).astype(bool), 16, axis=1)
+            assert np.array_equal(to_np(hs)[on], to_np(h)[on])
+            assert np.isnan(to_np(hs)[~on]).all()
+            ys = ops.spmm(hs, Wdn, active=active)
+            assert_close_bf16(to_np(ys), ref["y"], "y skip", ulps=8)
+    gu = ops.spmm(xd, Wgu)
+    assert_close_bf16(to_np(gu), oracle_spmm(x, spec["gate_up"]), "gu")
+
+
+def test_decode_gather_flags_worklist(dev):
+    """The work-list GEMV with the reference's row_act / col_act gather flags (route_flags)."""
+    d_model, d_ff, ncl, k, B = 512, 16 * 64, 64, 16, 3
+    spec = synth.synth_mlp(d_model, d_ff, 0.3, seed=70)
+    x = synth.synth_x(B, d_model, 71)
+    g_ref, _ = O.remoe_gates(synth.synth_logits(B, ncl, 72), k)
+    ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=g_ref)
+    gates = torch.from_numpy(g_ref).to(dev)
+    Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    ract, cact = ops.route_flags(gates, d_ff)
+    h = ops.gemv(to_dev(x, dev), Wgu, swiglu_out=True, gates=gates, row_act=ract)
+    y = ops.gemv(h, Wdn, col_act=cact)
+    assert_close_bf16(to_np(y), ref["y"], "flagged decode", ulps=8)
+
+
+@pytest.mark.parametrize("B,n_layers", [(3, 5), (12, 5), (2, 300)])
+def test_layer_stack_matches_single_launches(dev, B, n_layers):
+    """Layer-batched launch: n layers in one launch give bit-identical results to n separate launches."""
+    d_model, d_ff = 256, 16 * 380                                                    # down is K-segmented
+    specs = [synth.synth_mlp(d_model, d_ff, 0.25, seed=500 + i, zipf_s=1.2) for i in range(min(n_layers, 5))]
+    packs = [(synth.to_pack(s["gate_up"], dev), synth.to_pack(s["down"], dev)) for s in specs]
+    packs = [packs[i % len(packs)] for i in range(n_layers)]
+    xs = [to_dev(synth.synth_x(B, d_model, 520 + i), dev) for i in range(n_layers)]
+    hs = [torch.empty((B, d_ff), dtype=torch.bfloat16, device=dev) for _ in range(n_layers)]
+    ys = [torch.empty((B, d_model), dtype=torch.bfloat16, device=dev) for _ in range(n_layers)]
+    up = ops.LayerStack([p[0] for p in packs], xs, hs, swiglu=True)
+    dn = ops.LayerStack([p[1] for p in packs], hs, ys, swiglu=False)
+    for _ in range(2):
+        up.run()
+        dn.run()
+    for i in range(n_layers):
+        h1 = ops.gateup_swiglu(xs[i], packs[i][0])
+        assert torch.equal(h1, hs[i]), f"layer {i} h"
+        assert torch.equal(ops.spmm(h1, packs[i][1]), ys[i]), f"layer {i} y"
+    ref = O.swiglu_mlp(to_np(xs[1]), specs[1]["gate_up"], specs[1]["down"])
+    assert_close_bf16(to_np(ys[1]), ref["y"], "stack vs oracle", ulps=8)
+    with pytest.raises(ValueError):
+        ops.LayerStack([packs[0][0]], [to_dev(synth.synth_x(17, d_model, 1), dev)],
+                       [torch.empty((17, d_ff), dtype=torch.bfloat16, device=dev)], swiglu=True)
 
 
 @pytest.mark.parametrize("max_blocks", [3, 8])
@@ -289,7 +365,7 @@ def test_full_size_properties(dev):
     g_ref, a_ref = O.remoe_gates(lg, 88)
     gates, active = ops.remoe_gates(torch.from_numpy(lg).to(dev), 88)
     assert np.array_equal(active.cpu().numpy().astype(bool), a_ref)
-    cnt, lst = ops.remoe_route(active, ops.prefill_tile(Wgu))
+    cnt, lst = ops.remoe_route(active, ops.prefill_tile(Wgu, 4096))
     assert int(cnt.sum()) == int(a_ref.sum())
     hr = ops.gateup_swiglu(xd, Wgu, gates=gates, route=(cnt, lst))
     yr = ops.spmm(hr, Wdn, active=active)
