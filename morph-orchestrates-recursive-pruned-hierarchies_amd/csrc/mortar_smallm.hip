@@ -3,7 +3,7 @@
 // Replaces the reference's decode GEMV over packed ternary strips (morph/kernels/triton/fused_decode_step.py:
 // 1701-1842, mortar_gemv) for batches of up to 16 rows: the batch is one token tile of 4 or 16 tokens, so a
 // weight block is read once per launch and the kernel is bound by the weight stream.  Workgroups are small
-// (2 wavefronts) when one matrix has to cover the chip and 8 wavefronts when many layers share a launch.
+// (2 wavefronts) when one matrix has to cover the chip and 8 or 16 wavefronts when many layers share a launch.
 #include "mortar_spmm_core.h"
 
 namespace {
@@ -45,25 +45,43 @@ int mortar_smallm_tile(int Cb, int seg_cb, int64_t M, int kind) {
     return 0;
 }
 
+// Wavefronts per workgroup: 2 when one matrix has to cover the chip; otherwise 8, or 16 when the tile is so
+// large that only two workgroups fit in a CU's LDS (keeps 32 wavefronts per CU resident either way).
+static int pick_waves(int t, const SpmmParams &p, int layers) {
+    if ((int64_t)layers * p.n_units < 8 * 512) return 2;
+    const int bytes = t > 0 ? tile_bytes(t, p.Cb) : tile_bytes(16, p.seg_cb);
+    return bytes > 40 * 1024 ? 16 : 8;
+}
+
 int mortar_smallm_launch(int kind, SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
     if (t == 0) return -1;
     const bool resident = t > 0;
-    const bool wide = (int64_t)layers * p.n_units >= 8 * 512;   // enough units to fill the chip with 8-wave groups
-    if (t == 4) return wide ? launch_kind<4, 8>(kind, true, p, table, layers, st) : launch_kind<4, 2>(kind, true, p, table, layers, st);
-    return wide ? launch_kind<16, 8>(kind, resident, p, table, layers, st) : launch_kind<16, 2>(kind, resident, p, table, layers, st);
+    const int w = pick_waves(t, p, layers);
+    if (t == 4) {
+        if (w == 16) return launch_kind<4, 16>(kind, true, p, table, layers, st);
+        return w == 8 ? launch_kind<4, 8>(kind, true, p, table, layers, st) : launch_kind<4, 2>(kind, true, p, table, layers, st);
+    }
+    if (w == 16) return launch_kind<16, 16>(kind, resident, p, table, layers, st);
+    return w == 8 ? launch_kind<16, 8>(kind, resident, p, table, layers, st) : launch_kind<16, 2>(kind, resident, p, table, layers, st);
 }
 
 int mortar_smallm_shape(int kind, SpmmParams &p, int layers) {
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
     if (t == 0) return mortar_fail(MORTAR_ERR_LIMIT, "shape has no small-M kernel");
-    const bool wide = (int64_t)layers * p.n_units >= 8 * 512;
+    const int w = pick_waves(t, p, layers);
     if (t == 4) {
-        if (wide) mortar_resident_shape<4, 8>(p, layers); else mortar_resident_shape<4, 2>(p, layers);
+        if (w == 16) mortar_resident_shape<4, 16>(p, layers);
+        else if (w == 8) mortar_resident_shape<4, 8>(p, layers);
+        else mortar_resident_shape<4, 2>(p, layers);
     } else if (t == 16) {
-        if (wide) mortar_resident_shape<16, 8>(p, layers); else mortar_resident_shape<16, 2>(p, layers);
+        if (w == 16) mortar_resident_shape<16, 16>(p, layers);
+        else if (w == 8) mortar_resident_shape<16, 8>(p, layers);
+        else mortar_resident_shape<16, 2>(p, layers);
     } else {
-        if (wide) mortar_segmented_shape<16, 8, 1>(p); else mortar_segmented_shape<16, 2, 1>(p);
+        if (w == 16) mortar_segmented_shape<16, 16, 1>(p);
+        else if (w == 8) mortar_segmented_shape<16, 8, 1>(p);
+        else mortar_segmented_shape<16, 2, 1>(p);
     }
     return MORTAR_OK;
 }
