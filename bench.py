@@ -136,6 +136,28 @@ def main() -> None:
             dec[f"b{B}"] = {"us_per_mlp": t * 1e3, "tokens_per_s": B / (t * 1e-3),
                             "algorithmic_GBps": (wbytes + abytes) / (t * 1e-3) / 1e9}
         out["decode_warm"] = dec
+        # ---- the same, replayed from a HIP graph of 32 consecutive MLPs (no host launch cost in the figure) ----
+        gdec = {}
+        for B in (1, 4, 16):
+            xb = x[:B].contiguous()
+            hb = torch.empty((B, D_FF), dtype=torch.bfloat16, device=dev)
+            yb = torch.empty((B, D_MODEL), dtype=torch.bfloat16, device=dev)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    ops.gemv(xb, Wgu, swiglu_out=True, out=hb)
+                    ops.gemv(hb, Wdn, out=yb)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(32):
+                    ops.gemv(xb, Wgu, swiglu_out=True, out=hb)
+                    ops.gemv(hb, Wdn, out=yb)
+            t = event_time_ms(graph.replay, 20, 3) / 32
+            gdec[f"b{B}"] = {"us_per_mlp": t * 1e3, "tokens_per_s": B / (t * 1e-3),
+                             "algorithmic_GBps": (wbytes + B * (2 * D_MODEL + 2 * D_FF) * 2) / (t * 1e-3) / 1e9}
+        out["decode_graph"] = gdec
         # ---- decode, cold: stream distinct weight sets so that the Infinity Cache cannot hold them --------
         n_sets = 160                                                 # 160 x 2.37 MB = 379 MB > 256 MB
         packs = []
@@ -184,7 +206,7 @@ def main() -> None:
 
         def routed():
             gates, active = ops.remoe_gates(logits, TOP_K)
-            route = ops.remoe_route(active, ops.prefill_tile(Wgu))
+            route = ops.remoe_route(active, ops.route_tile(Wgu, TOKENS))
             ops.gateup_swiglu(x, Wgu, gates=gates, route=route, out=h)
             ops.spmm(h, Wdn, active=active, out=y)
         t = event_time_ms(routed, it)

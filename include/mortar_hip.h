@@ -26,8 +26,6 @@ extern "C" {
 #endif
 
 #define MORTAR_BLK 16            /* carved block edge (carve(blocking=16)) */
-#define MORTAR_PREFILL_MT 128    /* tokens per prefill workgroup tile */
-#define MORTAR_PREFILL_KCB 14    /* block-columns per prefill K-chunk */
 
 enum {
     MORTAR_OK = 0,
@@ -81,10 +79,8 @@ int mortar_encode_blocks_host(const uint8_t *packed, int64_t nnz, const float *s
 /* Inverse of the code part (for tests): device-layout dwords -> int8 codes [nnz,16,16]. */
 int mortar_decode_blocks_host(const uint32_t *codes, int64_t nnz, int8_t *codes_out);
 
-/* Prefill K-chunk table: out[r*(nkc+1)+c] = first block of row r whose column >= c*kcb
- * (nkc = ceil(Cb/kcb)); out host [Rb*(nkc+1)] int32.  Validates the BCSR (sorted, in range). */
-int mortar_chunk_ptr_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
-                          int32_t kcb, int32_t *out);
+/* Validates a BCSR (offsets start at 0 and never decrease, columns in range and strictly ascending in a row). */
+int mortar_validate_bcsr_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb);
 
 /* Octet stream of one matrix (see mortar_bcsr_t).  row_desc_out host [Rb*4] is always written; the return
  * value is the number of groups.  With codes_o_out == NULL only row_desc_out is filled (size query);
@@ -99,11 +95,19 @@ int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, int32_t Cb,
  * Cb <= this runs the single-segment prefill kernel.  Use seg_cb = ceil(Cb / ceil(Cb / max)). */
 int mortar_prefill_max_seg_cb(void);
 
-/* Row-unit schedule for uneven nnz: units sorted by descending block count and dealt so that every
- * workgroup of `group` units gets a similar total (longest-processing-time first).
- * rows_per_unit = 1 (plain) or 2 (gate row u and up row u + Rb/2).  order_out host [n_units]. */
+/* Row-unit order for uneven nnz: units sorted by descending block count and dealt into groups of `group`
+ * consecutive positions with similar totals (longest-processing-time first); use group = 16, the number of
+ * wavefronts of a prefill workgroup.  rows_per_unit = 1 (plain) or 2 (gate row u and up row u + Rb/2).
+ * order_out host [n_units]: the unit at each schedule position.  Uniform rows keep the natural order. */
 int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_t rows_per_unit, int32_t group,
                            int32_t *order_out);
+
+/* Part descriptors in schedule order, the form the kernels walk: for position pos, K segment sg and row a of
+ * the unit, sched_out[((pos*nseg + sg)*rows_per_unit + a)*4 ..] = {first octet, end octet, blocks, unit}, taken
+ * from row_desc (mortar_octet_layout_host) of row unit + a*n_units.  order: host [n_units] from
+ * mortar_unit_order_host, or NULL for the natural order.  sched_out host [n_units*nseg*rows_per_unit*4]. */
+int mortar_schedule_host(const int32_t *row_desc, int32_t Rb, int32_t nseg, int32_t rows_per_unit,
+                         const int32_t *order, int32_t *sched_out);
 
 /* Decode work list.  Splits every row unit into entries of <= max_blocks blocks inside one K segment of
  * kseg block-columns.  Each entry is 8 int32: {rowA, pA, cntA, rowB, pB, cntB, slot, seg}; rowB = -1 for
@@ -115,40 +119,37 @@ int64_t mortar_decode_worklist_host(const int32_t *row_ptr, const int16_t *col, 
                                     int32_t rows_per_unit, int32_t kseg, int32_t max_blocks,
                                     int32_t *entries_out, int32_t *nslots_out, int32_t *row_slots_out);
 
-/* ---- prefill (large M), bf16 MFMA, fp32 accumulate -------------------------------------------- */
+/* ---- SpMM on bf16 MFMA, fp32 accumulate (any M) -------------------------------------------------- */
 
-/* y[M, Rb*16] = x[M, Cb*16] @ W^T (bf16 in, bf16 out).  Replaces stk_dds(..., transpose_b=True).
- * chunk_ptr: device copy of mortar_chunk_ptr_host(kcb = MORTAR_PREFILL_KCB).
- * unit_order: device [Rb] from mortar_unit_order_host(rows_per_unit=1, group=mortar_prefill_group(0)) or NULL.
+/* y[M, Rb*16] = x[M, Cb*16] @ W^T (bf16 in, bf16 out).  Replaces stk_dds(..., transpose_b=True)
+ * (morph/sparse/stk/backend/custom_ops.py:35-56).
+ * sched: device copy of mortar_schedule_host(rows_per_unit = 1), or NULL for the natural row order.
  * ldx / ldy in elements; x and y 16-byte aligned, ldx % 8 == 0, ldy % 4 == 0. */
-int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int32_t *unit_order,
-                     const uint16_t *x, int64_t M, int64_t ldx, uint16_t *y, int64_t ldy, void *stream);
+int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M, int64_t ldx,
+                     uint16_t *y, int64_t ldy, void *stream);
 
 /* h[M, d_ff] = silu(gate) * up [* gates per cluster], gate_up = W [2*d_ff, d_model] with gate rows
  * [0, d_ff) and up rows [d_ff, 2*d_ff) (transformer.py:335-336,403-405).  Intermediates are rounded to
  * bf16 where the reference materialises a bf16 tensor.  gates: device fp32 [M, n_clusters] or NULL;
- * d_ff % n_clusters == 0.
- * Routed skipping (optional): tok_cnt/tok_list from mortar_remoe_route with tile = mortar_prefill_tile(Cb, M); when
- * given (requires cluster_size % 16 == 0) only active (token, block-row) tiles are computed and written;
- * inactive entries of h are left untouched and must be masked by the consumer (mortar_spmm_bf16_masked). */
-int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int32_t *unit_order,
-                              const uint16_t *x, int64_t M, int64_t ldx, uint16_t *h, int64_t ldh,
-                              const float *gates, int32_t n_clusters,
+ * d_ff % n_clusters == 0.  sched: mortar_schedule_host(rows_per_unit = 2) or NULL.
+ * Routed skipping (optional): tok_cnt/tok_list from mortar_remoe_route with tile = mortar_route_tile(Cb, M); when
+ * given (requires cluster_size % 16 == 0 and mortar_route_tile != 0) only active (token, block-row) tiles are
+ * computed and written; inactive entries of h are left untouched and must be masked by the consumer
+ * (mortar_spmm_bf16_masked). */
+int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M,
+                              int64_t ldx, uint16_t *h, int64_t ldh, const float *gates, int32_t n_clusters,
                               const int32_t *tok_cnt, const uint8_t *tok_list, void *stream);
 
 /* As mortar_spmm_bf16, but input element (m, c) is read as 0 when active[m, c / cluster_size] == 0
  * (active: device uint8 [M, n_clusters]); used for `down` after a routed mortar_gateup_swiglu_bf16. */
-int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *chunk_ptr, const int32_t *unit_order,
-                            const uint16_t *x, int64_t M, int64_t ldx, uint16_t *y, int64_t ldy,
-                            const uint8_t *active, int32_t n_clusters, void *stream);
+int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M,
+                            int64_t ldx, uint16_t *y, int64_t ldy, const uint8_t *active, int32_t n_clusters,
+                            void *stream);
 
-/* Token tile the gate_up kernels use for M rows against a matrix with Cb block-columns: the tile size that
- * mortar_remoe_route must be called with for routed mortar_gateup_swiglu_bf16 on that (matrix, M).
- * 4 or 16 for decode-sized M (<= 16), otherwise a multiple of 16 that depends on Cb only. */
-int mortar_prefill_tile(int32_t Cb, int64_t M);
-
-/* Units per prefill workgroup (for mortar_unit_order_host): swiglu = 0 plain, 1 gate/up pairs. */
-int mortar_prefill_group(int swiglu);
+/* Token tile of routed mortar_gateup_swiglu_bf16 for M rows against a matrix with Cb block-columns: the tile
+ * size mortar_remoe_route must be called with.  4 or 16 for decode-sized M (<= 16), otherwise 32, 64 or 96
+ * depending on Cb; 0 when in_features is too wide for routed skipping (one LDS tile must hold a row of x). */
+int mortar_route_tile(int32_t Cb, int64_t M);
 
 /* ---- ReMoE gating --------------------------------------------------------------------------- */
 
@@ -184,12 +185,13 @@ int mortar_route_flags(const float *gates, int64_t B, int32_t n_clusters, int64_
  *   mortar_stack_table_bytes  bytes of device memory the parameter table needs
  *   mortar_stack_prepare      validates the layers, writes the table (synchronous host-to-device copy);
  *                             W: host array [n_layers] of descriptors with device pointers, x / y: host arrays
- *                             of device pointers; swiglu = 0: y_l = x_l W_l^T, 1: y_l = silu(g) * u of gate_up W_l
+ *                             of device pointers, sched: host array of device schedules or NULL; swiglu = 0: y_l = x_l W_l^T, 1: y_l = silu(g) * u of gate_up W_l
  *   mortar_stack_run          launches the prepared table (any number of times); W0 = &W[0], same swiglu,
  *                             n_layers and M as prepared */
 int64_t mortar_stack_table_bytes(int32_t n_layers);
-int mortar_stack_prepare(int32_t swiglu, int32_t n_layers, const mortar_bcsr_t *W, const uint16_t *const *x,
-                         uint16_t *const *y, int64_t M, int64_t ldx, int64_t ldy, void *table_dev, void *stream);
+int mortar_stack_prepare(int32_t swiglu, int32_t n_layers, const mortar_bcsr_t *W, const int32_t *const *sched,
+                         const uint16_t *const *x, uint16_t *const *y, int64_t M, int64_t ldx, int64_t ldy,
+                         void *table_dev, void *stream);
 int mortar_stack_run(int32_t swiglu, int32_t n_layers, const mortar_bcsr_t *W0, int64_t M, const void *table_dev,
                      void *stream);
 

@@ -27,20 +27,20 @@ _SIGS = {
     "mortar_decode_blocks_host": (C.c_int, [c_vp, c_i64, c_vp]),
     "mortar_octet_layout_host": (c_i64, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "mortar_prefill_max_seg_cb": (C.c_int, []),
-    "mortar_chunk_ptr_host": (C.c_int, [c_vp, c_vp, c_i32, c_i32, c_i32, c_vp]),
+    "mortar_validate_bcsr_host": (C.c_int, [c_vp, c_vp, c_i32, c_i32]),
+    "mortar_schedule_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp]),
     "mortar_unit_order_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp]),
     "mortar_decode_worklist_host": (c_i64, [c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp]),
-    "mortar_spmm_bf16": (C.c_int, [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_i64, c_vp]),
-    "mortar_gateup_swiglu_bf16": (C.c_int, [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_i64, c_vp, c_i32,
+    "mortar_spmm_bf16": (C.c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_i64, c_vp]),
+    "mortar_gateup_swiglu_bf16": (C.c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_i64, c_vp, c_i32,
                                             c_vp, c_vp, c_vp]),
-    "mortar_spmm_bf16_masked": (C.c_int, [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_i64, c_vp, c_i32, c_vp]),
-    "mortar_prefill_group": (C.c_int, [C.c_int]),
-    "mortar_prefill_tile": (C.c_int, [c_i32, c_i64]),
+    "mortar_spmm_bf16_masked": (C.c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_i64, c_vp, c_i32, c_vp]),
+    "mortar_route_tile": (C.c_int, [c_i32, c_i64]),
     "mortar_remoe_gates": (C.c_int, [c_vp, c_i64, c_i32, c_i32, c_vp, c_vp, c_vp]),
     "mortar_remoe_route": (C.c_int, [c_vp, c_i64, c_i32, c_i32, c_vp, c_vp, c_vp]),
     "mortar_route_flags": (C.c_int, [c_vp, c_i64, c_i32, c_i64, c_i32, c_vp, c_i64, c_vp, c_i64, c_vp]),
     "mortar_stack_table_bytes": (c_i64, [c_i32]),
-    "mortar_stack_prepare": (C.c_int, [c_i32, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
+    "mortar_stack_prepare": (C.c_int, [c_i32, c_i32, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
     "mortar_stack_run": (C.c_int, [c_i32, c_i32, c_vp, c_i64, c_vp, c_vp]),
     "mortar_gemv_bf16": (C.c_int, [c_vp, c_vp, c_i64, c_i32, c_vp, c_i32, c_i32, c_vp, c_i32, c_i64, c_vp, c_i64,
                                    c_vp, c_vp, c_i32, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp]),

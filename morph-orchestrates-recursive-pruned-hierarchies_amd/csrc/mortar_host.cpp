@@ -106,21 +106,8 @@ int mortar_check_bcsr_host(const int32_t *row_ptr, const int16_t *col, int32_t R
     return MORTAR_OK;
 }
 
-extern "C" int mortar_chunk_ptr_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
-                                     int32_t kcb, int32_t *out) {
-    if (!out || kcb <= 0) return mortar_fail(MORTAR_ERR_ARG, "chunk_ptr: bad argument");
-    int rc = mortar_check_bcsr_host(row_ptr, col, Rb, Cb);
-    if (rc) return rc;
-    const int nkc = (Cb + kcb - 1) / kcb;
-    for (int r = 0; r < Rb; ++r) {
-        int p = row_ptr[r];
-        const int e = row_ptr[r + 1];
-        for (int c = 0; c <= nkc; ++c) {
-            while (p < e && col[p] < c * kcb) ++p;
-            out[(int64_t)r * (nkc + 1) + c] = (c == nkc) ? e : p;
-        }
-    }
-    return MORTAR_OK;
+extern "C" int mortar_validate_bcsr_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb) {
+    return mortar_check_bcsr_host(row_ptr, col, Rb, Cb);
 }
 
 extern "C" int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, int32_t Cb, int32_t seg_cb,
@@ -204,20 +191,34 @@ extern "C" int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_
         members[best].push_back(u);
         load[best] += cost[u];
     }
-    // inside a group the waves take consecutive runs; deal the sorted members across the runs
-    const int nw = 4, rw = std::max(1, group / nw);   // 4 wavefronts per prefill workgroup
+    // Wave w of a workgroup takes the positions w, w + group, ... of its window: every group hands one unit
+    // to each wave.  Members are in descending cost; odd groups are reversed so that no wave collects the
+    // heaviest unit of every group.
+    int o = 0;
     for (int g = 0; g < ng; ++g) {
         const int n = (int)members[g].size();
-        std::vector<int> placed(group, -1);
-        int k = 0;
-        for (int rnd = 0; rnd < rw && k < n; ++rnd)
-            for (int w = 0; w < nw && k < n; ++w) {
-                const int ww = (rnd & 1) ? nw - 1 - w : w;     // snake
-                placed[ww * rw + rnd] = members[g][k++];
+        for (int i = 0; i < n; ++i) order_out[o++] = members[g][(g & 1) ? n - 1 - i : i];
+    }
+    return MORTAR_OK;
+}
+
+extern "C" int mortar_schedule_host(const int32_t *row_desc, int32_t Rb, int32_t nseg, int32_t rows_per_unit,
+                                    const int32_t *order, int32_t *sched_out) {
+    if (!row_desc || !sched_out || Rb <= 0 || nseg <= 0 || (rows_per_unit != 1 && rows_per_unit != 2) ||
+        Rb % rows_per_unit)
+        return mortar_fail(MORTAR_ERR_ARG, "schedule: bad argument");
+    const int nu = Rb / rows_per_unit;
+    std::vector<char> seen((size_t)nu, 0);
+    for (int pos = 0; pos < nu; ++pos) {
+        const int u = order ? order[pos] : pos;
+        if (u < 0 || u >= nu || seen[(size_t)u]) return mortar_fail(MORTAR_ERR_ARG, "schedule: order is not a permutation");
+        seen[(size_t)u] = 1;
+        for (int sg = 0; sg < nseg; ++sg)
+            for (int a = 0; a < rows_per_unit; ++a) {
+                const int32_t *d = row_desc + 4 * ((int64_t)sg * Rb + u + (int64_t)a * nu);
+                int32_t *o = sched_out + 4 * (((int64_t)pos * nseg + sg) * rows_per_unit + a);
+                o[0] = d[0]; o[1] = d[1]; o[2] = d[2]; o[3] = u;
             }
-        int o = g * group;
-        for (int i = 0; i < group; ++i)
-            if (placed[i] >= 0) order_out[o++] = placed[i];
     }
     return MORTAR_OK;
 }

@@ -16,30 +16,24 @@
 #include "mortar_internal.h"
 
 struct SpmmParams {
-    const uint32_t *codes;
-    const uint32_t *sdup;
-    const int16_t *col;
-    const int32_t *chunk_ptr;
-    const int32_t *row_ptr;
     const u32x4_t *row_desc;  // octet stream: {first octet, end octet, blocks, 0} per (segment, block-row)
     const u32x4_t *codes_o;
     const u32x4_t *sd_o;
     const u32x4_t *col_o;
-    const int32_t *unit_order;
-    int n_units, nkc, Cb;
+    const u32x4_t *sched;     // part descriptors {first octet, end octet, blocks, unit} in schedule order
+                              // [(position * nseg + segment) * rows_per_unit + a], or null: position = unit
     const uint16_t *x;
-    int64_t ldx;
-    int M;
     uint16_t *y;
-    int64_t ldy;
     const float *gates;       // [M, n_clusters] fp32 or null
     const uint8_t *active;    // [M, n_clusters] input mask or null
     const int32_t *tok_cnt;   // routed: [n_mtiles, n_clusters]
     const uint8_t *tok_list;  // routed: [n_mtiles, n_clusters, MT]
+    int64_t ldx, ldy;
+    int n_units, Cb, M, Rb;
     int n_clusters, cluster_size;
-    int xcd_map, n_mtiles, n_groups;
-    int n_split;              // workgroups that share one token tile
-    int seg_cb, nseg, Rb;     // K segments of the octet stream
+    int n_mtiles, n_split;    // token tiles; workgroups that share one token tile
+    int seg_cb, nseg;         // K segments of the octet stream
+    int pad_[4];
 };
 
 // Device-side view of the launch parameters: the pointers carry the global address space in their type, so
@@ -47,9 +41,8 @@ struct SpmmParams {
 // would otherwise be generic and cost flat instructions).
 #define MORTAR_GLOBAL __attribute__((address_space(1)))
 struct SpmmView {
-    const MORTAR_GLOBAL u32x4_t *row_desc, *codes_o;
+    const MORTAR_GLOBAL u32x4_t *row_desc, *codes_o, *sched;
     const MORTAR_GLOBAL uint32_t *sd_dw, *cc_dw;      // scale patterns / block-columns of the octet stream as dwords
-    const MORTAR_GLOBAL int32_t *unit_order;
     const MORTAR_GLOBAL char *x;
     MORTAR_GLOBAL uint16_t *y;
     const MORTAR_GLOBAL float *gates;
@@ -72,8 +65,8 @@ __device__ __forceinline__ SpmmParams mortar_table_entry(const SpmmParams *table
 __device__ __forceinline__ SpmmView mortar_view(const SpmmParams &q) {
     SpmmView v;
     v.row_desc = (const MORTAR_GLOBAL u32x4_t *)q.row_desc; v.codes_o = (const MORTAR_GLOBAL u32x4_t *)q.codes_o;
+    v.sched = (const MORTAR_GLOBAL u32x4_t *)q.sched;
     v.sd_dw = (const MORTAR_GLOBAL uint32_t *)q.sd_o; v.cc_dw = (const MORTAR_GLOBAL uint32_t *)q.col_o;
-    v.unit_order = (const MORTAR_GLOBAL int32_t *)q.unit_order;
     v.x = (const MORTAR_GLOBAL char *)q.x; v.y = (MORTAR_GLOBAL uint16_t *)q.y;
     v.gates = (const MORTAR_GLOBAL float *)q.gates; v.active = (const MORTAR_GLOBAL uint8_t *)q.active;
     v.tok_cnt = (const MORTAR_GLOBAL int32_t *)q.tok_cnt; v.tok_list = (const MORTAR_GLOBAL uint8_t *)q.tok_list;
@@ -107,29 +100,43 @@ __device__ __forceinline__ uint32_t mortar_row_bcast(uint32_t v, int k) {
     }
 }
 
-// The batch loop of one row part: blocks [g0, g1) of the octet stream against the tile at `lx`.
+// One batch of the octet stream in registers: RES_GROUPS octets (8 blocks = 4 pairs each) = 16 block pairs.
+// A lane holds its code dwords of the 16 pairs (one 16-byte load per octet) and, as lane k of its 16-lane row,
+// the scale pattern and block-column of pair k (one dword each); pair u's metadata reaches the row by a DPP
+// broadcast when it is used.
+struct MortarBatch {
+    u32x4_t cw[RES_GROUPS];
+    uint32_t sdv, ccv;
+};
+
+// Loads the batch that starts at octet gq of a row part ending at octet g1 (octets past the end repeat the last).
+__device__ __forceinline__ void mortar_load_batch(const SpmmView &p, MortarBatch &b, int gq, int g1, int n, int bsel) {
+#pragma unroll
+    for (int k = 0; k < RES_GROUPS; ++k) {
+        const uint32_t gi = (uint32_t)(gq + k < g1 ? gq + k : g1 - 1) * 2u + (uint32_t)bsel;
+        b.cw[k] = p.codes_o[gi * 16u + n];
+    }
+    const int go = gq + (n >> 2);
+    const uint32_t mi = ((uint32_t)(go < g1 ? go : g1 - 1) * 2u + (uint32_t)bsel) * 4u + (uint32_t)(n & 3);
+    b.sdv = p.sd_dw[mi];
+    b.ccv = p.cc_dw[mi];
+}
+
+// One row part: octets [g0, g1) (nb blocks) of the stream against the tile at `lx`.
 // `xo_base` is the lane's unit offset inside a block-column (column half, token) plus the segment's origin.
 template <int MSUB, int LDM, bool ROUTED>
 __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *lx, int g0, int g1, int nb,
-                                                uint32_t xo_base, const uint32_t (&tk)[MSUB], int nsub,
-                                                int n, int bsel, int hsel, f32x4_t (&acc)[MSUB]) {
-    // One batch = RES_GROUPS octets (8 blocks = 4 pairs each) = 16 block pairs.  A lane loads its code dwords
-    // of the 16 pairs (one 16-byte load per octet) and, as lane k of its 16-lane row, the scale pattern and
-    // block-column of pair k (one dword each); pair u's metadata then reaches the row by a DPP broadcast.
+                                                uint32_t xo_base, const uint32_t (&tk)[MSUB], int nsub, int n,
+                                                int bsel, int hsel, f32x4_t (&acc)[MSUB]) {
     const unsigned char *lb = reinterpret_cast<const unsigned char *>(lx);
     for (int gq = g0; gq < g1; gq += RES_GROUPS) {
-        u32x4_t cw[RES_GROUPS];
-#pragma unroll
-        for (int k = 0; k < RES_GROUPS; ++k) {
-            const uint32_t gi = (uint32_t)(gq + k < g1 ? gq + k : g1 - 1) * 2u + (uint32_t)bsel;
-            cw[k] = p.codes_o[gi * 16u + n];
-        }
-        const int go = gq + (n >> 2);
-        const uint32_t mi = ((uint32_t)(go < g1 ? go : g1 - 1) * 2u + (uint32_t)bsel) * 4u + (uint32_t)(n & 3);
-        const uint32_t sdv = p.sd_dw[mi];
-        const uint32_t ccs = p.cc_dw[mi] * (uint32_t)(2 * LDM * 16);   // byte offset of the block-column in the tile
+        MortarBatch b;
+        mortar_load_batch(p, b, gq, g1, n, bsel);
+        const uint32_t ccs = __umul24(b.ccv, (uint32_t)(2 * LDM * 16));   // byte offset of the block-column in the tile
         const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;      // block pairs left in the row from this batch on
-        // activation operands are fetched two pairs ahead of the MFMAs that use them
+        // Activation operands are fetched two pairs ahead of the MFMAs that use them.  The only branches are
+        // per octet (a whole octet past the end of the part is skipped); inside an octet the four pairs run
+        // straight, pairs past the end being the all-zero padding blocks of the stream.
         constexpr int NP = 4 * RES_GROUPS;
         uint4 Bq[3][MSUB];
 #pragma unroll
@@ -139,21 +146,25 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
             for (int ms = 0; ms < MSUB; ++ms) Bq[d][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 16u : ms * 256u));
         }
 #pragma unroll
-        for (int u = 0; u < NP; ++u) {
-            if (u < pairs) {
-                const u32x4_t A = mortar_unpack8(cw[u >> 2][u & 3] << (8 * hsel), mortar_row_bcast(sdv, u));
-                if (u + 2 < NP) {
-                    const uint32_t xo = mortar_row_bcast(ccs, u + 2) + xo_base * 16u;
+        for (int k = 0; k < RES_GROUPS; ++k) {
+            if (4 * k < pairs) {
 #pragma unroll
-                    for (int ms = 0; ms < MSUB; ++ms)
-                        Bq[(u + 2) % 3][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 16u : ms * 256u));
-                }
+                for (int t = 0; t < 4; ++t) {
+                    const int u = 4 * k + t;
+                    const u32x4_t A = mortar_unpack8(b.cw[k][t] << (8 * hsel), mortar_row_bcast(b.sdv, u));
+                    if (u + 2 < NP) {
+                        const uint32_t xo = mortar_row_bcast(ccs, u + 2) + xo_base * 16u;
 #pragma unroll
-                for (int ms = 0; ms < MSUB; ++ms) {
-                    if (!ROUTED || ms < nsub) {
-                        const uint4 bq = Bq[u % 3][ms];
-                        const u32x4_t Bv = {bq.x, bq.y, bq.z, bq.w};
-                        acc[ms] = mortar_mfma(A, Bv, acc[ms]);
+                        for (int ms = 0; ms < MSUB; ++ms)
+                            Bq[(u + 2) % 3][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 16u : ms * 256u));
+                    }
+#pragma unroll
+                    for (int ms = 0; ms < MSUB; ++ms) {
+                        if (!ROUTED || ms < nsub) {
+                            const uint4 bq = Bq[u % 3][ms];
+                            const u32x4_t Bv = {bq.x, bq.y, bq.z, bq.w};
+                            acc[ms] = mortar_mfma(A, Bv, acc[ms]);
+                        }
                     }
                 }
             }
@@ -217,10 +228,21 @@ __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, i
     *(MORTAR_GLOBAL u32x2_t *)(p.y + (int64_t)tok * p.ldy + unit * 16 + 4 * g) = pk;
 }
 
+// Part descriptor of schedule position `pos`, segment `sg`, row `a` of the unit: {g0, g1, nb, unit}.
+template <int NACC>
+__device__ __forceinline__ u32x4_t mortar_part_desc(const SpmmView &p, int pos, int sg, int a) {
+    pos = pos < p.n_units ? pos : p.n_units - 1;
+    if (p.sched) return p.sched[((uint32_t)pos * (uint32_t)p.nseg + (uint32_t)sg) * NACC + a];
+    u32x4_t d = p.row_desc[sg * p.Rb + pos + a * p.n_units];
+    d[3] = (uint32_t)pos;
+    return d;
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // Resident kernel.  The workgroup stages x[MT, K] once; then every wave walks whole row units on its own,
 // streaming the unit's block pairs straight from global memory in batches (a row's blocks are contiguous).
-// No barrier after the first one; latency is hidden by the waves that share a SIMD.
+// No barrier after the first one.  A wave's work is a chain of row parts (unit, segment, row of the unit) whose
+// descriptors come from the schedule table one part ahead; latency is hidden by the waves that share a SIMD.
 // ---------------------------------------------------------------------------------------------------------
 template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE>
 __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmParams p0, const SpmmParams *table) {
@@ -236,27 +258,22 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
     const uint32_t lane_xo = (uint32_t)(hsel * LDM + (ROUTED ? 0 : n));
     const bool has_gates = p.gates != nullptr;
 
+    const int per = (p.n_units + p.n_split - 1) / p.n_split;
+    const int u_end = (sp + 1) * per < p.n_units ? (sp + 1) * per : p.n_units;
+    int pos = sp * per + wave;
+    // coordinates of the part after the current one; its descriptor is fetched while the current part runs
+    auto advance = [&](int &ps, int &s, int &a_) {
+        if (++a_ == NACC) { a_ = 0; if (++s == p.nseg) { s = 0; ps += WAVES; } }
+    };
+    int p1 = pos, s1 = 0, a1 = 0;
+    advance(p1, s1, a1);
+    u32x4_t d0 = mortar_part_desc<NACC>(p, pos, 0, 0);
+
     mortar_stage_tile<MT, WAVES, false>(p, lx, m0, 0, p.Cb, tid);
     __syncthreads();
 
-    const int per = (p.n_units + p.n_split - 1) / p.n_split;
-    const int u_end = (sp + 1) * per < p.n_units ? (sp + 1) * per : p.n_units;
-    // Unit ids are fetched two units ahead and row descriptors one row part ahead, so that no dependent global
-    // round trip (order -> descriptor -> blocks) is exposed between two units of a wave.
-    auto unit_of = [&](int pos_) { return (p.unit_order && pos_ < u_end) ? p.unit_order[pos_] : pos_; };
-    auto desc_of = [&](int unit_, int a_, int sg_) {
-        const int r = unit_ + a_ * p.n_units;
-        return p.row_desc[sg_ * p.Rb + (r < p.Rb ? r : 0)];
-    };
-    int pos = sp * per + wave;
-    int unit_v = unit_of(pos), unit_v1 = unit_of(pos + WAVES);
-    u32x4_t dcur[NACC], dnxt[NACC];
-#pragma unroll
-    for (int a = 0; a < NACC; ++a) dcur[a] = desc_of(unit_v, a, 0);
     for (; pos < u_end; pos += WAVES) {
-        const int unit = __builtin_amdgcn_readfirstlane(unit_v);
-        const int unit_v2 = unit_of(pos + 2 * WAVES);
-        const int unit_n = unit_v1 < p.n_units ? unit_v1 : 0;
+        const int unit = __builtin_amdgcn_readfirstlane((int)d0[3]);
         int cnt = MT;
         uint32_t tk[MSUB];
 #pragma unroll
@@ -281,24 +298,17 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
             for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
         for (int sg = 0; sg < p.nseg; ++sg) {
-            const bool last = sg + 1 == p.nseg;
-            int rg0[NACC], rg1[NACC], rnb[NACC];
-#pragma unroll
-            for (int a = 0; a < NACC; ++a) {
-                dnxt[a] = desc_of(last ? unit_n : unit, a, last ? 0 : sg + 1);
-                rg0[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][0]);
-                rg1[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][1]);
-                rnb[a] = __builtin_amdgcn_readfirstlane((int)dcur[a][2]);
-                dcur[a] = dnxt[a];
-            }
-            if (skip) continue;
             const uint32_t xo_base = lane_xo + (uint32_t)(sg * p.seg_cb) * (2 * LDM);
 #pragma unroll
-            for (int a = 0; a < NACC; ++a)
-                mortar_row_part<MSUB, LDM, ROUTED>(p, lx, rg0[a], rg1[a], rnb[a], xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+            for (int a = 0; a < NACC; ++a) {
+                const u32x4_t d1 = mortar_part_desc<NACC>(p, p1, s1, a1);
+                const int g0 = __builtin_amdgcn_readfirstlane((int)d0[0]), g1 = __builtin_amdgcn_readfirstlane((int)d0[1]);
+                const int nb = __builtin_amdgcn_readfirstlane((int)d0[2]);
+                if (!skip) mortar_row_part<MSUB, LDM, ROUTED>(p, lx, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+                d0 = d1;
+                advance(p1, s1, a1);
+            }
         }
-        unit_v = unit_v1;
-        unit_v1 = unit_v2;
         if (skip) continue;
 
 #pragma unroll
@@ -315,11 +325,13 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
 // ---------------------------------------------------------------------------------------------------------
 // Segmented kernel for matrices whose K does not fit in LDS at once (e.g. `down`, K = d_ff).  The workgroup
 // walks the K segments of the octet stream: per segment it stages x[MT, 16*seg_cb] (one barrier pair), and
-// every wave multiplies the segment's blocks of its own UPW row units.
+// every wave multiplies the segment's blocks of its own UPW row units, whose accumulators stay in registers.
+// The descriptors of the next segment are fetched before the barrier pair, so their latency hides behind the
+// staging.
 // ---------------------------------------------------------------------------------------------------------
 template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE>
 __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const SpmmParams p0, const SpmmParams *table) {
-    constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1;
+    constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1, NP = UPW * NACC;
     const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint4 *lx = reinterpret_cast<uint4 *>(smem);
@@ -331,16 +343,9 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
     const uint32_t lane_xo = (uint32_t)(hsel * LDM + n);
     const bool has_gates = p.gates != nullptr;
 
-    // this wave's units: positions sp*per + wave + WAVES*k of the schedule
+    // this wave's units: schedule positions sp*per + wave + WAVES*k
     constexpr int per = WAVES * UPW;
-    int units[UPW];
-#pragma unroll
-    for (int k = 0; k < UPW; ++k) {
-        const int pos = sp * per + wave + WAVES * k;
-        int u = -1;
-        if (pos < p.n_units) u = p.unit_order ? p.unit_order[pos] : pos;
-        units[k] = __builtin_amdgcn_readfirstlane(u);
-    }
+    const int pos0 = sp * per + wave;
     f32x4_t acc[UPW][NACC][MSUB];
     uint32_t tk[MSUB];
 #pragma unroll
@@ -352,29 +357,34 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
 #pragma unroll
             for (int ms = 0; ms < MSUB; ++ms) acc[k][a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
+    u32x4_t dn[NP];     // descriptors of the coming segment, part q = k * NACC + a
+#pragma unroll
+    for (int q = 0; q < NP; ++q) dn[q] = mortar_part_desc<NACC>(p, pos0 + WAVES * (q / NACC), 0, q % NACC);
+    int units[UPW];
+
     for (int sg = 0; sg < p.nseg; ++sg) {
         const int c0 = sg * p.seg_cb;
         const int ncb = p.Cb - c0 < p.seg_cb ? p.Cb - c0 : p.seg_cb;
-        // row descriptors of this segment (loaded before the barrier so that their latency is hidden)
-        u32x4_t desc[UPW][NACC];
+        int g0[NP], g1[NP], nb[NP];
 #pragma unroll
-        for (int k = 0; k < UPW; ++k)
+        for (int q = 0; q < NP; ++q) {
+            const bool on = pos0 + WAVES * (q / NACC) < p.n_units;
+            g0[q] = on ? __builtin_amdgcn_readfirstlane((int)dn[q][0]) : 0;
+            g1[q] = on ? __builtin_amdgcn_readfirstlane((int)dn[q][1]) : 0;
+            nb[q] = __builtin_amdgcn_readfirstlane((int)dn[q][2]);
+            if (q % NACC == 0) units[q / NACC] = on ? __builtin_amdgcn_readfirstlane((int)dn[q][3]) : -1;
+        }
+        if (sg + 1 < p.nseg) {
 #pragma unroll
-            for (int a = 0; a < NACC; ++a)
-                desc[k][a] = p.row_desc[(int64_t)sg * p.Rb + (units[k] < 0 ? 0 : units[k] + a * p.n_units)];
+            for (int q = 0; q < NP; ++q) dn[q] = mortar_part_desc<NACC>(p, pos0 + WAVES * (q / NACC), sg + 1, q % NACC);
+        }
         if (sg > 0) __syncthreads();
         mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, c0, ncb, tid);
         __syncthreads();
 #pragma unroll
-        for (int k = 0; k < UPW; ++k) {
-            if (units[k] < 0) continue;
-#pragma unroll
-            for (int a = 0; a < NACC; ++a) {
-                const int g0 = __builtin_amdgcn_readfirstlane((int)desc[k][a][0]);
-                const int g1 = __builtin_amdgcn_readfirstlane((int)desc[k][a][1]);
-                const int nb = __builtin_amdgcn_readfirstlane((int)desc[k][a][2]);
-                mortar_row_part<MSUB, LDM, false>(p, lx, g0, g1, nb, lane_xo, tk, MSUB, n, bsel, hsel, acc[k][a]);
-            }
+        for (int q = 0; q < NP; ++q) {
+            mortar_row_part<MSUB, LDM, false>(p, lx, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
+                                              acc[q / NACC][q % NACC]);
         }
     }
 
@@ -418,9 +428,11 @@ template <int MT, int WAVES>
 inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
     p.n_mtiles = (p.M + MT - 1) / MT;
     // Prefill tiles: enough workgroups to cover the 256 CUs twice (every workgroup stages a whole tile, so few
-    // large ones).  Decode tiles stage little: many small workgroups (about 12 per CU, at least `upw` units
-    // per wave) so that the hardware dispatcher evens out the load.
-    constexpr int upw = MT <= 4 ? 2 : (MT <= 16 ? 4 : 1);
+    // large ones).  Decode tiles stage little: many small workgroups (about 12 per CU) so that the hardware
+    // dispatcher evens out the load, with a few units per wave when many layers share the launch and one unit
+    // per wave when a single matrix has to be spread over the whole chip.
+    const bool wide = (int64_t)layers * p.n_units >= 8 * 512;
+    const int upw = MT > 16 || !wide ? 1 : (MT <= 4 ? 2 : 4);
     const int target = MT <= 16 ? 256 * 12 : 256 * 2;
     int split = (target + layers * p.n_mtiles - 1) / (layers * p.n_mtiles);
     const int max_split = (p.n_units + WAVES * upw - 1) / (WAVES * upw);

@@ -51,12 +51,13 @@ class MortarDecodeMLP:
         rt = getattr(self.mlp, "router", None)
         if gates is None and rt is not None:
             gates = rt(xn, iter_idx=self.iter_idx)[0].reshape(B, -1).float().contiguous()
-        if gates is not None and (self.d_ff // gates.shape[-1]) % 16 == 0:
+        tile = ops.route_tile(self.Mgu, B) if gates is not None and (self.d_ff // gates.shape[-1]) % 16 == 0 else 0
+        if tile:
             # gather-skip: only (stream, block-row) tiles of active clusters are computed; `down` reads the
             # hidden activations of inactive clusters as zero
             gates = gates.contiguous()
             active = (gates > 0).to(torch.uint8)
-            route = ops.remoe_route(active, ops.prefill_tile(self.Mgu, B))
+            route = ops.remoe_route(active, tile)
             h = ops.gateup_swiglu(xn, self.Mgu, gates=gates, route=route)
             return ops.spmm(h, self.Mdown, active=active).view(B, 1, -1)
         h = ops.gateup_swiglu(xn, self.Mgu, gates=gates.contiguous() if gates is not None else None)

@@ -11,7 +11,6 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from . import ops
-from .pack import PREFILL_MT
 from .sparsity import MortarLinear
 
 
@@ -112,10 +111,11 @@ class _SwiGLUMortar(nn.Module):
         N = xb.shape[0]
         # one path for prefill and decode: the library picks 4- or 16-token tiles for decode-sized N
         cs = self.d_ff // gates.shape[-1] if gates is not None else 0
-        if gates is not None and self.route_skip and cs % 16 == 0 and N > 0:
+        tile = ops.route_tile(Wgu, N) if (gates is not None and self.route_skip and cs % 16 == 0 and N > 0) else 0
+        if tile:
             if active is None:
                 active = (gates > 0).to(torch.uint8)
-            route = ops.remoe_route(active, ops.prefill_tile(Wgu, N))
+            route = ops.remoe_route(active, tile)
             h = ops.gateup_swiglu(xb, Wgu, gates=gates, route=route)
             y = ops.spmm(h, Wdn, active=active)
         else:

@@ -8,7 +8,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .pack import BLK, PREFILL_MT, MortarPack
+from .pack import BLK, MortarPack
 
 
 def _stream(t: Tensor):
@@ -49,15 +49,14 @@ def spmm(x: Tensor, W: MortarPack, out: Tensor | None = None, active: Tensor | N
     if M == 0:
         return y
     L = _lib.lib()
-    order = W.unit_order(1)
+    sched = W.sched(1)
     if active is None:
-        rc = L.mortar_spmm_bf16(C.byref(W.struct), _p(W.chunk_ptr), _p(order), _p(x), M, x.stride(0), _p(y),
-                                y.stride(0), _stream(x))
+        rc = L.mortar_spmm_bf16(C.byref(W.struct), _p(sched), _p(x), M, x.stride(0), _p(y), y.stride(0), _stream(x))
     else:
         if active.dtype != torch.uint8 or not active.is_contiguous():
             raise TypeError("spmm: active must be a contiguous uint8 tensor")
-        rc = L.mortar_spmm_bf16_masked(C.byref(W.struct), _p(W.chunk_ptr), _p(order), _p(x), M, x.stride(0), _p(y),
-                                       y.stride(0), _p(active), active.shape[1], _stream(x))
+        rc = L.mortar_spmm_bf16_masked(C.byref(W.struct), _p(sched), _p(x), M, x.stride(0), _p(y), y.stride(0),
+                                       _p(active), active.shape[1], _stream(x))
     _lib.check(rc, "mortar_spmm_bf16")
     return y
 
@@ -80,9 +79,8 @@ def gateup_swiglu(x: Tensor, W: MortarPack, gates: Tensor | None = None, route: 
             raise TypeError("gateup_swiglu: gates must be a contiguous float32 [M, n_clusters] tensor")
         ncl = gates.shape[1]
     cnt, lst = route if route is not None else (None, None)
-    rc = _lib.lib().mortar_gateup_swiglu_bf16(C.byref(W.struct), _p(W.chunk_ptr), _p(W.unit_order(2)), _p(x), M,
-                                              x.stride(0), _p(h), h.stride(0), _p(gates), ncl, _p(cnt), _p(lst),
-                                              _stream(x))
+    rc = _lib.lib().mortar_gateup_swiglu_bf16(C.byref(W.struct), _p(W.sched(2)), _p(x), M, x.stride(0), _p(h),
+                                              h.stride(0), _p(gates), ncl, _p(cnt), _p(lst), _stream(x))
     _lib.check(rc, "mortar_gateup_swiglu_bf16")
     return h
 
@@ -105,12 +103,13 @@ def remoe_gates(logits: Tensor, k: int) -> tuple[Tensor, Tensor]:
     return gates, active
 
 
-def prefill_tile(W: MortarPack, M: int = 0) -> int:
-    """Token tile of the gate_up kernels for M rows against this matrix (the tile remoe_route must use)."""
-    return int(_lib.lib().mortar_prefill_tile(W.Cb, int(M)))
+def route_tile(W: MortarPack, M: int = 0) -> int:
+    """Token tile of the routed gate_up kernels for M rows against this matrix (the tile remoe_route must use);
+    0 when the matrix is too wide for routed skipping (use the dense gated call)."""
+    return int(_lib.lib().mortar_route_tile(W.Cb, int(M)))
 
 
-def remoe_route(active: Tensor, tile: int = PREFILL_MT) -> tuple[Tensor, Tensor]:
+def remoe_route(active: Tensor, tile: int) -> tuple[Tensor, Tensor]:
     """Per (token tile, cluster): count and ascending list of the tile-local indices of active tokens."""
     _need_gpu(active, "remoe_route")
     if active.dtype != torch.uint8 or active.dim() != 2 or not active.is_contiguous():
@@ -213,10 +212,11 @@ class LayerStack:
         L = _lib.lib()
         self.packs, self.xs, self.ys, self.swiglu, self.M, self.n = packs, xs, ys, int(bool(swiglu)), M, n
         self._structs = (_lib.BcsrStruct * n)(*[p.struct for p in packs])
+        sp = (C.c_void_p * n)(*[p.sched(2 if swiglu else 1).data_ptr() for p in packs])
         xp = (C.c_void_p * n)(*[x.data_ptr() for x in xs])
         yp = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
         self.table = torch.empty(int(L.mortar_stack_table_bytes(n)), dtype=torch.uint8, device=xs[0].device)
-        _lib.check(L.mortar_stack_prepare(self.swiglu, n, self._structs, xp, yp, M, xs[0].stride(0), ys[0].stride(0),
+        _lib.check(L.mortar_stack_prepare(self.swiglu, n, self._structs, sp, xp, yp, M, xs[0].stride(0), ys[0].stride(0),
                                           _p(self.table), _stream(xs[0])), "mortar_stack_prepare")
 
     def run(self) -> list[Tensor]:

@@ -15,8 +15,7 @@ import torch
 from . import _lib
 
 BLK = 16
-PREFILL_KCB = 14
-PREFILL_MT = 128
+SCHED_GROUP = 16      # wavefronts of a prefill workgroup: the group size of the row-unit order
 
 
 def _np(a, dtype):
@@ -50,12 +49,9 @@ def decode_blocks(codes: np.ndarray) -> np.ndarray:
     return out
 
 
-def chunk_ptr(offsets, col, Rb: int, Cb: int, kcb: int = PREFILL_KCB) -> np.ndarray:
+def validate_bcsr(offsets, col, Rb: int, Cb: int) -> None:
     offsets, col = _np(offsets, np.int32), _np(col, np.int16)
-    nkc = -(-Cb // kcb)
-    out = np.empty((Rb, nkc + 1), dtype=np.int32)
-    _lib.check(_lib.lib().mortar_chunk_ptr_host(_vp(offsets), _vp(col), Rb, Cb, kcb, _vp(out)), "mortar_chunk_ptr_host")
-    return out
+    _lib.check(_lib.lib().mortar_validate_bcsr_host(_vp(offsets), _vp(col), Rb, Cb), "mortar_validate_bcsr_host")
 
 
 def octet_layout(offsets, Rb: int, Cb: int, seg_cb: int, codes: np.ndarray, sdup: np.ndarray, col):
@@ -75,11 +71,20 @@ def octet_layout(offsets, Rb: int, Cb: int, seg_cb: int, codes: np.ndarray, sdup
     return grp, codes_o, sd_o, col_o
 
 
-def unit_order(offsets, Rb: int, rows_per_unit: int) -> np.ndarray:
+def unit_order(offsets, Rb: int, rows_per_unit: int, group: int = SCHED_GROUP) -> np.ndarray:
     offsets = _np(offsets, np.int32)
-    group = _lib.lib().mortar_prefill_group(1 if rows_per_unit == 2 else 0)
     out = np.empty(Rb // rows_per_unit, dtype=np.int32)
     _lib.check(_lib.lib().mortar_unit_order_host(_vp(offsets), Rb, rows_per_unit, group, _vp(out)), "mortar_unit_order_host")
+    return out
+
+
+def schedule(row_desc: np.ndarray, Rb: int, nseg: int, rows_per_unit: int, order: np.ndarray | None) -> np.ndarray:
+    """Part descriptors in schedule order [n_units, nseg, rows_per_unit, 4] int32: see mortar_schedule_host."""
+    row_desc = _np(row_desc, np.int32)
+    out = np.empty((Rb // rows_per_unit, nseg, rows_per_unit, 4), dtype=np.int32)
+    o = _np(order, np.int32) if order is not None else None
+    _lib.check(_lib.lib().mortar_schedule_host(_vp(row_desc), Rb, nseg, rows_per_unit, _vp(o) if o is not None else None,
+                                               _vp(out)), "mortar_schedule_host")
     return out
 
 
@@ -121,22 +126,23 @@ class MortarPack:
             raise RuntimeError("carved matrix has a block-row with zero kept blocks")
         self.device = torch.device(device)
         codes, sdup = encode_blocks(packed, self.nnz, scale)
-        self.h_chunk_ptr = chunk_ptr(self.h_offsets, self.h_col, self.Rb, self.Cb)      # also validates the BCSR
+        validate_bcsr(self.h_offsets, self.h_col, self.Rb, self.Cb)
         dev = self.device
         self.codes = torch.from_numpy(codes.view(np.int32)).to(dev)
         self.sdup = torch.from_numpy(sdup.view(np.int32)).to(dev)
         self.col = torch.from_numpy(self.h_col).to(dev)
         self.row_ptr = torch.from_numpy(self.h_offsets).to(dev)
-        self.chunk_ptr = torch.from_numpy(self.h_chunk_ptr).to(dev)
         max_seg = int(_lib.lib().mortar_prefill_max_seg_cb())
         nseg = -(-self.Cb // max_seg)
         self.seg_cb = -(-self.Cb // nseg)
         grp, codes_o, sd_o, col_o = octet_layout(self.h_offsets, self.Rb, self.Cb, self.seg_cb, codes, sdup, self.h_col)
+        self.nseg = nseg
+        self.h_row_desc = grp
         self.row_desc = torch.from_numpy(grp).to(dev)
         self.codes_o = torch.from_numpy(codes_o.view(np.int32)).to(dev)
         self.sd_o = torch.from_numpy(sd_o.view(np.int32)).to(dev)
         self.col_o = torch.from_numpy(col_o).to(dev)
-        self._orders: dict[int, torch.Tensor] = {}
+        self._scheds: dict[int, torch.Tensor] = {}
         self._worklists: dict[tuple, tuple] = {}
         self.struct = self._make_struct()
 
@@ -145,11 +151,13 @@ class MortarPack:
                                self.row_ptr.data_ptr(), self.row_desc.data_ptr(), self.codes_o.data_ptr(),
                                self.sd_o.data_ptr(), self.col_o.data_ptr(), self.Rb, self.Cb, self.nnz, self.seg_cb)
 
-    def unit_order(self, rows_per_unit: int) -> torch.Tensor:
-        if rows_per_unit not in self._orders:
+    def sched(self, rows_per_unit: int) -> torch.Tensor:
+        """Device schedule (mortar_schedule_host over the balanced unit order) for plain (1) or gate/up (2) units."""
+        if rows_per_unit not in self._scheds:
             o = unit_order(self.h_offsets, self.Rb, rows_per_unit)
-            self._orders[rows_per_unit] = torch.from_numpy(o).to(self.device)
-        return self._orders[rows_per_unit]
+            sc = schedule(self.h_row_desc, self.Rb, self.nseg, rows_per_unit, o)
+            self._scheds[rows_per_unit] = torch.from_numpy(sc).to(self.device)
+        return self._scheds[rows_per_unit]
 
     def worklist(self, rows_per_unit: int, kseg: int, max_blocks: int):
         key = (rows_per_unit, kseg, max_blocks)
@@ -167,9 +175,9 @@ class MortarPack:
         """A second resident copy (own device buffers and schedules) of the same matrix."""
         import copy
         c = copy.copy(self)
-        for name in ("codes", "sdup", "col", "row_ptr", "chunk_ptr", "row_desc", "codes_o", "sd_o", "col_o"):
+        for name in ("codes", "sdup", "col", "row_ptr", "row_desc", "codes_o", "sd_o", "col_o"):
             setattr(c, name, getattr(self, name).clone())
-        c._orders = {k: v.clone() for k, v in self._orders.items()}
+        c._scheds = {k: v.clone() for k, v in self._scheds.items()}
         c._worklists = {k: (v[0].clone(), v[1], v[2].clone(), v[3]) for k, v in self._worklists.items()}
         c.struct = c._make_struct()
         return c

@@ -125,7 +125,7 @@ def test_mlp_with_gates_and_skip(dev):
     xd = to_dev(x, dev)
     h_dense = ops.gateup_swiglu(xd, Wgu, gates=gates)
     assert_close_bf16(to_np(h_dense), ref["h"], "h gated", ulps=4)
-    cnt, lst = ops.remoe_route(active, ops.prefill_tile(Wgu, M))
+    cnt, lst = ops.remoe_route(active, ops.route_tile(Wgu, M))
     h_skip = torch.full_like(h_dense, float("nan"))                             # untouched entries stay NaN
     ops.gateup_swiglu(xd, Wgu, gates=gates, route=(cnt, lst), out=h_skip)
     hs, hd = to_np(h_skip), to_np(h_dense)
@@ -215,7 +215,7 @@ def test_decode_small_tiles(dev, B, dims):
         assert_close_bf16(to_np(y), ref["y"], "y", ulps=8)
         if gates is not None:                                                        # gather-skip form
             active = (gd > 0).to(torch.uint8)
-            tile = ops.prefill_tile(Wgu, B)
+            tile = ops.route_tile(Wgu, B)
             assert tile == (4 if B <= 4 else 16)
             route = ops.remoe_route(active, tile)
             hs = torch.full_like(h, float("nan"))
@@ -365,7 +365,7 @@ def test_full_size_properties(dev):
     g_ref, a_ref = O.remoe_gates(lg, 88)
     gates, active = ops.remoe_gates(torch.from_numpy(lg).to(dev), 88)
     assert np.array_equal(active.cpu().numpy().astype(bool), a_ref)
-    cnt, lst = ops.remoe_route(active, ops.prefill_tile(Wgu, 4096))
+    cnt, lst = ops.remoe_route(active, ops.route_tile(Wgu, 4096))
     assert int(cnt.sum()) == int(a_ref.sum())
     hr = ops.gateup_swiglu(xd, Wgu, gates=gates, route=(cnt, lst))
     yr = ops.spmm(hr, Wdn, active=active)

@@ -67,22 +67,58 @@ def test_encode_scalar_scale_and_errors():
     assert not dw0.any() and not sd0.any()
 
 
-def test_chunk_ptr_partitions_rows():
+def test_validate_bcsr_rejects_bad_layouts():
     m = synth.synth_matrix(16 * 9, 16 * 50, 0.3, 3, zipf_s=1.2)
-    cp = P.chunk_ptr(m["offsets"], m["col_idx"], 9, 50, 14)
-    assert cp.shape == (9, 5)
-    for r in range(9):
-        assert cp[r, 0] == m["offsets"][r] and cp[r, -1] == m["offsets"][r + 1]
-        for c in range(4):
-            cols = m["col_idx"][cp[r, c]:cp[r, c + 1]]
-            assert ((cols >= c * 14) & (cols < (c + 1) * 14)).all()
+    P.validate_bcsr(m["offsets"], m["col_idx"], 9, 50)
     bad = m["col_idx"].copy(); bad[1] = bad[0]
     with pytest.raises(ValueError, match="ascending"):
-        P.chunk_ptr(m["offsets"], bad, 9, 50, 14)
+        P.validate_bcsr(m["offsets"], bad, 9, 50)
+    bad = m["col_idx"].copy(); bad[0] = 50
+    with pytest.raises(ValueError, match="out of range"):
+        P.validate_bcsr(m["offsets"], bad, 9, 50)
+    off = m["offsets"].copy(); off[3] = off[2] - 1
+    with pytest.raises(ValueError, match="decrease"):
+        P.validate_bcsr(off, m["col_idx"], 9, 50)
 
 
-def test_unit_order_is_balanced_permutation():
+@pytest.mark.parametrize("seg_cb", [50, 17, 7])
+def test_octet_stream_holds_every_block_once(seg_cb):
+    """Decoding the octet stream back (codes, scale pattern, column) reproduces the BCSR exactly, for one and
+    for several K segments; padding blocks are all-zero."""
+    Rb, Cb = 9, 50
+    m = synth.synth_matrix(16 * Rb, 16 * Cb, 0.3, 3, zipf_s=1.2)
+    nnz = int(m["offsets"][-1])
+    dw, sdup = P.encode_blocks(O.pack_ternary_codes(m["codes"]), nnz, m["scales"])
+    desc, codes_o, sd_o, col_o = P.octet_layout(m["offsets"], Rb, Cb, seg_cb, dw, sdup, m["col_idx"])
+    nseg = -(-Cb // seg_cb)
+    desc = desc.reshape(nseg, Rb, 4)
+    codes_o = codes_o.reshape(-1, 2, 16, 4); sd_o = sd_o.reshape(-1, 2, 4); col_o = col_o.reshape(-1, 2, 4)
+    used = np.zeros(codes_o.shape[0], bool)
+    for r in range(Rb):
+        got = []
+        for sg in range(nseg):
+            g0, g1, nb, _ = desc[sg, r]
+            assert g1 - g0 == -(-nb // 8) and not used[g0:g1].any()
+            used[g0:g1] = True
+            for b in range(8 * (g1 - g0)):
+                g, t, s2 = g0 + b // 8, (b % 8) // 2, b % 2
+                if b < nb:
+                    got.append((int(col_o[g, s2, t]) + sg * seg_cb, int(sd_o[g, s2, t]), codes_o[g, s2, :, t].copy()))
+                    assert 0 <= col_o[g, s2, t] < seg_cb
+                else:
+                    assert sd_o[g, s2, t] == 0 and not codes_o[g, s2, :, t].any()
+        lo, hi = m["offsets"][r], m["offsets"][r + 1]
+        assert [c for c, _, _ in got] == m["col_idx"][lo:hi].tolist()
+        assert [s for _, s, _ in got] == sdup[lo:hi].tolist()
+        assert np.array_equal(np.stack([w for _, _, w in got]), dw.reshape(-1, 16)[lo:hi])
+    assert used.all()
+
+
+def test_unit_order_and_schedule():
     m = synth.synth_matrix(16 * 64, 16 * 40, 0.25, 4, zipf_s=1.2)
+    nnz = int(m["offsets"][-1])
+    dw, sdup = P.encode_blocks(O.pack_ternary_codes(m["codes"]), nnz, m["scales"])
+    desc, _, _, _ = P.octet_layout(m["offsets"], 64, 40, 17, dw, sdup, m["col_idx"])
     for rpu in (1, 2):
         o = P.unit_order(m["offsets"], 64, rpu)
         nu = 64 // rpu
@@ -90,12 +126,32 @@ def test_unit_order_is_balanced_permutation():
         cost = np.diff(m["offsets"])
         if rpu == 2:
             cost = cost[:nu] + cost[nu:]
-        group = _lib.lib().mortar_prefill_group(rpu == 2)
+        group = P.SCHED_GROUP
         loads = [cost[o[g:g + group]].sum() for g in range(0, nu, group)]
         naive = [cost[g:g + group].sum() for g in range(0, nu, group)]
         assert max(loads) <= max(naive)
+        sc = P.schedule(desc, 64, 3, rpu, o)                                            # [nu, nseg, rpu, 4]
+        d3 = desc.reshape(3, 64, 4)
+        for pos in (0, 1, nu - 1):
+            for sg in range(3):
+                for a in range(rpu):
+                    assert sc[pos, sg, a, :3].tolist() == d3[sg, o[pos] + a * nu, :3].tolist()
+                    assert sc[pos, sg, a, 3] == o[pos]
+        ident = P.schedule(desc, 64, 3, rpu, None)
+        assert ident[:, 0, 0, 3].tolist() == list(range(nu))
+        with pytest.raises(ValueError, match="permutation"):
+            P.schedule(desc, 64, 3, rpu, np.zeros(nu, np.int32))
     u = synth.synth_matrix(16 * 8, 16 * 8, 0.25, 5)
     assert P.unit_order(u["offsets"], 8, 1).tolist() == list(range(8))             # uniform rows keep natural order
+
+
+def test_tile_queries():
+    L = _lib.lib()
+    assert L.mortar_prefill_max_seg_cb() == 151
+    assert L.mortar_route_tile(128, 4096) == 32 and L.mortar_route_tile(48, 4096) == 96
+    assert L.mortar_route_tile(128, 1) == 4 and L.mortar_route_tile(128, 16) == 16
+    assert L.mortar_route_tile(352, 4096) == 0                                      # too wide for routed skipping
+    assert L.mortar_stack_table_bytes(3) % 16 == 0 and L.mortar_stack_table_bytes(0) == 0
 
 
 @pytest.mark.parametrize("rpu,kseg,mb", [(1, 1000, 1 << 20), (2, 1000, 1 << 20), (1, 7, 3), (2, 16, 4)])
