@@ -214,6 +214,14 @@ def main() -> None:
         out["routed_prefill"] = {"ms": t, "tokens_per_s": TOKENS / (t * 1e-3),
                                  "active_fraction": n_act / (TOKENS * N_CLUSTERS)}
 
+    # A plain device-to-device copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE counters when this
+    # command runs under `rocprofv3 --pmc` (counter KiB per byte copied), and a practical HBM bandwidth figure.
+    cal_src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).fill_(1)
+    cal_dst = torch.empty_like(cal_src)
+    t_cal = event_time_ms(lambda: cal_dst.copy_(cal_src), 10, 2)
+    out["copy_calibration"] = {"bytes_read": cal_src.numel(), "bytes_written": cal_dst.numel(), "ms": t_cal,
+                               "GBps_read_plus_write": 2 * cal_src.numel() / (t_cal * 1e-3) / 1e9}
+
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(spec, args.cpu_tokens)
     else:

@@ -79,9 +79,9 @@ int mortar_smallm_shape(int kind, SpmmParams &p, int layers) {
         else if (w == 8) mortar_resident_shape<16, 8>(p, layers);
         else mortar_resident_shape<16, 2>(p, layers);
     } else {
-        if (w == 16) mortar_segmented_shape<16, 16, 1>(p);
-        else if (w == 8) mortar_segmented_shape<16, 8, 1>(p);
-        else mortar_segmented_shape<16, 2, 1>(p);
+        if (w == 16) mortar_segmented_shape<16, 16, 1>(p, layers);
+        else if (w == 8) mortar_segmented_shape<16, 8, 1>(p, layers);
+        else mortar_segmented_shape<16, 2, 1>(p, layers);
     }
     return MORTAR_OK;
 }

@@ -33,7 +33,8 @@ struct SpmmParams {
     int n_clusters, cluster_size;
     int n_mtiles, n_split;    // token tiles; workgroups that share one token tile
     int seg_cb, nseg;         // K segments of the octet stream
-    int pad_[4];
+    int xcd_map;              // 1: workgroup ids are renumbered per XCD (grid padded to a multiple of 8)
+    int pad_[3];
 };
 
 // Device-side view of the launch parameters: the pointers carry the global address space in their type, so
@@ -50,7 +51,7 @@ struct SpmmView {
     const MORTAR_GLOBAL int32_t *tok_cnt;
     const MORTAR_GLOBAL uint8_t *tok_list;
     int64_t ldx, ldy;
-    int n_units, Cb, M, n_clusters, cluster_size, n_split, seg_cb, nseg, Rb;
+    int n_units, Cb, M, n_clusters, cluster_size, n_mtiles, n_split, seg_cb, nseg, Rb, xcd_map;
 };
 static_assert(sizeof(SpmmParams) % 16 == 0, "table entries are copied in 16-byte words");
 // Entry i of a parameter table in device memory (uniform address: scalar loads).
@@ -71,7 +72,7 @@ __device__ __forceinline__ SpmmView mortar_view(const SpmmParams &q) {
     v.gates = (const MORTAR_GLOBAL float *)q.gates; v.active = (const MORTAR_GLOBAL uint8_t *)q.active;
     v.tok_cnt = (const MORTAR_GLOBAL int32_t *)q.tok_cnt; v.tok_list = (const MORTAR_GLOBAL uint8_t *)q.tok_list;
     v.ldx = q.ldx; v.ldy = q.ldy; v.n_units = q.n_units; v.Cb = q.Cb; v.M = q.M; v.n_clusters = q.n_clusters;
-    v.cluster_size = q.cluster_size; v.n_split = q.n_split; v.seg_cb = q.seg_cb; v.nseg = q.nseg; v.Rb = q.Rb;
+    v.cluster_size = q.cluster_size; v.n_mtiles = q.n_mtiles; v.n_split = q.n_split; v.seg_cb = q.seg_cb; v.nseg = q.nseg; v.Rb = q.Rb; v.xcd_map = q.xcd_map;
     return v;
 }
 
@@ -253,7 +254,11 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
-    const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
+    // Workgroups are dealt round-robin over the 8 XCDs (each with its own L2): renumber them so that the
+    // n_split workgroups that stage the same token tile run on one XCD and share its copy of the tile.
+    const int wg = p.xcd_map ? (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    if (wg >= p.n_mtiles * p.n_split) return;
+    const int mt = wg / p.n_split, sp = wg % p.n_split;
     const int m0 = mt * MT;
     const uint32_t lane_xo = (uint32_t)(hsel * LDM + (ROUTED ? 0 : n));
     const bool has_gates = p.gates != nullptr;
@@ -338,7 +343,11 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
-    const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
+    // Workgroups are dealt round-robin over the 8 XCDs (each with its own L2): renumber them so that the
+    // n_split workgroups that stage the same token tile run on one XCD and share its copy of the tile.
+    const int wg = p.xcd_map ? (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    if (wg >= p.n_mtiles * p.n_split) return;
+    const int mt = wg / p.n_split, sp = wg % p.n_split;
     const int m0 = mt * MT;
     const uint32_t lane_xo = (uint32_t)(hsel * LDM + n);
     const bool has_gates = p.gates != nullptr;
@@ -423,6 +432,14 @@ inline int mortar_launch_check(int64_t grid, int layers) {
     return MORTAR_OK;
 }
 
+// Grid width for n_mtiles * n_split workgroups.  When several workgroups share a token tile of a large single
+// launch, the ids are renumbered per XCD in the kernel and the grid is padded to a multiple of 8.
+inline int64_t mortar_grid_width(SpmmParams &p, int layers) {
+    const int64_t n = (int64_t)p.n_mtiles * p.n_split;
+    p.xcd_map = layers == 1 && p.n_split > 1 && n >= 64;
+    return p.xcd_map ? (n + 7) / 8 * 8 : n;
+}
+
 // Fills the launch-shape fields of `p` for the resident kernel and returns the grid width.
 template <int MT, int WAVES>
 inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
@@ -438,7 +455,7 @@ inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
     const int max_split = (p.n_units + WAVES * upw - 1) / (WAVES * upw);
     split = split < 1 ? 1 : (split > max_split ? max_split : split);
     p.n_split = split;
-    return (int64_t)p.n_mtiles * split;
+    return mortar_grid_width(p, layers);
 }
 
 template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE = false>
@@ -459,10 +476,10 @@ int mortar_launch_resident(SpmmParams &p, const SpmmParams *table, int layers, h
 }
 
 template <int MT, int WAVES, int UPW>
-inline int64_t mortar_segmented_shape(SpmmParams &p) {
+inline int64_t mortar_segmented_shape(SpmmParams &p, int layers) {
     p.n_mtiles = (p.M + MT - 1) / MT;
     p.n_split = (p.n_units + WAVES * UPW - 1) / (WAVES * UPW);
-    return (int64_t)p.n_mtiles * p.n_split;
+    return mortar_grid_width(p, layers);
 }
 
 template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE = false>
@@ -474,7 +491,7 @@ int mortar_launch_segmented(SpmmParams &p, const SpmmParams *table, int layers, 
     auto kern = mortar_segmented_kernel<MT, NACC, MASKED, WAVES, UPW, TABLE>;
     int rc = mortar_allow_big_lds(kern, attr_done);
     if (rc) return rc;
-    const int64_t grid = mortar_segmented_shape<MT, WAVES, UPW>(p);
+    const int64_t grid = mortar_segmented_shape<MT, WAVES, UPW>(p, layers);
     if ((rc = mortar_launch_check(grid, layers))) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)layers), dim3(WAVES * 64), smem, st, p, table);
     hipError_t e = hipGetLastError();
