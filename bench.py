@@ -22,6 +22,12 @@ if ROOT not in sys.path:
 D_MODEL, D_FF, DENSITY, TOKENS = 2048, 5632, 0.25, 4096
 N_CLUSTERS, TOP_K = 352, 88
 PEAK_BF16_TFLOPS, PEAK_HBM_GBS = 2500.0, 8000.0
+# HBM-side bytes per launch (read + written) measured with `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` on this
+# workload and calibrated on a plain copy; the runs and factors are in profiles/bench_prefill_step_hbm_traffic_pmc.md
+# and profiles/bench_all_legs_hbm_traffic_pmc.md.  Not measured live: counters need the profiler.
+TRAFFIC_GATE_UP_BYTES = 42.84e6 + 46.14e6
+TRAFFIC_DOWN_BYTES = 53.74e6 + 16.78e6
+TRAFFIC_DECODE_STACK_BYTES = (263.92e6 + 4.53e6) + (166.32e6 + 1.64e6)   # gate_up + down launches, 160 layers, b = 1
 
 
 def event_time_ms(fn, iters: int, warmup: int = 2) -> float:
@@ -49,7 +55,7 @@ def cpu_baseline(spec, sample_tokens: int) -> dict:
     t0 = time.perf_counter()
     c_oracle.mlp_bf16(x, spec["gate_up"], spec["down"], D_FF)
     t1 = time.perf_counter() - t0
-    reps = max(1, min(400, int(round(12.0 / max(t1, 1e-3)))))                # about 12 s of CPU work in total
+    reps = max(1, min(800, int(round(18.0 / max(t1, 1e-3)))))                # 10-20 s of CPU work in total
     t0 = time.perf_counter()
     for _ in range(reps):
         c_oracle.mlp_bf16(x, spec["gate_up"], spec["down"], D_FF)
@@ -112,11 +118,12 @@ def main() -> None:
         "effective_tflops": (flops_gu + flops_dn) / (ms * 1e-3) / 1e12,
         "roofline": {"bound": "mfma", "kernel": "mortar_resident_kernel<32 tokens, gate_up + SwiGLU>",
                      "achieved": flops_gu / (ms_gu * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops_gu / (ms_gu * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
-                     "ms": ms_gu},
+                     "frac": flops_gu / (ms_gu * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_GATE_UP_BYTES,
+                     "algorithmic_bytes": TOKENS * (D_MODEL + D_FF) * 2 + Wgu.weight_bytes, "ms": ms_gu},
         "roofline_down": {"bound": "mfma", "kernel": "mortar_segmented_kernel<32 tokens, plain> (down)",
                           "achieved": flops_dn / (ms_dn * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                          "frac": flops_dn / (ms_dn * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "ms": ms_dn},
+                          "frac": flops_dn / (ms_dn * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_DOWN_BYTES,
+                          "algorithmic_bytes": TOKENS * (D_MODEL + D_FF) * 2 + Wdn.weight_bytes, "ms": ms_dn},
     }
 
     if not args.no_extras:
@@ -200,7 +207,8 @@ def main() -> None:
         out["decode_stack"] = stack
         out["roofline_decode"] = {"bound": "hbm", "kernel": "mortar_resident_kernel<4 tokens> (160 layers per launch, b=1)",
                                   "achieved": stack["b1"]["algorithmic_GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                  "frac": stack["b1"]["frac_hbm"], "traffic": None}
+                                  "frac": stack["b1"]["frac_hbm"], "traffic": TRAFFIC_DECODE_STACK_BYTES,
+                                  "algorithmic_bytes": n_sets * (wbytes + (2 * D_MODEL + 2 * D_FF) * 2)}
         # ---- ReMoE-routed prefill (BASELINE config 3) ----------------------------------------------------
         logits = torch.from_numpy(synth.synth_logits(TOKENS, N_CLUSTERS, seed=2)).to(dev)
 
@@ -213,6 +221,43 @@ def main() -> None:
         n_act = int(ops.remoe_gates(logits, TOP_K)[1].sum())
         out["routed_prefill"] = {"ms": t, "tokens_per_s": TOKENS / (t * 1e-3),
                                  "active_fraction": n_act / (TOKENS * N_CLUSTERS)}
+
+    if not args.no_extras:
+        # ---- BASELINE config 1: base-width MLP (d_model 768, d_ff 2048), 4 x 4096 tokens ---------------------
+        spec1 = synth.synth_mlp(768, 2048, DENSITY, seed=10)
+        G1, D1 = synth.to_pack(spec1["gate_up"], dev), synth.to_pack(spec1["down"], dev)
+        x1 = torch.from_numpy(synth.synth_x(16384, 768, seed=11)).to(torch.bfloat16).to(dev)
+        h1 = torch.empty((16384, 2048), dtype=torch.bfloat16, device=dev)
+        y1 = torch.empty((16384, 768), dtype=torch.bfloat16, device=dev)
+
+        def step1():
+            ops.gateup_swiglu(x1, G1, out=h1)
+            ops.spmm(h1, D1, out=y1)
+        t = event_time_ms(step1, it)
+        fl = 2.0 * 16384 * 256 * (G1.nnz + D1.nnz)
+        out["base_width_prefill"] = {"ms": t, "tokens_per_s": 16384 / (t * 1e-3), "effective_tflops": fl / (t * 1e-3) / 1e12,
+                                     "frac_mfma": fl / (t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+        del x1, h1, y1
+        # ---- BASELINE config 4: 8 shared blocks x 6 iterations, Zipf(1.2) rows, RMS-normalised input ----------
+        specs = [synth.synth_mlp(D_MODEL, D_FF, DENSITY, seed=20 + i, zipf_s=1.2) for i in range(8)]
+        packs4 = [(synth.to_pack(sp["gate_up"], dev), synth.to_pack(sp["down"], dev)) for sp in specs]
+        xs = [x, torch.empty_like(x)]
+
+        def looped():
+            cur = 0
+            for _ in range(6):
+                for g4, d4 in packs4:
+                    xn = ops.rmsnorm(xs[cur])
+                    ops.gateup_swiglu(xn, g4, out=h)
+                    ops.spmm(h, d4, out=xs[1 - cur] if cur == 0 else xs[1])
+                    cur = 1
+        t = event_time_ms(looped, 3, 1)
+        fl = 6 * sum(2.0 * TOKENS * 256 * (g4.nnz + d4.nnz) for g4, d4 in packs4)
+        out["looped_stack"] = {"ms": t, "mlp_calls": 48, "ms_per_mlp": t / 48, "tokens_per_s": TOKENS / (t * 1e-3),
+                               "effective_tflops": fl / (t * 1e-3) / 1e12,
+                               "frac_mfma": fl / (t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                               "note": "includes one RMSNorm launch per MLP; rows follow Zipf(1.2) clipped to 5-60 %"}
+        del specs, packs4
 
     # A plain device-to-device copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE counters when this
     # command runs under `rocprofv3 --pmc` (counter KiB per byte copied), and a practical HBM bandwidth figure.

@@ -12,6 +12,34 @@ from util import assert_close_bf16, oracle_spmm, to_dev, to_np
 pytestmark = pytest.mark.gpu
 
 
+# ---------------------------------------------------------------------------------------------- committed fixtures
+
+def test_golden_fixtures(dev):
+    """The HIP path against the committed vectors (tests/golden): config 0 whole and an MLP slice with gating."""
+    import golden_util as G
+    z = G.load("c0_spmm.npz")
+    m = G.matrix(z)
+    W = synth.to_pack(m, dev)
+    x = torch.from_numpy(z["x_bits"].view(np.int16)).view(torch.bfloat16).to(dev)
+    ref = O.bf16_from_bits(z["y_bits"])
+    assert_close_bf16(to_np(ops.spmm(x, W)), ref, "c0 spmm (64 rows)")
+    assert_close_bf16(to_np(ops.spmm(x[:3], W)), ref[:3], "c0 spmm (3 rows, decode tile)")
+    z = G.load("mlp_slice.npz")
+    Wgu, Wdn = synth.to_pack(G.matrix(z, "gate_up_"), dev), synth.to_pack(G.matrix(z, "down_"), dev)
+    x = torch.from_numpy(z["x_bits"].view(np.int16)).view(torch.bfloat16).to(dev)
+    logits = torch.from_numpy(z["logits_bits"].view(np.float32)).to(dev)
+    gates, active = ops.remoe_gates(logits, 11)
+    assert np.array_equal(active.cpu().numpy(), z["active"])                       # tile selection bit-exact
+    np.testing.assert_allclose(gates.cpu().numpy(), z["gates_bits"].view(np.float32), rtol=2e-6, atol=0)
+    h = ops.gateup_swiglu(x, Wgu)
+    assert_close_bf16(to_np(h), O.bf16_from_bits(z["h_bits"]), "h", ulps=4)
+    assert_close_bf16(to_np(ops.spmm(h, Wdn)), O.bf16_from_bits(z["y_bits"]), "y", ulps=8)
+    route = ops.remoe_route(active, ops.route_tile(Wgu, 8))
+    hr = ops.gateup_swiglu(x, Wgu, gates=gates, route=route)
+    yr = ops.spmm(hr, Wdn, active=active)
+    assert_close_bf16(to_np(yr), O.bf16_from_bits(z["y_routed_bits"]), "y routed", ulps=8)
+
+
 # ---------------------------------------------------------------------------------------------- prefill SpMM
 
 def test_c0_single_spmm(dev):

@@ -284,3 +284,41 @@ def test_bf16_round_matches_torch():
     a = np.random.default_rng(70).standard_normal(10000).astype(np.float32) * 1e3
     a[:4] = [0.1, 1.00390625, 1.005859375, -1.00390625]                           # ties-to-even cases
     assert np.array_equal(O.bf16_round(a), torch.from_numpy(a).to(torch.bfloat16).float().numpy())
+
+
+# ---------------------------------------------------------------------------------------------- committed fixtures
+
+def test_golden_c0_pins_numpy_and_c_oracle():
+    """The committed config-0 vectors: both restatements reproduce the stored bf16 output bit for bit."""
+    import golden_util as G
+    from oracle import c_oracle
+    z = G.load("c0_spmm.npz")
+    m = G.matrix(z)
+    x = O.bf16_from_bits(z["x_bits"])
+    assert m["shape"] == (2048, 768) and int(m["offsets"][-1]) == 1536 and z["x_bits"].shape == (64, 768)
+    y = O.bcsr_spmm(x, m["codes"], m["scales"], m["col_idx"], m["offsets"], m["shape"])
+    assert np.array_equal(O.bf16_bits(y), z["y_bits"])
+    yc = c_oracle.bcsr_spmm_bf16(z["x_bits"], m["codes"], m["scales"], m["col_idx"], m["offsets"])
+    assert np.array_equal(yc, z["y_bits"])
+    # and the stored output is what a dense fp64 matmul of the scattered weight gives (library routine)
+    dense = O.to_dense(O.effective_blocks(m["codes"], m["scales"]), m["row_idx"], m["col_idx"], m["shape"])
+    assert np.array_equal(O.bf16_bits(x.astype(np.float64) @ dense.astype(np.float64).T), z["y_bits"])
+
+
+def test_golden_mlp_slice_pins_swiglu_and_gating():
+    import golden_util as G
+    from oracle import c_oracle
+    z = G.load("mlp_slice.npz")
+    gu, dn = G.matrix(z, "gate_up_"), G.matrix(z, "down_")
+    x = O.bf16_from_bits(z["x_bits"])
+    logits = z["logits_bits"].view(np.float32)
+    gates, active = O.remoe_gates(logits, 11)
+    assert np.array_equal(gates.astype(np.float32).view(np.uint32), z["gates_bits"])
+    assert np.array_equal(active.astype(np.uint8), z["active"])
+    assert (z["active"].sum(1) <= 10).all()                                    # strict threshold: at most k-1 active
+    for g, hk, yk in ((None, "h_bits", "y_bits"), (gates, "h_routed_bits", "y_routed_bits")):
+        r = O.swiglu_mlp(x, gu, dn, gates=g)
+        assert np.array_equal(O.bf16_bits(r["h"]), z[hk]) and np.array_equal(O.bf16_bits(r["y"]), z[yk])
+        _, hc, yc = c_oracle.mlp_bf16(z["x_bits"], gu, dn, 704, gates=None if g is None else g.astype(np.float32))
+        assert np.abs(O.bf16_from_bits(hc) - O.bf16_from_bits(z[hk])).max() <= 2 ** -7 * np.abs(O.bf16_from_bits(z[hk])).max()
+        assert np.abs(O.bf16_from_bits(yc) - O.bf16_from_bits(z[yk])).max() <= 1e-2 * np.abs(O.bf16_from_bits(z[yk])).max()
