@@ -147,7 +147,7 @@ int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *sched, const 
                             void *stream);
 
 /* Token tile of routed mortar_gateup_swiglu_bf16 for M rows against a matrix with Cb block-columns: the tile
- * size mortar_remoe_route must be called with.  4 or 16 for decode-sized M (<= 16), otherwise 32, 64 or 96
+ * size mortar_remoe_route must be called with.  4 for M <= 4, 16 for M <= 64, otherwise 32, 64 or 96
  * depending on Cb; 0 when in_features is too wide for routed skipping (one LDS tile must hold a row of x). */
 int mortar_route_tile(int32_t Cb, int64_t M);
 
@@ -174,8 +174,8 @@ int mortar_route_flags(const float *gates, int64_t B, int32_t n_clusters, int64_
 /* ---- decode (M <= 64) ------------------------------------------------------------------------ */
 
 /* mortar_spmm_bf16 / mortar_gateup_swiglu_bf16 / mortar_spmm_bf16_masked serve decode batches directly: for
- * M <= 16 they run small-tile variants (4- or 16-token tile, small workgroups) that read every weight block
- * once per launch.  That path replaces mortar_gemv of fused_decode_step.py:1701-1842 for the MLP pair.
+ * M <= 64 they run small-tile variants (4- or 16-token tiles, small workgroups) that read every weight block
+ * from HBM once per launch.  That path replaces mortar_gemv of fused_decode_step.py:1701-1842 for the MLP pair.
  *
  * Layer-batched form for M <= 16: ONE launch runs the same operation on n_layers independent
  * (matrix, input, output) triples of identical shape (Rb, Cb, seg_cb).  No counterpart in the reference,

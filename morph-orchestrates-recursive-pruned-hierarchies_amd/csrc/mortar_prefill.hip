@@ -62,7 +62,7 @@ constexpr int SEG_WAVES = 16, SEG_UPW = 4;
 
 // kind: 0 spmm, 1 gate_up + SwiGLU, 2 routed gate_up + SwiGLU, 3 spmm with an input mask
 int dispatch(int kind, SpmmParams &p, hipStream_t st) {
-    if (p.M <= 16) {
+    if (p.M <= MORTAR_SMALLM_MAX) {
         const int rc = mortar_smallm_launch(kind, p, nullptr, 1, st);
         if (rc >= 0) return rc;
     }
@@ -85,7 +85,7 @@ int dispatch(int kind, SpmmParams &p, hipStream_t st) {
 extern "C" int mortar_prefill_max_seg_cb(void) { return (LDS_BUDGET / 16 - LDS_PAD) / (2 * 33); }
 
 extern "C" int mortar_route_tile(int32_t Cb, int64_t M) {
-    if (M > 0 && M <= 16) {
+    if (M > 0 && M <= MORTAR_SMALLM_MAX) {
         const int t = mortar_smallm_tile(Cb, Cb, M, 2);
         if (t > 0) return t;
     }

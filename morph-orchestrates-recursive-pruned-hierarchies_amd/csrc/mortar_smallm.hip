@@ -1,8 +1,9 @@
-// Small-M (decode, M <= 16) instantiations of the octet-stream SpMM kernels.
+// Small-M (decode, M <= 64) instantiations of the octet-stream SpMM kernels.
 //
 // Replaces the reference's decode GEMV over packed ternary strips (morph/kernels/triton/fused_decode_step.py:
-// 1701-1842, mortar_gemv) for batches of up to 16 rows: the batch is one token tile of 4 or 16 tokens, so a
-// weight block is read once per launch and the kernel is bound by the weight stream.  Workgroups are small
+// 1701-1842, mortar_gemv) for batches of up to 64 rows: the batch is one token tile of 4 or 16 tokens (up to four
+// 16-token tiles above 16 rows), so a weight block is read from HBM once per launch and the kernel is bound by
+// the weight stream.  Workgroups are small
 // (2 wavefronts) when one matrix has to cover the chip and 8 or 16 wavefronts when many layers share a launch.
 #include "mortar_spmm_core.h"
 
@@ -38,7 +39,7 @@ bool fits(int mt, int ncb) { return tile_bytes(mt, ncb) <= LDS_BUDGET; }
 int mortar_smallm_tile(int Cb, int seg_cb, int64_t M, int kind) {
     (void)seg_cb;
     if (M <= 4 && kind != 3 && fits(4, Cb)) return 4;
-    if (M <= 16) {
+    if (M <= MORTAR_SMALLM_MAX) {      // up to four 16-token tiles
         if (kind != 3 && fits(16, Cb)) return 16;
         if (kind == 0 || kind == 3) return -16;
     }
@@ -53,11 +54,40 @@ static int pick_waves(int t, const SpmmParams &p, int layers) {
     return bytes > 40 * 1024 ? 16 : 8;
 }
 
+// Part-split launch for one matrix: PW waves per unit, PW = 4, 3 or 2 dividing the unit's part count.
+template <int MT>
+static int launch_partsplit(int kind, SpmmParams &p, hipStream_t st) {
+    const int nacc = (kind == 0 || kind == 3) ? 1 : 2, nparts = p.nseg * nacc;
+    const int pw = nparts % 4 == 0 ? 4 : (nparts % 3 == 0 ? 3 : (nparts % 2 == 0 ? 2 : 0));
+    if (pw == 0 || tile_bytes(MT, p.Cb) + 16 * 2 * 1024 > 160 * 1024) return -1;
+    switch (kind * 10 + pw) {
+        case 2: return mortar_launch_partsplit<MT, 1, false, false, 2, 4>(p, st);
+        case 3: return mortar_launch_partsplit<MT, 1, false, false, 3, 4>(p, st);
+        case 4: return mortar_launch_partsplit<MT, 1, false, false, 4, 4>(p, st);
+        case 12: return mortar_launch_partsplit<MT, 2, false, false, 2, 4>(p, st);
+        case 13: return mortar_launch_partsplit<MT, 2, false, false, 3, 4>(p, st);
+        case 14: return mortar_launch_partsplit<MT, 2, false, false, 4, 4>(p, st);
+        case 22: return mortar_launch_partsplit<MT, 2, true, false, 2, 4>(p, st);
+        case 23: return mortar_launch_partsplit<MT, 2, true, false, 3, 4>(p, st);
+        case 24: return mortar_launch_partsplit<MT, 2, true, false, 4, 4>(p, st);
+        case 32: return mortar_launch_partsplit<MT, 1, false, true, 2, 4>(p, st);
+        case 33: return mortar_launch_partsplit<MT, 1, false, true, 3, 4>(p, st);
+        case 34: return mortar_launch_partsplit<MT, 1, false, true, 4, 4>(p, st);
+    }
+    return -1;
+}
+
 int mortar_smallm_launch(int kind, SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
     if (t == 0) return -1;
     const bool resident = t > 0;
     const int w = pick_waves(t, p, layers);
+    if (!table && layers == 1 && w == 2) {      // one matrix over the whole chip: latency form
+        int rc = -1;
+        if (resident) rc = t == 4 ? launch_partsplit<4>(kind, p, st) : launch_partsplit<16>(kind, p, st);
+        else if (fits(8, p.Cb)) rc = launch_partsplit<8>(kind, p, st);      // 8-token tiles of all K instead of K segments
+        if (rc >= 0) return rc;
+    }
     if (t == 4) {
         if (w == 16) return launch_kind<4, 16>(kind, true, p, table, layers, st);
         return w == 8 ? launch_kind<4, 8>(kind, true, p, table, layers, st) : launch_kind<4, 2>(kind, true, p, table, layers, st);

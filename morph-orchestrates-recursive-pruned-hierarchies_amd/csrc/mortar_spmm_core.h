@@ -1,4 +1,4 @@
-// Octet-stream SpMM kernels shared by the prefill (large M) and decode (M <= 16) entry points.
+// Octet-stream SpMM kernels shared by the prefill (large M) and decode (M <= 64) entry points.
 //
 // Both kernels keep a token tile of the activations in LDS and let every wavefront walk whole row units of
 // the octet weight stream: unpack the ternary codes of two blocks in registers, read the activation operand
@@ -76,6 +76,7 @@ __device__ __forceinline__ SpmmView mortar_view(const SpmmParams &q) {
     return v;
 }
 
+constexpr int MORTAR_SMALLM_MAX = 64;    // rows up to which the small-tile (decode) instantiations are used
 constexpr int RES_GROUPS = 4;            // octets (4 block pairs each) loaded per batch
 constexpr int LDS_BUDGET = 156 * 1024;   // bytes of LDS a token tile may take
 constexpr int LDS_PAD = 16;              // 16-byte units past the tile that idle lanes of a narrow tile may read
@@ -125,14 +126,14 @@ __device__ __forceinline__ void mortar_load_batch(const SpmmView &p, MortarBatch
 
 // One row part: octets [g0, g1) (nb blocks) of the stream against the tile at `lx`.
 // `xo_base` is the lane's unit offset inside a block-column (column half, token) plus the segment's origin.
+// `b` holds the part's first batch, loaded by the caller (mortar_load_batch at g0) where it suits it.
 template <int MSUB, int LDM, bool ROUTED>
-__device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *lx, int g0, int g1, int nb,
-                                                uint32_t xo_base, const uint32_t (&tk)[MSUB], int nsub, int n,
+__device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *lx, MortarBatch b, int g0, int g1,
+                                                int nb, uint32_t xo_base, const uint32_t (&tk)[MSUB], int nsub, int n,
                                                 int bsel, int hsel, f32x4_t (&acc)[MSUB]) {
     const unsigned char *lb = reinterpret_cast<const unsigned char *>(lx);
     for (int gq = g0; gq < g1; gq += RES_GROUPS) {
-        MortarBatch b;
-        mortar_load_batch(p, b, gq, g1, n, bsel);
+        if (gq != g0) mortar_load_batch(p, b, gq, g1, n, bsel);
         const uint32_t ccs = __umul24(b.ccv, (uint32_t)(2 * LDM * 16));   // byte offset of the block-column in the tile
         const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;      // block pairs left in the row from this batch on
         // Activation operands are fetched two pairs ahead of the MFMAs that use them.  The only branches are
@@ -175,16 +176,18 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
 
 // Stages x[m0 .. m0+MT, 16*c0 .. 16*(c0+ncb)] into the tile: unit (ch, row) <- 8 values of column half ch.
 // A wavefront takes whole rows (row = wave, wave + WAVES, ...), its lanes consecutive 16-byte units of the row,
-// so that addresses need no division: uniform row base + lane offset.  Rows past M repeat the last row.
+// so that addresses need no division: uniform row base + lane offset.  Rows past M are not staged: their LDS
+// units keep whatever they held and only feed accumulator columns that are never stored.
 // With MASKED, units of (token, input cluster) pairs that are off are zeroed.
 template <int MT, int WAVES, bool MASKED>
 __device__ __forceinline__ void mortar_stage_tile(const SpmmView &p, uint4 *lx, int m0, int c0, int ncb, int tid) {
-    constexpr int LDM = MT + 1, RU = 2, CU = 4;     // rows x 64-unit chunks in flight per lane
+    // rows x 64-unit chunks in flight per lane: a small workgroup keeps up to 32 loads per lane in flight
+    constexpr int LDM = MT + 1, CU = 4, RU = MT / WAVES >= 8 ? 8 : (MT / WAVES >= 4 ? 4 : 2);
     const int nch = 2 * ncb;
     const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const MORTAR_GLOBAL char *xt = p.x + (int64_t)m0 * p.ldx * 2 + (int64_t)c0 * 32;
-    for (int r0 = wave; r0 < MT; r0 += WAVES * RU) {
+    for (int r0 = wave; r0 <= rlast; r0 += WAVES * RU) {
         for (int ch0 = 0; ch0 < nch; ch0 += 64 * CU) {
             u32x4_t v[RU][CU];
 #pragma unroll
@@ -207,7 +210,7 @@ __device__ __forceinline__ void mortar_stage_tile(const SpmmView &p, uint4 *lx, 
 #pragma unroll
                 for (int b = 0; b < CU; ++b) {
                     const int ch = ch0 + b * 64 + lane;
-                    if (row < MT && ch < nch) reinterpret_cast<u32x4_t *>(lx)[ch * LDM + row] = v[a][b];
+                    if (row <= rlast && ch < nch) reinterpret_cast<u32x4_t *>(lx)[ch * LDM + row] = v[a][b];
                 }
             }
         }
@@ -309,7 +312,11 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
                 const u32x4_t d1 = mortar_part_desc<NACC>(p, p1, s1, a1);
                 const int g0 = __builtin_amdgcn_readfirstlane((int)d0[0]), g1 = __builtin_amdgcn_readfirstlane((int)d0[1]);
                 const int nb = __builtin_amdgcn_readfirstlane((int)d0[2]);
-                if (!skip) mortar_row_part<MSUB, LDM, ROUTED>(p, lx, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+                if (!skip && g0 < g1) {
+                    MortarBatch b;
+                    mortar_load_batch(p, b, g0, g1, n, bsel);
+                    mortar_row_part<MSUB, LDM, ROUTED>(p, lx, b, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+                }
                 d0 = d1;
                 advance(p1, s1, a1);
             }
@@ -392,8 +399,12 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
         __syncthreads();
 #pragma unroll
         for (int q = 0; q < NP; ++q) {
-            mortar_row_part<MSUB, LDM, false>(p, lx, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
-                                              acc[q / NACC][q % NACC]);
+            if (g0[q] < g1[q]) {
+                MortarBatch b;
+                mortar_load_batch(p, b, g0[q], g1[q], n, bsel);
+                mortar_row_part<MSUB, LDM, false>(p, lx, b, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
+                                                  acc[q / NACC][q % NACC]);
+            }
         }
     }
 
@@ -408,6 +419,111 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
             if (tok >= p.M) continue;
             mortar_store_unit<NACC>(p, units[k], tok, g, has_gates, acc[k][0][ms], acc[k][NACC - 1][ms]);
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Part-split kernel: the latency form for ONE small-M product that has to be spread over the whole chip.
+// The row parts of a unit (its K segments x its gate/up rows) are dealt to PW waves that run side by side;
+// their partial accumulators meet in LDS and the unit's first wave applies the epilogue.  A workgroup holds UW
+// units (PW * UW waves) and one resident token tile.  Every wave fetches its first descriptor and weight batch
+// before the tile is staged, so the only serial global round trips are descriptor -> batch.
+// ---------------------------------------------------------------------------------------------------------
+template <int MT, int NACC, bool ROUTED, bool MASKED, int PW, int UW>
+__global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const SpmmParams p0) {
+    constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1, WAVES = PW * UW;
+    const SpmmView p = mortar_view(p0);
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint4 *lx = reinterpret_cast<uint4 *>(smem);
+    f32x4_t *red = reinterpret_cast<f32x4_t *>(smem + tile_bytes(MT, p.Cb));   // [WAVES][NACC][MSUB][64]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
+    const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
+    const int m0 = mt * MT;
+    const uint32_t lane_xo = (uint32_t)(hsel * LDM + (ROUTED ? 0 : n));
+    const bool has_gates = p.gates != nullptr;
+    const int ug = wave / PW, wq = wave % PW;            // unit slot in the workgroup, this wave's share of its parts
+    const int pos = sp * UW + ug;
+    const bool valid = pos < p.n_units;
+    const int nparts = p.nseg * NACC;
+
+    // first part of this wave: q = wq  (q = segment * NACC + a)
+    MortarBatch first;
+    u32x4_t d = u32x4_t{0u, 0u, 0u, 0u};
+    if (valid && wq < nparts) {
+        d = mortar_part_desc<NACC>(p, pos, wq / NACC, wq % NACC);
+        const int g0 = __builtin_amdgcn_readfirstlane((int)d[0]), g1 = __builtin_amdgcn_readfirstlane((int)d[1]);
+        if (g0 < g1) mortar_load_batch(p, first, g0, g1, n, bsel);
+    }
+    const int unit = valid ? __builtin_amdgcn_readfirstlane((int)mortar_part_desc<NACC>(p, pos, 0, 0)[3]) : 0;
+
+    int cnt = MT;
+    uint32_t tk[MSUB];
+#pragma unroll
+    for (int ms = 0; ms < MSUB; ++ms) tk[ms] = ms * 16 + n;
+    bool skip = !valid;
+    if (ROUTED && valid) {
+        const int cl = (unit * 16) / p.cluster_size;
+        const int64_t e = (int64_t)mt * p.n_clusters + cl;
+        cnt = __builtin_amdgcn_readfirstlane(p.tok_cnt[e]);
+        skip = cnt == 0;
+#pragma unroll
+        for (int ms = 0; ms < MSUB; ++ms) {
+            const int i = ms * 16 + n;
+            tk[ms] = i < cnt ? p.tok_list[e * MT + i] : 0;
+        }
+    }
+    const int nsub = ROUTED ? (cnt + 15) >> 4 : MSUB;
+
+    mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, 0, p.Cb, tid);
+    __syncthreads();
+
+    f32x4_t acc[NACC][MSUB];
+#pragma unroll
+    for (int a = 0; a < NACC; ++a)
+#pragma unroll
+        for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (!skip) {
+        for (int sg = 0; sg < p.nseg; ++sg) {
+            const uint32_t xo_base = lane_xo + (uint32_t)(sg * p.seg_cb) * (2 * LDM);
+#pragma unroll
+            for (int a = 0; a < NACC; ++a) {
+                const int q = sg * NACC + a;
+                if (q % PW != wq) continue;
+                const bool is_first = q == wq;
+                const u32x4_t dq = is_first ? d : mortar_part_desc<NACC>(p, pos, sg, a);
+                const int g0 = __builtin_amdgcn_readfirstlane((int)dq[0]), g1 = __builtin_amdgcn_readfirstlane((int)dq[1]);
+                const int nb = __builtin_amdgcn_readfirstlane((int)dq[2]);
+                if (g0 >= g1) continue;
+                if (!is_first) mortar_load_batch(p, first, g0, g1, n, bsel);
+                mortar_row_part<MSUB, LDM, ROUTED>(p, lx, first, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+            }
+        }
+    }
+    // partial sums of the unit's waves meet in LDS; its first wave finishes the unit
+    if (PW > 1) {
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int ms = 0; ms < MSUB; ++ms) red[((wave * NACC + a) * MSUB + ms) * 64 + lane] = acc[a][ms];
+        __syncthreads();
+        if (wq != 0) return;
+#pragma unroll
+        for (int w = 1; w < PW; ++w)
+#pragma unroll
+            for (int a = 0; a < NACC; ++a)
+#pragma unroll
+                for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] += red[(((wave + w) * NACC + a) * MSUB + ms) * 64 + lane];
+    }
+    if (skip) return;
+#pragma unroll
+    for (int ms = 0; ms < MSUB; ++ms) {
+        const int li = ms * 16 + n;
+        if (li >= (ROUTED ? cnt : MT)) continue;
+        const int tok = m0 + (int)tk[ms];
+        if (tok >= p.M) continue;
+        mortar_store_unit<NACC>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
     }
 }
 
@@ -494,6 +610,26 @@ int mortar_launch_segmented(SpmmParams &p, const SpmmParams *table, int layers, 
     const int64_t grid = mortar_segmented_shape<MT, WAVES, UPW>(p, layers);
     if ((rc = mortar_launch_check(grid, layers))) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)layers), dim3(WAVES * 64), smem, st, p, table);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "spmm launch: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}
+
+template <int MT, int NACC, bool ROUTED, bool MASKED, int PW, int UW>
+int mortar_launch_partsplit(SpmmParams &p, hipStream_t st) {
+    constexpr int WAVES = PW * UW;
+    const int smem = tile_bytes(MT, p.Cb) + WAVES * NACC * ((MT + 15) / 16) * 64 * 16;
+    if (smem > 160 * 1024) return mortar_fail(MORTAR_ERR_LIMIT, "part-split tile of %d bytes does not fit LDS", smem);
+    static bool attr_done = false;
+    auto kern = mortar_partsplit_kernel<MT, NACC, ROUTED, MASKED, PW, UW>;
+    int rc = mortar_allow_big_lds(kern, attr_done);
+    if (rc) return rc;
+    p.n_mtiles = (p.M + MT - 1) / MT;
+    p.n_split = (p.n_units + UW - 1) / UW;
+    p.xcd_map = 0;
+    const int64_t grid = (int64_t)p.n_mtiles * p.n_split;
+    if ((rc = mortar_launch_check(grid, 1))) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WAVES * 64), smem, st, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "spmm launch: %s", hipGetErrorString(e));
     return MORTAR_OK;

@@ -274,7 +274,8 @@ def test_decode_gather_flags_worklist(dev):
 
 @pytest.mark.parametrize("B,n_layers", [(3, 5), (12, 5), (2, 300)])
 def test_layer_stack_matches_single_launches(dev, B, n_layers):
-    """Layer-batched launch: n layers in one launch give bit-identical results to n separate launches."""
+    """Layer-batched launch: n layers in one launch match n separate launches (to fp32 summation order: the
+    single-matrix launches split a row's K segments over several waves) and the oracle."""
     d_model, d_ff = 256, 16 * 380                                                    # down is K-segmented
     specs = [synth.synth_mlp(d_model, d_ff, 0.25, seed=500 + i, zipf_s=1.2) for i in range(min(n_layers, 5))]
     packs = [(synth.to_pack(s["gate_up"], dev), synth.to_pack(s["down"], dev)) for s in specs]
@@ -289,8 +290,8 @@ def test_layer_stack_matches_single_launches(dev, B, n_layers):
         dn.run()
     for i in range(n_layers):
         h1 = ops.gateup_swiglu(xs[i], packs[i][0])
-        assert torch.equal(h1, hs[i]), f"layer {i} h"
-        assert torch.equal(ops.spmm(h1, packs[i][1]), ys[i]), f"layer {i} y"
+        assert_close_bf16(to_np(hs[i]), to_np(h1), f"layer {i} h", ulps=2)
+        assert_close_bf16(to_np(ys[i]), to_np(ops.spmm(hs[i], packs[i][1])), f"layer {i} y", ulps=2)
     ref = O.swiglu_mlp(to_np(xs[1]), specs[1]["gate_up"], specs[1]["down"])
     assert_close_bf16(to_np(ys[1]), ref["y"], "stack vs oracle", ulps=8)
     with pytest.raises(ValueError):
