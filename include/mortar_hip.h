@@ -147,7 +147,7 @@ int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *sched, const 
                             void *stream);
 
 /* Token tile of routed mortar_gateup_swiglu_bf16 for M rows against a matrix with Cb block-columns: the tile
- * size mortar_remoe_route must be called with.  4 for M <= 4, 16 for M <= 64, otherwise 32, 64 or 96
+ * size mortar_remoe_route must be called with.  4 for M <= 4, 16 for M <= 64, otherwise 32 or 64
  * depending on Cb; 0 when in_features is too wide for routed skipping (one LDS tile must hold a row of x). */
 int mortar_route_tile(int32_t Cb, int64_t M);
 

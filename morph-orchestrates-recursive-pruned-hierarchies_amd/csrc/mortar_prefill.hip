@@ -3,7 +3,7 @@
 // Replaces the reference's stk dds forward (morph/sparse/stk/backend/triton_kernels.py:170-230 behind
 // custom_ops.py:35-56) and, in gate_up mode, fuses the SwiGLU of _SwiGLUMortar.forward
 // (morph/model/transformer.py:402-431) into the epilogue.  The kernels live in mortar_spmm_core.h:
-//   mortar_resident_kernel   in_features fits LDS for a 32..96-token tile
+//   mortar_resident_kernel   in_features fits LDS for a 32- or 64-token tile
 //   mortar_segmented_kernel  wide K (e.g. `down`): K cut into LDS-sized segments, 32-token tile
 // Batches of up to 16 rows go to the small-tile instantiations in mortar_smallm.hip.
 #include "mortar_spmm_core.h"
@@ -43,16 +43,16 @@ void fill(SpmmParams &p, const mortar_bcsr_t *W, const int32_t *sched, const uin
 
 // Token tile of the resident prefill kernel for a matrix with Cb block-columns (0 = does not fit).
 int resident_mt(int Cb) {
-    for (int mt : {96, 64, 32})
+    for (int mt : {64, 32})
         if (tile_bytes(mt, Cb) <= LDS_BUDGET) return mt;
     return 0;
 }
 
-// prefill tiles: 16 wavefronts (4 per SIMD) for the 32-token tile, 8 for larger tiles
+// prefill tiles: 16 wavefronts (4 per SIMD) for the 32-token tile, 8 for the 64-token tile (measured: a 96-token
+// tile of a narrow matrix leaves only two waves per SIMD and is slower)
 template <int NACC, bool ROUTED>
 int launch_resident_any(SpmmParams &p, hipStream_t st) {
     switch (resident_mt(p.Cb)) {
-        case 96: return mortar_launch_resident<96, NACC, ROUTED, 8>(p, nullptr, 1, st);
         case 64: return mortar_launch_resident<64, NACC, ROUTED, 8>(p, nullptr, 1, st);
         default: return mortar_launch_resident<32, NACC, ROUTED, 16>(p, nullptr, 1, st);
     }

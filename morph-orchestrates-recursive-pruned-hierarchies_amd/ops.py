@@ -11,8 +11,14 @@ from . import _lib
 from .pack import BLK, MortarPack
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: Tensor):
-    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+    """The current stream of t's device as a raw handle (ctypes converts the int to void*)."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
+    return torch.cuda.current_stream(t.device).cuda_stream
 
 
 def _need_gpu(t: Tensor, what: str):
@@ -32,7 +38,7 @@ def _bf16_2d(x: Tensor, what: str) -> Tensor:
 
 
 def _p(t):
-    return C.c_void_p(t.data_ptr()) if t is not None else None
+    return t.data_ptr() if t is not None else None
 
 
 # ----------------------------------------------------------------------------- prefill
@@ -51,11 +57,11 @@ def spmm(x: Tensor, W: MortarPack, out: Tensor | None = None, active: Tensor | N
     L = _lib.lib()
     sched = W.sched(1)
     if active is None:
-        rc = L.mortar_spmm_bf16(C.byref(W.struct), _p(sched), _p(x), M, x.stride(0), _p(y), y.stride(0), _stream(x))
+        rc = L.mortar_spmm_bf16(W.ref, _p(sched), _p(x), M, x.stride(0), _p(y), y.stride(0), _stream(x))
     else:
         if active.dtype != torch.uint8 or not active.is_contiguous():
             raise TypeError("spmm: active must be a contiguous uint8 tensor")
-        rc = L.mortar_spmm_bf16_masked(C.byref(W.struct), _p(sched), _p(x), M, x.stride(0), _p(y), y.stride(0),
+        rc = L.mortar_spmm_bf16_masked(W.ref, _p(sched), _p(x), M, x.stride(0), _p(y), y.stride(0),
                                        _p(active), active.shape[1], _stream(x))
     _lib.check(rc, "mortar_spmm_bf16")
     return y
@@ -79,7 +85,7 @@ def gateup_swiglu(x: Tensor, W: MortarPack, gates: Tensor | None = None, route: 
             raise TypeError("gateup_swiglu: gates must be a contiguous float32 [M, n_clusters] tensor")
         ncl = gates.shape[1]
     cnt, lst = route if route is not None else (None, None)
-    rc = _lib.lib().mortar_gateup_swiglu_bf16(C.byref(W.struct), _p(W.sched(2)), _p(x), M, x.stride(0), _p(h),
+    rc = _lib.lib().mortar_gateup_swiglu_bf16(W.ref, _p(W.sched(2)), _p(x), M, x.stride(0), _p(h),
                                               h.stride(0), _p(gates), ncl, _p(cnt), _p(lst), _stream(x))
     _lib.check(rc, "mortar_gateup_swiglu_bf16")
     return h
@@ -185,7 +191,7 @@ def gemv(x: Tensor, W: MortarPack, swiglu_out: bool = False, gates: Tensor | Non
         if f is not None and (f.dtype != torch.int32 or f.stride(1) != 1):
             raise TypeError("gemv: row_act / col_act must be int32 with unit inner stride")
     rc = _lib.lib().mortar_gemv_bf16(
-        C.byref(W.struct), _p(ent), ent.shape[0], nslots, _p(row_slots), kseg, 1 if swiglu_out else 0,
+        W.ref, _p(ent), ent.shape[0], nslots, _p(row_slots), kseg, 1 if swiglu_out else 0,
         _p(x), B, x.stride(0), _p(y), y.stride(0), _p(part), _p(gates), ncl, ldg,
         _p(row_act), row_act.stride(0) if row_act is not None else 0,
         _p(col_act), col_act.stride(0) if col_act is not None else 0, _stream(x))

@@ -145,6 +145,7 @@ class MortarPack:
         self._scheds: dict[int, torch.Tensor] = {}
         self._worklists: dict[tuple, tuple] = {}
         self.struct = self._make_struct()
+        self.ref = C.byref(self.struct)
 
     def _make_struct(self):
         return _lib.BcsrStruct(self.codes.data_ptr(), self.sdup.data_ptr(), self.col.data_ptr(),
@@ -180,4 +181,5 @@ class MortarPack:
         c._scheds = {k: v.clone() for k, v in self._scheds.items()}
         c._worklists = {k: (v[0].clone(), v[1], v[2].clone(), v[3]) for k, v in self._worklists.items()}
         c.struct = c._make_struct()
+        c.ref = C.byref(c.struct)
         return c
