@@ -83,6 +83,7 @@ constexpr int LDS_PAD = 16;              // 16-byte units past the tile that idl
 
 // LDS bytes of a token tile of MT tokens and ncb block-columns (token stride MT + 1 keeps reads conflict-free).
 constexpr int tile_bytes(int mt, int ncb) { return (2 * ncb * (mt + 1) + LDS_PAD) * 16; }
+constexpr int LDS_EXTRA = 16;            // bytes after the tile: the resident kernel's unit counter
 
 // Lane k of every 16-lane row broadcast to the whole row (DPP row_newbcast); K must fold to a constant.
 template <int K>
@@ -233,12 +234,17 @@ __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, i
 }
 
 // Part descriptor of schedule position `pos`, segment `sg`, row `a` of the unit: {g0, g1, nb, unit}.
+// One load site for both sources (schedule table, or row descriptors in natural order) so that the compiler can
+// keep the load in flight instead of waiting at a control-flow join.
 template <int NACC>
 __device__ __forceinline__ u32x4_t mortar_part_desc(const SpmmView &p, int pos, int sg, int a) {
     pos = pos < p.n_units ? pos : p.n_units - 1;
-    if (p.sched) return p.sched[((uint32_t)pos * (uint32_t)p.nseg + (uint32_t)sg) * NACC + a];
-    u32x4_t d = p.row_desc[sg * p.Rb + pos + a * p.n_units];
-    d[3] = (uint32_t)pos;
+    const bool sc = p.sched != nullptr;
+    const MORTAR_GLOBAL u32x4_t *base = sc ? p.sched : p.row_desc;
+    const uint32_t idx = sc ? ((uint32_t)pos * (uint32_t)p.nseg + (uint32_t)sg) * NACC + a
+                            : (uint32_t)(sg * p.Rb + pos + a * p.n_units);
+    u32x4_t d = base[idx];
+    d[3] = sc ? d[3] : (uint32_t)pos;
     return d;
 }
 
@@ -268,19 +274,29 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
 
     const int per = (p.n_units + p.n_split - 1) / p.n_split;
     const int u_end = (sp + 1) * per < p.n_units ? (sp + 1) * per : p.n_units;
-    int pos = sp * per + wave;
-    // coordinates of the part after the current one; its descriptor is fetched while the current part runs
-    auto advance = [&](int &ps, int &s, int &a_) {
-        if (++a_ == NACC) { a_ = 0; if (++s == p.nseg) { s = 0; ps += WAVES; } }
-    };
-    int p1 = pos, s1 = 0, a1 = 0;
-    advance(p1, s1, a1);
+    // Units are handed out dynamically: a wave starts with position `wave` of the workgroup's window and draws
+    // its next position from a counter in LDS when it begins a unit (one unit ahead, so that the descriptor of the
+    // next unit's first part can still be fetched early).  The SIMD arbiter favours the oldest wave, so with a
+    // fixed assignment the waves of a SIMD would finish one after another and leave it with one or two waves;
+    // drawing positions keeps all waves busy until the window is empty.
+    uint32_t *next_unit = reinterpret_cast<uint32_t *>(smem + tile_bytes(MT, p.Cb));
+    if (tid == 0) *next_unit = WAVES;
+    const int base = sp * per;
+    int pos = base + wave;
     u32x4_t d0 = mortar_part_desc<NACC>(p, pos, 0, 0);
 
     mortar_stage_tile<MT, WAVES, false>(p, lx, m0, 0, p.Cb, tid);
     __syncthreads();
 
-    for (; pos < u_end; pos += WAVES) {
+    while (pos < u_end) {
+        uint32_t drawn = 0;
+        if (lane == 0) drawn = atomicAdd(next_unit, 1u);
+        // coordinates of the part after the current one; its descriptor is fetched while the current part runs
+        int p1 = pos, s1 = 0, a1 = 0;
+        int npos = -1;       // position of this wave's next unit, known from the second part on
+        auto advance = [&](int &ps, int &s, int &a_) {
+            if (++a_ == NACC) { a_ = 0; if (++s == p.nseg) { s = 0; ps = npos; } }
+        };
         const int unit = __builtin_amdgcn_readfirstlane((int)d0[3]);
         int cnt = MT;
         uint32_t tk[MSUB];
@@ -309,6 +325,9 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
             const uint32_t xo_base = lane_xo + (uint32_t)(sg * p.seg_cb) * (2 * LDM);
 #pragma unroll
             for (int a = 0; a < NACC; ++a) {
+                const bool last_part = sg + 1 == p.nseg && a + 1 == NACC;
+                if (last_part) npos = base + (int)__builtin_amdgcn_readfirstlane(drawn);
+                advance(p1, s1, a1);
                 const u32x4_t d1 = mortar_part_desc<NACC>(p, p1, s1, a1);
                 const int g0 = __builtin_amdgcn_readfirstlane((int)d0[0]), g1 = __builtin_amdgcn_readfirstlane((int)d0[1]);
                 const int nb = __builtin_amdgcn_readfirstlane((int)d0[2]);
@@ -318,9 +337,9 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
                     mortar_row_part<MSUB, LDM, ROUTED>(p, lx, b, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
                 }
                 d0 = d1;
-                advance(p1, s1, a1);
             }
         }
+        pos = npos;
         if (skip) continue;
 
 #pragma unroll
@@ -577,8 +596,8 @@ inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
 template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE = false>
 int mortar_launch_resident(SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     if (TABLE != (table != nullptr)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: parameter table mismatch");
-    const int smem = tile_bytes(MT, p.Cb);
-    if (smem > LDS_BUDGET + LDS_PAD * 16) return mortar_fail(MORTAR_ERR_LIMIT, "resident tile of %d bytes does not fit LDS", smem);
+    const int smem = tile_bytes(MT, p.Cb) + LDS_EXTRA;
+    if (smem > LDS_BUDGET + LDS_PAD * 16 + LDS_EXTRA) return mortar_fail(MORTAR_ERR_LIMIT, "resident tile of %d bytes does not fit LDS", smem);
     static bool attr_done = false;
     auto kern = mortar_resident_kernel<MT, NACC, ROUTED, WAVES, TABLE>;
     int rc = mortar_allow_big_lds(kern, attr_done);
