@@ -25,9 +25,9 @@ PEAK_BF16_TFLOPS, PEAK_HBM_GBS = 2500.0, 8000.0
 # HBM-side bytes per launch (read + written) measured with `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` on this
 # workload and calibrated on a plain copy; the runs and factors are in profiles/bench_prefill_step_hbm_traffic_pmc.md
 # and profiles/bench_all_legs_hbm_traffic_pmc.md.  Not measured live: counters need the profiler.
-TRAFFIC_GATE_UP_BYTES = 42.84e6 + 46.14e6
-TRAFFIC_DOWN_BYTES = 53.74e6 + 16.78e6
-TRAFFIC_DECODE_STACK_BYTES = (263.92e6 + 4.53e6) + (166.32e6 + 1.64e6)   # gate_up + down launches, 160 layers, b = 1
+TRAFFIC_GATE_UP_BYTES = 42.45e6 + 46.78e6
+TRAFFIC_DOWN_BYTES = 53.83e6 + 16.78e6
+TRAFFIC_DECODE_STACK_BYTES = (263.93e6 + 4.54e6) + (166.81e6 + 1.65e6)   # gate_up + down launches, 160 layers, b = 1
 
 
 def event_time_ms(fn, iters: int, warmup: int = 2) -> float:
@@ -205,7 +205,7 @@ def main() -> None:
                               "frac_hbm": (b_up + b_dn) / ((t_up + t_dn) * 1e-3) / 1e9 / PEAK_HBM_GBS}
             del up, dn, hs, ys
         out["decode_stack"] = stack
-        out["roofline_decode"] = {"bound": "hbm", "kernel": "mortar_resident_kernel<4 tokens> (160 layers per launch, b=1)",
+        out["roofline_decode"] = {"bound": "hbm", "kernel": "mortar_resident_kernel<4 tokens>, gate_up + down launches of 160 layers each, b=1",
                                   "achieved": stack["b1"]["algorithmic_GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                   "frac": stack["b1"]["frac_hbm"], "traffic": TRAFFIC_DECODE_STACK_BYTES,
                                   "algorithmic_bytes": n_sets * (wbytes + (2 * D_MODEL + 2 * D_FF) * 2)}
