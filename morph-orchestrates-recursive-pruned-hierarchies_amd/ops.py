@@ -73,6 +73,8 @@ def gateup_swiglu(x: Tensor, W: MortarPack, gates: Tensor | None = None, route: 
     route = (tok_cnt, tok_list) from remoe_route switches on active-tile skipping."""
     x = _bf16_2d(x, "gateup_swiglu")
     M = x.shape[0]
+    if W.Rb % 2:
+        raise ValueError(f"gateup_swiglu: gate_up has an odd number of block-rows ({W.Rb}): not a [2*d_ff, d_model] matrix")
     d_ff = W.out_features // 2
     if x.shape[1] != W.in_features:
         raise ValueError(f"gateup_swiglu: x has {x.shape[1]} features, matrix expects {W.in_features}")

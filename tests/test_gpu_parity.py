@@ -400,3 +400,30 @@ def test_full_size_properties(dev):
     yr = ops.spmm(hr, Wdn, active=active)
     refr = O.swiglu_mlp(x[rows], spec["gate_up"], spec["down"], gates=g_ref[rows])
     assert_close_bf16(to_np(yr)[rows], refr["y"], "routed y rows", ulps=8)
+
+
+# ---------------------------------------------------------------------------------------------- error behaviour
+
+def test_argument_errors_are_raised_before_launch(dev):
+    """Host-side checks of the C-ABI surface: every bad call raises (ValueError for arguments / limits) and
+    nothing is launched."""
+    m = synth.synth_matrix(16 * 4, 16 * 8, 0.5, seed=1)
+    W = synth.to_pack(m, dev)
+    x = to_dev(synth.synth_x(8, 128, 2), dev)
+    with pytest.raises(ValueError, match="features"):
+        ops.spmm(x[:, :64], W)
+    with pytest.raises(TypeError):
+        ops.spmm(x.float(), W)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        ops.spmm(x.cpu(), W)
+    with pytest.raises(ValueError, match="odd number of block-rows"):
+        ops.gateup_swiglu(x, synth.to_pack(synth.synth_matrix(16 * 3, 16 * 8, 0.5, seed=2), dev))
+    with pytest.raises(ValueError, match="multiple of 4"):                       # d_ff / n_clusters = 32 / 16 = 2
+        ops.gateup_swiglu(x, W, gates=torch.ones((8, 16), device=dev))
+    with pytest.raises(ValueError, match="tile must be"):
+        ops.remoe_route(torch.ones((8, 4), dtype=torch.uint8, device=dev), 24)
+    wide = synth.to_pack(synth.synth_matrix(16 * 4, 16 * 400, 0.1, seed=3), dev)  # K too wide for routed skipping
+    assert ops.route_tile(wide, 4096) == 0 and ops.route_tile(wide, 2) == 4
+    assert ops.spmm(x[:0], W).shape == (0, 64)                                    # empty batch: no launch, empty result
+    y = ops.spmm(x, W)                                                            # and the good call still works
+    assert_close_bf16(to_np(y), oracle_spmm(to_np(x), m), "after errors")

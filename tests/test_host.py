@@ -267,3 +267,9 @@ def test_synth_generators_are_deterministic_and_shaped():
     cnt = np.diff(z["offsets"])
     assert cnt.min() >= round(0.05 * 352) and cnt.max() <= round(0.60 * 352)
     assert abs(cnt.mean() / 352 - 0.25) < 0.02 and cnt.std() > 10
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess, sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "ONE GPU" in (r.stderr + r.stdout)
