@@ -10,7 +10,7 @@
 
 namespace {
 
-constexpr int MAXPL = 16;   // logits per lane -> n <= 1024
+constexpr int MAXPL_LIMIT = 16;   // logits per lane -> n <= 1024
 
 __device__ __forceinline__ uint32_t order_key(float f) {
     const uint32_t u = __builtin_bit_cast(uint32_t, f);
@@ -30,6 +30,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 // One wavefront per token.  The k-th largest logit is found exactly by an MSB-first radix select on
 // order-preserving keys: for each bit the wave counts (ballot + popcount) the keys >= the candidate
 // prefix.  Ties need no special care: the result is a VALUE, and the gate rule is `logit > kth`.
+template <int MAXPL>      // logits per lane this instantiation holds: n <= 64 * MAXPL
 __global__ void __launch_bounds__(256) remoe_gates_kernel(const float *logits, int64_t M, int n, int k,
                                                            float *gates, uint8_t *active) {
     const int lane = threadIdx.x & 63;
@@ -48,13 +49,11 @@ __global__ void __launch_bounds__(256) remoe_gates_kernel(const float *logits, i
     const bool thresh = k < n;
     if (thresh) {
         uint32_t prefix = 0;
-        const int npl = (n + 63) >> 6;
         for (int bit = 31; bit >= 0; --bit) {
             const uint32_t cand = prefix | (1u << bit);
             int c = 0;
 #pragma unroll
-            for (int i = 0; i < MAXPL; ++i)
-                if (i < npl) c += __popcll(__ballot(key[i] >= cand));
+            for (int i = 0; i < MAXPL; ++i) c += __popcll(__ballot(key[i] >= cand));     // padding keys are 0 < cand
             if (c >= k) prefix = cand;
         }
         kth = key_to_float(prefix);
@@ -164,9 +163,16 @@ extern "C" int mortar_remoe_gates(const float *logits, int64_t M, int32_t n, int
                                   uint8_t *active, void *stream) {
     if (!logits || !gates) return mortar_fail(MORTAR_ERR_ARG, "remoe_gates: null pointer");
     if (M <= 0 || n <= 0 || k <= 0) return mortar_fail(MORTAR_ERR_ARG, "remoe_gates: M, n, k must be positive");
-    if (n > 64 * MAXPL) return mortar_fail(MORTAR_ERR_LIMIT, "remoe_gates: n=%d exceeds %d clusters", n, 64 * MAXPL);
-    hipLaunchKernelGGL(remoe_gates_kernel, dim3((unsigned)((M + 3) / 4)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), logits, M, n, k, gates, active);
+    if (n > 64 * MAXPL_LIMIT) return mortar_fail(MORTAR_ERR_LIMIT, "remoe_gates: n=%d exceeds %d clusters", n, 64 * MAXPL_LIMIT);
+    const dim3 grid((unsigned)((M + 3) / 4)), block(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int npl = (n + 63) / 64;
+    if (npl <= 1) hipLaunchKernelGGL(remoe_gates_kernel<1>, grid, block, 0, st, logits, M, n, k, gates, active);
+    else if (npl <= 2) hipLaunchKernelGGL(remoe_gates_kernel<2>, grid, block, 0, st, logits, M, n, k, gates, active);
+    else if (npl <= 4) hipLaunchKernelGGL(remoe_gates_kernel<4>, grid, block, 0, st, logits, M, n, k, gates, active);
+    else if (npl <= 6) hipLaunchKernelGGL(remoe_gates_kernel<6>, grid, block, 0, st, logits, M, n, k, gates, active);
+    else if (npl <= 8) hipLaunchKernelGGL(remoe_gates_kernel<8>, grid, block, 0, st, logits, M, n, k, gates, active);
+    else hipLaunchKernelGGL(remoe_gates_kernel<16>, grid, block, 0, st, logits, M, n, k, gates, active);
     return check_launch("remoe_gates");
 }
 
