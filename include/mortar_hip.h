@@ -41,14 +41,20 @@ enum {
  *   sdup    [nnz] uint32: per-block scale pattern produced by mortar_encode_blocks_host
  *   col     [nnz] the reference's mortar_column_indices (int16, unchanged)
  *   row_ptr [Rb+1] the reference's mortar_offsets (int32, unchanged)
- * Octet stream (second copy for the prefill kernels, from mortar_octet_layout_host): the block-columns are cut
+ * Octet stream (the copy every SpMM kernel reads, prefill and decode; from mortar_octet_layout_host): the block-columns are cut
  * into nseg = ceil(Cb / seg_cb) K segments, and every (segment, row) run of blocks into groups of 8 blocks
  * (the last one padded with all-zero blocks) so that one 16-byte load per lane fetches the lane's code dwords
  * of four consecutive block pairs:
  *   row_desc [nseg*Rb*4] int32 per (segment, row): {first group, end group, number of blocks, 0}
  *   col_o holds block-columns relative to the segment start
  *   codes_o [ngroups*2*16*4] uint32: ((group*2 + s)*16 + n)*4 + t = row n of block 8*g + 2*t + s of the row
- *   sd_o    [ngroups*2*4] uint32 and col_o [ngroups*2*4] int32: (group*2 + s)*4 + t, same block             */
+ *   sd_o    [ngroups*2*4] uint32 and col_o [ngroups*2*4] int32: (group*2 + s)*4 + t, same block
+ * Optional 4-bit copy of the code stream for prefill-sized launches (M > 64), from mortar_fp4_stream_host; NULL =
+ * prefill unpacks the 2-bit stream.  Same octets, every ternary code as an FP4 (E2M1) value (0 -> 0x0, +1 -> 0x2,
+ * -1 -> 0xA) so that one hardware conversion per register replaces the shift and mask of the 2-bit unpack:
+ *   codes4_o [ngroups*4*16*4] uint32: ((group*4 + 2*s + h)*16 + n)*4 + t = columns 8h .. 8h+7 of row n of block
+ *            8*g + 2*t + s, column 8h + q in bits [4q, 4q+3]
+ * Decode-sized launches always read the 2-bit stream (half the bytes).                                          */
 typedef struct {
     const uint32_t *codes;
     const uint32_t *sdup;
@@ -58,6 +64,7 @@ typedef struct {
     const uint32_t *codes_o;
     const uint32_t *sd_o;
     const int32_t *col_o;
+    const uint32_t *codes4_o;
     int32_t Rb, Cb, nnz;
     int32_t seg_cb;   /* block-columns per K segment of the octet stream (>= Cb: one segment) */
 } mortar_bcsr_t;
@@ -90,6 +97,10 @@ int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, int32_t Cb,
                                  const uint32_t *codes, const uint32_t *sdup, const int16_t *col,
                                  int32_t *row_desc_out, uint32_t *codes_o_out, uint32_t *sd_o_out,
                                  int32_t *col_o_out);
+
+/* 4-bit copy of an octet code stream: codes_o host [ngroups*128] (from mortar_octet_layout_host) ->
+ * codes4_o_out host [ngroups*256], layout as described at mortar_bcsr_t.  No counterpart in the reference. */
+int mortar_fp4_stream_host(const uint32_t *codes_o, int64_t ngroups, uint32_t *codes4_o_out);
 
 /* Largest K segment (in block-columns) whose 32-token activation tile fits in LDS; a matrix with
  * Cb <= this runs the single-segment prefill kernel.  Use seg_cb = ceil(Cb / ceil(Cb / max)). */

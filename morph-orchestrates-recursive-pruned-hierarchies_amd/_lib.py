@@ -16,7 +16,8 @@ c_i32, c_i64, c_vp, c_f32 = C.c_int32, C.c_int64, C.c_void_p, C.c_float
 class BcsrStruct(C.Structure):
     """mortar_bcsr_t"""
     _fields_ = [("codes", c_vp), ("sdup", c_vp), ("col", c_vp), ("row_ptr", c_vp), ("row_desc", c_vp),
-                ("codes_o", c_vp), ("sd_o", c_vp), ("col_o", c_vp), ("Rb", c_i32), ("Cb", c_i32), ("nnz", c_i32),
+                ("codes_o", c_vp), ("sd_o", c_vp), ("col_o", c_vp), ("codes4_o", c_vp),
+                ("Rb", c_i32), ("Cb", c_i32), ("nnz", c_i32),
                 ("seg_cb", c_i32)]
 
 
@@ -26,6 +27,7 @@ _SIGS = {
     "mortar_encode_blocks_host": (C.c_int, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp]),
     "mortar_decode_blocks_host": (C.c_int, [c_vp, c_i64, c_vp]),
     "mortar_octet_layout_host": (c_i64, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
+    "mortar_fp4_stream_host": (C.c_int, [c_vp, c_i64, c_vp]),
     "mortar_prefill_max_seg_cb": (C.c_int, []),
     "mortar_validate_bcsr_host": (C.c_int, [c_vp, c_vp, c_i32, c_i32]),
     "mortar_schedule_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp]),

@@ -34,6 +34,19 @@ __device__ __forceinline__ u32x4_t mortar_unpack8(uint32_t t, uint32_t sd) {
     return r;
 }
 
+// Same result from the 4-bit stream: `t` holds the lane's 8 codes as FP4 (E2M1) values 0 / +1 / -1, byte i =
+// {column 2i (low nibble), column 2i+1 (high nibble)}.  One scaled conversion per register (scale 2.0 makes the
+// bf16 patterns 0x4000 / 0xC000 / 0, i.e. fp16 +-2 / 0 as above), then the same multiply.
+__device__ __forceinline__ u32x4_t mortar_unpack8_fp4(uint32_t t, uint32_t sd) {
+    const f16x2_t s = __builtin_bit_cast(f16x2_t, sd);
+    u32x4_t r;
+    r[0] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(t, 2.0f, 0)));
+    r[1] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(t, 2.0f, 1)));
+    r[2] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(t, 2.0f, 2)));
+    r[3] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(t, 2.0f, 3)));
+    return r;
+}
+
 __device__ __forceinline__ f32x4_t mortar_mfma(u32x4_t a, u32x4_t b, f32x4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
                                                    __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);

@@ -25,7 +25,7 @@ int mortar_fail(int code, const char *fmt, ...) {
 }
 
 extern "C" const char *mortar_last_error(void) { return g_err; }
-extern "C" int mortar_abi_version(void) { return 1; }
+extern "C" int mortar_abi_version(void) { return 2; }
 
 static inline uint16_t f32_to_bf16_bits(float f) {
     uint32_t u;
@@ -157,6 +157,26 @@ extern "C" int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, 
         }
     }
     return ng;
+}
+
+extern "C" int mortar_fp4_stream_host(const uint32_t *codes_o, int64_t ngroups, uint32_t *codes4_o_out) {
+    if (!codes_o || !codes4_o_out || ngroups < 0) return mortar_fail(MORTAR_ERR_ARG, "fp4_stream: bad argument");
+    for (int64_t gs = 0; gs < ngroups * 2; ++gs)          // (octet, s)
+        for (int n = 0; n < 16; ++n)
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t w = codes_o[(gs * 16 + n) * 4 + t];
+                for (int h = 0; h < 2; ++h) {
+                    uint32_t o = 0;
+                    for (int q = 0; q < 8; ++q) {
+                        const int c = 8 * h + q;
+                        const uint32_t enc = (w >> (2 * slot_of_col(c))) & 3u;
+                        o |= (enc == 1u ? 0x2u : (enc == 3u ? 0xAu : 0u)) << (4 * q);
+                    }
+                    const int64_t g = gs >> 1, s2 = gs & 1;
+                    codes4_o_out[(((g * 4 + 2 * s2 + h) * 16) + n) * 4 + t] = o;
+                }
+            }
+    return MORTAR_OK;
 }
 
 extern "C" int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_t rows_per_unit,

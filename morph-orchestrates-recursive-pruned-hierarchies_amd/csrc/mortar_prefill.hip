@@ -50,34 +50,45 @@ int resident_mt(int Cb) {
 
 // prefill tiles: 16 wavefronts (4 per SIMD) for the 32-token tile, 8 for the 64-token tile (measured: a 96-token
 // tile of a narrow matrix leaves only two waves per SIMD and is slower)
-template <int NACC, bool ROUTED>
+template <int NACC, bool ROUTED, bool FP4>
 int launch_resident_any(SpmmParams &p, hipStream_t st) {
     switch (resident_mt(p.Cb)) {
-        case 64: return mortar_launch_resident<64, NACC, ROUTED, 8>(p, nullptr, 1, st);
-        default: return mortar_launch_resident<32, NACC, ROUTED, 16>(p, nullptr, 1, st);
+        case 64: return mortar_launch_resident<64, NACC, ROUTED, 8, false, FP4>(p, nullptr, 1, st);
+        default: return mortar_launch_resident<32, NACC, ROUTED, 16, false, FP4>(p, nullptr, 1, st);
     }
 }
 
 constexpr int SEG_WAVES = 16, SEG_UPW = 4;
 
-// kind: 0 spmm, 1 gate_up + SwiGLU, 2 routed gate_up + SwiGLU, 3 spmm with an input mask
-int dispatch(int kind, SpmmParams &p, hipStream_t st) {
+template <bool FP4>
+int dispatch_prefill(int kind, SpmmParams &p, hipStream_t st) {
+    switch (kind) {
+        case 0:
+            if (p.nseg == 1) return launch_resident_any<1, false, FP4>(p, st);
+            return mortar_launch_segmented<32, 1, false, SEG_WAVES, SEG_UPW, false, FP4>(p, nullptr, 1, st);
+        case 1:
+            if (p.nseg == 1) return launch_resident_any<2, false, FP4>(p, st);
+            return mortar_launch_segmented<32, 2, false, SEG_WAVES, 2, false, FP4>(p, nullptr, 1, st);
+        case 2:
+            return launch_resident_any<2, true, FP4>(p, st);
+        default:
+            return mortar_launch_segmented<32, 1, true, SEG_WAVES, SEG_UPW, false, FP4>(p, nullptr, 1, st);
+    }
+}
+
+// kind: 0 spmm, 1 gate_up + SwiGLU, 2 routed gate_up + SwiGLU, 3 spmm with an input mask.
+// Prefill-sized launches read the 4-bit code stream when the matrix carries one (cheaper unpack: one conversion
+// per register instead of shift + mask); decode-sized launches always stream the 2-bit codes (half the bytes).
+int dispatch(int kind, SpmmParams &p, const mortar_bcsr_t *W, hipStream_t st) {
     if (p.M <= MORTAR_SMALLM_MAX) {
         const int rc = mortar_smallm_launch(kind, p, nullptr, 1, st);
         if (rc >= 0) return rc;
     }
-    switch (kind) {
-        case 0:
-            if (p.nseg == 1) return launch_resident_any<1, false>(p, st);
-            return mortar_launch_segmented<32, 1, false, SEG_WAVES, SEG_UPW>(p, nullptr, 1, st);
-        case 1:
-            if (p.nseg == 1) return launch_resident_any<2, false>(p, st);
-            return mortar_launch_segmented<32, 2, false, SEG_WAVES, 2>(p, nullptr, 1, st);
-        case 2:
-            return launch_resident_any<2, true>(p, st);
-        default:
-            return mortar_launch_segmented<32, 1, true, SEG_WAVES, SEG_UPW>(p, nullptr, 1, st);
+    if (W->codes4_o) {
+        p.codes_o = reinterpret_cast<const u32x4_t *>(W->codes4_o);
+        return dispatch_prefill<true>(kind, p, st);
     }
+    return dispatch_prefill<false>(kind, p, st);
 }
 
 }  // namespace
@@ -99,7 +110,7 @@ extern "C" int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *sched, co
     SpmmParams p;
     fill(p, W, sched, x, M, ldx, y, ldy);
     p.n_units = W->Rb;
-    return dispatch(0, p, static_cast<hipStream_t>(stream));
+    return dispatch(0, p, W, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M,
@@ -113,7 +124,7 @@ extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *sc
     fill(p, W, sched, x, M, ldx, y, ldy);
     p.n_units = W->Rb;
     p.active = active; p.n_clusters = n_clusters; p.cluster_size = (W->Cb * 16) / n_clusters;
-    return dispatch(3, p, static_cast<hipStream_t>(stream));
+    return dispatch(3, p, W, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M,
@@ -139,9 +150,9 @@ extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *
             return mortar_fail(MORTAR_ERR_LIMIT, "gateup: routed mode needs in_features to fit one LDS tile "
                                "(mortar_route_tile() == 0: call without tok_cnt / tok_list)");
         p.tok_cnt = tok_cnt; p.tok_list = tok_list;
-        return dispatch(2, p, static_cast<hipStream_t>(stream));
+        return dispatch(2, p, W, static_cast<hipStream_t>(stream));
     }
-    return dispatch(1, p, static_cast<hipStream_t>(stream));
+    return dispatch(1, p, W, static_cast<hipStream_t>(stream));
 }
 
 // ---- layer-batched small-M launches ---------------------------------------------------------------------

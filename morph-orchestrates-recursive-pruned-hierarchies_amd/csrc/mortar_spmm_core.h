@@ -113,10 +113,15 @@ struct MortarBatch {
 };
 
 // Loads the batch that starts at octet gq of a row part ending at octet g1 (octets past the end repeat the last).
-__device__ __forceinline__ void mortar_load_batch(const SpmmView &p, MortarBatch &b, int gq, int g1, int n, int bsel) {
+// FP4: the code stream is the 4-bit one (a lane's dword holds the 8 codes of its own column half, so the four
+// lane groups read four different 16-byte runs per octet instead of two).
+template <bool FP4 = false>
+__device__ __forceinline__ void mortar_load_batch(const SpmmView &p, MortarBatch &b, int gq, int g1, int n, int bsel,
+                                                  int hsel = 0) {
 #pragma unroll
     for (int k = 0; k < RES_GROUPS; ++k) {
-        const uint32_t gi = (uint32_t)(gq + k < g1 ? gq + k : g1 - 1) * 2u + (uint32_t)bsel;
+        const uint32_t go = (uint32_t)(gq + k < g1 ? gq + k : g1 - 1);
+        const uint32_t gi = FP4 ? go * 4u + (uint32_t)(bsel * 2 + hsel) : go * 2u + (uint32_t)bsel;
         b.cw[k] = p.codes_o[gi * 16u + n];
     }
     const int go = gq + (n >> 2);
@@ -128,18 +133,18 @@ __device__ __forceinline__ void mortar_load_batch(const SpmmView &p, MortarBatch
 // One row part: octets [g0, g1) (nb blocks) of the stream against the tile at `lx`.
 // `xo_base` is the lane's unit offset inside a block-column (column half, token) plus the segment's origin.
 // `b` holds the part's first batch, loaded by the caller (mortar_load_batch at g0) where it suits it.
-template <int MSUB, int LDM, bool ROUTED>
+template <int MSUB, int LDM, bool ROUTED, bool FP4 = false>
 __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *lx, MortarBatch b, int g0, int g1,
                                                 int nb, uint32_t xo_base, const uint32_t (&tk)[MSUB], int nsub, int n,
                                                 int bsel, int hsel, f32x4_t (&acc)[MSUB]) {
     const unsigned char *lb = reinterpret_cast<const unsigned char *>(lx);
     for (int gq = g0; gq < g1; gq += RES_GROUPS) {
-        if (gq != g0) mortar_load_batch(p, b, gq, g1, n, bsel);
+        if (gq != g0) mortar_load_batch<FP4>(p, b, gq, g1, n, bsel, hsel);
         const uint32_t ccs = __umul24(b.ccv, (uint32_t)(2 * LDM * 16));   // byte offset of the block-column in the tile
         const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;      // block pairs left in the row from this batch on
         // Activation operands are fetched two pairs ahead of the MFMAs that use them.  The only branches are
-        // per octet (a whole octet past the end of the part is skipped); inside an octet the four pairs run
-        // straight, pairs past the end being the all-zero padding blocks of the stream.
+        // per octet (a whole octet past the end of the part is skipped) and, for prefill tiles, per half octet;
+        // otherwise the pairs run straight, pairs past the end being the all-zero padding blocks of the stream.
         constexpr int NP = 4 * RES_GROUPS;
         uint4 Bq[3][MSUB];
 #pragma unroll
@@ -154,7 +159,9 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const int u = 4 * k + t;
-                    const u32x4_t A = mortar_unpack8(b.cw[k][t] << (8 * hsel), mortar_row_bcast(b.sdv, u));
+                    if (MSUB >= 2 && t == 2 && u >= pairs) break;     // prefill tiles: the padded half of the last octet
+                    const uint32_t sdu = mortar_row_bcast(b.sdv, u);
+                    const u32x4_t A = FP4 ? mortar_unpack8_fp4(b.cw[k][t], sdu) : mortar_unpack8(b.cw[k][t] << (8 * hsel), sdu);
                     if (u + 2 < NP) {
                         const uint32_t xo = mortar_row_bcast(ccs, u + 2) + xo_base * 16u;
 #pragma unroll
@@ -254,7 +261,7 @@ __device__ __forceinline__ u32x4_t mortar_part_desc(const SpmmView &p, int pos, 
 // No barrier after the first one.  A wave's work is a chain of row parts (unit, segment, row of the unit) whose
 // descriptors come from the schedule table one part ahead; latency is hidden by the waves that share a SIMD.
 // ---------------------------------------------------------------------------------------------------------
-template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE>
+template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE, bool FP4>
 __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmParams p0, const SpmmParams *table) {
     constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1;
     const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
@@ -333,8 +340,8 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
                 const int nb = __builtin_amdgcn_readfirstlane((int)d0[2]);
                 if (!skip && g0 < g1) {
                     MortarBatch b;
-                    mortar_load_batch(p, b, g0, g1, n, bsel);
-                    mortar_row_part<MSUB, LDM, ROUTED>(p, lx, b, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+                    mortar_load_batch<FP4>(p, b, g0, g1, n, bsel, hsel);
+                    mortar_row_part<MSUB, LDM, ROUTED, FP4>(p, lx, b, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
                 }
                 d0 = d1;
             }
@@ -360,7 +367,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
 // The descriptors of the next segment are fetched before the barrier pair, so their latency hides behind the
 // staging.
 // ---------------------------------------------------------------------------------------------------------
-template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE>
+template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE, bool FP4>
 __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const SpmmParams p0, const SpmmParams *table) {
     constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1, NP = UPW * NACC;
     const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
@@ -420,8 +427,8 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
         for (int q = 0; q < NP; ++q) {
             if (g0[q] < g1[q]) {
                 MortarBatch b;
-                mortar_load_batch(p, b, g0[q], g1[q], n, bsel);
-                mortar_row_part<MSUB, LDM, false>(p, lx, b, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
+                mortar_load_batch<FP4>(p, b, g0[q], g1[q], n, bsel, hsel);
+                mortar_row_part<MSUB, LDM, false, FP4>(p, lx, b, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
                                                   acc[q / NACC][q % NACC]);
             }
         }
@@ -579,13 +586,13 @@ inline int64_t mortar_grid_width(SpmmParams &p, int layers) {
 template <int MT, int WAVES>
 inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
     p.n_mtiles = (p.M + MT - 1) / MT;
-    // Prefill tiles: enough workgroups to cover the 256 CUs twice (every workgroup stages a whole tile, so few
-    // large ones).  Decode tiles stage little: many small workgroups (about 12 per CU) so that the hardware
+    // Prefill tiles: one workgroup per CU (every workgroup stages a whole tile and the last units of its window
+    // leave waves idle, so few large ones: one round measured faster than two).  Decode tiles stage little: many small workgroups (about 12 per CU) so that the hardware
     // dispatcher evens out the load, with a few units per wave when many layers share the launch and one unit
     // per wave when a single matrix has to be spread over the whole chip.
     const bool wide = (int64_t)layers * p.n_units >= 8 * 512;
     const int upw = MT > 16 || !wide ? 1 : (MT <= 4 ? 2 : 4);
-    const int target = MT <= 16 ? 256 * 12 : 256 * 2;
+        const int target = MT <= 16 ? 256 * 12 : 256;
     int split = (target + layers * p.n_mtiles - 1) / (layers * p.n_mtiles);
     const int max_split = (p.n_units + WAVES * upw - 1) / (WAVES * upw);
     split = split < 1 ? 1 : (split > max_split ? max_split : split);
@@ -593,13 +600,13 @@ inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
     return mortar_grid_width(p, layers);
 }
 
-template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE = false>
+template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE = false, bool FP4 = false>
 int mortar_launch_resident(SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     if (TABLE != (table != nullptr)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: parameter table mismatch");
     const int smem = tile_bytes(MT, p.Cb) + LDS_EXTRA;
     if (smem > LDS_BUDGET + LDS_PAD * 16 + LDS_EXTRA) return mortar_fail(MORTAR_ERR_LIMIT, "resident tile of %d bytes does not fit LDS", smem);
     static bool attr_done = false;
-    auto kern = mortar_resident_kernel<MT, NACC, ROUTED, WAVES, TABLE>;
+    auto kern = mortar_resident_kernel<MT, NACC, ROUTED, WAVES, TABLE, FP4>;
     int rc = mortar_allow_big_lds(kern, attr_done);
     if (rc) return rc;
     const int64_t grid = mortar_resident_shape<MT, WAVES>(p, layers);
@@ -617,13 +624,13 @@ inline int64_t mortar_segmented_shape(SpmmParams &p, int layers) {
     return mortar_grid_width(p, layers);
 }
 
-template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE = false>
+template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE = false, bool FP4 = false>
 int mortar_launch_segmented(SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     if (TABLE != (table != nullptr)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: parameter table mismatch");
     const int smem = tile_bytes(MT, p.seg_cb);
     if (smem > LDS_BUDGET + LDS_PAD * 16) return mortar_fail(MORTAR_ERR_LIMIT, "segment tile of %d bytes does not fit LDS", smem);
     static bool attr_done = false;
-    auto kern = mortar_segmented_kernel<MT, NACC, MASKED, WAVES, UPW, TABLE>;
+    auto kern = mortar_segmented_kernel<MT, NACC, MASKED, WAVES, UPW, TABLE, FP4>;
     int rc = mortar_allow_big_lds(kern, attr_done);
     if (rc) return rc;
     const int64_t grid = mortar_segmented_shape<MT, WAVES, UPW>(p, layers);

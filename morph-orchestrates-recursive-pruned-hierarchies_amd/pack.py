@@ -71,6 +71,14 @@ def octet_layout(offsets, Rb: int, Cb: int, seg_cb: int, codes: np.ndarray, sdup
     return grp, codes_o, sd_o, col_o
 
 
+def fp4_stream(codes_o: np.ndarray) -> np.ndarray:
+    """4-bit (FP4) copy of an octet code stream: see mortar_fp4_stream_host."""
+    codes_o = _np(codes_o, np.uint32)
+    out = np.empty(codes_o.size * 2, dtype=np.uint32)
+    _lib.check(_lib.lib().mortar_fp4_stream_host(_vp(codes_o), codes_o.size // 128, _vp(out)), "mortar_fp4_stream_host")
+    return out
+
+
 def unit_order(offsets, Rb: int, rows_per_unit: int, group: int = SCHED_GROUP) -> np.ndarray:
     offsets = _np(offsets, np.int32)
     out = np.empty(Rb // rows_per_unit, dtype=np.int32)
@@ -107,10 +115,13 @@ class MortarPack:
 
     Built from the reference's buffers: ``packed`` = mortar_packed (flat 2-bit codes over [nnz,16,16]),
     ``scale`` = mortar_scale (scalar) or a per-block fp32 vector, ``col`` = mortar_column_indices,
-    ``offsets`` = mortar_offsets.
+    ``offsets`` = mortar_offsets.  ``prefill_stream`` also keeps the 4-bit copy of the code stream that
+    prefill-sized launches (M > 64) unpack faster (+128 bytes per block of device memory); without it they
+    unpack the 2-bit stream.
     """
 
-    def __init__(self, packed, scale, col, offsets, out_features: int, in_features: int, device):
+    def __init__(self, packed, scale, col, offsets, out_features: int, in_features: int, device,
+                 prefill_stream: bool = True):
         if out_features % BLK or in_features % BLK:
             raise ValueError(f"[{out_features},{in_features}] not divisible by blocking {BLK}")
         self.out_features, self.in_features = int(out_features), int(in_features)
@@ -142,6 +153,7 @@ class MortarPack:
         self.codes_o = torch.from_numpy(codes_o.view(np.int32)).to(dev)
         self.sd_o = torch.from_numpy(sd_o.view(np.int32)).to(dev)
         self.col_o = torch.from_numpy(col_o).to(dev)
+        self.codes4_o = torch.from_numpy(fp4_stream(codes_o).view(np.int32)).to(dev) if prefill_stream else None
         self._scheds: dict[int, torch.Tensor] = {}
         self._worklists: dict[tuple, tuple] = {}
         self.struct = self._make_struct()
@@ -150,7 +162,9 @@ class MortarPack:
     def _make_struct(self):
         return _lib.BcsrStruct(self.codes.data_ptr(), self.sdup.data_ptr(), self.col.data_ptr(),
                                self.row_ptr.data_ptr(), self.row_desc.data_ptr(), self.codes_o.data_ptr(),
-                               self.sd_o.data_ptr(), self.col_o.data_ptr(), self.Rb, self.Cb, self.nnz, self.seg_cb)
+                               self.sd_o.data_ptr(), self.col_o.data_ptr(),
+                               self.codes4_o.data_ptr() if self.codes4_o is not None else None,
+                               self.Rb, self.Cb, self.nnz, self.seg_cb)
 
     def sched(self, rows_per_unit: int) -> torch.Tensor:
         """Device schedule (mortar_schedule_host over the balanced unit order) for plain (1) or gate/up (2) units."""
@@ -176,8 +190,9 @@ class MortarPack:
         """A second resident copy (own device buffers and schedules) of the same matrix."""
         import copy
         c = copy.copy(self)
-        for name in ("codes", "sdup", "col", "row_ptr", "row_desc", "codes_o", "sd_o", "col_o"):
-            setattr(c, name, getattr(self, name).clone())
+        for name in ("codes", "sdup", "col", "row_ptr", "row_desc", "codes_o", "sd_o", "col_o", "codes4_o"):
+            if getattr(self, name) is not None:
+                setattr(c, name, getattr(self, name).clone())
         c._scheds = {k: v.clone() for k, v in self._scheds.items()}
         c._worklists = {k: (v[0].clone(), v[1], v[2].clone(), v[3]) for k, v in self._worklists.items()}
         c.struct = c._make_struct()

@@ -166,6 +166,31 @@ def test_mlp_with_gates_and_skip(dev):
     assert torch.equal(y2, y)
 
 
+@pytest.mark.parametrize("d_model,d_ff", [(256, 16 * 40), (2048, 16 * 24), (16 * 30, 16 * 352)])
+def test_prefill_code_streams_agree(dev, d_model, d_ff):
+    """Prefill kernels over the 4-bit code stream and over the 2-bit one do the same arithmetic: identical bits
+    (64- and 32-token resident tiles, K-segmented `down`; plain, gated + routed, masked)."""
+    M, ncl = 200, d_ff // 16
+    spec = synth.synth_mlp(d_model, d_ff, 0.25, seed=33, zipf_s=1.2)
+    xd = to_dev(synth.synth_x(M, d_model, 34), dev)
+    gates, active = ops.remoe_gates(torch.from_numpy(synth.synth_logits(M, ncl, 35)).to(dev), ncl // 4)
+    outs = []
+    for stream in (True, False):
+        Wgu, Wdn = (synth.to_pack(spec[k], dev, prefill_stream=stream) for k in ("gate_up", "down"))
+        assert (Wgu.codes4_o is not None) == stream
+        h = ops.gateup_swiglu(xd, Wgu)
+        res = [h, ops.spmm(h, Wdn)]
+        tile = ops.route_tile(Wgu, M)
+        if tile:
+            hr = torch.zeros_like(h)
+            ops.gateup_swiglu(xd, Wgu, gates=gates, route=ops.remoe_route(active, tile), out=hr)
+            res += [hr, ops.spmm(hr, Wdn, active=active)]
+        outs.append(res)
+    assert_close_bf16(to_np(outs[0][1]), O.swiglu_mlp(synth.synth_x(M, d_model, 34), spec["gate_up"], spec["down"])["y"], "y", ulps=8)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+
+
 def test_remoe_route_lists_exact(dev):
     rng = np.random.default_rng(40)
     act = (rng.random((333, 70)) < 0.25).astype(np.uint8)

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in mortar_hip.h but not exported"
     assert declared == set(_lib.EXPORTS)
-    assert _lib.lib().mortar_abi_version() == 1
+    assert _lib.lib().mortar_abi_version() == 2
 
 
 def test_encode_round_trip_and_bit_layout():
@@ -112,6 +112,28 @@ def test_octet_stream_holds_every_block_once(seg_cb):
         assert [s for _, s, _ in got] == sdup[lo:hi].tolist()
         assert np.array_equal(np.stack([w for _, _, w in got]), dw.reshape(-1, 16)[lo:hi])
     assert used.all()
+
+
+def test_fp4_stream_holds_the_same_codes():
+    """The 4-bit copy of the code stream decodes (FP4 E2M1: 0x2 = +1, 0xA = -1, 0 = 0) to the ternary codes of the
+    block it mirrors, column 8h + q of row n in nibble q of dword (octet, 2s + h, n, t)."""
+    Rb, Cb = 9, 50
+    m = synth.synth_matrix(16 * Rb, 16 * Cb, 0.3, 5, zipf_s=1.2)
+    nnz = int(m["offsets"][-1])
+    dw, sdup = P.encode_blocks(O.pack_ternary_codes(m["codes"]), nnz, m["scales"])
+    desc, codes_o, _, _ = P.octet_layout(m["offsets"], Rb, Cb, 17, dw, sdup, m["col_idx"])
+    c4 = P.fp4_stream(codes_o).reshape(-1, 2, 2, 16, 4)                       # octet, s, h, n, t
+    assert c4.shape[0] * 128 == codes_o.size
+    nib = (c4[..., None] >> (4 * np.arange(8, dtype=np.uint32))) & 0xF        # ..., q
+    assert np.isin(nib, [0x0, 0x2, 0xA]).all()
+    val = np.where(nib == 0x2, 1, np.where(nib == 0xA, -1, 0)).astype(np.int8)
+    # the 2-bit stream's blocks, decoded with the library's own inverse: [octet, s, t] -> [16 rows, 16 cols]
+    blocks = codes_o.reshape(-1, 2, 16, 4).transpose(0, 1, 3, 2).reshape(-1, 16)    # (octet, s, t) x n
+    dec = np.empty((blocks.shape[0], 16, 16), np.int8)
+    _lib.check(_lib.lib().mortar_decode_blocks_host(P._vp(np.ascontiguousarray(blocks)), blocks.shape[0], P._vp(dec)), "decode")
+    dec = dec.reshape(-1, 2, 4, 16, 2, 8)                                      # octet, s, t, n, h, q
+    assert np.array_equal(val, dec.transpose(0, 1, 4, 3, 2, 5))               # -> octet, s, h, n, t, q
+    assert np.abs(dec).sum() == np.abs(m["codes"]).sum()                      # every kept code once, padding is zero
 
 
 def test_unit_order_and_schedule():
