@@ -50,8 +50,8 @@ enum {
  *   codes_o [ngroups*2*16*4] uint32: ((group*2 + s)*16 + n)*4 + t = row n of block 8*g + 2*t + s of the row
  *   sd_o    [ngroups*2*4] uint32 and col_o [ngroups*2*4] int32: (group*2 + s)*4 + t, same block
  * Optional 4-bit copy of the code stream for prefill-sized launches (M > 64), from mortar_fp4_stream_host; NULL =
- * prefill unpacks the 2-bit stream.  Same octets, every ternary code as an FP4 (E2M1) value (0 -> 0x0, +1 -> 0x2,
- * -1 -> 0xA) so that one hardware conversion per register replaces the shift and mask of the 2-bit unpack:
+ * prefill unpacks the 2-bit stream.  Same octets, every ternary code as the FP4 (E2M1) nibble the unpack feeds the
+ * hardware conversion with (0 -> 0x0, +1 -> 0x4, -1 -> 0xC), which saves the shift and mask of the 2-bit unpack:
  *   codes4_o [ngroups*4*16*4] uint32: ((group*4 + 2*s + h)*16 + n)*4 + t = columns 8h .. 8h+7 of row n of block
  *            8*g + 2*t + s, column 8h + q in bits [4q, 4q+3]
  * Decode-sized launches always read the 2-bit stream (half the bytes).                                          */

@@ -60,7 +60,7 @@ __device__ __forceinline__ void run_blocks(const GemvParams &p, int p0, int cnt,
             if (q0 + 2 * u < cnt) {
                 bool on = ok[u];
                 if (colflag) on = on && colflag[c[u]] != 0u;
-                const u32x4_t A = mortar_unpack8(on ? (w[u] << (8 * hsel)) : 0u, sd[u]);
+                const u32x4_t A = mortar_unpack8(on ? (w[u] << (2 * hsel)) : 0u, sd[u]);
                 const uint32_t xo = (uint32_t)((c[u] * 2 + hsel) * LDB + n);
 #pragma unroll
                 for (int ms = 0; ms < MSUB; ++ms) {

@@ -18,34 +18,30 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 // The accumulator lane holds D[4g + v][n], v = 0..3: four consecutive output features of token n.
 
 // 8 ternary codes -> 8 bf16 weights (+-bf16(scale) or 0) in four dwords.
-// `t` is the row dword already shifted left by 8*hsel; the pair (2i, 2i+1) of this column half then sits
-// in the top two bits of the half-words of (t << 2i): bit 15/31 = negative, bit 14/30 = non-zero.  Read as
-// 16-bit floats those half-words are -2, 0 or +2; `sd` holds the block scale's bf16 pattern minus one
-// 16-bit-float exponent step in both halves, so one packed half multiply returns exactly +-scale or 0 in bf16
-// bits (a power-of-two product is exact; the host rejects scales whose pattern would leave the normal range).
-__device__ __forceinline__ u32x4_t mortar_unpack8(uint32_t t, uint32_t sd) {
+// A row dword holds its 16 two-bit codes (bit 1 = negative, bit 0 = non-zero) interleaved: column c < 8 in slot
+// 2c + 1, column c >= 8 in slot 2(c - 8).  `t` is the dword shifted left by 2*hsel, so that the lane's 8 columns
+// sit in the odd slots: masked with 0xCCCCCCCC every nibble is {sign, non-zero, 0, 0}, which read as FP4 (E2M1) is
+// -2, 0 or +2, and one hardware conversion per register (v_cvt_scalef32_pk_bf16_fp4, scale 1) gives the two bf16
+// patterns 0xC000 / 0 / 0x4000 of a column pair.  Read as 16-bit floats those are -2, 0, +2 as well; `sd` holds
+// the block scale's bf16 pattern minus one 16-bit-float exponent step in both halves, so one packed half multiply
+// returns exactly +-scale or 0 in bf16 bits (a power-of-two product is exact; the host rejects scales whose
+// pattern would leave the normal range).
+__device__ __forceinline__ u32x4_t mortar_scale4(uint32_t nib, uint32_t sd) {
     const f16x2_t s = __builtin_bit_cast(f16x2_t, sd);
     u32x4_t r;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t f = (t << (2 * i)) & 0xC000C000u;
-        r[i] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, f));
-    }
+    r[0] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, 1.0f, 0)));
+    r[1] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, 1.0f, 1)));
+    r[2] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, 1.0f, 2)));
+    r[3] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, 1.0f, 3)));
     return r;
+}
+__device__ __forceinline__ u32x4_t mortar_unpack8(uint32_t t, uint32_t sd) {
+    return mortar_scale4(t & 0xCCCCCCCCu, sd);
 }
 
-// Same result from the 4-bit stream: `t` holds the lane's 8 codes as FP4 (E2M1) values 0 / +1 / -1, byte i =
-// {column 2i (low nibble), column 2i+1 (high nibble)}.  One scaled conversion per register (scale 2.0 makes the
-// bf16 patterns 0x4000 / 0xC000 / 0, i.e. fp16 +-2 / 0 as above), then the same multiply.
-__device__ __forceinline__ u32x4_t mortar_unpack8_fp4(uint32_t t, uint32_t sd) {
-    const f16x2_t s = __builtin_bit_cast(f16x2_t, sd);
-    u32x4_t r;
-    r[0] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(t, 2.0f, 0)));
-    r[1] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(t, 2.0f, 1)));
-    r[2] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(t, 2.0f, 2)));
-    r[3] = __builtin_bit_cast(uint32_t, s * __builtin_bit_cast(f16x2_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(t, 2.0f, 3)));
-    return r;
-}
+// Same result from the 4-bit stream: `t` holds the lane's 8 codes as FP4 nibbles {sign, non-zero, 0, 0} already,
+// byte i = {column 2i (low nibble), column 2i+1 (high nibble)}.
+__device__ __forceinline__ u32x4_t mortar_unpack8_fp4(uint32_t t, uint32_t sd) { return mortar_scale4(t, sd); }
 
 __device__ __forceinline__ f32x4_t mortar_mfma(u32x4_t a, u32x4_t b, f32x4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),

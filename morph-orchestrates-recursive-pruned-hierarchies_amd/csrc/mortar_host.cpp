@@ -35,10 +35,10 @@ static inline uint16_t f32_to_bf16_bits(float f) {
     return (uint16_t)(u >> 16);
 }
 
-// Bit position (in 2-bit slots) of column c inside a row dword: the even columns of each pair sit in the
-// low half-word and the odd columns in the high half-word, so that (dword << 2*(c/2)) & 0xC000C000
-// isolates the pair (c&~1, c|1) in the two top bit pairs of the half-words.
-static inline int slot_of_col(int c) { return ((c & 1) ? 15 : 7) - (c >> 1); }
+// Bit position (in 2-bit slots) of column c inside a row dword: columns 0..7 in the odd slots, columns 8..15 in
+// the even slots, so that (dword << 2*(c/8)) & 0xCCCCCCCC leaves the 8 codes of a column half as the top two
+// bits of the 8 nibbles, in column order.
+static inline int slot_of_col(int c) { return c < 8 ? 2 * c + 1 : 2 * (c - 8); }
 
 extern "C" int mortar_encode_blocks_host(const uint8_t *packed, int64_t nnz, const float *scale,
                                          int64_t scale_count, uint32_t *codes_out, uint32_t *sdup_out) {
@@ -170,7 +170,7 @@ extern "C" int mortar_fp4_stream_host(const uint32_t *codes_o, int64_t ngroups, 
                     for (int q = 0; q < 8; ++q) {
                         const int c = 8 * h + q;
                         const uint32_t enc = (w >> (2 * slot_of_col(c))) & 3u;
-                        o |= (enc == 1u ? 0x2u : (enc == 3u ? 0xAu : 0u)) << (4 * q);
+                        o |= (enc << 2) << (4 * q);
                     }
                     const int64_t g = gs >> 1, s2 = gs & 1;
                     codes4_o_out[(((g * 4 + 2 * s2 + h) * 16) + n) * 4 + t] = o;

@@ -161,7 +161,7 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
                     const int u = 4 * k + t;
                     if (MSUB >= 2 && t == 2 && u >= pairs) break;     // prefill tiles: the padded half of the last octet
                     const uint32_t sdu = mortar_row_bcast(b.sdv, u);
-                    const u32x4_t A = FP4 ? mortar_unpack8_fp4(b.cw[k][t], sdu) : mortar_unpack8(b.cw[k][t] << (8 * hsel), sdu);
+                    const u32x4_t A = FP4 ? mortar_unpack8_fp4(b.cw[k][t], sdu) : mortar_unpack8(b.cw[k][t] << (2 * hsel), sdu);
                     if (u + 2 < NP) {
                         const uint32_t xo = mortar_row_bcast(ccs, u + 2) + xo_base * 16u;
 #pragma unroll

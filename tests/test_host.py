@@ -32,13 +32,12 @@ def test_encode_round_trip_and_bit_layout():
     scale = rng.uniform(0.01, 0.1, 9).astype(np.float32)
     dw, sdup = P.encode_blocks(O.pack_ternary_codes(codes), 9, scale)
     assert np.array_equal(P.decode_blocks(dw), codes)
-    # the pair (2i, 2i+1) of column half h is isolated by (w << 8h << 2i) & 0xC000C000: bit 15/31 sign, 14/30 non-zero
-    for j, n, h, i in itertools.product((0, 8), (0, 7, 15), (0, 1), range(4)):
+    # the 8 columns of column half h are the top two bits (sign, non-zero) of the 8 nibbles of (w << 2h) & 0xCCCCCCCC,
+    # in column order: as FP4 (E2M1) those nibbles are 0x4 = +2, 0xC = -2, 0 = 0
+    for j, n, h, q in itertools.product((0, 8), (0, 7, 15), (0, 1), range(8)):
         w = int(dw[j * 16 + n])
-        f = ((w << (8 * h + 2 * i)) & 0xFFFFFFFF) & 0xC000C000
-        for half, c in ((0, 8 * h + 2 * i), (1, 8 * h + 2 * i + 1)):
-            bits = (f >> (16 * half + 14)) & 3
-            assert {0: 0, 1: 1, 3: -1}[bits] == codes[j, n, c]
+        nib = ((((w << (2 * h)) & 0xFFFFFFFF) & 0xCCCCCCCC) >> (4 * q)) & 0xF
+        assert {0x0: 0, 0x4: 1, 0xC: -1}[nib] == codes[j, n, 8 * h + q]
     # scale pattern: bf16 bits minus one 16-bit-float exponent step, in both halves
     s16 = O.bf16_bits(scale).astype(np.uint32) - 0x400
     assert np.array_equal(sdup, s16 | (s16 << 16))
@@ -115,7 +114,7 @@ def test_octet_stream_holds_every_block_once(seg_cb):
 
 
 def test_fp4_stream_holds_the_same_codes():
-    """The 4-bit copy of the code stream decodes (FP4 E2M1: 0x2 = +1, 0xA = -1, 0 = 0) to the ternary codes of the
+    """The 4-bit copy of the code stream decodes (FP4 E2M1: 0x4 = +2, 0xC = -2, 0 = 0, for codes +1 / -1 / 0) to the ternary codes of the
     block it mirrors, column 8h + q of row n in nibble q of dword (octet, 2s + h, n, t)."""
     Rb, Cb = 9, 50
     m = synth.synth_matrix(16 * Rb, 16 * Cb, 0.3, 5, zipf_s=1.2)
@@ -125,8 +124,8 @@ def test_fp4_stream_holds_the_same_codes():
     c4 = P.fp4_stream(codes_o).reshape(-1, 2, 2, 16, 4)                       # octet, s, h, n, t
     assert c4.shape[0] * 128 == codes_o.size
     nib = (c4[..., None] >> (4 * np.arange(8, dtype=np.uint32))) & 0xF        # ..., q
-    assert np.isin(nib, [0x0, 0x2, 0xA]).all()
-    val = np.where(nib == 0x2, 1, np.where(nib == 0xA, -1, 0)).astype(np.int8)
+    assert np.isin(nib, [0x0, 0x4, 0xC]).all()
+    val = np.where(nib == 0x4, 1, np.where(nib == 0xC, -1, 0)).astype(np.int8)
     # the 2-bit stream's blocks, decoded with the library's own inverse: [octet, s, t] -> [16 rows, 16 cols]
     blocks = codes_o.reshape(-1, 2, 16, 4).transpose(0, 1, 3, 2).reshape(-1, 16)    # (octet, s, t) x n
     dec = np.empty((blocks.shape[0], 16, 16), np.int8)
