@@ -587,12 +587,22 @@ template <int MT, int WAVES>
 inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
     p.n_mtiles = (p.M + MT - 1) / MT;
     // Prefill tiles: one workgroup per CU (every workgroup stages a whole tile and the last units of its window
-    // leave waves idle, so few large ones: one round measured faster than two).  Decode tiles stage little: many small workgroups (about 12 per CU) so that the hardware
-    // dispatcher evens out the load, with a few units per wave when many layers share the launch and one unit
-    // per wave when a single matrix has to be spread over the whole chip.
+    // leave waves idle, so few large ones: one round measured faster than two).  Decode tiles stage little: many
+    // small workgroups (about 12 per CU) so that the hardware dispatcher evens out the load, with a few units
+    // per wave when many layers share the launch and one unit per wave when a single matrix has to be spread
+    // over the whole chip.
     const bool wide = (int64_t)layers * p.n_units >= 8 * 512;
-    const int upw = MT > 16 || !wide ? 1 : (MT <= 4 ? 2 : 4);
-        const int target = MT <= 16 ? 256 * 12 : 256;
+    int upw = 1;
+    if (MT <= 16 && wide) {
+        // up to 4 units per wave (fewer workgroups, each staging its tile once), but never so few workgroups that
+        // the launch cannot fill the chip's resident slots about once: a second, mostly empty round is what a
+        // count just above the slot count costs, and half-empty CUs what a count far below it costs
+        const int by_lds = (160 * 1024) / (tile_bytes(MT, p.Cb) + LDS_EXTRA), by_waves = 32 / WAVES;
+        const int64_t slots = 256 * (int64_t)(by_lds < by_waves ? by_lds : by_waves);
+        for (upw = 4; upw > 1; --upw)
+            if ((int64_t)layers * p.n_mtiles * ((p.n_units + WAVES * upw - 1) / (WAVES * upw)) * 10 >= slots * 9) break;
+    }
+    const int target = MT <= 16 ? 256 * 12 : 256;
     int split = (target + layers * p.n_mtiles - 1) / (layers * p.n_mtiles);
     const int max_split = (p.n_units + WAVES * upw - 1) / (WAVES * upw);
     split = split < 1 ? 1 : (split > max_split ? max_split : split);
