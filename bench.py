@@ -256,7 +256,7 @@ def main() -> None:
         out["looped_stack"] = {"ms": t, "mlp_calls": 48, "ms_per_mlp": t / 48, "tokens_per_s": TOKENS / (t * 1e-3),
                                "effective_tflops": fl / (t * 1e-3) / 1e12,
                                "frac_mfma": fl / (t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-                               "note": "includes one RMSNorm launch per MLP; rows follow Zipf(1.2) clipped to 5-60 %"}
+                               "note": "RMSNorm before every MLP, applied while gate_up stages x (no separate launch); rows follow Zipf(1.2) clipped to 5-60 %"}
         del specs, packs4
 
     # A plain device-to-device copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE counters when this

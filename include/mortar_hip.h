@@ -225,6 +225,18 @@ int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_e
 
 /* ---- RMSNorm ---------------------------------------------------------------------------------- */
 
+/* mortar_gateup_swiglu_bf16 with the RMSNorm in front of the MLP (attention.RMSNorm, morph/model/attention.py:133-141,
+ * called as mlp(norm_mlp(x)) in morph/model/mhc.py:249-250) applied to the rows of x while they are staged: the
+ * normalised activations never go to memory.  norm_w: bf16 [in_features], 16-byte aligned, or NULL for no weight.
+ * Same bits as mortar_rmsnorm_bf16 followed by mortar_gateup_swiglu_bf16.  The reference fuses the same norm into
+ * its dense ternary GEMV (X_MODE = 1, morph/kernels/triton/fused_decode_step.py:1149-1169).
+ * Available when mortar_norm_fusable(Cb) != 0 (in_features <= 2048 in one K segment); otherwise MORTAR_ERR_LIMIT. */
+int mortar_norm_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M,
+                                   int64_t ldx, const uint16_t *norm_w, float norm_eps, uint16_t *h, int64_t ldh,
+                                   const float *gates, int32_t n_clusters, const int32_t *tok_cnt,
+                                   const uint8_t *tok_list, void *stream);
+int mortar_norm_fusable(int32_t Cb);
+
 /* y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) per row; x, y bf16 [M, d]; w bf16 [d] or NULL (= 1). */
 int mortar_rmsnorm_bf16(const uint16_t *x, int64_t M, int32_t d, int64_t ldx, const uint16_t *w, float eps,
                         uint16_t *y, int64_t ldy, void *stream);

@@ -59,6 +59,40 @@ __device__ __forceinline__ uint32_t bf16_bits_rne(float f) { return bf16_pack2(f
 __device__ __forceinline__ float bf16_to_f32(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
 __device__ __forceinline__ float bf16r(float f) { return __builtin_bit_cast(float, bf16_pack2(0.f, f) & 0xffff0000u); }
 
+// ---- RMSNorm pieces shared by the stand-alone kernel and the fused staging of gate_up, so that both round alike.
+// A row is handled by one wavefront in 16-byte units (8 bf16): a lane adds the squares of its units in ascending
+// unit order (fused multiply-adds, low half-word first), the lanes meet in a xor butterfly.
+__device__ __forceinline__ float rms_sumsq8(u32x4_t u, float s) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lo = __builtin_bit_cast(float, u[j] << 16), hi = __builtin_bit_cast(float, u[j] & 0xffff0000u);
+        s = __builtin_fmaf(lo, lo, s);
+        s = __builtin_fmaf(hi, hi, s);
+    }
+    return s;
+}
+__device__ __forceinline__ float rms_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float rms_scale(float sumsq, int d, float eps) { return 1.0f / sqrtf(sumsq / (float)d + eps); }
+// bf16(bf16(x * r) * w) on 8 values; has_w = false leaves out the weight.
+__device__ __forceinline__ u32x4_t rms_apply8(u32x4_t u, float r, u32x4_t w, bool has_w) {
+    u32x4_t o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lo = __builtin_bit_cast(float, u[j] << 16), hi = __builtin_bit_cast(float, u[j] & 0xffff0000u);
+        uint32_t pk = bf16_pack2(lo * r, hi * r);
+        if (has_w) {
+            const float wl = __builtin_bit_cast(float, w[j] << 16), wh = __builtin_bit_cast(float, w[j] & 0xffff0000u);
+            pk = bf16_pack2(__builtin_bit_cast(float, pk << 16) * wl, __builtin_bit_cast(float, pk & 0xffff0000u) * wh);
+        }
+        o[j] = pk;
+    }
+    return o;
+}
+
 // silu in fp32 from a bf16-rounded input; the result is rounded to bf16 by the caller, which absorbs the
 // 1-ulp error of the hardware exp and reciprocal.
 __device__ __forceinline__ float silu_f32(float g) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)); }

@@ -127,10 +127,32 @@ extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *sc
     return dispatch(3, p, W, static_cast<hipStream_t>(stream));
 }
 
+namespace {
+int gateup_common(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M, int64_t ldx, bool norm,
+                  const uint16_t *norm_w, float norm_eps, uint16_t *h, int64_t ldh, const float *gates,
+                  int32_t n_clusters, const int32_t *tok_cnt, const uint8_t *tok_list, void *stream);
+}
+
 extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M,
                                          int64_t ldx, uint16_t *h, int64_t ldh, const float *gates,
                                          int32_t n_clusters, const int32_t *tok_cnt, const uint8_t *tok_list,
                                          void *stream) {
+    return gateup_common(W, sched, x, M, ldx, false, nullptr, 0.f, h, ldh, gates, n_clusters, tok_cnt, tok_list, stream);
+}
+
+extern "C" int mortar_norm_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x,
+                                              int64_t M, int64_t ldx, const uint16_t *norm_w, float norm_eps,
+                                              uint16_t *h, int64_t ldh, const float *gates, int32_t n_clusters,
+                                              const int32_t *tok_cnt, const uint8_t *tok_list, void *stream) {
+    return gateup_common(W, sched, x, M, ldx, true, norm_w, norm_eps, h, ldh, gates, n_clusters, tok_cnt, tok_list, stream);
+}
+
+extern "C" int mortar_norm_fusable(int32_t Cb) { return Cb > 0 && Cb <= NORM_MAX_CB && resident_mt(Cb) != 0; }
+
+namespace {
+int gateup_common(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M, int64_t ldx, bool norm,
+                  const uint16_t *norm_w, float norm_eps, uint16_t *h, int64_t ldh, const float *gates,
+                  int32_t n_clusters, const int32_t *tok_cnt, const uint8_t *tok_list, void *stream) {
     if (W && (W->Rb & 1)) return mortar_fail(MORTAR_ERR_ARG, "gateup: odd number of block-rows");
     const int64_t d_ff = W ? (int64_t)W->Rb * 8 : 0;
     int rc = check_common(W, x, M, ldx, h, ldh, d_ff);
@@ -138,6 +160,14 @@ extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *
     SpmmParams p;
     fill(p, W, sched, x, M, ldx, h, ldh);
     p.n_units = W->Rb / 2;
+    if (norm) {
+        if (!mortar_norm_fusable(W->Cb) || p.nseg != 1)
+            return mortar_fail(MORTAR_ERR_LIMIT, "gateup: the fused RMSNorm needs in_features <= %d in one K segment "
+                               "(mortar_norm_fusable() == 0: call mortar_rmsnorm_bf16 first)", NORM_MAX_CB * 16);
+        if (!(norm_eps >= 0.f)) return mortar_fail(MORTAR_ERR_ARG, "gateup: norm_eps must be >= 0");
+        if (reinterpret_cast<uintptr_t>(norm_w) & 15) return mortar_fail(MORTAR_ERR_ARG, "gateup: norm_w must be 16-byte aligned");
+        p.norm = 1; p.norm_eps = norm_eps; p.norm_w = norm_w;
+    }
     if (gates) {
         if (n_clusters <= 0 || d_ff % n_clusters || (d_ff / n_clusters) % 4)
             return mortar_fail(MORTAR_ERR_ARG, "gateup: d_ff / n_clusters must be a whole multiple of 4");
@@ -154,6 +184,7 @@ extern "C" int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *
     }
     return dispatch(1, p, W, static_cast<hipStream_t>(stream));
 }
+}  // namespace
 
 // ---- layer-batched small-M launches ---------------------------------------------------------------------
 

@@ -129,6 +129,25 @@ __global__ void __launch_bounds__(256) route_flags_kernel(const float *gates, in
     }
 }
 
+// One wavefront per row, in 16-byte units, with the summation order and rounding steps of the fused form in
+// the gate_up staging (rms_* in mortar_device.h): both give the same bits.
+__global__ void __launch_bounds__(256) rmsnorm_rows_kernel(const uint16_t *x, int64_t M, int d, int64_t ldx,
+                                                            const uint16_t *w, float eps, uint16_t *y, int64_t ldy) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const u32x4_t *xp = reinterpret_cast<const u32x4_t *>(x + row * ldx);
+    const u32x4_t *wp = reinterpret_cast<const u32x4_t *>(w);
+    u32x4_t *yp = reinterpret_cast<u32x4_t *>(y + row * ldy);
+    const int nch = d / 8;
+    float ss = 0.f;
+    for (int ch = lane; ch < nch; ch += 64) ss = rms_sumsq8(xp[ch], ss);
+    const float r = rms_scale(rms_wave_sum(ss), d, eps);
+    for (int ch = lane; ch < nch; ch += 64)
+        yp[ch] = rms_apply8(xp[ch], r, w ? wp[ch] : u32x4_t{0u, 0u, 0u, 0u}, w != nullptr);
+}
+
+// Any d / alignment: element-wise (its sums are ordered differently; no fused counterpart exists for such rows).
 __global__ void __launch_bounds__(256) rmsnorm_kernel(const uint16_t *x, int64_t M, int d, int64_t ldx,
                                                        const uint16_t *w, float eps, uint16_t *y, int64_t ldy) {
     __shared__ float red[4];
@@ -202,7 +221,13 @@ extern "C" int mortar_rmsnorm_bf16(const uint16_t *x, int64_t M, int32_t d, int6
                                    float eps, uint16_t *y, int64_t ldy, void *stream) {
     if (!x || !y) return mortar_fail(MORTAR_ERR_ARG, "rmsnorm: null pointer");
     if (M <= 0 || d <= 0 || ldx < d || ldy < d) return mortar_fail(MORTAR_ERR_ARG, "rmsnorm: bad shape");
-    hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)M), dim3(256), 0, static_cast<hipStream_t>(stream), x, M, d,
-                       ldx, w, eps, y, ldy);
+    const bool units = d % 8 == 0 && ldx % 8 == 0 && ldy % 8 == 0 &&
+                       ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(w)) & 15) == 0;
+    if (units)
+        hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           x, M, d, ldx, w, eps, y, ldy);
+    else
+        hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)M), dim3(256), 0, static_cast<hipStream_t>(stream), x, M, d,
+                           ldx, w, eps, y, ldy);
     return check_launch("rmsnorm");
 }

@@ -34,7 +34,10 @@ struct SpmmParams {
     int n_mtiles, n_split;    // token tiles; workgroups that share one token tile
     int seg_cb, nseg;         // K segments of the octet stream
     int xcd_map;              // 1: workgroup ids are renumbered per XCD (grid padded to a multiple of 8)
+    int norm;                 // 1: rows of x are RMS-normalised while they are staged (single-segment tiles only)
+    float norm_eps;
     int pad_[3];
+    const uint16_t *norm_w;   // bf16 [in_features] weight of that norm, or null for none
 };
 
 // Device-side view of the launch parameters: the pointers carry the global address space in their type, so
@@ -51,7 +54,9 @@ struct SpmmView {
     const MORTAR_GLOBAL int32_t *tok_cnt;
     const MORTAR_GLOBAL uint8_t *tok_list;
     int64_t ldx, ldy;
-    int n_units, Cb, M, n_clusters, cluster_size, n_mtiles, n_split, seg_cb, nseg, Rb, xcd_map;
+    int n_units, Cb, M, n_clusters, cluster_size, n_mtiles, n_split, seg_cb, nseg, Rb, xcd_map, norm;
+    float norm_eps;
+    const MORTAR_GLOBAL u32x4_t *norm_w;
 };
 static_assert(sizeof(SpmmParams) % 16 == 0, "table entries are copied in 16-byte words");
 // Entry i of a parameter table in device memory (uniform address: scalar loads).
@@ -73,6 +78,7 @@ __device__ __forceinline__ SpmmView mortar_view(const SpmmParams &q) {
     v.tok_cnt = (const MORTAR_GLOBAL int32_t *)q.tok_cnt; v.tok_list = (const MORTAR_GLOBAL uint8_t *)q.tok_list;
     v.ldx = q.ldx; v.ldy = q.ldy; v.n_units = q.n_units; v.Cb = q.Cb; v.M = q.M; v.n_clusters = q.n_clusters;
     v.cluster_size = q.cluster_size; v.n_mtiles = q.n_mtiles; v.n_split = q.n_split; v.seg_cb = q.seg_cb; v.nseg = q.nseg; v.Rb = q.Rb; v.xcd_map = q.xcd_map;
+    v.norm = q.norm; v.norm_eps = q.norm_eps; v.norm_w = (const MORTAR_GLOBAL u32x4_t *)q.norm_w;
     return v;
 }
 
@@ -84,6 +90,7 @@ constexpr int LDS_PAD = 16;              // 16-byte units past the tile that idl
 // LDS bytes of a token tile of MT tokens and ncb block-columns (token stride MT + 1 keeps reads conflict-free).
 constexpr int tile_bytes(int mt, int ncb) { return (2 * ncb * (mt + 1) + LDS_PAD) * 16; }
 constexpr int LDS_EXTRA = 16;            // bytes after the tile: the resident kernel's unit counter
+constexpr int NORM_MAX_CB = 128;         // block-columns up to which a row fits the registers of the staging wave
 
 // Lane k of every 16-lane row broadcast to the whole row (DPP row_newbcast); K must fold to a constant.
 template <int K>
@@ -225,6 +232,56 @@ __device__ __forceinline__ void mortar_stage_tile(const SpmmView &p, uint4 *lx, 
     }
 }
 
+// The same staging with the rows RMS-normalised on the way (gate_up with the block's norm folded in): a wave holds
+// a whole row in registers (at most 256 units: the host admits the fused norm for ncb <= NORM_MAX_CB only), two
+// rows at a time, adds the squares, and writes bf16(bf16(x * r) * w).
+template <int MT, int WAVES>
+__device__ __forceinline__ void mortar_stage_tile_norm(const SpmmView &p, uint4 *lx, int m0, int ncb, int tid) {
+    constexpr int LDM = MT + 1, CU = 4, RU = 2;
+    const int nch = 2 * ncb;
+    const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const MORTAR_GLOBAL char *xt = p.x + (int64_t)m0 * p.ldx * 2;
+    const bool has_w = p.norm_w != nullptr;
+    u32x4_t wv[CU];
+#pragma unroll
+    for (int b = 0; b < CU; ++b) {
+        int ch = b * 64 + lane;
+        ch = ch < nch ? ch : nch - 1;
+        wv[b] = has_w ? p.norm_w[ch] : u32x4_t{0u, 0u, 0u, 0u};
+    }
+    for (int r0 = wave; r0 <= rlast; r0 += WAVES * RU) {
+        u32x4_t v[RU][CU];
+#pragma unroll
+        for (int a = 0; a < RU; ++a) {
+            int row = r0 + a * WAVES;
+            row = row < rlast ? row : rlast;
+            const MORTAR_GLOBAL char *xr = xt + (int64_t)row * p.ldx * 2;
+#pragma unroll
+            for (int b = 0; b < CU; ++b) {
+                int ch = b * 64 + lane;
+                ch = ch < nch ? ch : nch - 1;
+                v[a][b] = *(const MORTAR_GLOBAL u32x4_t *)(xr + (uint32_t)ch * 16u);
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < RU; ++a) {
+            const int row = r0 + a * WAVES;
+            float ss = 0.f;
+#pragma unroll
+            for (int b = 0; b < CU; ++b)
+                if (b * 64 + lane < nch) ss = rms_sumsq8(v[a][b], ss);
+            const float r = rms_scale(rms_wave_sum(ss), 8 * nch, p.norm_eps);
+#pragma unroll
+            for (int b = 0; b < CU; ++b) {
+                const int ch = b * 64 + lane;
+                if (row <= rlast && ch < nch)
+                    reinterpret_cast<u32x4_t *>(lx)[ch * LDM + row] = rms_apply8(v[a][b], r, wv[b], has_w);
+            }
+        }
+    }
+}
+
 // Epilogue of one row unit for the 16 tokens of sub-tile `ms`: the lane holds D[4g+v][token].
 template <int NACC>
 __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, int tok, int g, bool has_gates,
@@ -292,7 +349,8 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
     int pos = base + wave;
     u32x4_t d0 = mortar_part_desc<NACC>(p, pos, 0, 0);
 
-    mortar_stage_tile<MT, WAVES, false>(p, lx, m0, 0, p.Cb, tid);
+    if (NACC == 2 && p.norm) mortar_stage_tile_norm<MT, WAVES>(p, lx, m0, p.Cb, tid);      // gate_up may carry the norm
+    else mortar_stage_tile<MT, WAVES, false>(p, lx, m0, 0, p.Cb, tid);
     __syncthreads();
 
     while (pos < u_end) {
@@ -502,7 +560,8 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
     }
     const int nsub = ROUTED ? (cnt + 15) >> 4 : MSUB;
 
-    mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, 0, p.Cb, tid);
+    if (NACC == 2 && !MASKED && p.norm) mortar_stage_tile_norm<MT, WAVES>(p, lx, m0, p.Cb, tid);
+    else mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, 0, p.Cb, tid);
     __syncthreads();
 
     f32x4_t acc[NACC][MSUB];

@@ -47,8 +47,13 @@ class MortarDecodeMLP:
     @torch.no_grad()
     def __call__(self, x: Tensor, gates: Tensor | None = None) -> Tensor:
         B = x.shape[0]
-        xn = ops.rmsnorm(x.reshape(B, -1).to(torch.bfloat16), self.norm_weight, self.eps)
         rt = getattr(self.mlp, "router", None)
+        if (gates is not None or rt is None) and ops.norm_fusable(self.Mgu):
+            # no router to feed: the norm rides on the gate_up launch (the reference folds it into its dense
+            # ternary GEMV the same way, fused_decode_step.py X_MODE = 1)
+            return self.mlp(x.reshape(B, -1).to(torch.bfloat16), iter_idx=self.iter_idx, gates=gates,
+                            norm=(self.norm_weight, self.eps)).view(B, 1, -1)
+        xn = ops.rmsnorm(x.reshape(B, -1).to(torch.bfloat16), self.norm_weight, self.eps)
         if gates is None and rt is not None:
             gates = rt(xn, iter_idx=self.iter_idx)[0].reshape(B, -1).float().contiguous()
         tile = ops.route_tile(self.Mgu, B) if gates is not None and (self.d_ff // gates.shape[-1]) % 16 == 0 else 0
@@ -72,5 +77,5 @@ def looped_core_forward(mlps, x: Tensor, n_iters: int, norm_weights=None, eps: f
     for t in range(n_iters):
         for i, m in enumerate(mlps):
             w = norm_weights[i] if norm_weights is not None else None
-            x = m(ops.rmsnorm(x, w, eps), iter_idx=t)
+            x = m(x, iter_idx=t, norm=(w, eps))
     return x

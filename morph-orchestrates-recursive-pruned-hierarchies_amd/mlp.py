@@ -74,9 +74,24 @@ class _SwiGLUMortar(nn.Module):
     def _carved(self) -> bool:
         return self.gate_up._cms._mortar and self.down._cms._mortar
 
-    def forward(self, x: Tensor, iter_idx: int = 0, gates: Tensor | None = None) -> Tensor:
+    def forward(self, x: Tensor, iter_idx: int = 0, gates: Tensor | None = None, norm: tuple | None = None) -> Tensor:
         """x [..., d_model] -> [..., d_model].  ``gates`` overrides the router output (fp32 [N, n_clusters]);
-        it exists so that a caller which already evaluated the router (or holds seeded logits) can feed it."""
+        it exists so that a caller which already evaluated the router (or holds seeded logits) can feed it.
+        ``norm`` = (weight or None, eps): x is the activation BEFORE the block's RMSNorm (norm_mlp) and the norm is
+        applied here, inside the gate_up launch when the matrix allows it; same result as mlp(rmsnorm(x))."""
+        if norm is not None:
+            fused = (self._carved() and x.is_cuda and (self.router is None or gates is not None)
+                     and ops.norm_fusable(self.gate_up._cms.mortar_pack()))
+            if not fused:
+                nw, eps = norm
+                if self._carved() and x.is_cuda:
+                    x = ops.rmsnorm(x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16), nw, eps)
+                else:
+                    xn = (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype)
+                    x = xn * nw.to(x.dtype) if nw is not None else xn
+                norm = None
+            elif norm[0] is not None and norm[0].dtype != torch.bfloat16:
+                norm = (norm[0].to(torch.bfloat16), norm[1])
         if not self._carved():
             gu = self.gate_up(x)
             gate, up = gu.chunk(2, dim=-1)
@@ -116,10 +131,10 @@ class _SwiGLUMortar(nn.Module):
             if active is None:
                 active = (gates > 0).to(torch.uint8)
             route = ops.remoe_route(active, tile)
-            h = ops.gateup_swiglu(xb, Wgu, gates=gates, route=route)
+            h = ops.gateup_swiglu(xb, Wgu, gates=gates, route=route, norm=norm)
             y = ops.spmm(h, Wdn, active=active)
         else:
-            h = ops.gateup_swiglu(xb, Wgu, gates=gates)
+            h = ops.gateup_swiglu(xb, Wgu, gates=gates, norm=norm)
             y = ops.spmm(h, Wdn)
         if y.dtype != x.dtype:
             y = y.to(x.dtype)

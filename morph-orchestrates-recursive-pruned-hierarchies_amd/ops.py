@@ -67,10 +67,17 @@ def spmm(x: Tensor, W: MortarPack, out: Tensor | None = None, active: Tensor | N
     return y
 
 
+def norm_fusable(W: MortarPack) -> bool:
+    """True if gateup_swiglu can apply the RMSNorm in front of the MLP while it stages x (in_features <= 2048)."""
+    return bool(_lib.lib().mortar_norm_fusable(W.Cb)) and W.nseg == 1
+
+
 def gateup_swiglu(x: Tensor, W: MortarPack, gates: Tensor | None = None, route: tuple | None = None,
-                  out: Tensor | None = None) -> Tensor:
+                  out: Tensor | None = None, norm: tuple | None = None) -> Tensor:
     """h[M, d_ff] = silu(gate) * up [* gates per cluster] with gate_up = W [2*d_ff, d_model].
-    route = (tok_cnt, tok_list) from remoe_route switches on active-tile skipping."""
+    route = (tok_cnt, tok_list) from remoe_route switches on active-tile skipping.
+    norm = (weight bf16 [d_model] or None, eps): x is RMS-normalised on the way in (same bits as rmsnorm() first);
+    needs norm_fusable(W)."""
     x = _bf16_2d(x, "gateup_swiglu")
     M = x.shape[0]
     if W.Rb % 2:
@@ -87,6 +94,16 @@ def gateup_swiglu(x: Tensor, W: MortarPack, gates: Tensor | None = None, route: 
             raise TypeError("gateup_swiglu: gates must be a contiguous float32 [M, n_clusters] tensor")
         ncl = gates.shape[1]
     cnt, lst = route if route is not None else (None, None)
+    if norm is not None:
+        nw, eps = norm
+        if nw is not None:
+            if nw.dtype != torch.bfloat16 or nw.dim() != 1 or nw.shape[0] != W.in_features or not nw.is_contiguous():
+                raise TypeError("gateup_swiglu: norm weight must be a contiguous bfloat16 [in_features] tensor")
+            _need_gpu(nw, "gateup_swiglu")
+        rc = _lib.lib().mortar_norm_gateup_swiglu_bf16(W.ref, _p(W.sched(2)), _p(x), M, x.stride(0), _p(nw), float(eps),
+                                                       _p(h), h.stride(0), _p(gates), ncl, _p(cnt), _p(lst), _stream(x))
+        _lib.check(rc, "mortar_norm_gateup_swiglu_bf16")
+        return h
     rc = _lib.lib().mortar_gateup_swiglu_bf16(W.ref, _p(W.sched(2)), _p(x), M, x.stride(0), _p(h),
                                               h.stride(0), _p(gates), ncl, _p(cnt), _p(lst), _stream(x))
     _lib.check(rc, "mortar_gateup_swiglu_bf16")

@@ -379,6 +379,49 @@ def test_rmsnorm(dev):
     assert_close_bf16(to_np(y).reshape(37, 2048), O.rmsnorm(x), "rmsnorm unit weight", ulps=2)
 
 
+@pytest.mark.parametrize("d_model,M", [(256, 1), (256, 3), (256, 16), (256, 40), (256, 200), (2048, 1), (2048, 5),
+                                       (2048, 200), (16 * 47, 130)])
+def test_norm_fused_into_gate_up(dev, d_model, M):
+    """RMSNorm applied while gate_up stages x gives the bits of rmsnorm() followed by gateup_swiglu(), for the decode
+    tiles (part-split and small workgroups), the 64- and 32-token prefill tiles, with and without weight, gated and
+    routed; and agrees with the oracle."""
+    d_ff = 16 * 24
+    spec = synth.synth_mlp(d_model, d_ff, 0.25, seed=60, zipf_s=1.2)
+    x = O.bf16_round(synth.synth_x(M, d_model, 61) * 2.5)
+    w = O.bf16_round(1.0 + 0.1 * synth.synth_x(1, d_model, 62)[0])
+    Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    assert ops.norm_fusable(Wgu)
+    xd, wd = to_dev(x, dev), to_dev(w, dev)
+    gates, active = ops.remoe_gates(torch.from_numpy(synth.synth_logits(M, d_ff // 16, 63)).to(dev), 6)
+    for nw, eps in ((wd, 1e-6), (None, 1e-5)):
+        xn = ops.rmsnorm(xd, nw, eps)
+        assert torch.equal(ops.gateup_swiglu(xd, Wgu, norm=(nw, eps)), ops.gateup_swiglu(xn, Wgu))
+        assert torch.equal(ops.gateup_swiglu(xd, Wgu, gates=gates, norm=(nw, eps)), ops.gateup_swiglu(xn, Wgu, gates=gates))
+        tile = ops.route_tile(Wgu, M)
+        route = ops.remoe_route(active, tile)
+        a, b = torch.zeros((M, d_ff), dtype=torch.bfloat16, device=dev), torch.zeros((M, d_ff), dtype=torch.bfloat16, device=dev)
+        ops.gateup_swiglu(xd, Wgu, gates=gates, route=route, norm=(nw, eps), out=a)
+        ops.gateup_swiglu(xn, Wgu, gates=gates, route=route, out=b)
+        assert torch.equal(a, b)
+    ref = O.swiglu_mlp(O.rmsnorm(x, w), spec["gate_up"], spec["down"])
+    h = ops.gateup_swiglu(xd, Wgu, norm=(wd, 1e-6))
+    assert_close_bf16(to_np(h), ref["h"], "h of normalised x", ulps=8)
+    mlp = synth.mlp_module(spec, dev)
+    assert torch.equal(mlp(xd, norm=(wd, 1e-6)), mlp(ops.rmsnorm(xd, wd, 1e-6)))
+
+
+def test_norm_fusion_limits(dev):
+    """Matrices too wide for the fused norm are refused by the C-ABI; the module falls back to a separate launch."""
+    spec = synth.synth_mlp(16 * 130, 16 * 8, 0.25, seed=64)
+    Wgu = synth.to_pack(spec["gate_up"], dev)
+    xd = to_dev(synth.synth_x(20, 16 * 130, 65), dev)
+    assert not ops.norm_fusable(Wgu)
+    with pytest.raises(ValueError, match="fused RMSNorm"):
+        ops.gateup_swiglu(xd, Wgu, norm=(None, 1e-6))
+    mlp = synth.mlp_module(spec, dev)
+    assert torch.equal(mlp(xd, norm=(None, 1e-6)), mlp(ops.rmsnorm(xd, None, 1e-6)))
+
+
 def test_looped_core_stack_small(dev):
     """BASELINE config 4 call pattern at reduced size: shared blocks x iterations, RMS-normalised input, Zipf rows."""
     d_model, d_ff, M = 256, 16 * 44, 150
