@@ -165,6 +165,37 @@ def main() -> None:
             gdec[f"b{B}"] = {"us_per_mlp": t * 1e3, "tokens_per_s": B / (t * 1e-3),
                              "algorithmic_GBps": (wbytes + B * (2 * D_MODEL + 2 * D_FF) * 2) / (t * 1e-3) / 1e9}
         out["decode_graph"] = gdec
+        # ---- routed decode: RMSNorm -> router (two-launch HIP front end) -> tile lists -> routed gate_up -> masked down.
+        # 16 clusters of 352 neurons, 4 x 4 product keys, k = 8: the reference's deploy router shape (fused_router.py).
+        from mortar_amd.engine import MortarDecodeMLP
+        rmlp = synth.mlp_module(spec, dev)
+        rmlp.enable_routing(n_clusters=16, activation_ratio=0.5, n_sub_keys=4)
+        rdec_mlp = MortarDecodeMLP(rmlp)
+        rt = rmlp.router
+        rdec = {}
+        with torch.no_grad():
+            for B in (1, 16):
+                xb = x[:B].contiguous()
+                xn = ops.rmsnorm(xb)
+                t_fused = event_time_ms(lambda: rt.route(xn), 100, 10)
+                t_torch = event_time_ms(lambda: ops.remoe_gates(rt.group_logits(xn, 0), rt.activation_k), 100, 10)
+                t_eager = event_time_ms(lambda: rdec_mlp(xb), 100, 10)
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    for _ in range(3):
+                        rdec_mlp(xb)
+                torch.cuda.current_stream().wait_stream(side)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for _ in range(16):
+                        rdec_mlp(xb)
+                t_graph = event_time_ms(graph.replay, 20, 3) / 16
+                rdec[f"b{B}"] = {"us_per_mlp_graph": t_graph * 1e3, "us_per_mlp_eager": t_eager * 1e3,
+                                 "router_us_eager": t_fused * 1e3, "router_us_eager_torch_ops": t_torch * 1e3}
+                del graph
+        out["decode_routed"] = rdec
+        del rmlp, rdec_mlp
         # ---- decode, cold: stream distinct weight sets so that the Infinity Cache cannot hold them --------
         n_sets = 160                                                 # 160 x 2.37 MB = 379 MB > 256 MB
         packs = []

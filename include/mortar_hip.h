@@ -182,6 +182,24 @@ int mortar_remoe_route(const uint8_t *active, int64_t M, int32_t n, int32_t tile
 int mortar_route_flags(const float *gates, int64_t B, int32_t n_clusters, int64_t ldg, int32_t d_ff,
                        int32_t *row_act, int64_t ldr, int32_t *col_act, int64_t ldc, void *stream);
 
+/* Decode-side router front end + gating tail in two launches, for 1..64 tokens: TileRouter.forward steps 1-8
+ * (morph/model/routing.py:181-284); the reference's fused form is morph/kernels/triton/fused_router.py:43-140
+ * (projection GEMV + one tail kernel, B == 1).
+ *   qv = x Wq^T + iter_vec;  q = LayerNorm(qv; ln_w, ln_b, ln_eps);  sa = q[:d/2] Ka^T;  sb = q[d/2:] Kb^T
+ *   logits[g] = sa[p / nsk] + sb[p % nsk] + bias[g],  p = g mod nsk^2   (nsk^2 == n: the 1:1 product map of
+ *   fused_router.py; nsk^2 < n: the reference's wrap, routing.py:227-230; nsk^2 > n is refused: MORTAR_ERR_LIMIT)
+ *   gates / active as mortar_remoe_gates.
+ * x: [B, d] bf16 (x_is_f32 = 0) or fp32 (1), row stride ldx; wq fp32 [d, d] row-major (query_proj.weight);
+ * iter_vec fp32 [d] (iter_embed[it]) or NULL; ln_w, ln_b fp32 [d]; ka, kb fp32 [nsk, d/2]; bias fp32 [n].
+ * qv: caller workspace fp32 [B, d].  logits_out fp32 [B, n] or NULL; gates fp32 [B, n]; active uint8 [B, n] or NULL.
+ * All arithmetic fp32 (the deploy router stays fp32, fused_router.py:26-28); sums are ordered differently from a
+ * library GEMM, so gates agree with the eager path to rounding (the reference's own gate: active mismatch 0,
+ * max gate error 2e-6, away from exact ties at the threshold). */
+int mortar_router_bf16(const void *x, int32_t x_is_f32, int64_t B, int32_t d, int64_t ldx, const float *wq,
+                       const float *iter_vec, const float *ln_w, const float *ln_b, float ln_eps, const float *ka,
+                       const float *kb, int32_t nsk, const float *bias, int32_t n, int32_t k, float *qv,
+                       float *logits_out, float *gates, uint8_t *active, void *stream);
+
 /* ---- decode (M <= 64) ------------------------------------------------------------------------ */
 
 /* mortar_spmm_bf16 / mortar_gateup_swiglu_bf16 / mortar_spmm_bf16_masked serve decode batches directly: for

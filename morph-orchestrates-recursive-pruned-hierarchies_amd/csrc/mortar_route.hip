@@ -27,16 +27,12 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// One wavefront per token.  The k-th largest logit is found exactly by an MSB-first radix select on
-// order-preserving keys: for each bit the wave counts (ballot + popcount) the keys >= the candidate
+// Gating tail of one token on one wavefront.  The k-th largest logit is found exactly by an MSB-first radix
+// select on order-preserving keys: for each bit the wave counts (ballot + popcount) the keys >= the candidate
 // prefix.  Ties need no special care: the result is a VALUE, and the gate rule is `logit > kth`.
+// `lp` may point to global memory or LDS; gates / active are this token's output rows.
 template <int MAXPL>      // logits per lane this instantiation holds: n <= 64 * MAXPL
-__global__ void __launch_bounds__(256) remoe_gates_kernel(const float *logits, int64_t M, int n, int k,
-                                                           float *gates, uint8_t *active) {
-    const int lane = threadIdx.x & 63;
-    const int64_t tok = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (tok >= M) return;
-    const float *lp = logits + tok * n;
+__device__ __forceinline__ void remoe_gates_wave(const float *lp, int n, int k, float *gates, uint8_t *active, int lane) {
     float v[MAXPL];
     uint32_t key[MAXPL];
 #pragma unroll
@@ -76,10 +72,181 @@ __global__ void __launch_bounds__(256) remoe_gates_kernel(const float *logits, i
         const int idx = i * 64 + lane;
         if (idx < n) {
             const float gv = g0[i] * t;
-            gates[tok * n + idx] = gv;
-            if (active) active[tok * n + idx] = gv > 0.f;
+            gates[idx] = gv;
+            if (active) active[idx] = gv > 0.f;
         }
     }
+}
+
+template <int MAXPL>
+__global__ void __launch_bounds__(256) remoe_gates_kernel(const float *logits, int64_t M, int n, int k,
+                                                           float *gates, uint8_t *active) {
+    const int64_t tok = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tok >= M) return;
+    remoe_gates_wave<MAXPL>(logits + tok * n, n, k, gates + tok * n, active ? active + tok * n : nullptr, threadIdx.x & 63);
+}
+
+// ---- decode-side router front end (TileRouter.forward steps 1-4 in front of the gating tail) -------------------
+// Launch 1: qv[b, o] = sum_i x[b, i] * Wq[o, i] + iter_vec[o].  One wavefront per output row o; the row of Wq is
+// read once per group of TB tokens (16-byte loads, fp32), x comes from L2.
+template <int TB, bool XF32>
+__global__ void __launch_bounds__(256) router_project_kernel(const void *xv, int B, int d, int64_t ldx, const float *wq,
+                                                              const float *iter_vec, float *qv) {
+    const int lane = threadIdx.x & 63;
+    const int o = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (o >= d) return;
+    const float4 *wr = reinterpret_cast<const float4 *>(wq + (int64_t)o * d);
+    const float bias = iter_vec ? iter_vec[o] : 0.f;
+    const int n4 = d / 4;
+    for (int b0 = 0; b0 < B; b0 += TB) {
+        float acc[TB];
+#pragma unroll
+        for (int t = 0; t < TB; ++t) acc[t] = 0.f;
+        // four 16-byte loads of the weight row in flight per lane (the row is read from HBM exactly once per token
+        // group; the loop is latency-bound otherwise)
+        for (int i0 = lane; i0 < n4; i0 += 256) {
+            float4 w[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i4 = i0 + 64 * u;
+                w[u] = i4 < n4 ? wr[i4] : float4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i4 = i0 + 64 * u < n4 ? i0 + 64 * u : n4 - 1;
+#pragma unroll
+                for (int t = 0; t < TB; ++t) {
+                    const int b = b0 + t < B ? b0 + t : B - 1;
+                    float x0, x1, x2, x3;
+                    if (XF32) {
+                        const float4 xx = reinterpret_cast<const float4 *>(static_cast<const float *>(xv) + (int64_t)b * ldx)[i4];
+                        x0 = xx.x; x1 = xx.y; x2 = xx.z; x3 = xx.w;
+                    } else {
+                        const uint2 xx = reinterpret_cast<const uint2 *>(static_cast<const uint16_t *>(xv) + (int64_t)b * ldx)[i4];
+                        x0 = __builtin_bit_cast(float, xx.x << 16); x1 = __builtin_bit_cast(float, xx.x & 0xffff0000u);
+                        x2 = __builtin_bit_cast(float, xx.y << 16); x3 = __builtin_bit_cast(float, xx.y & 0xffff0000u);
+                    }
+                    acc[t] = __builtin_fmaf(x3, w[u].w, __builtin_fmaf(x2, w[u].z, __builtin_fmaf(x1, w[u].y, __builtin_fmaf(x0, w[u].x, acc[t]))));
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TB; ++t) {
+            const float s = wave_sum(acc[t]);
+            if (lane == 0 && b0 + t < B) qv[(int64_t)(b0 + t) * d + o] = s + bias;
+        }
+    }
+}
+
+__device__ __forceinline__ float block_sum256(float v, float *red) {      // red: 4 floats of LDS; all 256 threads call
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+
+// Launch 2, one workgroup per token: LayerNorm(qv) -> sub-key scores of the two query halves -> product-key logits
+// (+ group bias) -> gating tail.  P = nsk * nsk products map to the n groups one to one (P == n) or wrap (P < n).
+// PRE (d <= 2048, nsk <= 4): every parameter a thread needs (LayerNorm weights, its slices of the sub-keys, its
+// bias) is fetched into registers before the first reduction, so the kernel pays one memory round trip instead of
+// one per phase.
+template <int MAXPL, bool PRE>
+__global__ void __launch_bounds__(256) router_tail_kernel(const float *qv, int d, const float *ln_w, const float *ln_b,
+                                                           float ln_eps, const float *ka, const float *kb, int nsk,
+                                                           const float *bias, int n, int k, float *logits_out,
+                                                           float *gates, uint8_t *active) {
+    extern __shared__ __attribute__((aligned(16))) float sm[];       // qn[d] | s[2 * nsk] | logits[n] | red[4]
+    float *qn = sm, *sc = sm + d, *lg = sc + 2 * nsk, *red = lg + n;
+    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float *q = qv + (int64_t)b * d;
+    const int d2 = d / 2, n4 = d2 / 4;          // d % 8 == 0: both halves are whole float4 runs
+    constexpr int QE = 8, DPW = 2, KU = 4;      // PRE: entries per thread, sub-key dots per wave, float4 per lane and dot
+    float qe[QE], lw[QE], lbv[QE];
+    float4 kreg[DPW][KU];
+    if (PRE) {
+#pragma unroll
+        for (int j = 0; j < QE; ++j) {
+            const int i = tid + 256 * j, ic = i < d ? i : d - 1;
+            qe[j] = q[ic]; lw[j] = ln_w[ic]; lbv[j] = ln_b[ic];
+        }
+#pragma unroll
+        for (int cc = 0; cc < DPW; ++cc) {
+            int c = wave + 4 * cc;
+            c = c < 2 * nsk ? c : 2 * nsk - 1;
+            const float4 *kr = reinterpret_cast<const float4 *>(c < nsk ? ka + (int64_t)c * d2 : kb + (int64_t)(c - nsk) * d2);
+#pragma unroll
+            for (int u = 0; u < KU; ++u) kreg[cc][u] = lane + 64 * u < n4 ? kr[lane + 64 * u] : float4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    float s = 0.f;
+    if (PRE) {
+#pragma unroll
+        for (int j = 0; j < QE; ++j) s += tid + 256 * j < d ? qe[j] : 0.f;
+    } else {
+        for (int i = tid; i < d; i += 256) { const float t = q[i]; qn[i] = t; s += t; }      // a thread re-reads its own entries
+    }
+    const float mean = block_sum256(s, red) / (float)d;
+    float v = 0.f;
+    if (PRE) {
+#pragma unroll
+        for (int j = 0; j < QE; ++j) { const float c = tid + 256 * j < d ? qe[j] - mean : 0.f; v = __builtin_fmaf(c, c, v); }
+    } else {
+        for (int i = tid; i < d; i += 256) { const float c = qn[i] - mean; v = __builtin_fmaf(c, c, v); }
+    }
+    const float rstd = 1.0f / sqrtf(block_sum256(v, red) / (float)d + ln_eps);
+    if (PRE) {
+#pragma unroll
+        for (int j = 0; j < QE; ++j)
+            if (tid + 256 * j < d) qn[tid + 256 * j] = (qe[j] - mean) * rstd * lw[j] + lbv[j];
+    } else {
+        for (int i = tid; i < d; i += 256) qn[i] = (qn[i] - mean) * rstd * ln_w[i] + ln_b[i];
+    }
+    __syncthreads();
+    if (PRE) {
+#pragma unroll
+        for (int cc = 0; cc < DPW; ++cc) {
+            const int c = wave + 4 * cc;
+            const float4 *qh = reinterpret_cast<const float4 *>(c < nsk ? qn : qn + d2);
+            float a = 0.f;
+#pragma unroll
+            for (int u = 0; u < KU; ++u) {
+                const float4 qq = qh[lane + 64 * u < n4 ? lane + 64 * u : n4 - 1];
+                a = __builtin_fmaf(qq.w, kreg[cc][u].w, __builtin_fmaf(qq.z, kreg[cc][u].z, __builtin_fmaf(qq.y, kreg[cc][u].y, __builtin_fmaf(qq.x, kreg[cc][u].x, a))));
+            }
+            a = wave_sum(a);
+            if (lane == 0 && c < 2 * nsk) sc[c] = a;
+        }
+    } else {
+        for (int c = wave; c < 2 * nsk; c += 4) {
+            const float4 *kr = reinterpret_cast<const float4 *>(c < nsk ? ka + (int64_t)c * d2 : kb + (int64_t)(c - nsk) * d2);
+            const float4 *qh = reinterpret_cast<const float4 *>(c < nsk ? qn : qn + d2);
+            float a = 0.f;
+            for (int i0 = lane; i0 < n4; i0 += 256) {
+                float4 kv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) kv[u] = i0 + 64 * u < n4 ? kr[i0 + 64 * u] : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const float4 qq = qh[i0 + 64 * u < n4 ? i0 + 64 * u : n4 - 1];
+                    a = __builtin_fmaf(qq.w, kv[u].w, __builtin_fmaf(qq.z, kv[u].z, __builtin_fmaf(qq.y, kv[u].y, __builtin_fmaf(qq.x, kv[u].x, a))));
+                }
+            }
+            a = wave_sum(a);
+            if (lane == 0) sc[c] = a;
+        }
+    }
+    __syncthreads();
+    const int P = nsk * nsk;
+    for (int g = tid; g < n; g += 256) {
+        const int pr = g % P;
+        const float l = (sc[pr / nsk] + sc[nsk + pr % nsk]) + bias[g];
+        lg[g] = l;
+        if (logits_out) logits_out[(int64_t)b * n + g] = l;
+    }
+    __syncthreads();
+    if (wave == 0)
+        remoe_gates_wave<MAXPL>(lg, n, k, gates + (int64_t)b * n, active ? active + (int64_t)b * n : nullptr, lane);
 }
 
 // Workgroup = (token tile, chunk of 64 clusters).  The tile's active bytes for the chunk are staged in LDS
@@ -193,6 +360,49 @@ extern "C" int mortar_remoe_gates(const float *logits, int64_t M, int32_t n, int
     else if (npl <= 8) hipLaunchKernelGGL(remoe_gates_kernel<8>, grid, block, 0, st, logits, M, n, k, gates, active);
     else hipLaunchKernelGGL(remoe_gates_kernel<16>, grid, block, 0, st, logits, M, n, k, gates, active);
     return check_launch("remoe_gates");
+}
+
+extern "C" int mortar_router_bf16(const void *x, int32_t x_is_f32, int64_t B, int32_t d, int64_t ldx, const float *wq,
+                                  const float *iter_vec, const float *ln_w, const float *ln_b, float ln_eps,
+                                  const float *ka, const float *kb, int32_t nsk, const float *bias, int32_t n,
+                                  int32_t k, float *qv, float *logits_out, float *gates, uint8_t *active,
+                                  void *stream) {
+    if (!x || !wq || !ln_w || !ln_b || !ka || !kb || !bias || !qv || !gates)
+        return mortar_fail(MORTAR_ERR_ARG, "router: null pointer");
+    if (B <= 0 || B > 64) return mortar_fail(MORTAR_ERR_LIMIT, "router: the fused front end serves 1..64 tokens (got %lld)", (long long)B);
+    if (d <= 0 || d % 8 || d > 8192 || ldx < d || ldx % (x_is_f32 ? 4 : 8))
+        return mortar_fail(MORTAR_ERR_ARG, "router: d must be a multiple of 8 up to 8192 and ldx >= d, 16-byte aligned rows");
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wq) | reinterpret_cast<uintptr_t>(ka) | reinterpret_cast<uintptr_t>(kb)) & 15)
+        return mortar_fail(MORTAR_ERR_ARG, "router: x, wq, ka and kb must be 16-byte aligned");
+    if (n <= 0 || k <= 0 || nsk <= 0) return mortar_fail(MORTAR_ERR_ARG, "router: n, k, nsk must be positive");
+    if (n > 64 * MAXPL_LIMIT) return mortar_fail(MORTAR_ERR_LIMIT, "router: n=%d exceeds %d clusters", n, 64 * MAXPL_LIMIT);
+    if ((int64_t)nsk * nsk > n)
+        return mortar_fail(MORTAR_ERR_LIMIT, "router: %d x %d product keys exceed the %d groups (the reference ranks the "
+                           "products with topk there; not served by the fused front end)", nsk, nsk, n);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 pg((unsigned)((d + 3) / 4)), blk(256);
+#define MORTAR_PROJ(TB, F) hipLaunchKernelGGL((router_project_kernel<TB, F>), pg, blk, 0, st, x, (int)B, d, ldx, wq, iter_vec, qv)
+    if (x_is_f32) { if (B == 1) MORTAR_PROJ(1, true); else if (B <= 4) MORTAR_PROJ(4, true); else MORTAR_PROJ(8, true); }
+    else { if (B == 1) MORTAR_PROJ(1, false); else if (B <= 4) MORTAR_PROJ(4, false); else MORTAR_PROJ(8, false); }
+#undef MORTAR_PROJ
+    int rc = check_launch("router projection");
+    if (rc) return rc;
+    const size_t smem = (size_t)(d + 2 * nsk + n + 4) * sizeof(float);
+    const dim3 tg((unsigned)B);
+    const int npl = (n + 63) / 64;
+    const bool pre = d <= 2048 && nsk <= 4;
+#define MORTAR_TAIL(PL) do { if (pre) hipLaunchKernelGGL((router_tail_kernel<PL, true>), tg, blk, smem, st, qv, d, ln_w, ln_b, ln_eps, \
+                                      ka, kb, nsk, bias, n, k, logits_out, gates, active); \
+        else hipLaunchKernelGGL((router_tail_kernel<PL, false>), tg, blk, smem, st, qv, d, ln_w, ln_b, ln_eps, ka, kb, nsk, \
+                                bias, n, k, logits_out, gates, active); } while (0)
+    if (npl <= 1) MORTAR_TAIL(1);
+    else if (npl <= 2) MORTAR_TAIL(2);
+    else if (npl <= 4) MORTAR_TAIL(4);
+    else if (npl <= 6) MORTAR_TAIL(6);
+    else if (npl <= 8) MORTAR_TAIL(8);
+    else MORTAR_TAIL(16);
+#undef MORTAR_TAIL
+    return check_launch("router tail");
 }
 
 extern "C" int mortar_remoe_route(const uint8_t *active, int64_t M, int32_t n, int32_t tile, int32_t *tok_cnt,

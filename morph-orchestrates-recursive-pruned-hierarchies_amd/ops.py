@@ -128,6 +128,36 @@ def remoe_gates(logits: Tensor, k: int) -> tuple[Tensor, Tensor]:
     return gates, active
 
 
+ROUTER_MAX_TOKENS = 64
+
+
+def router_fused(x: Tensor, wq: Tensor, iter_vec: Tensor | None, ln_w: Tensor, ln_b: Tensor, ln_eps: float,
+                 ka: Tensor, kb: Tensor, bias: Tensor, k: int, want_logits: bool = False):
+    """Decode-side TileRouter in two launches (projection, then LayerNorm + product keys + gating tail).
+    x [B <= 64, d] bf16 or fp32; all parameters fp32.  -> (gates fp32 [B, n], active uint8 [B, n][, logits])."""
+    _need_gpu(x, "router_fused")
+    if x.dim() != 2 or x.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("router_fused: x must be a 2-D bfloat16 or float32 tensor")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    B, d = x.shape
+    n, nsk = bias.numel(), ka.shape[0]
+    for name, t, shp in (("wq", wq, (d, d)), ("ln_w", ln_w, (d,)), ("ln_b", ln_b, (d,)), ("ka", ka, (nsk, d // 2)),
+                         ("kb", kb, (nsk, d // 2)), ("bias", bias, (n,))) + ((("iter_vec", iter_vec, (d,)),) if iter_vec is not None else ()):
+        if t.dtype != torch.float32 or tuple(t.shape) != shp or not t.is_contiguous() or t.device != x.device:
+            raise TypeError(f"router_fused: {name} must be a contiguous float32 {shp} tensor on {x.device}")
+    qv = torch.empty((B, d), dtype=torch.float32, device=x.device)
+    gates = torch.empty((B, n), dtype=torch.float32, device=x.device)
+    active = torch.empty((B, n), dtype=torch.uint8, device=x.device)
+    logits = torch.empty((B, n), dtype=torch.float32, device=x.device) if want_logits else None
+    if B:
+        rc = _lib.lib().mortar_router_bf16(_p(x), int(x.dtype == torch.float32), B, d, x.stride(0), _p(wq), _p(iter_vec),
+                                           _p(ln_w), _p(ln_b), float(ln_eps), _p(ka), _p(kb), nsk, _p(bias), n, int(k),
+                                           _p(qv), _p(logits), _p(gates), _p(active), _stream(x))
+        _lib.check(rc, "mortar_router_bf16")
+    return (gates, active, logits) if want_logits else (gates, active)
+
+
 def route_tile(W: MortarPack, M: int = 0) -> int:
     """Token tile of the routed gate_up kernels for M rows against this matrix (the tile remoe_route must use);
     0 when the matrix is too wide for routed skipping (use the dense gated call)."""

@@ -2,8 +2,9 @@
 
 Interface mirror of the reference's morph/model/routing.py (same parameters, forward signature, outputs).
 The gating tail (steps 5-8: k-th largest threshold, ReLU, normalise to sum k, active mask) runs in the HIP
-kernel for inference; the query projection / LayerNorm / sub-key scores in front of it are library GEMMs
-through torch.  With autograd enabled the tail stays in differentiable torch ops.
+kernel for inference.  For decode-sized calls (up to 64 rows) the front end (query projection, LayerNorm, sub-key
+scores, product-key logits) runs in HIP as well, two launches in all; larger calls use library GEMMs through torch.
+With autograd enabled the tail stays in differentiable torch ops.
 """
 from __future__ import annotations
 
@@ -63,12 +64,39 @@ class TileRouter(nn.Module):
         idx = torch.arange(self.n_tile_groups, device=x_flat.device) % n_products
         return ps[:, idx] + self.group_bias.unsqueeze(0)
 
+    def _fused_ok(self, x_flat: Tensor) -> bool:
+        """Decode-sized inference calls on the GPU with fp32 router parameters go through the two-launch HIP router."""
+        return (x_flat.is_cuda and 0 < x_flat.shape[0] <= ops.ROUTER_MAX_TOKENS and not torch.is_grad_enabled()
+                and x_flat.dtype in (torch.bfloat16, torch.float32) and self.query_proj.weight.dtype == torch.float32
+                and self.n_sub_keys * self.n_sub_keys <= self.n_tile_groups and self.d_model % 8 == 0
+                and self.n_tile_groups <= 1024)
+
+    @torch.no_grad()
+    def route(self, x_flat: Tensor, iter_idx: int = 0) -> Tuple[Tensor, Tensor]:
+        """Inference-only routing of [N, d_model] rows: (gates fp32 [N, n], active uint8 [N, n]) and nothing else (no
+        load statistics, no auxiliary loss), as the reference's decode engine calls its fused router
+        (morph/kernels/triton/fused_router.py:100-140).  Two launches for decode-sized N, torch GEMMs + the gating
+        kernel otherwise."""
+        if self._fused_ok(x_flat):
+            it = max(0, min(int(iter_idx), self.n_iters - 1))
+            return ops.router_fused(x_flat, self.query_proj.weight, self.iter_embed[it], self.query_norm.weight,
+                                    self.query_norm.bias, self.query_norm.eps, self.sub_keys_a, self.sub_keys_b,
+                                    self.group_bias, self.activation_k)
+        return gates_from_logits(self.group_logits(x_flat, iter_idx), self.activation_k)
+
     def forward(self, x: Tensor, iter_idx: int = 0) -> Tuple[Tensor, Tensor]:
         orig_shape = x.shape
         x_flat = x.reshape(-1, orig_shape[-1])
-        logits = self.group_logits(x_flat, iter_idx)
         k = self.activation_k
-        if torch.is_grad_enabled() and logits.requires_grad:
+        if self._fused_ok(x_flat):
+            gates, active = self.route(x_flat, iter_idx)
+            self.last_active = active
+            logits = None
+        else:
+            logits = self.group_logits(x_flat, iter_idx)
+        if logits is None:
+            pass
+        elif torch.is_grad_enabled() and logits.requires_grad:
             if k < self.n_tile_groups:
                 kth = logits.topk(k, dim=-1).values[:, -1:]
                 gates = F.relu(logits - kth)

@@ -264,6 +264,28 @@ def kth_largest(logits: np.ndarray, k: int) -> np.ndarray:
     return np.sort(logits, axis=-1)[:, ::-1][:, k - 1]
 
 
+def router_logits(x, wq, iter_vec, ln_w, ln_b, ln_eps, ka, kb, bias) -> np.ndarray:
+    """TileRouter.forward steps 1-4, morph/model/routing.py:181-230 (float64 here): q = LayerNorm(x Wq^T + iter_vec);
+    sa = q[:, :d/2] Ka^T, sb = q[:, d/2:] Kb^T; product scores ps[a*nsk + b] = sa[a] + sb[b]; group logits = ps + bias
+    when nsk^2 == n (:205-211), ps[g mod nsk^2] + bias when nsk^2 < n (:227-230).  LayerNorm uses the biased variance
+    (torch.nn.LayerNorm).  The nsk^2 > n branch (topk over products, :212-222) is not restated."""
+    x = np.asarray(x, np.float64)
+    qv = x @ np.asarray(wq, np.float64).T
+    if iter_vec is not None:
+        qv = qv + np.asarray(iter_vec, np.float64)
+    mean = qv.mean(axis=-1, keepdims=True)
+    var = ((qv - mean) ** 2).mean(axis=-1, keepdims=True)
+    q = (qv - mean) / np.sqrt(var + ln_eps) * np.asarray(ln_w, np.float64) + np.asarray(ln_b, np.float64)
+    d2 = q.shape[1] // 2
+    sa = q[:, :d2] @ np.asarray(ka, np.float64).T
+    sb = q[:, d2:] @ np.asarray(kb, np.float64).T
+    nsk = sa.shape[1]
+    ps = (sa[:, :, None] + sb[:, None, :]).reshape(x.shape[0], nsk * nsk)
+    n = np.asarray(bias).size
+    assert nsk * nsk <= n
+    return ps[:, np.arange(n) % (nsk * nsk)] + np.asarray(bias, np.float64)
+
+
 def remoe_gates(logits: np.ndarray, k: int):
     """TileRouter.forward steps 5-8, morph/model/routing.py:232-284:
     kth = k-th largest value; g0 = relu(logits - kth); gates = g0 * (k / clamp(sum g0, 1e-6));

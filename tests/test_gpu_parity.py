@@ -220,6 +220,55 @@ def test_remoe_gates_ties_and_edges(dev):
         ops.remoe_gates(torch.zeros(2, 2000, device=dev), 5)
 
 
+@pytest.mark.parametrize("B,d,nsk,n,xdt", [(1, 256, 4, 16, "bf16"), (5, 768, 4, 16, "bf16"), (16, 2048, 8, 64, "bf16"),
+                                          (3, 2048, 18, 352, "f32"), (64, 512, 4, 16, "f32"), (2, 264, 3, 9, "bf16")])
+def test_fused_router_front_end(dev, B, d, nsk, n, xdt):
+    """Two-launch decode router (projection; LayerNorm + product keys + gating tail) against the float64 oracle:
+    logits to fp32 rounding, the active set exactly except where a logit sits within rounding of the threshold,
+    gates to 1e-4; and against the torch ops of TileRouter.group_logits + the stand-alone gates kernel."""
+    rng = np.random.default_rng(70 + B)
+    k = max(1, n // 4)
+    x = O.bf16_round(rng.standard_normal((B, d)).astype(np.float32)) if xdt == "bf16" else rng.standard_normal((B, d)).astype(np.float32)
+    wq = (rng.standard_normal((d, d)) / np.sqrt(d)).astype(np.float32); it = (0.1 * rng.standard_normal(d)).astype(np.float32)
+    lw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32); lb = (0.1 * rng.standard_normal(d)).astype(np.float32)
+    ka = (rng.standard_normal((nsk, d // 2)) / np.sqrt(d // 2)).astype(np.float32)
+    kb = (rng.standard_normal((nsk, d // 2)) / np.sqrt(d // 2)).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(n)).astype(np.float32)
+    T = lambda a: torch.from_numpy(a).to(dev)
+    xd = to_dev(x, dev) if xdt == "bf16" else T(x)
+    gates, active, logits = ops.router_fused(xd, T(wq), T(it), T(lw), T(lb), 1e-5, T(ka), T(kb), T(bias), k, want_logits=True)
+    ref = O.router_logits(x, wq, it, lw, lb, 1e-5, ka, kb, bias)
+    np.testing.assert_allclose(logits.cpu().numpy(), ref, rtol=0, atol=2e-5 * max(1.0, np.abs(ref).max()))
+    g_ref, a_ref = O.remoe_gates(ref.astype(np.float32), k)
+    kth = O.kth_largest(ref.astype(np.float32), k)[:, None] if k < n else np.full((B, 1), -np.inf)
+    clear = np.abs(ref - kth) > 1e-4                       # logits not within rounding of the threshold
+    assert np.array_equal(active.cpu().numpy().astype(bool)[clear], a_ref[clear])
+    np.testing.assert_allclose(gates.cpu().numpy(), g_ref, rtol=0, atol=2e-4)
+    # the fused tail equals the stand-alone gates kernel on the fused logits, bit for bit
+    g2, a2 = ops.remoe_gates(logits, k)
+    assert torch.equal(g2, gates) and torch.equal(a2, active)
+    # module path: TileRouter picks the fused router for decode-sized inference calls
+    from mortar_amd.routing import TileRouter
+    rt = TileRouter(n, d, activation_ratio=k / n, n_sub_keys=nsk, n_iters=2).to(dev)
+    with torch.no_grad():
+        rt.query_proj.weight.copy_(T(wq)); rt.iter_embed[1].copy_(T(it)); rt.query_norm.weight.copy_(T(lw))
+        rt.query_norm.bias.copy_(T(lb)); rt.sub_keys_a.copy_(T(ka)); rt.sub_keys_b.copy_(T(kb)); rt.group_bias.copy_(T(bias))
+        assert rt.activation_k == k and rt._fused_ok(xd)
+        gm, _ = rt(xd, iter_idx=1)
+        assert torch.equal(gm, gates)
+        lt = rt.group_logits(xd, 1)                       # eager torch ops (library GEMMs)
+    np.testing.assert_allclose(lt.cpu().numpy(), ref, rtol=0, atol=2e-5 * max(1.0, np.abs(ref).max()))
+
+
+def test_fused_router_limits(dev):
+    T = lambda *s: torch.zeros(s, dtype=torch.float32, device=dev)
+    x = torch.zeros((65, 64), dtype=torch.bfloat16, device=dev)
+    with pytest.raises(ValueError, match="1..64 tokens"):
+        ops.router_fused(x, T(64, 64), None, T(64), T(64), 1e-5, T(4, 32), T(4, 32), T(16), 4)
+    with pytest.raises(ValueError, match="product keys exceed"):
+        ops.router_fused(x[:2], T(64, 64), None, T(64), T(64), 1e-5, T(5, 32), T(5, 32), T(16), 4)
+
+
 def test_route_flags_exact(dev):
     for ncl, d_ff in ((352, 5632), (16, 2048), (256, 2048), (44, 5632)):
         lg = synth.synth_logits(5, ncl, ncl)
