@@ -78,6 +78,7 @@ def main() -> None:
         sys.exit("bench.py: this build runs on ONE GPU (the path shards by tokens with replicated weights; "
                  "no multi-GPU code is part of it). Use --gpus 1.")
 
+    import numpy as np
     import torch
     import mortar_amd
     from mortar_amd import ops, synth
@@ -252,6 +253,31 @@ def main() -> None:
         n_act = int(ops.remoe_gates(logits, TOP_K)[1].sum())
         out["routed_prefill"] = {"ms": t, "tokens_per_s": TOKENS / (t * 1e-3),
                                  "active_fraction": n_act / (TOKENS * N_CLUSTERS)}
+        # ---- the reference's own deploy format: ONE scale per matrix (pack_mortar_ternary), same shapes ----------
+        spec_u = {k: dict(spec[k]) for k in ("gate_up", "down")}
+        spec_u["gate_up"]["scales"], spec_u["down"]["scales"] = np.float32(0.05), np.float32(0.03)
+        Ugu, Udn = synth.to_pack(spec_u["gate_up"], dev), synth.to_pack(spec_u["down"], dev)
+
+        def ustep():
+            ops.gateup_swiglu(x, Ugu, out=h)
+            ops.spmm(h, Udn, out=y)
+        t = event_time_ms(ustep, it)
+        xb = x[:1].contiguous()
+        upacks = [(Ugu, Udn) if i == 0 else (Ugu.clone_weights(), Udn.clone_weights()) for i in range(n_sets)]
+        hs = [torch.empty((1, D_FF), dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
+        ys = [torch.empty((1, D_MODEL), dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
+        up = ops.LayerStack([g for g, _ in upacks], [xb] * n_sets, hs, swiglu=True)
+        dn = ops.LayerStack([d for _, d in upacks], hs, ys, swiglu=False)
+        t_s = event_time_ms(up.run, 10, 2) + event_time_ms(dn.run, 10, 2)
+        b_s = n_sets * (wbytes - 4 * (Wgu.nnz + Wdn.nnz) + (2 * D_MODEL + 2 * D_FF) * 2)     # no scale per block to read
+        out["per_tensor_scale"] = {"prefill_ms": t, "prefill_tokens_per_s": TOKENS / (t * 1e-3),
+                                   "prefill_effective_tflops": (flops_gu + flops_dn) / (t * 1e-3) / 1e12,
+                                   "decode_stack_b1_us_per_mlp": t_s * 1e3 / n_sets,
+                                   "decode_stack_b1_GBps": b_s / (t_s * 1e-3) / 1e9,
+                                   "decode_stack_b1_frac_hbm": b_s / (t_s * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                   "note": "blocks multiplied as +-2 / 0, fp32 sums scaled once (scale-after-sum, as the "
+                                           "reference's decode kernel); the headline uses per-block scales"}
+        del up, dn, hs, ys, upacks, Ugu, Udn
 
     if not args.no_extras:
         # ---- BASELINE config 1: base-width MLP (d_model 768, d_ff 2048), 4 x 4096 tokens ---------------------

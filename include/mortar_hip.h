@@ -67,6 +67,12 @@ typedef struct {
     const uint32_t *codes4_o;
     int32_t Rb, Cb, nnz;
     int32_t seg_cb;   /* block-columns per K segment of the octet stream (>= Cb: one segment) */
+    float uniform_scale;   /* != 0: every block has this (bf16-representable) scale, the reference's per-tensor
+                              mortar_scale (deploy_quant.py:344-374); from mortar_uniform_scale_host.  The kernels then
+                              multiply +-2 / 0 blocks and scale the fp32 sums once, as the reference's decode kernel
+                              does (fused_decode_step.py:1441-1443), instead of scaling every block's weights.
+                              0: per-block scales (always valid, also for a uniform matrix). */
+    int32_t reserved_;
 } mortar_bcsr_t;
 
 const char *mortar_last_error(void);
@@ -82,6 +88,10 @@ int mortar_abi_version(void);
  * (0 is allowed and zeroes the block). */
 int mortar_encode_blocks_host(const uint8_t *packed, int64_t nnz, const float *scale, int64_t scale_count,
                               uint32_t *codes_out, uint32_t *sdup_out);
+
+/* The scale shared by all blocks, from the sdup patterns of mortar_encode_blocks_host: *scale_out = that bf16 value
+ * as float, or 0 if the blocks differ (or the scale is 0).  Put it into mortar_bcsr_t.uniform_scale. */
+int mortar_uniform_scale_host(const uint32_t *sdup, int64_t nnz, float *scale_out);
 
 /* Inverse of the code part (for tests): device-layout dwords -> int8 codes [nnz,16,16]. */
 int mortar_decode_blocks_host(const uint32_t *codes, int64_t nnz, int8_t *codes_out);

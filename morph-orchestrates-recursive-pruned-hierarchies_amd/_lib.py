@@ -18,13 +18,14 @@ class BcsrStruct(C.Structure):
     _fields_ = [("codes", c_vp), ("sdup", c_vp), ("col", c_vp), ("row_ptr", c_vp), ("row_desc", c_vp),
                 ("codes_o", c_vp), ("sd_o", c_vp), ("col_o", c_vp), ("codes4_o", c_vp),
                 ("Rb", c_i32), ("Cb", c_i32), ("nnz", c_i32),
-                ("seg_cb", c_i32)]
+                ("seg_cb", c_i32), ("uniform_scale", c_f32), ("reserved_", c_i32)]
 
 
 _SIGS = {
     "mortar_last_error": (C.c_char_p, []),
     "mortar_abi_version": (C.c_int, []),
     "mortar_encode_blocks_host": (C.c_int, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp]),
+    "mortar_uniform_scale_host": (C.c_int, [c_vp, c_i64, c_vp]),
     "mortar_decode_blocks_host": (C.c_int, [c_vp, c_i64, c_vp]),
     "mortar_octet_layout_host": (c_i64, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "mortar_fp4_stream_host": (C.c_int, [c_vp, c_i64, c_vp]),

@@ -38,6 +38,15 @@ __device__ __forceinline__ u32x4_t mortar_scale4(uint32_t nib, uint32_t sd) {
 __device__ __forceinline__ u32x4_t mortar_unpack8(uint32_t t, uint32_t sd) {
     return mortar_scale4(t & 0xCCCCCCCCu, sd);
 }
+// The conversions alone: bf16 +-2 / 0 for the eight nibbles (matrices with one scale, applied after the sums).
+__device__ __forceinline__ u32x4_t mortar_nib4(uint32_t nib) {
+    u32x4_t r;
+    r[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, 1.0f, 0));
+    r[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, 1.0f, 1));
+    r[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, 1.0f, 2));
+    r[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, 1.0f, 3));
+    return r;
+}
 
 // Same result from the 4-bit stream: `t` holds the lane's 8 codes as FP4 nibbles {sign, non-zero, 0, 0} already,
 // byte i = {column 2i (low nibble), column 2i+1 (high nibble)}.

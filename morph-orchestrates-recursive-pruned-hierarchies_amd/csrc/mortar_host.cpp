@@ -78,6 +78,17 @@ extern "C" int mortar_encode_blocks_host(const uint8_t *packed, int64_t nnz, con
     return MORTAR_OK;
 }
 
+extern "C" int mortar_uniform_scale_host(const uint32_t *sdup, int64_t nnz, float *scale_out) {
+    if (!sdup || !scale_out || nnz <= 0) return mortar_fail(MORTAR_ERR_ARG, "uniform_scale: bad argument");
+    *scale_out = 0.f;
+    for (int64_t j = 1; j < nnz; ++j)
+        if (sdup[j] != sdup[0]) return MORTAR_OK;
+    if (sdup[0] == 0u) return MORTAR_OK;
+    const uint32_t bits = ((sdup[0] & 0xffffu) + 0x0400u) << 16;     // undo the exponent step: bf16 bits of the scale
+    memcpy(scale_out, &bits, 4);
+    return MORTAR_OK;
+}
+
 extern "C" int mortar_decode_blocks_host(const uint32_t *codes, int64_t nnz, int8_t *codes_out) {
     if (!codes || !codes_out) return mortar_fail(MORTAR_ERR_ARG, "decode_blocks: null pointer");
     for (int64_t j = 0; j < nnz; ++j)

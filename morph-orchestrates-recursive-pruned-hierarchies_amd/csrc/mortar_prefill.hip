@@ -39,6 +39,7 @@ void fill(SpmmParams &p, const mortar_bcsr_t *W, const int32_t *sched, const uin
     p.Cb = W->Cb;
     p.x = x; p.ldx = ldx; p.M = (int)M; p.y = y; p.ldy = ldy;
     p.n_clusters = 1; p.cluster_size = 1 << 30;
+    p.uscale = 0.5f * W->uniform_scale;
 }
 
 // Token tile of the resident prefill kernel for a matrix with Cb block-columns (0 = does not fit).
@@ -50,35 +51,37 @@ int resident_mt(int Cb) {
 
 // prefill tiles: 16 wavefronts (4 per SIMD) for the 32-token tile, 8 for the 64-token tile (measured: a 96-token
 // tile of a narrow matrix leaves only two waves per SIMD and is slower)
-template <int NACC, bool ROUTED, bool FP4>
+template <int NACC, bool ROUTED, int CODE>
 int launch_resident_any(SpmmParams &p, hipStream_t st) {
     switch (resident_mt(p.Cb)) {
-        case 64: return mortar_launch_resident<64, NACC, ROUTED, 8, false, FP4>(p, nullptr, 1, st);
-        default: return mortar_launch_resident<32, NACC, ROUTED, 16, false, FP4>(p, nullptr, 1, st);
+        case 64: return mortar_launch_resident<64, NACC, ROUTED, 8, false, CODE>(p, nullptr, 1, st);
+        default: return mortar_launch_resident<32, NACC, ROUTED, 16, false, CODE>(p, nullptr, 1, st);
     }
 }
 
 constexpr int SEG_WAVES = 16, SEG_UPW = 4;
 
-template <bool FP4>
+template <int CODE>
 int dispatch_prefill(int kind, SpmmParams &p, hipStream_t st) {
     switch (kind) {
         case 0:
-            if (p.nseg == 1) return launch_resident_any<1, false, FP4>(p, st);
-            return mortar_launch_segmented<32, 1, false, SEG_WAVES, SEG_UPW, false, FP4>(p, nullptr, 1, st);
+            if (p.nseg == 1) return launch_resident_any<1, false, CODE>(p, st);
+            return mortar_launch_segmented<32, 1, false, SEG_WAVES, SEG_UPW, false, CODE>(p, nullptr, 1, st);
         case 1:
-            if (p.nseg == 1) return launch_resident_any<2, false, FP4>(p, st);
-            return mortar_launch_segmented<32, 2, false, SEG_WAVES, 2, false, FP4>(p, nullptr, 1, st);
+            if (p.nseg == 1) return launch_resident_any<2, false, CODE>(p, st);
+            return mortar_launch_segmented<32, 2, false, SEG_WAVES, 2, false, CODE>(p, nullptr, 1, st);
         case 2:
-            return launch_resident_any<2, true, FP4>(p, st);
+            return launch_resident_any<2, true, CODE>(p, st);
         default:
-            return mortar_launch_segmented<32, 1, true, SEG_WAVES, SEG_UPW, false, FP4>(p, nullptr, 1, st);
+            return mortar_launch_segmented<32, 1, true, SEG_WAVES, SEG_UPW, false, CODE>(p, nullptr, 1, st);
     }
 }
 
 // kind: 0 spmm, 1 gate_up + SwiGLU, 2 routed gate_up + SwiGLU, 3 spmm with an input mask.
 // Prefill-sized launches read the 4-bit code stream when the matrix carries one (cheaper unpack: one conversion
 // per register instead of shift + mask); decode-sized launches always stream the 2-bit codes (half the bytes).
+// A matrix with one scale (uniform_scale != 0) runs the kernels that multiply +-2 / 0 blocks and scale the
+// accumulators once (decode-sized launches always, prefill-sized ones through the 4-bit stream).
 int dispatch(int kind, SpmmParams &p, const mortar_bcsr_t *W, hipStream_t st) {
     if (p.M <= MORTAR_SMALLM_MAX) {
         const int rc = mortar_smallm_launch(kind, p, nullptr, 1, st);
@@ -86,9 +89,11 @@ int dispatch(int kind, SpmmParams &p, const mortar_bcsr_t *W, hipStream_t st) {
     }
     if (W->codes4_o) {
         p.codes_o = reinterpret_cast<const u32x4_t *>(W->codes4_o);
-        return dispatch_prefill<true>(kind, p, st);
+        if (p.uscale != 0.f) return dispatch_prefill<CODE_4BIT | CODE_UNIFORM>(kind, p, st);
+        return dispatch_prefill<CODE_4BIT>(kind, p, st);
     }
-    return dispatch_prefill<false>(kind, p, st);
+    p.uscale = 0.f;      // per-block path: the 2-bit prefill kernels multiply every block by its own pattern
+    return dispatch_prefill<CODE_2BIT>(kind, p, st);
 }
 
 }  // namespace
@@ -203,6 +208,9 @@ extern "C" int mortar_stack_prepare(int32_t swiglu, int32_t n_layers, const mort
         if (W[l].Rb != W[0].Rb || W[l].Cb != W[0].Cb || W[l].seg_cb != W[0].seg_cb)
             return mortar_fail(MORTAR_ERR_ARG, "stack_prepare: layer %d differs in shape from layer 0", l);
         if (swiglu && (W[l].Rb & 1)) return mortar_fail(MORTAR_ERR_ARG, "stack_prepare: odd number of block-rows");
+        if ((W[l].uniform_scale != 0.f) != (W[0].uniform_scale != 0.f))
+            return mortar_fail(MORTAR_ERR_ARG, "stack_prepare: layer %d and layer 0 differ in having a uniform scale "
+                               "(set uniform_scale = 0 on all layers to run them together)", l);
         const int64_t out_cols = swiglu ? (int64_t)W[l].Rb * 8 : (int64_t)W[l].Rb * 16;
         int rc = check_common(&W[l], x[l], M, ldx, y[l], ldy, out_cols);
         if (rc) return rc;

@@ -9,22 +9,22 @@
 
 namespace {
 
-template <int MT, int WAVES>
+template <int MT, int WAVES, int CODE>
 int launch_kind(int kind, bool resident, SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     if (table) {      // layer-batched: plain products and unrouted gate_up only
-        if (resident && kind == 0) return mortar_launch_resident<MT, 1, false, WAVES, true>(p, table, layers, st);
-        if (resident && kind == 1) return mortar_launch_resident<MT, 2, false, WAVES, true>(p, table, layers, st);
-        if (!resident && kind == 0 && MT == 16) return mortar_launch_segmented<16, 1, false, WAVES, 1, true>(p, table, layers, st);
+        if (resident && kind == 0) return mortar_launch_resident<MT, 1, false, WAVES, true, CODE>(p, table, layers, st);
+        if (resident && kind == 1) return mortar_launch_resident<MT, 2, false, WAVES, true, CODE>(p, table, layers, st);
+        if (!resident && kind == 0 && MT == 16) return mortar_launch_segmented<16, 1, false, WAVES, 1, true, CODE>(p, table, layers, st);
     } else if (resident) {
         switch (kind) {
-            case 0: return mortar_launch_resident<MT, 1, false, WAVES>(p, nullptr, 1, st);
-            case 1: return mortar_launch_resident<MT, 2, false, WAVES>(p, nullptr, 1, st);
-            case 2: return mortar_launch_resident<MT, 2, true, WAVES>(p, nullptr, 1, st);
+            case 0: return mortar_launch_resident<MT, 1, false, WAVES, false, CODE>(p, nullptr, 1, st);
+            case 1: return mortar_launch_resident<MT, 2, false, WAVES, false, CODE>(p, nullptr, 1, st);
+            case 2: return mortar_launch_resident<MT, 2, true, WAVES, false, CODE>(p, nullptr, 1, st);
         }
     } else if (MT == 16) {
         switch (kind) {
-            case 0: return mortar_launch_segmented<16, 1, false, WAVES, 1>(p, nullptr, 1, st);
-            case 3: return mortar_launch_segmented<16, 1, true, WAVES, 1>(p, nullptr, 1, st);
+            case 0: return mortar_launch_segmented<16, 1, false, WAVES, 1, false, CODE>(p, nullptr, 1, st);
+            case 3: return mortar_launch_segmented<16, 1, true, WAVES, 1, false, CODE>(p, nullptr, 1, st);
         }
     }
     return mortar_fail(MORTAR_ERR_ARG, "small-M dispatch: no kernel for kind %d", kind);
@@ -55,45 +55,52 @@ static int pick_waves(int t, const SpmmParams &p, int layers) {
 }
 
 // Part-split launch for one matrix: PW waves per unit, PW = 4, 3 or 2 dividing the unit's part count.
-template <int MT>
+template <int MT, int CODE>
 static int launch_partsplit(int kind, SpmmParams &p, hipStream_t st) {
     const int nacc = (kind == 0 || kind == 3) ? 1 : 2, nparts = p.nseg * nacc;
     const int pw = nparts % 4 == 0 ? 4 : (nparts % 3 == 0 ? 3 : (nparts % 2 == 0 ? 2 : 0));
     if (pw == 0 || tile_bytes(MT, p.Cb) + 16 * 2 * 1024 > 160 * 1024) return -1;
     switch (kind * 10 + pw) {
-        case 2: return mortar_launch_partsplit<MT, 1, false, false, 2, 4>(p, st);
-        case 3: return mortar_launch_partsplit<MT, 1, false, false, 3, 4>(p, st);
-        case 4: return mortar_launch_partsplit<MT, 1, false, false, 4, 4>(p, st);
-        case 12: return mortar_launch_partsplit<MT, 2, false, false, 2, 4>(p, st);
-        case 13: return mortar_launch_partsplit<MT, 2, false, false, 3, 4>(p, st);
-        case 14: return mortar_launch_partsplit<MT, 2, false, false, 4, 4>(p, st);
-        case 22: return mortar_launch_partsplit<MT, 2, true, false, 2, 4>(p, st);
-        case 23: return mortar_launch_partsplit<MT, 2, true, false, 3, 4>(p, st);
-        case 24: return mortar_launch_partsplit<MT, 2, true, false, 4, 4>(p, st);
-        case 32: return mortar_launch_partsplit<MT, 1, false, true, 2, 4>(p, st);
-        case 33: return mortar_launch_partsplit<MT, 1, false, true, 3, 4>(p, st);
-        case 34: return mortar_launch_partsplit<MT, 1, false, true, 4, 4>(p, st);
+        case 2: return mortar_launch_partsplit<MT, 1, false, false, 2, 4, CODE>(p, st);
+        case 3: return mortar_launch_partsplit<MT, 1, false, false, 3, 4, CODE>(p, st);
+        case 4: return mortar_launch_partsplit<MT, 1, false, false, 4, 4, CODE>(p, st);
+        case 12: return mortar_launch_partsplit<MT, 2, false, false, 2, 4, CODE>(p, st);
+        case 13: return mortar_launch_partsplit<MT, 2, false, false, 3, 4, CODE>(p, st);
+        case 14: return mortar_launch_partsplit<MT, 2, false, false, 4, 4, CODE>(p, st);
+        case 22: return mortar_launch_partsplit<MT, 2, true, false, 2, 4, CODE>(p, st);
+        case 23: return mortar_launch_partsplit<MT, 2, true, false, 3, 4, CODE>(p, st);
+        case 24: return mortar_launch_partsplit<MT, 2, true, false, 4, 4, CODE>(p, st);
+        case 32: return mortar_launch_partsplit<MT, 1, false, true, 2, 4, CODE>(p, st);
+        case 33: return mortar_launch_partsplit<MT, 1, false, true, 3, 4, CODE>(p, st);
+        case 34: return mortar_launch_partsplit<MT, 1, false, true, 4, 4, CODE>(p, st);
     }
     return -1;
 }
 
-int mortar_smallm_launch(int kind, SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
+template <int CODE>
+static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
     if (t == 0) return -1;
     const bool resident = t > 0;
     const int w = pick_waves(t, p, layers);
     if (!table && layers == 1 && w == 2) {      // one matrix over the whole chip: latency form
         int rc = -1;
-        if (resident) rc = t == 4 ? launch_partsplit<4>(kind, p, st) : launch_partsplit<16>(kind, p, st);
-        else if (fits(8, p.Cb)) rc = launch_partsplit<8>(kind, p, st);      // 8-token tiles of all K instead of K segments
+        if (resident) rc = t == 4 ? launch_partsplit<4, CODE>(kind, p, st) : launch_partsplit<16, CODE>(kind, p, st);
+        else if (fits(8, p.Cb)) rc = launch_partsplit<8, CODE>(kind, p, st);      // 8-token tiles of all K instead of K segments
         if (rc >= 0) return rc;
     }
     if (t == 4) {
-        if (w == 16) return launch_kind<4, 16>(kind, true, p, table, layers, st);
-        return w == 8 ? launch_kind<4, 8>(kind, true, p, table, layers, st) : launch_kind<4, 2>(kind, true, p, table, layers, st);
+        if (w == 16) return launch_kind<4, 16, CODE>(kind, true, p, table, layers, st);
+        return w == 8 ? launch_kind<4, 8, CODE>(kind, true, p, table, layers, st) : launch_kind<4, 2, CODE>(kind, true, p, table, layers, st);
     }
-    if (w == 16) return launch_kind<16, 16>(kind, resident, p, table, layers, st);
-    return w == 8 ? launch_kind<16, 8>(kind, resident, p, table, layers, st) : launch_kind<16, 2>(kind, resident, p, table, layers, st);
+    if (w == 16) return launch_kind<16, 16, CODE>(kind, resident, p, table, layers, st);
+    return w == 8 ? launch_kind<16, 8, CODE>(kind, resident, p, table, layers, st) : launch_kind<16, 2, CODE>(kind, resident, p, table, layers, st);
+}
+
+// p.uscale != 0 (set by the caller for a matrix with one scale) selects the kernels that scale after the sums.
+int mortar_smallm_launch(int kind, SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
+    return p.uscale != 0.f ? smallm_launch_code<CODE_UNIFORM>(kind, p, table, layers, st)
+                           : smallm_launch_code<CODE_2BIT>(kind, p, table, layers, st);
 }
 
 int mortar_smallm_shape(int kind, SpmmParams &p, int layers) {

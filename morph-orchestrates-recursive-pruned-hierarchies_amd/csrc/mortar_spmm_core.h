@@ -36,7 +36,8 @@ struct SpmmParams {
     int xcd_map;              // 1: workgroup ids are renumbered per XCD (grid padded to a multiple of 8)
     int norm;                 // 1: rows of x are RMS-normalised while they are staged (single-segment tiles only)
     float norm_eps;
-    int pad_[3];
+    float uscale;             // CODE_UNIFORM kernels: half the matrix's (bf16-rounded) scale
+    int pad_[2];
     const uint16_t *norm_w;   // bf16 [in_features] weight of that norm, or null for none
 };
 
@@ -55,7 +56,7 @@ struct SpmmView {
     const MORTAR_GLOBAL uint8_t *tok_list;
     int64_t ldx, ldy;
     int n_units, Cb, M, n_clusters, cluster_size, n_mtiles, n_split, seg_cb, nseg, Rb, xcd_map, norm;
-    float norm_eps;
+    float norm_eps, uscale;
     const MORTAR_GLOBAL u32x4_t *norm_w;
 };
 static_assert(sizeof(SpmmParams) % 16 == 0, "table entries are copied in 16-byte words");
@@ -78,9 +79,14 @@ __device__ __forceinline__ SpmmView mortar_view(const SpmmParams &q) {
     v.tok_cnt = (const MORTAR_GLOBAL int32_t *)q.tok_cnt; v.tok_list = (const MORTAR_GLOBAL uint8_t *)q.tok_list;
     v.ldx = q.ldx; v.ldy = q.ldy; v.n_units = q.n_units; v.Cb = q.Cb; v.M = q.M; v.n_clusters = q.n_clusters;
     v.cluster_size = q.cluster_size; v.n_mtiles = q.n_mtiles; v.n_split = q.n_split; v.seg_cb = q.seg_cb; v.nseg = q.nseg; v.Rb = q.Rb; v.xcd_map = q.xcd_map;
-    v.norm = q.norm; v.norm_eps = q.norm_eps; v.norm_w = (const MORTAR_GLOBAL u32x4_t *)q.norm_w;
+    v.norm = q.norm; v.norm_eps = q.norm_eps; v.uscale = q.uscale; v.norm_w = (const MORTAR_GLOBAL u32x4_t *)q.norm_w;
     return v;
 }
+
+// How a kernel reads the code stream (template parameter CODE): bit 0 = the 4-bit stream, bit 1 = one scale for the
+// whole matrix (the reference's per-tensor mortar_scale): the blocks are multiplied as +-2 / 0 and the accumulators
+// are scaled once in the epilogue, which saves the packed multiplies and the scale broadcast of every pair.
+constexpr int CODE_2BIT = 0, CODE_4BIT = 1, CODE_UNIFORM = 2;
 
 constexpr int MORTAR_SMALLM_MAX = 64;    // rows up to which the small-tile (decode) instantiations are used
 constexpr int RES_GROUPS = 4;            // octets (4 block pairs each) loaded per batch
@@ -122,31 +128,31 @@ struct MortarBatch {
 // Loads the batch that starts at octet gq of a row part ending at octet g1 (octets past the end repeat the last).
 // FP4: the code stream is the 4-bit one (a lane's dword holds the 8 codes of its own column half, so the four
 // lane groups read four different 16-byte runs per octet instead of two).
-template <bool FP4 = false>
+template <int CODE = 0>
 __device__ __forceinline__ void mortar_load_batch(const SpmmView &p, MortarBatch &b, int gq, int g1, int n, int bsel,
                                                   int hsel = 0) {
 #pragma unroll
     for (int k = 0; k < RES_GROUPS; ++k) {
         const uint32_t go = (uint32_t)(gq + k < g1 ? gq + k : g1 - 1);
-        const uint32_t gi = FP4 ? go * 4u + (uint32_t)(bsel * 2 + hsel) : go * 2u + (uint32_t)bsel;
+        const uint32_t gi = (CODE & CODE_4BIT) ? go * 4u + (uint32_t)(bsel * 2 + hsel) : go * 2u + (uint32_t)bsel;
         b.cw[k] = p.codes_o[gi * 16u + n];
     }
     const int go = gq + (n >> 2);
     const uint32_t mi = ((uint32_t)(go < g1 ? go : g1 - 1) * 2u + (uint32_t)bsel) * 4u + (uint32_t)(n & 3);
-    b.sdv = p.sd_dw[mi];
+    b.sdv = (CODE & CODE_UNIFORM) ? 0u : p.sd_dw[mi];
     b.ccv = p.cc_dw[mi];
 }
 
 // One row part: octets [g0, g1) (nb blocks) of the stream against the tile at `lx`.
 // `xo_base` is the lane's unit offset inside a block-column (column half, token) plus the segment's origin.
 // `b` holds the part's first batch, loaded by the caller (mortar_load_batch at g0) where it suits it.
-template <int MSUB, int LDM, bool ROUTED, bool FP4 = false>
+template <int MSUB, int LDM, bool ROUTED, int CODE = 0>
 __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *lx, MortarBatch b, int g0, int g1,
                                                 int nb, uint32_t xo_base, const uint32_t (&tk)[MSUB], int nsub, int n,
                                                 int bsel, int hsel, f32x4_t (&acc)[MSUB]) {
     const unsigned char *lb = reinterpret_cast<const unsigned char *>(lx);
     for (int gq = g0; gq < g1; gq += RES_GROUPS) {
-        if (gq != g0) mortar_load_batch<FP4>(p, b, gq, g1, n, bsel, hsel);
+        if (gq != g0) mortar_load_batch<CODE>(p, b, gq, g1, n, bsel, hsel);
         const uint32_t ccs = __umul24(b.ccv, (uint32_t)(2 * LDM * 16));   // byte offset of the block-column in the tile
         const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;      // block pairs left in the row from this batch on
         // Activation operands are fetched two pairs ahead of the MFMAs that use them.  The only branches are
@@ -167,8 +173,8 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
                 for (int t = 0; t < 4; ++t) {
                     const int u = 4 * k + t;
                     if (MSUB >= 2 && t == 2 && u >= pairs) break;     // prefill tiles: the padded half of the last octet
-                    const uint32_t sdu = mortar_row_bcast(b.sdv, u);
-                    const u32x4_t A = FP4 ? mortar_unpack8_fp4(b.cw[k][t], sdu) : mortar_unpack8(b.cw[k][t] << (2 * hsel), sdu);
+                    const uint32_t nib = (CODE & CODE_4BIT) ? b.cw[k][t] : ((b.cw[k][t] << (2 * hsel)) & 0xCCCCCCCCu);
+                    const u32x4_t A = (CODE & CODE_UNIFORM) ? mortar_nib4(nib) : mortar_scale4(nib, mortar_row_bcast(b.sdv, u));
                     if (u + 2 < NP) {
                         const uint32_t xo = mortar_row_bcast(ccs, u + 2) + xo_base * 16u;
 #pragma unroll
@@ -283,9 +289,13 @@ __device__ __forceinline__ void mortar_stage_tile_norm(const SpmmView &p, uint4 
 }
 
 // Epilogue of one row unit for the 16 tokens of sub-tile `ms`: the lane holds D[4g+v][token].
-template <int NACC>
+template <int NACC, int CODE = 0>
 __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, int tok, int g, bool has_gates,
-                                                  const f32x4_t &a0, const f32x4_t &a1) {
+                                                  f32x4_t a0, f32x4_t a1) {
+    if (CODE & CODE_UNIFORM) {      // the blocks were multiplied as +-2: p.uscale is half the matrix's scale
+        a0 *= p.uscale;
+        if (NACC == 2) a1 *= p.uscale;
+    }
     u32x2_t pk;
     if (NACC == 1) {
         pk = u32x2_t{bf16_pack2(a0[0], a0[1]), bf16_pack2(a0[2], a0[3])};
@@ -318,7 +328,7 @@ __device__ __forceinline__ u32x4_t mortar_part_desc(const SpmmView &p, int pos, 
 // No barrier after the first one.  A wave's work is a chain of row parts (unit, segment, row of the unit) whose
 // descriptors come from the schedule table one part ahead; latency is hidden by the waves that share a SIMD.
 // ---------------------------------------------------------------------------------------------------------
-template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE, bool FP4>
+template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE, int CODE>
 __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmParams p0, const SpmmParams *table) {
     constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1;
     const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
@@ -398,8 +408,8 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
                 const int nb = __builtin_amdgcn_readfirstlane((int)d0[2]);
                 if (!skip && g0 < g1) {
                     MortarBatch b;
-                    mortar_load_batch<FP4>(p, b, g0, g1, n, bsel, hsel);
-                    mortar_row_part<MSUB, LDM, ROUTED, FP4>(p, lx, b, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+                    mortar_load_batch<CODE>(p, b, g0, g1, n, bsel, hsel);
+                    mortar_row_part<MSUB, LDM, ROUTED, CODE>(p, lx, b, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
                 }
                 d0 = d1;
             }
@@ -413,7 +423,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
             if (li >= (ROUTED ? cnt : MT)) continue;
             const int tok = m0 + (int)tk[ms];
             if (tok >= p.M) continue;
-            mortar_store_unit<NACC>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
+            mortar_store_unit<NACC, CODE>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
         }
     }
 }
@@ -425,7 +435,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
 // The descriptors of the next segment are fetched before the barrier pair, so their latency hides behind the
 // staging.
 // ---------------------------------------------------------------------------------------------------------
-template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE, bool FP4>
+template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE, int CODE>
 __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const SpmmParams p0, const SpmmParams *table) {
     constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1, NP = UPW * NACC;
     const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
@@ -485,8 +495,8 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
         for (int q = 0; q < NP; ++q) {
             if (g0[q] < g1[q]) {
                 MortarBatch b;
-                mortar_load_batch<FP4>(p, b, g0[q], g1[q], n, bsel, hsel);
-                mortar_row_part<MSUB, LDM, false, FP4>(p, lx, b, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
+                mortar_load_batch<CODE>(p, b, g0[q], g1[q], n, bsel, hsel);
+                mortar_row_part<MSUB, LDM, false, CODE>(p, lx, b, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
                                                   acc[q / NACC][q % NACC]);
             }
         }
@@ -501,7 +511,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
             if (li >= MT) continue;
             const int tok = m0 + li;
             if (tok >= p.M) continue;
-            mortar_store_unit<NACC>(p, units[k], tok, g, has_gates, acc[k][0][ms], acc[k][NACC - 1][ms]);
+            mortar_store_unit<NACC, CODE>(p, units[k], tok, g, has_gates, acc[k][0][ms], acc[k][NACC - 1][ms]);
         }
     }
 }
@@ -513,7 +523,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
 // units (PW * UW waves) and one resident token tile.  Every wave fetches its first descriptor and weight batch
 // before the tile is staged, so the only serial global round trips are descriptor -> batch.
 // ---------------------------------------------------------------------------------------------------------
-template <int MT, int NACC, bool ROUTED, bool MASKED, int PW, int UW>
+template <int MT, int NACC, bool ROUTED, bool MASKED, int PW, int UW, int CODE>
 __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const SpmmParams p0) {
     constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1, WAVES = PW * UW;
     const SpmmView p = mortar_view(p0);
@@ -538,7 +548,7 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
     if (valid && wq < nparts) {
         d = mortar_part_desc<NACC>(p, pos, wq / NACC, wq % NACC);
         const int g0 = __builtin_amdgcn_readfirstlane((int)d[0]), g1 = __builtin_amdgcn_readfirstlane((int)d[1]);
-        if (g0 < g1) mortar_load_batch(p, first, g0, g1, n, bsel);
+        if (g0 < g1) mortar_load_batch<CODE>(p, first, g0, g1, n, bsel, hsel);
     }
     const int unit = valid ? __builtin_amdgcn_readfirstlane((int)mortar_part_desc<NACC>(p, pos, 0, 0)[3]) : 0;
 
@@ -581,8 +591,8 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
                 const int g0 = __builtin_amdgcn_readfirstlane((int)dq[0]), g1 = __builtin_amdgcn_readfirstlane((int)dq[1]);
                 const int nb = __builtin_amdgcn_readfirstlane((int)dq[2]);
                 if (g0 >= g1) continue;
-                if (!is_first) mortar_load_batch(p, first, g0, g1, n, bsel);
-                mortar_row_part<MSUB, LDM, ROUTED>(p, lx, first, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+                if (!is_first) mortar_load_batch<CODE>(p, first, g0, g1, n, bsel, hsel);
+                mortar_row_part<MSUB, LDM, ROUTED, CODE>(p, lx, first, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
             }
         }
     }
@@ -608,7 +618,7 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
         if (li >= (ROUTED ? cnt : MT)) continue;
         const int tok = m0 + (int)tk[ms];
         if (tok >= p.M) continue;
-        mortar_store_unit<NACC>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
+        mortar_store_unit<NACC, CODE>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
     }
 }
 
@@ -669,13 +679,13 @@ inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
     return mortar_grid_width(p, layers);
 }
 
-template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE = false, bool FP4 = false>
+template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE = false, int CODE = 0>
 int mortar_launch_resident(SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     if (TABLE != (table != nullptr)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: parameter table mismatch");
     const int smem = tile_bytes(MT, p.Cb) + LDS_EXTRA;
     if (smem > LDS_BUDGET + LDS_PAD * 16 + LDS_EXTRA) return mortar_fail(MORTAR_ERR_LIMIT, "resident tile of %d bytes does not fit LDS", smem);
     static bool attr_done = false;
-    auto kern = mortar_resident_kernel<MT, NACC, ROUTED, WAVES, TABLE, FP4>;
+    auto kern = mortar_resident_kernel<MT, NACC, ROUTED, WAVES, TABLE, CODE>;
     int rc = mortar_allow_big_lds(kern, attr_done);
     if (rc) return rc;
     const int64_t grid = mortar_resident_shape<MT, WAVES>(p, layers);
@@ -693,13 +703,13 @@ inline int64_t mortar_segmented_shape(SpmmParams &p, int layers) {
     return mortar_grid_width(p, layers);
 }
 
-template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE = false, bool FP4 = false>
+template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE = false, int CODE = 0>
 int mortar_launch_segmented(SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     if (TABLE != (table != nullptr)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: parameter table mismatch");
     const int smem = tile_bytes(MT, p.seg_cb);
     if (smem > LDS_BUDGET + LDS_PAD * 16) return mortar_fail(MORTAR_ERR_LIMIT, "segment tile of %d bytes does not fit LDS", smem);
     static bool attr_done = false;
-    auto kern = mortar_segmented_kernel<MT, NACC, MASKED, WAVES, UPW, TABLE, FP4>;
+    auto kern = mortar_segmented_kernel<MT, NACC, MASKED, WAVES, UPW, TABLE, CODE>;
     int rc = mortar_allow_big_lds(kern, attr_done);
     if (rc) return rc;
     const int64_t grid = mortar_segmented_shape<MT, WAVES, UPW>(p, layers);
@@ -710,13 +720,13 @@ int mortar_launch_segmented(SpmmParams &p, const SpmmParams *table, int layers, 
     return MORTAR_OK;
 }
 
-template <int MT, int NACC, bool ROUTED, bool MASKED, int PW, int UW>
+template <int MT, int NACC, bool ROUTED, bool MASKED, int PW, int UW, int CODE = 0>
 int mortar_launch_partsplit(SpmmParams &p, hipStream_t st) {
     constexpr int WAVES = PW * UW;
     const int smem = tile_bytes(MT, p.Cb) + WAVES * NACC * ((MT + 15) / 16) * 64 * 16;
     if (smem > 160 * 1024) return mortar_fail(MORTAR_ERR_LIMIT, "part-split tile of %d bytes does not fit LDS", smem);
     static bool attr_done = false;
-    auto kern = mortar_partsplit_kernel<MT, NACC, ROUTED, MASKED, PW, UW>;
+    auto kern = mortar_partsplit_kernel<MT, NACC, ROUTED, MASKED, PW, UW, CODE>;
     int rc = mortar_allow_big_lds(kern, attr_done);
     if (rc) return rc;
     p.n_mtiles = (p.M + MT - 1) / MT;

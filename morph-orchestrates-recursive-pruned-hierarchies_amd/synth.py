@@ -67,10 +67,10 @@ def flat_pack(codes: np.ndarray) -> np.ndarray:
     return (u[:, 0] | (u[:, 1] << 2) | (u[:, 2] << 4) | (u[:, 3] << 6)).astype(np.uint8)
 
 
-def to_pack(mat: dict, device, prefill_stream: bool = True) -> MortarPack:
+def to_pack(mat: dict, device, prefill_stream: bool = True, scale_after_sum: bool = True) -> MortarPack:
     out_f, in_f = mat["shape"]
     return MortarPack(flat_pack(mat["codes"]), mat["scales"], mat["col_idx"], mat["offsets"], out_f, in_f, device,
-                      prefill_stream=prefill_stream)
+                      prefill_stream=prefill_stream, scale_after_sum=scale_after_sum)
 
 
 def synth_mlp(d_model: int, d_ff: int, density: float = 0.25, seed: int = 0, zipf_s: float | None = None) -> dict:

@@ -191,6 +191,42 @@ def test_prefill_code_streams_agree(dev, d_model, d_ff):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("d_model,d_ff,M", [(256, 16 * 40, 200), (2048, 16 * 24, 130), (16 * 30, 16 * 352, 100),
+                                            (256, 16 * 40, 1), (2048, 16 * 24, 5), (16 * 30, 16 * 352, 16), (768, 2048, 40)])
+def test_one_scale_per_matrix(dev, d_model, d_ff, M):
+    """Matrices with one scale (the reference's per-tensor mortar_scale): the kernels that scale the fp32 sums once
+    against the oracle and against the per-block kernels on the same data (plain, gated, routed, masked), for the
+    prefill tiles, the K-segmented `down`, the decode tiles and a layer-batched launch."""
+    spec = synth.synth_mlp(d_model, d_ff, 0.25, seed=77, zipf_s=1.2)
+    spec["gate_up"]["scales"] = np.float32(0.0437)
+    spec["down"]["scales"] = np.float32(0.0291)
+    x = synth.synth_x(M, d_model, 78)
+    xd = to_dev(x, dev)
+    ncl = d_ff // 16
+    gates, active = ops.remoe_gates(torch.from_numpy(synth.synth_logits(M, ncl, 79)).to(dev), ncl // 4)
+    outs = []
+    for after in (True, False):
+        Wgu, Wdn = (synth.to_pack(spec[k], dev, scale_after_sum=after) for k in ("gate_up", "down"))
+        assert (Wgu.uniform_scale != 0) == after and (Wdn.uniform_scale != 0) == after
+        h = ops.gateup_swiglu(xd, Wgu)
+        res = [h, ops.spmm(h, Wdn), ops.gateup_swiglu(xd, Wgu, gates=gates)]
+        tile = ops.route_tile(Wgu, M)
+        if tile:
+            hr = torch.zeros_like(h)
+            ops.gateup_swiglu(xd, Wgu, gates=gates, route=ops.remoe_route(active, tile), out=hr)
+            res += [hr, ops.spmm(hr, Wdn, active=active)]
+        if M <= 16:
+            hs = [torch.empty_like(h) for _ in range(3)]
+            ops.LayerStack([Wgu] * 3, [xd] * 3, hs, swiglu=True).run()
+            res += hs[1:2]
+        outs.append(res)
+    ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
+    assert_close_bf16(to_np(outs[0][0]), ref["h"], "h", ulps=4)
+    assert_close_bf16(to_np(outs[0][1]), ref["y"], "y", ulps=8)
+    for a, b in zip(*outs):
+        assert_close_bf16(to_np(a), to_np(b).astype(np.float32), "scale after sum vs per block", ulps=8)
+
+
 def test_remoe_route_lists_exact(dev):
     rng = np.random.default_rng(40)
     act = (rng.random((333, 70)) < 0.25).astype(np.uint8)

@@ -1,5 +1,6 @@
 """CPU tests of the host logic: C-ABI exports, device-format encoding, schedules, module state (no GPU compute)."""
 import ctypes
+import ctypes as C
 import itertools
 import os
 import re
@@ -47,6 +48,21 @@ def test_encode_round_trip_and_bit_layout():
         prod = (half.astype(np.float32) * np.float32(sign)).astype(np.float16).view(np.uint16)
         want = O.bf16_bits(scale) | (0x8000 if sign < 0 else 0)
         assert np.array_equal(prod, want)
+
+
+def test_uniform_scale_is_detected():
+    codes = np.ones((5, 16, 16), np.int8)
+    L = _lib.lib()
+    us = C.c_float(-1.0)
+    _, sdup = P.encode_blocks(O.pack_ternary_codes(codes), 5, np.float32(0.0371))
+    _lib.check(L.mortar_uniform_scale_host(P._vp(sdup), 5, C.byref(us)), "uniform")
+    assert us.value == O.bf16_round(np.float32(0.0371))                  # the bf16 value the kernels multiply by
+    _, sdup = P.encode_blocks(O.pack_ternary_codes(codes), 5, np.linspace(0.01, 0.1, 5).astype(np.float32))
+    _lib.check(L.mortar_uniform_scale_host(P._vp(sdup), 5, C.byref(us)), "uniform")
+    assert us.value == 0.0                                               # per-block scales
+    _, sdup = P.encode_blocks(O.pack_ternary_codes(codes), 5, np.float32(0.0))
+    _lib.check(L.mortar_uniform_scale_host(P._vp(sdup), 5, C.byref(us)), "uniform")
+    assert us.value == 0.0
 
 
 def test_encode_scalar_scale_and_errors():
