@@ -2,7 +2,7 @@
 
 Step = one pass of the carved SwiGLU MLP (gate_up with fused SwiGLU, then down) over one batch of synthetic
 tokens.  Workload at N=1: d_model 2048, d_ff 5632, 16x16 BCSR at 25 % block density, ternary codes with one
-fp32 scale per block, 4096-token prefill (the shapes of BASELINE.json configs 2/3).  The same run also times
+fp32 scale per block, 4096-token prefill (the shapes of benchmark configs 2/3).  The same run also times
 the decode GEMVs (batch 1/4/16/64), the ReMoE-routed prefill, and a bounded CPU baseline on the host cores.
 
 Prints ONE JSON line.  `value` = prefill tokens/s with inputs resident in HBM.
@@ -114,7 +114,7 @@ def main() -> None:
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "carved SwiGLU MLP prefill, d_model 2048 / d_ff 5632, 16x16 BCSR 25 % uniform, "
-                               "ternary + per-block scale, 4096 tokens bf16 (BASELINE configs 2/3 shapes)",
+                               "ternary + per-block scale, 4096 tokens bf16 (benchmark configs 2/3 shapes)",
                    "tokens": TOKENS, "nnz_blocks": [Wgu.nnz, Wdn.nnz]},
         "effective_tflops": (flops_gu + flops_dn) / (ms * 1e-3) / 1e12,
         "roofline": {"bound": "mfma", "kernel": "mortar_resident_kernel<32 tokens, gate_up + SwiGLU>",
@@ -241,7 +241,7 @@ def main() -> None:
                                   "achieved": stack["b1"]["algorithmic_GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                   "frac": stack["b1"]["frac_hbm"], "traffic": TRAFFIC_DECODE_STACK_BYTES,
                                   "algorithmic_bytes": n_sets * (wbytes + (2 * D_MODEL + 2 * D_FF) * 2)}
-        # ---- ReMoE-routed prefill (BASELINE config 3) ----------------------------------------------------
+        # ---- ReMoE-routed prefill (benchmark config 3) ----------------------------------------------------
         logits = torch.from_numpy(synth.synth_logits(TOKENS, N_CLUSTERS, seed=2)).to(dev)
 
         def routed():
@@ -280,7 +280,7 @@ def main() -> None:
         del up, dn, hs, ys, upacks, Ugu, Udn
 
     if not args.no_extras:
-        # ---- BASELINE config 1: base-width MLP (d_model 768, d_ff 2048), 4 x 4096 tokens ---------------------
+        # ---- benchmark config 1: base-width MLP (d_model 768, d_ff 2048), 4 x 4096 tokens ---------------------
         spec1 = synth.synth_mlp(768, 2048, DENSITY, seed=10)
         G1, D1 = synth.to_pack(spec1["gate_up"], dev), synth.to_pack(spec1["down"], dev)
         x1 = torch.from_numpy(synth.synth_x(16384, 768, seed=11)).to(torch.bfloat16).to(dev)
@@ -295,7 +295,7 @@ def main() -> None:
         out["base_width_prefill"] = {"ms": t, "tokens_per_s": 16384 / (t * 1e-3), "effective_tflops": fl / (t * 1e-3) / 1e12,
                                      "frac_mfma": fl / (t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
         del x1, h1, y1
-        # ---- BASELINE config 4: 8 shared blocks x 6 iterations, Zipf(1.2) rows, RMS-normalised input ----------
+        # ---- benchmark config 4: 8 shared blocks x 6 iterations, Zipf(1.2) rows, RMS-normalised input ----------
         specs = [synth.synth_mlp(D_MODEL, D_FF, DENSITY, seed=20 + i, zipf_s=1.2) for i in range(8)]
         packs4 = [(synth.to_pack(sp["gate_up"], dev), synth.to_pack(sp["down"], dev)) for sp in specs]
         xs = [x, torch.empty_like(x)]

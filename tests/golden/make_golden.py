@@ -21,7 +21,7 @@ from oracle import mortar_oracle as O  # noqa: E402
 
 
 def c0():
-    """BASELINE config 0 whole: x [64, 768] bf16, W [2048, 768] at 25 % block density, ternary (.3/.4/.3),
+    """benchmark config 0 whole: x [64, 768] bf16, W [2048, 768] at 25 % block density, ternary (.3/.4/.3),
     per-block scale U(.01, .1)."""
     m = synth.synth_matrix(2048, 768, 0.25, seed=100)
     x = synth.synth_x(64, 768, seed=101)

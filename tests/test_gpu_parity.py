@@ -43,7 +43,7 @@ def test_golden_fixtures(dev):
 # ---------------------------------------------------------------------------------------------- prefill SpMM
 
 def test_c0_single_spmm(dev):
-    """BASELINE config 0: x 64x768, W 768->2048, 25 % uniform, ternary p=(.3,.4,.3), scale U(.01,.1)."""
+    """benchmark config 0: x 64x768, W 768->2048, 25 % uniform, ternary p=(.3,.4,.3), scale U(.01,.1)."""
     m = synth.synth_matrix(2048, 768, 0.25, seed=100)
     x = synth.synth_x(64, 768, seed=101)
     W = synth.to_pack(m, dev)
@@ -122,7 +122,7 @@ def test_stk_dds_operator_signature(dev):
 
 @pytest.mark.parametrize("M", [64, 200])
 def test_mlp_base_config_slice(dev, M):
-    """BASELINE config 1 shapes (d_model 768, d_ff 2048) on a token slice the oracle finishes quickly."""
+    """benchmark config 1 shapes (d_model 768, d_ff 2048) on a token slice the oracle finishes quickly."""
     spec = synth.synth_mlp(768, 2048, 0.25, seed=20)
     x = synth.synth_x(M, 768, 21)
     ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
@@ -248,7 +248,7 @@ def test_remoe_gates_ties_and_edges(dev):
         g, a = ops.remoe_gates(torch.from_numpy(lg).to(dev), k)
         assert np.array_equal(a.cpu().numpy().astype(bool), a_ref), (n, k)
         np.testing.assert_allclose(g.cpu().numpy(), g_ref, rtol=3e-6, atol=0)
-    lg = synth.synth_logits(4096, 352, 42)                                      # BASELINE config 3 router
+    lg = synth.synth_logits(4096, 352, 42)                                      # benchmark config 3 router
     g_ref, a_ref = O.remoe_gates(lg, 88)
     g, a = ops.remoe_gates(torch.from_numpy(lg).to(dev), 88)
     assert np.array_equal(a.cpu().numpy().astype(bool), a_ref) and (a_ref.sum(1) == 87).all()
@@ -319,7 +319,7 @@ def test_route_flags_exact(dev):
 
 @pytest.mark.parametrize("B", [1, 4, 16, 17, 64])
 def test_decode_mlp_cloud_width(dev, B):
-    """BASELINE config 2: d_model 2048, d_ff 5632, batch of single-token rows."""
+    """benchmark config 2: d_model 2048, d_ff 5632, batch of single-token rows."""
     spec = synth.synth_mlp(2048, 5632, 0.25, seed=50)
     x = synth.synth_x(B, 2048, 51 + B)
     ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
@@ -508,7 +508,7 @@ def test_norm_fusion_limits(dev):
 
 
 def test_looped_core_stack_small(dev):
-    """BASELINE config 4 call pattern at reduced size: shared blocks x iterations, RMS-normalised input, Zipf rows."""
+    """benchmark config 4 call pattern at reduced size: shared blocks x iterations, RMS-normalised input, Zipf rows."""
     d_model, d_ff, M = 256, 16 * 44, 150
     specs = [synth.synth_mlp(d_model, d_ff, 0.25, seed=200 + i, zipf_s=1.2) for i in range(2)]
     x = synth.synth_x(M, d_model, 210)
@@ -524,7 +524,7 @@ def test_looped_core_stack_small(dev):
 # ---------------------------------------------------------------------------------------------- full size, by properties
 
 def test_full_size_properties(dev):
-    """BASELINE config 3 shapes (d_model 2048, d_ff 5632, 4096 tokens): size-independent checks.
+    """benchmark config 3 shapes (d_model 2048, d_ff 5632, 4096 tokens): size-independent checks.
     (1) rows sampled from the prefill output equal the oracle on those rows; (2) prefill and decode kernels
     agree on the same rows; (3) linearity in a power-of-two scale is exact."""
     spec = synth.synth_mlp(2048, 5632, 0.25, seed=300)
