@@ -26,6 +26,7 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 // the block scale's bf16 pattern minus one 16-bit-float exponent step in both halves, so one packed half multiply
 // returns exactly +-scale or 0 in bf16 bits (a power-of-two product is exact; the host rejects scales whose
 // pattern would leave the normal range).
+// The 4-bit stream stores the nibbles themselves (byte i = {column 2i, column 2i + 1}): no shift, no mask.
 __device__ __forceinline__ u32x4_t mortar_scale4(uint32_t nib, uint32_t sd) {
     const f16x2_t s = __builtin_bit_cast(f16x2_t, sd);
     u32x4_t r;
@@ -47,10 +48,6 @@ __device__ __forceinline__ u32x4_t mortar_nib4(uint32_t nib) {
     r[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(nib, 1.0f, 3));
     return r;
 }
-
-// Same result from the 4-bit stream: `t` holds the lane's 8 codes as FP4 nibbles {sign, non-zero, 0, 0} already,
-// byte i = {column 2i (low nibble), column 2i+1 (high nibble)}.
-__device__ __forceinline__ u32x4_t mortar_unpack8_fp4(uint32_t t, uint32_t sd) { return mortar_scale4(t, sd); }
 
 __device__ __forceinline__ f32x4_t mortar_mfma(u32x4_t a, u32x4_t b, f32x4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
