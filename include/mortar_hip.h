@@ -112,6 +112,20 @@ int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, int32_t Cb,
  * codes4_o_out host [ngroups*256], layout as described at mortar_bcsr_t.  No counterpart in the reference. */
 int mortar_fp4_stream_host(const uint32_t *codes_o, int64_t ngroups, uint32_t *codes4_o_out);
 
+/* Position of every block in the octet streams (the index the device-side re-pack scatters to):
+ * pos_out host [nnz], pos_out[j] = (group*2 + s)*4 + t of block j, for the same seg_cb as mortar_octet_layout_host. */
+int mortar_octet_positions_host(const int32_t *row_ptr, int32_t Rb, int32_t Cb, int32_t seg_cb, const int16_t *col,
+                                int32_t *pos_out);
+
+/* Topology of W^T (reference: stk matrix.py:107-125 `_transpose`, which yields mortar_offsets_t,
+ * mortar_column_indices_t and mortar_block_offsets_t): offsets_t_out host [Cb+1], col_t_out host [nnz] = block-row
+ * of each block in transposed order, src_block_out host [nnz] = its index in the original order.  Blocks of one
+ * column keep ascending row order (the reference leaves that order to the sort backend).  A pack built over
+ * (offsets_t, col_t) and filled by mortar_requantize(..., src_block, transpose = 1) multiplies by W^T: the dX
+ * product stk_dds(..., transpose_b=False) (custom_ops.py:35-56). */
+int mortar_transpose_topology_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
+                                   int32_t *offsets_t_out, int16_t *col_t_out, int32_t *src_block_out);
+
 /* Largest K segment (in block-columns) whose 32-token activation tile fits in LDS; a matrix with
  * Cb <= this runs the single-segment prefill kernel.  Use seg_cb = ceil(Cb / ceil(Cb / max)). */
 int mortar_prefill_max_seg_cb(void);
@@ -268,6 +282,33 @@ int mortar_norm_fusable(int32_t Cb);
 /* y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) per row; x, y bf16 [M, d]; w bf16 [d] or NULL (= 1). */
 int mortar_rmsnorm_bf16(const uint16_t *x, int64_t M, int32_t d, int64_t ldx, const uint16_t *w, float eps,
                         uint16_t *y, int64_t ldy, void *stream);
+
+/* ---- device-side re-pack ------------------------------------------------------------------------ */
+
+/* Ternarise block values on the device and rewrite the matrix's value arrays (codes, sdup, codes_o, sd_o and,
+ * when present, codes4_o) in place; the topology arrays are not touched.  One launch (two with scale_mode 0)
+ * replaces the reference's per-forward torch ternarisation of mortar_data (block_sparse.py:909-919) and its
+ * deploy pack (deploy_quant.py:81-95, 344-374) followed by a host re-pack.
+ *   values     device [nnz,16,16], bf16 (values_f32 = 0) or fp32 (1): the reference's mortar_data
+ *   pos        device int32 [nnz] from mortar_octet_positions_host
+ *   src_block  device int32 [nnz] or NULL: block j of W takes the values of block src_block[j] (NULL: block j)
+ *   transpose  != 0: the source block is read transposed.  src_block + transpose fill the W^T pack of
+ *              mortar_transpose_topology_host from the values of W.
+ *   scale_mode 0: one scale per matrix, mean|w| over all values clamped to >= 1e-8 (deploy_quant.py:91)
+ *              1: one scale per block, mean|w| of the (source) block clamped to >= 1e-6 (block_sparse.py:397)
+ *              2: scale_in device fp32 [1];  3: scale_in device fp32 [nnz], indexed by source block
+ *   code = sign(w/s) where |w/s| > threshold (fp32 division, strict compare), else 0; means are summed in fp64
+ *   in a fixed order.  The kernels multiply by bf16(s) (round to nearest even), as the reference's bf16 autocast does.
+ *   scale_out  device fp32, [1] for modes 0 and 2, [nnz] for 1 and 3 (order of W's blocks), or NULL
+ *   status     device int32 [1] or NULL: set to 0, then to 1 if bf16(s) of some block lies outside
+ *              [2^-100, 2^100] (that block is zeroed; the host packer returns MORTAR_ERR_SCALE for it)
+ *   workspace  device, mortar_requantize_workspace_bytes() bytes, 8-byte aligned; needed for scale_mode 0 only
+ * mortar_bcsr_t.uniform_scale is host state: after modes 0 / 2 the caller may set it to bf16(s) to select the
+ * scale-after-sum kernels, or leave it 0 (per-block kernels, always valid). */
+int64_t mortar_requantize_workspace_bytes(void);
+int mortar_requantize(const mortar_bcsr_t *W, const void *values, int32_t values_f32, const int32_t *pos,
+                      const int32_t *src_block, int32_t transpose, int32_t scale_mode, float threshold,
+                      const float *scale_in, float *scale_out, int32_t *status, void *workspace, void *stream);
 
 #ifdef __cplusplus
 }

@@ -29,6 +29,10 @@ _SIGS = {
     "mortar_decode_blocks_host": (C.c_int, [c_vp, c_i64, c_vp]),
     "mortar_octet_layout_host": (c_i64, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "mortar_fp4_stream_host": (C.c_int, [c_vp, c_i64, c_vp]),
+    "mortar_octet_positions_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp]),
+    "mortar_transpose_topology_host": (C.c_int, [c_vp, c_vp, c_i32, c_i32, c_vp, c_vp, c_vp]),
+    "mortar_requantize_workspace_bytes": (c_i64, []),
+    "mortar_requantize": (C.c_int, [c_vp, c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_f32, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "mortar_prefill_max_seg_cb": (C.c_int, []),
     "mortar_validate_bcsr_host": (C.c_int, [c_vp, c_vp, c_i32, c_i32]),
     "mortar_schedule_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp]),

@@ -25,7 +25,7 @@ int mortar_fail(int code, const char *fmt, ...) {
 }
 
 extern "C" const char *mortar_last_error(void) { return g_err; }
-extern "C" int mortar_abi_version(void) { return 3; }
+extern "C" int mortar_abi_version(void) { return 4; }
 
 static inline uint16_t f32_to_bf16_bits(float f) {
     uint32_t u;
@@ -168,6 +168,53 @@ extern "C" int64_t mortar_octet_layout_host(const int32_t *row_ptr, int32_t Rb, 
         }
     }
     return ng;
+}
+
+extern "C" int mortar_octet_positions_host(const int32_t *row_ptr, int32_t Rb, int32_t Cb, int32_t seg_cb,
+                                           const int16_t *col, int32_t *pos_out) {
+    if (!row_ptr || !col || !pos_out || Rb <= 0 || Cb <= 0 || seg_cb <= 0)
+        return mortar_fail(MORTAR_ERR_ARG, "octet_positions: bad argument");
+    const int nseg = (Cb + seg_cb - 1) / seg_cb;
+    // same walk as mortar_octet_layout_host: segments outermost, rows inside, 8 blocks per octet
+    std::vector<int32_t> lo((size_t)nseg * Rb), hi((size_t)nseg * Rb);
+    for (int r = 0; r < Rb; ++r) {
+        int p = row_ptr[r];
+        for (int sg = 0; sg < nseg; ++sg) {
+            lo[(size_t)sg * Rb + r] = p;
+            while (p < row_ptr[r + 1] && col[p] < (sg + 1) * seg_cb) ++p;
+            hi[(size_t)sg * Rb + r] = p;
+        }
+    }
+    int64_t ng = 0;
+    for (int64_t v = 0; v < (int64_t)nseg * Rb; ++v) {
+        const int nb = hi[v] - lo[v];
+        for (int b = 0; b < nb; ++b) {
+            const int64_t g = ng + b / 8;
+            pos_out[lo[v] + b] = (int32_t)((g * 2 + (b & 1)) * 4 + ((b & 7) >> 1));
+        }
+        ng += (nb + 7) / 8;
+    }
+    return MORTAR_OK;
+}
+
+extern "C" int mortar_transpose_topology_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
+                                              int32_t *offsets_t_out, int16_t *col_t_out, int32_t *src_block_out) {
+    if (!offsets_t_out || !col_t_out || !src_block_out)
+        return mortar_fail(MORTAR_ERR_ARG, "transpose_topology: null pointer");
+    const int rc = mortar_check_bcsr_host(row_ptr, col, Rb, Cb);
+    if (rc) return rc;
+    const int32_t nnz = row_ptr[Rb];
+    std::fill(offsets_t_out, offsets_t_out + Cb + 1, 0);
+    for (int32_t j = 0; j < nnz; ++j) ++offsets_t_out[col[j] + 1];
+    for (int c = 0; c < Cb; ++c) offsets_t_out[c + 1] += offsets_t_out[c];
+    std::vector<int32_t> fill(offsets_t_out, offsets_t_out + Cb);
+    for (int r = 0; r < Rb; ++r)                        // ascending rows: blocks of one column stay in row order
+        for (int32_t j = row_ptr[r]; j < row_ptr[r + 1]; ++j) {
+            const int32_t o = fill[col[j]]++;
+            col_t_out[o] = (int16_t)r;
+            src_block_out[o] = j;
+        }
+    return MORTAR_OK;
 }
 
 extern "C" int mortar_fp4_stream_host(const uint32_t *codes_o, int64_t ngroups, uint32_t *codes4_o_out) {

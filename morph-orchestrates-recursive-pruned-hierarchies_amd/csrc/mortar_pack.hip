@@ -1,0 +1,161 @@
+// Device-side re-pack: ternarise block values and rewrite a matrix's code and scale arrays in place.
+//
+// The reference ternarises carved blocks in torch (deploy_quant.py:81-95 for the deploy pack,
+// block_sparse.py:909-919 on every QAT forward: scale = mean|w|, q = sign(w/s) * (|w/s| > threshold)) and keeps the
+// transposed topology for the dX product as index arrays over the same data (stk matrix.py:107-125).  Here the
+// topology of a pack (columns, offsets, octet positions) is fixed once on the host, and this kernel refreshes the
+// values: one wavefront per block reads the 256 values (optionally of another block, transposed: the dX pack),
+// forms the scale, and writes the row dwords into `codes`, the octet stream and its 4-bit copy.
+#include <hip/hip_runtime.h>
+
+#include "mortar_internal.h"
+
+namespace {
+
+constexpr int PARTIALS = 256;           // workgroups of the |w| reduction; the workspace holds one double each
+
+__device__ __forceinline__ float load_val(const void *v, int64_t i, bool f32) {
+    if (f32) return reinterpret_cast<const float *>(v)[i];
+    return __uint_as_float((uint32_t) reinterpret_cast<const uint16_t *>(v)[i] << 16);
+}
+
+__device__ __forceinline__ double wave_sum(double x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    return x;
+}
+
+// sum |w| over all values -> partial[blockIdx] (fixed order: the result does not depend on timing)
+__global__ __launch_bounds__(256) void abs_sum_kernel(const void *values, int64_t n, int f32, double *partial) {
+    __shared__ double wsum[4];
+    double s = 0.0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)PARTIALS * 256)
+        s += (double)fabsf(load_val(values, i, f32 != 0));
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) partial[blockIdx.x] = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
+}
+
+__global__ void clear_status_kernel(int32_t *status) {
+    if (threadIdx.x == 0) *status = 0;
+}
+
+struct RequantArgs {
+    uint32_t *codes, *sdup, *codes_o, *sd_o, *codes4_o;
+    const void *values;
+    const int32_t *pos, *src_block;
+    const float *scale_in;
+    float *scale_out;
+    int32_t *status;
+    const double *partial;
+    int32_t nnz, f32, transpose, mode;
+    float threshold;
+};
+
+// mode 0: one scale per matrix from the partial sums, 1: one per block, 2: scale_in[0], 3: scale_in[source block]
+__global__ __launch_bounds__(256) void requant_kernel(RequantArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int j = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (j >= a.nnz) return;
+    const int src = a.src_block ? a.src_block[j] : j;
+    const int n = lane >> 2, q = lane & 3;
+    float w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int c = 4 * q + e;
+        w[e] = load_val(a.values, (int64_t)src * 256 + (a.transpose ? c * 16 + n : n * 16 + c), a.f32 != 0);
+    }
+    float s;
+    if (a.mode == 0) {
+        const double t = wave_sum((a.partial[lane] + a.partial[lane + 64]) + (a.partial[lane + 128] + a.partial[lane + 192]));
+        s = fmaxf((float)(t / ((double)a.nnz * 256.0)), 1e-8f);
+    } else if (a.mode == 1) {
+        const double t = wave_sum(((double)fabsf(w[0]) + (double)fabsf(w[1])) + ((double)fabsf(w[2]) + (double)fabsf(w[3])));
+        s = fmaxf((float)(t * (1.0 / 256.0)), 1e-6f);
+    } else {
+        s = a.scale_in[a.mode == 2 ? 0 : src];
+    }
+    // scale pattern: bf16(s) one exponent step down, in both halves (0 zeroes the block)
+    uint32_t u = __float_as_uint(s);
+    uint32_t sb = (u & 0x7fffffffu) > 0x7f800000u ? 0x7fc0u : ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+    uint32_t sd = 0;
+    if ((sb & 0x7fffu) != 0) {
+        const uint32_t e8 = (sb >> 7) & 0xffu;
+        if (e8 < 27 || e8 > 227) {
+            if (lane == 0 && a.status) *a.status = 1;
+        } else {
+            const uint32_t adj = sb - 0x0400u;
+            sd = adj | (adj << 16);
+        }
+    }
+    uint32_t row = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int c = 4 * q + e;
+        const float wn = w[e] / s;
+        const uint32_t enc = (fabsf(wn) > a.threshold && wn != 0.f && sd != 0) ? (wn < 0.f ? 3u : 1u) : 0u;
+        row |= enc << (2 * (c < 8 ? 2 * c + 1 : 2 * (c - 8)));
+    }
+    row |= __shfl_xor(row, 1);
+    row |= __shfl_xor(row, 2);
+    const int P = a.pos[j];
+    if (q == 0) {
+        a.codes[(int64_t)j * 16 + n] = row;
+    } else if (q == 1) {
+        a.codes_o[(int64_t)(P >> 2) * 64 + n * 4 + (P & 3)] = row;
+    } else if (a.codes4_o) {
+        const int h = q - 2;
+        const int64_t g = P >> 3, s2 = (P >> 2) & 1;
+        a.codes4_o[((g * 4 + 2 * s2 + h) * 16 + n) * 4 + (P & 3)] = (row << (2 * h)) & 0xCCCCCCCCu;
+    }
+    if (lane == 0) {
+        a.sdup[j] = sd;
+        a.sd_o[P] = sd;
+        if (a.scale_out) a.scale_out[(a.mode == 0 || a.mode == 2) ? 0 : j] = s;
+    }
+}
+
+}  // namespace
+
+extern "C" int64_t mortar_requantize_workspace_bytes(void) { return (int64_t)PARTIALS * sizeof(double); }
+
+extern "C" int mortar_requantize(const mortar_bcsr_t *W, const void *values, int32_t values_f32, const int32_t *pos,
+                                 const int32_t *src_block, int32_t transpose, int32_t scale_mode, float threshold,
+                                 const float *scale_in, float *scale_out, int32_t *status, void *workspace,
+                                 void *stream) {
+    if (!W || !values || !pos) return mortar_fail(MORTAR_ERR_ARG, "requantize: null pointer");
+    if (!W->codes || !W->sdup || !W->codes_o || !W->sd_o || W->nnz <= 0)
+        return mortar_fail(MORTAR_ERR_ARG, "requantize: incomplete matrix");
+    if (scale_mode < 0 || scale_mode > 3) return mortar_fail(MORTAR_ERR_ARG, "requantize: scale_mode %d not in 0..3", scale_mode);
+    if (scale_mode >= 2 && !scale_in) return mortar_fail(MORTAR_ERR_ARG, "requantize: scale_mode %d needs scale_in", scale_mode);
+    if (scale_mode == 0 && !workspace) return mortar_fail(MORTAR_ERR_ARG, "requantize: scale_mode 0 needs the workspace");
+    if (!(threshold >= 0.f)) return mortar_fail(MORTAR_ERR_ARG, "requantize: threshold must be >= 0");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (status) hipLaunchKernelGGL(clear_status_kernel, dim3(1), dim3(64), 0, st, status);
+    if (scale_mode == 0)
+        hipLaunchKernelGGL(abs_sum_kernel, dim3(PARTIALS), dim3(256), 0, st, values, (int64_t)W->nnz * 256, values_f32,
+                           static_cast<double *>(workspace));
+    RequantArgs a;
+    a.codes = const_cast<uint32_t *>(W->codes);
+    a.sdup = const_cast<uint32_t *>(W->sdup);
+    a.codes_o = const_cast<uint32_t *>(W->codes_o);
+    a.sd_o = const_cast<uint32_t *>(W->sd_o);
+    a.codes4_o = const_cast<uint32_t *>(W->codes4_o);
+    a.values = values;
+    a.pos = pos;
+    a.src_block = src_block;
+    a.scale_in = scale_in;
+    a.scale_out = scale_out;
+    a.status = status;
+    a.partial = static_cast<const double *>(workspace);
+    a.nnz = W->nnz;
+    a.f32 = values_f32;
+    a.transpose = transpose;
+    a.mode = scale_mode;
+    a.threshold = threshold;
+    hipLaunchKernelGGL(requant_kernel, dim3((W->nnz + 3) / 4), dim3(256), 0, st, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "requantize: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}

@@ -79,6 +79,26 @@ def fp4_stream(codes_o: np.ndarray) -> np.ndarray:
     return out
 
 
+def octet_positions(offsets, Rb: int, Cb: int, seg_cb: int, col) -> np.ndarray:
+    """Index of every block in the octet streams: see mortar_octet_positions_host."""
+    offsets, col = _np(offsets, np.int32), _np(col, np.int16)
+    out = np.empty(col.size, dtype=np.int32)
+    _lib.check(_lib.lib().mortar_octet_positions_host(_vp(offsets), Rb, Cb, seg_cb, _vp(col), _vp(out)),
+               "mortar_octet_positions_host")
+    return out
+
+
+def transpose_topology(offsets, col, Rb: int, Cb: int):
+    """-> (offsets_t [Cb+1] int32, col_t [nnz] int16, src_block [nnz] int32): see mortar_transpose_topology_host."""
+    offsets, col = _np(offsets, np.int32), _np(col, np.int16)
+    off_t = np.empty(Cb + 1, dtype=np.int32)
+    col_t = np.empty(col.size, dtype=np.int16)
+    src = np.empty(col.size, dtype=np.int32)
+    _lib.check(_lib.lib().mortar_transpose_topology_host(_vp(offsets), _vp(col), Rb, Cb, _vp(off_t), _vp(col_t), _vp(src)),
+               "mortar_transpose_topology_host")
+    return off_t, col_t, src
+
+
 def unit_order(offsets, Rb: int, rows_per_unit: int, group: int = SCHED_GROUP) -> np.ndarray:
     offsets = _np(offsets, np.int32)
     out = np.empty(Rb // rows_per_unit, dtype=np.int32)
@@ -120,6 +140,10 @@ class MortarPack:
     unpack the 2-bit stream.  When all blocks share one scale (the reference's per-tensor mortar_scale) and
     ``scale_after_sum`` is on, the kernels scale the fp32 sums once instead of every block's weights
     (``uniform_scale``; about a third fewer vector instructions per block pair).
+
+    ``packed=None`` builds the topology with all-zero blocks, to be filled on the device by ``requantize`` from
+    block values (the reference's ``mortar_data``): the device-side pack used for QAT forwards and for the W^T
+    pack of the dX product (``transposed()``).
     """
 
     def __init__(self, packed, scale, col, offsets, out_features: int, in_features: int, device,
@@ -138,10 +162,14 @@ class MortarPack:
         if (np.diff(self.h_offsets) <= 0).any():
             raise RuntimeError("carved matrix has a block-row with zero kept blocks")
         self.device = torch.device(device)
-        codes, sdup = encode_blocks(packed, self.nnz, scale)
+        if packed is None:
+            codes, sdup = np.zeros(self.nnz * 16, dtype=np.uint32), np.zeros(self.nnz, dtype=np.uint32)
+        else:
+            codes, sdup = encode_blocks(packed, self.nnz, scale)
         validate_bcsr(self.h_offsets, self.h_col, self.Rb, self.Cb)
         us = C.c_float(0.0)
         _lib.check(_lib.lib().mortar_uniform_scale_host(_vp(sdup), self.nnz, C.byref(us)), "mortar_uniform_scale_host")
+        self.scale_after_sum = bool(scale_after_sum)
         self.uniform_scale = float(us.value) if scale_after_sum else 0.0
         dev = self.device
         self.codes = torch.from_numpy(codes.view(np.int32)).to(dev)
@@ -161,6 +189,8 @@ class MortarPack:
         self.codes4_o = torch.from_numpy(fp4_stream(codes_o).view(np.int32)).to(dev) if prefill_stream else None
         self._scheds: dict[int, torch.Tensor] = {}
         self._worklists: dict[tuple, tuple] = {}
+        self._pos = self._ws = self._status = self.src_block = None
+        self._transposed: "MortarPack | None" = None
         self.struct = self._make_struct()
         self.ref = C.byref(self.struct)
 
@@ -170,6 +200,65 @@ class MortarPack:
                                self.sd_o.data_ptr(), self.col_o.data_ptr(),
                                self.codes4_o.data_ptr() if self.codes4_o is not None else None,
                                self.Rb, self.Cb, self.nnz, self.seg_cb, self.uniform_scale, 0)
+
+    # ---- device-side re-pack ----------------------------------------------------------------------------------
+
+    def requantize(self, values: torch.Tensor, per_block: bool = False, threshold: float = 0.5,
+                   scale: torch.Tensor | None = None, transpose: bool = False, sync: bool = True) -> torch.Tensor:
+        """Ternarise ``values`` [nnz,16,16] (bf16 or fp32, on this device) into this pack, in place, on the current
+        stream: scale = mean|w| over the matrix (reference deploy_quant.py:81-95, block_sparse.py:909-919) or per
+        block (``per_block``), or the given ``scale`` (fp32 [1] or [nnz], indexed like ``values``); code =
+        sign(w/s) * (|w/s| > threshold).  A pack from ``transposed()`` reads the blocks of the original matrix
+        (its ``src_block`` map) and pass ``transpose=True``.  Returns the scale tensor (fp32 [1] or [nnz], in this
+        pack's block order).  ``sync=True`` waits, raises if a scale left the representable window, and selects the
+        scale-after-sum kernels for a one-scale matrix; ``sync=False`` only enqueues (per-block kernels)."""
+        if values.device != self.device or values.dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("requantize: values must be bf16 or fp32 on the pack's device")
+        if tuple(values.shape) != (self.nnz, BLK, BLK) or not values.is_contiguous():
+            raise ValueError(f"requantize: values must be contiguous [{self.nnz}, 16, 16], got {tuple(values.shape)}")
+        L = _lib.lib()
+        if self._pos is None:
+            self._pos = torch.from_numpy(octet_positions(self.h_offsets, self.Rb, self.Cb, self.seg_cb, self.h_col)).to(self.device)
+            self._ws = torch.empty(int(L.mortar_requantize_workspace_bytes()) // 8, dtype=torch.float64, device=self.device)
+            self._status = torch.zeros(1, dtype=torch.int32, device=self.device)
+        if scale is not None:
+            scale = scale.detach().to(device=self.device, dtype=torch.float32).reshape(-1).contiguous()
+            if scale.numel() not in (1, self.nnz):
+                raise ValueError(f"requantize: scale must have 1 or {self.nnz} entries")
+            mode = 2 if scale.numel() == 1 else 3
+        else:
+            mode = 1 if per_block else 0
+        out = torch.empty(1 if mode in (0, 2) else self.nnz, dtype=torch.float32, device=self.device)
+        st = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(L.mortar_requantize(self.ref, values.data_ptr(), int(values.dtype == torch.float32), self._pos.data_ptr(),
+                                       self.src_block.data_ptr() if self.src_block is not None else None,
+                                       int(bool(transpose)), mode, float(threshold),
+                                       scale.data_ptr() if scale is not None else None, out.data_ptr(),
+                                       self._status.data_ptr(), self._ws.data_ptr(), st), "mortar_requantize")
+        us = 0.0
+        if sync:
+            if int(self._status.item()):
+                raise ValueError("requantize: a block scale lies outside [2^-100, 2^100] (block zeroed)")
+            if mode in (0, 2) and self.scale_after_sum:
+                us = float(out.to(torch.bfloat16).float().item())
+        if us != self.uniform_scale:
+            self.uniform_scale = us
+            self.struct.uniform_scale = us
+        return out
+
+    def transposed(self) -> "MortarPack":
+        """The pack of W^T [in, out] over the transposed topology (reference: stk matrix.py:107-125), all-zero until
+        ``requantize(values_of_W, transpose=True)`` fills it.  x_grad = y_grad @ W is ``ops.spmm(y_grad, W.transposed())``:
+        the reference's stk_dds(..., transpose_b=False)."""
+        if self._transposed is None:
+            off_t, col_t, src = transpose_topology(self.h_offsets, self.h_col, self.Rb, self.Cb)
+            if (np.diff(off_t) <= 0).any():
+                raise RuntimeError("carved matrix has a block-column with zero kept blocks: W^T cannot be packed")
+            t = MortarPack(None, None, col_t, off_t, self.in_features, self.out_features, self.device,
+                           prefill_stream=self.codes4_o is not None, scale_after_sum=self.scale_after_sum)
+            t.src_block = torch.from_numpy(src).to(self.device)
+            self._transposed = t
+        return self._transposed
 
     def sched(self, rows_per_unit: int) -> torch.Tensor:
         """Device schedule (mortar_schedule_host over the balanced unit order) for plain (1) or gate/up (2) units."""
@@ -200,6 +289,7 @@ class MortarPack:
                 setattr(c, name, getattr(self, name).clone())
         c._scheds = {k: v.clone() for k, v in self._scheds.items()}
         c._worklists = {k: (v[0].clone(), v[1], v[2].clone(), v[3]) for k, v in self._worklists.items()}
+        c._transposed = None
         c.struct = c._make_struct()
         c.ref = C.byref(c.struct)
         return c

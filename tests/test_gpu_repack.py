@@ -1,0 +1,143 @@
+"""GPU parity of the device-side re-pack (ternarise + encode on the device) and of the W^T pack it fills for the
+dX product, against the CPU oracle and the host packer.  Codes and layouts bit-exact; bf16 outputs to 1e-2."""
+import numpy as np
+import pytest
+import torch
+
+from mortar_amd import ops, synth
+from mortar_amd.pack import MortarPack, decode_blocks
+from oracle import mortar_oracle as O
+from util import assert_close_bf16, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+ARRAYS = ("codes", "sdup", "codes_o", "sd_o", "codes4_o")
+
+
+def _values(nnz, seed, dtype):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    v = rng.standard_normal((nnz, 16, 16), dtype=np.float32) * rng.uniform(0.01, 0.1, (nnz, 1, 1)).astype(np.float32)
+    v[rng.random((nnz, 16, 16)) < 0.05] = 0.0
+    v[0, 0, :4] = [0.0, -0.0, 1e-30, -1e-30]
+    t = torch.from_numpy(v).to(dtype)
+    return t, t.float().numpy()
+
+
+def _rule(w, s, thr):
+    """The reference's rule with the scale given, in fp32 as torch computes it (deploy_quant.py:92-94)."""
+    wn = w / np.float32(1.0) / s
+    return (np.sign(wn) * (np.abs(wn) > np.float32(thr))).astype(np.int8)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("per_block", [False, True])
+@pytest.mark.parametrize("shape,seg", [((16 * 12, 16 * 30), None), ((16 * 6, 16 * 352), None)])
+def test_requantize_equals_the_host_pack(dev, dtype, per_block, shape, seg):
+    m = synth.synth_matrix(shape[0], shape[1], 0.25, seed=11, zipf_s=1.2)
+    nnz = m["col_idx"].size
+    vt, v = _values(nnz, 12, dtype)
+    W = MortarPack(None, None, m["col_idx"], m["offsets"], shape[0], shape[1], dev)
+    thr = 0.5
+    s_dev = W.requantize(vt.to(dev), per_block=per_block, threshold=thr).cpu().numpy()
+    # scale: the oracle's mean|w| (fp32 pairwise) against the device's (fp64 sum, rounded once): a few ulps apart at most
+    qo, so = (O.ternary_quantize_per_block if per_block else O.ternary_quantize)(v, thr)
+    np.testing.assert_allclose(s_dev, np.atleast_1d(so), rtol=4e-7, atol=0)
+    # codes: exactly the rule under the device's own scale, and the oracle's codes except on the threshold itself
+    s_full = s_dev[:, None, None] if per_block else s_dev[0]
+    q = _rule(v, s_full, thr)
+    got = decode_blocks(W.codes.cpu().numpy().view(np.uint32))
+    assert np.array_equal(got, q)
+    differ = got != qo
+    assert differ.mean() < 1e-5 and np.all(np.abs(np.abs(v / s_full)[differ] - thr) < 1e-5)
+    # every device array equals what the host packer builds from the same codes and scales
+    H = MortarPack(synth.flat_pack(q), s_dev if per_block else s_dev[:1], m["col_idx"], m["offsets"], shape[0], shape[1], dev)
+    for name in ARRAYS:
+        assert torch.equal(getattr(W, name), getattr(H, name)), name
+    assert W.uniform_scale == H.uniform_scale and (W.uniform_scale != 0) == (not per_block)
+    # and the product through it
+    x = synth.synth_x(70, shape[1], seed=13)
+    ref = O.bcsr_spmm(x, q, O.bf16_round(np.broadcast_to(s_dev, (nnz,)) if per_block else np.full(nnz, s_dev[0], np.float32)),
+                      m["col_idx"], m["offsets"])
+    assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), ref, "spmm after requantize")
+
+
+def test_requantize_given_scales_and_refresh(dev):
+    """Given scales (one or per block), a second refresh with other values, and the asynchronous form."""
+    m = synth.synth_matrix(16 * 8, 16 * 24, 0.3, seed=21)
+    nnz = m["col_idx"].size
+    W = MortarPack(None, None, m["col_idx"], m["offsets"], 16 * 8, 16 * 24, dev)
+    for seed, scale in ((1, np.array([0.037], np.float32)), (2, np.linspace(0.01, 0.2, nnz).astype(np.float32))):
+        vt, v = _values(nnz, seed, torch.bfloat16)
+        s = W.requantize(vt.to(dev), scale=torch.from_numpy(scale), threshold=0.7, sync=False)
+        assert np.array_equal(s.cpu().numpy(), scale) and W.uniform_scale == 0.0
+        q = _rule(v, scale[:, None, None] if scale.size > 1 else scale[0], 0.7)
+        H = MortarPack(synth.flat_pack(q), scale, m["col_idx"], m["offsets"], 16 * 8, 16 * 24, dev)
+        for name in ARRAYS:
+            assert torch.equal(getattr(W, name), getattr(H, name)), (seed, name)
+
+
+def test_requantize_rejects_bad_input(dev):
+    m = synth.synth_matrix(16 * 4, 16 * 8, 0.5, seed=3)
+    nnz = m["col_idx"].size
+    W = MortarPack(None, None, m["col_idx"], m["offsets"], 64, 128, dev)
+    with pytest.raises(ValueError):
+        W.requantize(torch.zeros(nnz, 16, 16, device=dev, dtype=torch.float16))
+    with pytest.raises(ValueError):
+        W.requantize(torch.zeros(nnz + 1, 16, 16, device=dev))
+    with pytest.raises(ValueError):
+        W.requantize(torch.zeros(nnz, 16, 16, device=dev), threshold=-1.0)
+    with pytest.raises(ValueError):                      # scale far outside the bf16 window the kernels accept
+        W.requantize(torch.ones(nnz, 16, 16, device=dev), scale=torch.tensor([1e35]))
+    # all-zero values: scale clamps (1e-8 / 1e-6), every code is 0, products are 0
+    W.requantize(torch.zeros(nnz, 16, 16, device=dev), per_block=True)
+    assert int(W.codes.abs().sum()) == 0
+    y = ops.spmm(torch.ones(5, 128, device=dev, dtype=torch.bfloat16), W)
+    assert float(y.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("per_block", [False, True])
+@pytest.mark.parametrize("M", [3, 200])
+def test_transposed_pack_gives_the_dx_product(dev, per_block, M):
+    """dX = dY @ W through the W^T pack (the reference's dds with the transposed metadata, transpose_b=False)."""
+    shape = (16 * 20, 16 * 12)
+    m = synth.synth_matrix(shape[0], shape[1], 0.3, seed=31, zipf_s=1.2)
+    nnz = m["col_idx"].size
+    vt, v = _values(nnz, 32, torch.bfloat16)
+    W = MortarPack(None, None, m["col_idx"], m["offsets"], shape[0], shape[1], dev)
+    s = W.requantize(vt.to(dev), per_block=per_block).cpu().numpy()
+    Wt = W.transposed()
+    st = Wt.requantize(vt.to(dev), per_block=per_block, transpose=True).cpu().numpy()
+    src = Wt.src_block.cpu().numpy()
+    assert np.array_equal(st, s[src] if per_block else s)
+    # W^T's blocks are W's blocks transposed, in the transposed order
+    cw = decode_blocks(W.codes.cpu().numpy().view(np.uint32))
+    ct = decode_blocks(Wt.codes.cpu().numpy().view(np.uint32))
+    assert np.array_equal(ct, cw[src].transpose(0, 2, 1))
+    dense = O.to_dense(cw.astype(np.float32) * O.bf16_round(np.broadcast_to(s, (nnz,)))[:, None, None],
+                       m["row_idx"], m["col_idx"], shape)
+    dy = synth.synth_x(M, shape[0], seed=33)
+    ref = O.bf16_round(dy).astype(np.float64) @ dense.astype(np.float64)
+    assert_close_bf16(to_np(ops.spmm(to_dev(dy, dev), Wt)), ref.astype(np.float32), "dX")
+
+
+def test_stk_dds_both_orientations(dev):
+    """The operator signature with transpose_b=False (dX = dY @ W) next to the forward orientation, and a refresh
+    after the data tensor changed in place."""
+    import mortar_amd
+    m = synth.synth_matrix(16 * 8, 16 * 6, 0.5, seed=41)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    data = t(O.effective_blocks(m["codes"], m["scales"])).to(torch.bfloat16)
+    dense = O.to_dense(data.float().cpu().numpy(), m["row_idx"], m["col_idx"], (128, 96)).astype(np.float64)
+    z32, z16 = torch.zeros(1, dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int16, device=dev)
+    args = (t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32)
+    x, dy = synth.synth_x(40, 96, seed=42), synth.synth_x(40, 128, seed=43)
+    y = mortar_amd.stk_dds(to_dev(x, dev), data, *args, 96, 128, True)
+    dx = mortar_amd.stk_dds(to_dev(dy, dev), data, *args, 128, 96, False)
+    assert y.shape == (40, 128) and dx.shape == (40, 96) and dx.dtype == torch.bfloat16
+    assert_close_bf16(to_np(y), (O.bf16_round(x) @ dense.T).astype(np.float32), "forward")
+    assert_close_bf16(to_np(dx), (O.bf16_round(dy) @ dense).astype(np.float32), "dX")
+    data.mul_(-2.0)                                     # same storage, new version: both packs must follow
+    y2 = mortar_amd.stk_dds(to_dev(x, dev), data, *args, 96, 128, True)
+    dx2 = mortar_amd.stk_dds(to_dev(dy, dev), data, *args, 128, 96, False)
+    assert_close_bf16(to_np(y2), (-2.0 * (O.bf16_round(x) @ dense.T)).astype(np.float32), "forward refreshed")
+    assert_close_bf16(to_np(dx2), (-2.0 * (O.bf16_round(dy) @ dense)).astype(np.float32), "dX refreshed")

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in mortar_hip.h but not exported"
     assert declared == set(_lib.EXPORTS)
-    assert _lib.lib().mortar_abi_version() == 3
+    assert _lib.lib().mortar_abi_version() == 4
 
 
 def test_encode_round_trip_and_bit_layout():
@@ -310,3 +310,32 @@ def test_bench_refuses_more_than_one_gpu():
     import subprocess, sys
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=60)
     assert r.returncode != 0 and "ONE GPU" in (r.stderr + r.stdout)
+
+
+def test_octet_positions_match_the_octet_layout():
+    """pos[j] must be where mortar_octet_layout_host put block j, for one and for several K segments."""
+    from mortar_amd import pack, synth
+    for shape, seg in (((16 * 9, 16 * 40), 40), ((16 * 7, 16 * 50), 17), ((16 * 5, 16 * 352), 118)):
+        m = synth.synth_matrix(shape[0], shape[1], 0.3, seed=3, zipf_s=1.2)
+        Rb, Cb = shape[0] // 16, shape[1] // 16
+        nnz = m["col_idx"].size
+        codes = (np.arange(nnz * 16, dtype=np.uint64) * 2654435761 % (1 << 32)).astype(np.uint32)
+        sdup = np.arange(1, nnz + 1, dtype=np.uint32)
+        grp, codes_o, sd_o, col_o = pack.octet_layout(m["offsets"], Rb, Cb, seg, codes, sdup, m["col_idx"])
+        pos = pack.octet_positions(m["offsets"], Rb, Cb, seg, m["col_idx"])
+        assert len(set(pos.tolist())) == nnz and pos.max() < sd_o.size
+        assert np.array_equal(sd_o[pos], sdup)
+        co = codes_o.reshape(-1, 16, 4)
+        for j in range(0, nnz, 7):
+            assert np.array_equal(co[pos[j] >> 2, :, pos[j] & 3], codes[j * 16:(j + 1) * 16])
+
+
+def test_transpose_topology_against_the_oracle():
+    """The W^T topology equals the oracle's restatement of stk's _transpose (stable order inside a column)."""
+    from mortar_amd import pack, synth
+    m = synth.synth_matrix(16 * 12, 16 * 30, 0.2, seed=5, zipf_s=1.2)
+    off_t, col_t, src = pack.transpose_topology(m["offsets"], m["col_idx"], 12, 30)
+    ct, ot, bt = O.transpose_meta((16 * 12, 16 * 30), 16, m["row_idx"], m["col_idx"])
+    assert np.array_equal(off_t, ot) and np.array_equal(col_t, ct) and np.array_equal(src, bt)
+    with pytest.raises(ValueError):
+        pack.transpose_topology(m["offsets"], m["col_idx"][::-1].copy(), 12, 30)
