@@ -310,6 +310,24 @@ int mortar_requantize(const mortar_bcsr_t *W, const void *values, int32_t values
                       const int32_t *src_block, int32_t transpose, int32_t scale_mode, float threshold,
                       const float *scale_in, float *scale_out, int32_t *status, void *workspace, void *stream);
 
+/* ---- weight gradient on the topology ------------------------------------------------------------ */
+
+/* out[j] = a[:, 16 rows of block j]^T @ b[:, 16 columns of block j] for every kept block: the dW product of the
+ * carved linear, the reference's stk_sdd_at_b(a, b, data, offsets, row_indices, column_indices) -> [nnz, blk, blk]
+ * (morph/sparse/stk/backend/custom_ops.py:78-96; forward y = x W^T: a = dY [M, out], b = x [M, in]).  bf16 operands,
+ * fp32 accumulation over the M tokens, bf16 result (round to nearest even).
+ *   mortar_sdd_plan_host: the work partition for a topology (host, once).  plan_out = NULL returns the number of
+ *     int32 words needed; otherwise fills plan_out (plan_words = its capacity) and returns the words used;
+ *     plan_out[0] = n_wg.  Upload the plan to the device.
+ *   mortar_sdd_bf16: plan device int32; a bf16 [M, lda >= Rb*16], b bf16 [M, ldb >= Cb*16], 16-byte aligned with
+ *     leading dimensions multiples of 8; acc device fp32 [nnz*256] workspace (token ranges are combined in it with
+ *     atomic adds, so the last fp32 bit of a sum can differ between runs); out device bf16 [nnz,16,16], 16-byte
+ *     aligned.  M = 0 gives zeros. */
+int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb, int32_t *plan_out,
+                             int64_t plan_words);
+int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t Rb, int32_t Cb, int32_t nnz, const uint16_t *a,
+                    int64_t lda, const uint16_t *b, int64_t ldb, int64_t M, float *acc, uint16_t *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -195,6 +195,27 @@ def route_flags(gates: Tensor, d_ff: int, row_act: Tensor | None = None, col_act
     return row_act, col_act
 
 
+def sdd(a: Tensor, b: Tensor, W: MortarPack, out: Tensor | None = None) -> Tensor:
+    """Weight gradient on W's topology: out[j] = a[:, rows of block j]^T @ b[:, columns of block j], bf16 [nnz,16,16]
+    (reference stk_sdd_at_b; for y = x W^T pass a = dY [M, out_features], b = x [M, in_features])."""
+    a, b = _bf16_2d(a, "sdd"), _bf16_2d(b, "sdd")
+    if a.shape[0] != b.shape[0] or a.shape[1] != W.out_features or b.shape[1] != W.in_features:
+        raise ValueError(f"sdd: a {tuple(a.shape)} / b {tuple(b.shape)} do not match the matrix [{W.out_features}, {W.in_features}]")
+    if a.stride(0) % 8 or a.data_ptr() % 16:
+        a = a.contiguous()
+    if b.stride(0) % 8 or b.data_ptr() % 16:
+        b = b.contiguous()
+    plan, n_wg = W.sdd_plan()
+    if out is None:
+        out = torch.empty((W.nnz, BLK, BLK), dtype=torch.bfloat16, device=a.device)
+    elif out.dtype != torch.bfloat16 or tuple(out.shape) != (W.nnz, BLK, BLK) or not out.is_contiguous():
+        raise TypeError("sdd: out must be a contiguous bfloat16 [nnz, 16, 16] tensor")
+    acc = torch.empty(W.nnz * BLK * BLK, dtype=torch.float32, device=a.device)
+    _lib.check(_lib.lib().mortar_sdd_bf16(_p(plan), n_wg, W.Rb, W.Cb, W.nnz, _p(a), a.stride(0), _p(b), b.stride(0),
+                                          a.shape[0], _p(acc), _p(out), _stream(a)), "mortar_sdd_bf16")
+    return out
+
+
 # ----------------------------------------------------------------------------- decode
 
 

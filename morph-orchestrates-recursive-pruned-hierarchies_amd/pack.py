@@ -189,7 +189,7 @@ class MortarPack:
         self.codes4_o = torch.from_numpy(fp4_stream(codes_o).view(np.int32)).to(dev) if prefill_stream else None
         self._scheds: dict[int, torch.Tensor] = {}
         self._worklists: dict[tuple, tuple] = {}
-        self._pos = self._ws = self._status = self.src_block = None
+        self._pos = self._ws = self._status = self.src_block = self._sdd = None
         self._transposed: "MortarPack | None" = None
         self.struct = self._make_struct()
         self.ref = C.byref(self.struct)
@@ -259,6 +259,18 @@ class MortarPack:
             t.src_block = torch.from_numpy(src).to(self.device)
             self._transposed = t
         return self._transposed
+
+    def sdd_plan(self) -> tuple[torch.Tensor, int]:
+        """(device plan, workgroups) of the weight-gradient kernel for this topology: see mortar_sdd_plan_host."""
+        if self._sdd is None:
+            L = _lib.lib()
+            n = _lib.check(L.mortar_sdd_plan_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, None, 0),
+                           "mortar_sdd_plan_host")
+            plan = np.empty(n, dtype=np.int32)
+            _lib.check(L.mortar_sdd_plan_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, _vp(plan), n),
+                       "mortar_sdd_plan_host")
+            self._sdd = (torch.from_numpy(plan).to(self.device), int(plan[0]), plan)
+        return self._sdd[0], self._sdd[1]
 
     def sched(self, rows_per_unit: int) -> torch.Tensor:
         """Device schedule (mortar_schedule_host over the balanced unit order) for plain (1) or gate/up (2) units."""

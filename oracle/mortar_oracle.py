@@ -12,6 +12,8 @@ reference checkout).  How each function is pinned (no reference import is needed
   pack/unpack_ternary      exhaustive over all 256 byte values
   pack_strips / work_list  closed form + partition invariants
   bcsr_spmm                reduces to dense scatter + float64 matmul; special cases
+  dds_dx / sdd_at_b        (backward) reduce to dense float64 matmuls + a gather of the
+                           kept blocks; the adjoint identity <dY, x W^T> = <dY W, x> = <dW, W>
   swiglu_mlp               textbook x*sigmoid(x) + the above
   remoe_gates              brute force on tiny inputs incl. ties; invariants
   route_flags              closed form
@@ -202,6 +204,27 @@ def bcsr_spmm(x: np.ndarray, codes: np.ndarray, scales, col_idx: np.ndarray, off
         y[:, r * blk:(r + 1) * blk] = np.einsum("mjc,jnc->mn", xs, w[lo:hi], optimize=True)
     y = y.astype(np.float32)
     return bf16_round(y) if round_out else y
+
+
+def dds_dx(dy: np.ndarray, codes: np.ndarray, scales, row_idx, col_idx, shape, blk: int = 16,
+           round_out: bool = True) -> np.ndarray:
+    """dX = dY @ W: the dds product with transpose_b=False over the transposed metadata
+    (morph/sparse/stk/backend/custom_ops.py:113-119; kernel triton_kernels.py:170-230 without trans_B).
+    dy float32 array of bf16-representable values [M, out] -> float32 [M, in], rounded to bf16 when round_out."""
+    W = to_dense(effective_blocks(codes, scales), row_idx, col_idx, shape, blk).astype(np.float64)
+    dx = (dy.astype(np.float64) @ W).astype(np.float32)
+    return bf16_round(dx) if round_out else dx
+
+
+def sdd_at_b(a: np.ndarray, b: np.ndarray, row_idx, col_idx, blk: int = 16, round_out: bool = True) -> np.ndarray:
+    """a^T @ b restricted to the kept blocks: out[j, lr, c] = sum_m a[m, row_j*blk+lr] * b[m, col_j*blk+c]
+    (stk_sdd_at_b, morph/sparse/stk/backend/custom_ops.py:78-96; the dW of the carved forward with a = dY, b = x).
+    a [M, out], b [M, in] float32 arrays of bf16-representable values -> float32 [nnz, blk, blk]."""
+    M = a.shape[0]
+    at = a.astype(np.float64).reshape(M, -1, blk)[:, np.asarray(row_idx, dtype=np.int64), :]     # [M, nnz, blk]
+    bt = b.astype(np.float64).reshape(M, -1, blk)[:, np.asarray(col_idx, dtype=np.int64), :]
+    out = np.einsum("mjl,mjc->jlc", at, bt, optimize=True).astype(np.float32)
+    return bf16_round(out) if round_out else out
 
 
 def dense_linear(x: np.ndarray, codes, scales, row_idx, col_idx, shape, blk=16) -> np.ndarray:

@@ -141,3 +141,49 @@ def test_stk_dds_both_orientations(dev):
     dx2 = mortar_amd.stk_dds(to_dev(dy, dev), data, *args, 128, 96, False)
     assert_close_bf16(to_np(y2), (-2.0 * (O.bf16_round(x) @ dense.T)).astype(np.float32), "forward refreshed")
     assert_close_bf16(to_np(dx2), (-2.0 * (O.bf16_round(dy) @ dense)).astype(np.float32), "dX refreshed")
+
+
+# ---------------------------------------------------------------------------------------------- weight gradient
+
+@pytest.mark.parametrize("shape,density,zipf,M", [((16 * 4, 16 * 6), 1.0, None, 32), ((16 * 20, 16 * 12), 0.3, 1.2, 1),
+                                                   ((16 * 20, 16 * 12), 0.3, 1.2, 77), ((16 * 40, 16 * 30), 0.25, None, 600),
+                                                   ((16 * 6, 16 * 352), 0.25, 1.2, 200), ((16 * 70, 16 * 16), 0.1, None, 4096)])
+def test_sdd_weight_gradient(dev, shape, density, zipf, M):
+    """dW on the topology against the oracle (one and several K segments, ragged token counts, split token ranges)."""
+    m = synth.synth_matrix(shape[0], shape[1], density, seed=51, zipf_s=zipf)
+    W = synth.to_pack(m, dev)
+    a, b = synth.synth_x(M, shape[0], seed=52), synth.synth_x(M, shape[1], seed=53)
+    got = to_np(ops.sdd(to_dev(a, dev), to_dev(b, dev), W))
+    ref = O.sdd_at_b(O.bf16_round(a), O.bf16_round(b), m["row_idx"], m["col_idx"])
+    assert_close_bf16(got, ref, f"dW {shape} M={M}")
+
+
+def test_sdd_exact_positions(dev):
+    """One-hot operands: a single token with a single 1 in a and in b gives a single 1 in exactly one block element."""
+    m = synth.synth_matrix(16 * 3, 16 * 5, 1.0, seed=1)
+    W = synth.to_pack(m, dev)
+    for tok, fa, fb in ((0, 0, 0), (5, 17, 33), (31, 47, 79), (40, 16, 15)):
+        a = torch.zeros(41, 48, dtype=torch.bfloat16, device=dev); a[tok, fa] = 1.0
+        b = torch.zeros(41, 80, dtype=torch.bfloat16, device=dev); b[tok, fb] = 1.0
+        got = ops.sdd(a, b, W).float().cpu().numpy()
+        want = np.zeros_like(got)
+        j = int(np.nonzero((m["row_idx"] == fa // 16) & (m["col_idx"] == fb // 16))[0][0])
+        want[j, fa % 16, fb % 16] = 1.0
+        assert np.array_equal(got, want), (tok, fa, fb)
+
+
+def test_sdd_edge_cases(dev):
+    m = synth.synth_matrix(16 * 4, 16 * 6, 0.5, seed=2)
+    W = synth.to_pack(m, dev)
+    z = ops.sdd(torch.zeros(0, 64, dtype=torch.bfloat16, device=dev), torch.zeros(0, 96, dtype=torch.bfloat16, device=dev), W)
+    assert z.shape == (W.nnz, 16, 16) and float(z.float().abs().max()) == 0.0
+    with pytest.raises(ValueError):
+        ops.sdd(torch.zeros(4, 64, dtype=torch.bfloat16, device=dev), torch.zeros(5, 96, dtype=torch.bfloat16, device=dev), W)
+    with pytest.raises(ValueError):
+        ops.sdd(torch.zeros(4, 96, dtype=torch.bfloat16, device=dev), torch.zeros(4, 96, dtype=torch.bfloat16, device=dev), W)
+    # strided views of wider buffers
+    a = torch.randn(50, 128, device=dev).to(torch.bfloat16)
+    b = torch.randn(50, 192, device=dev).to(torch.bfloat16)
+    got = to_np(ops.sdd(a[:, 64:], b[:, :96], W))
+    ref = O.sdd_at_b(to_np(a[:, 64:]), to_np(b[:, :96]), m["row_idx"], m["col_idx"])
+    assert_close_bf16(got, ref, "strided")

@@ -339,3 +339,34 @@ def test_transpose_topology_against_the_oracle():
     assert np.array_equal(off_t, ot) and np.array_equal(col_t, ct) and np.array_equal(src, bt)
     with pytest.raises(ValueError):
         pack.transpose_topology(m["offsets"], m["col_idx"][::-1].copy(), 12, 30)
+
+
+def test_sdd_plan_partitions_the_blocks():
+    """Every kept block appears exactly once, inside its workgroup's row window and K segment."""
+    from mortar_amd import synth
+    L = _lib.lib()
+    for shape in ((16 * 40, 16 * 30), (16 * 9, 16 * 352), (16 * 704, 16 * 128)):
+        m = synth.synth_matrix(shape[0], shape[1], 0.25, seed=9, zipf_s=1.2)
+        Rb, Cb = shape[0] // 16, shape[1] // 16
+        off, col = np.ascontiguousarray(m["offsets"], np.int32), np.ascontiguousarray(m["col_idx"], np.int16)
+        vp = lambda a: a.ctypes.data_as(C.c_void_p)
+        n = L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, None, 0)
+        plan = np.empty(n, np.int32)
+        assert L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, vp(plan), n) == n
+        assert L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, vp(plan), n - 1) < 0
+        n_wg, seg_cb, nseg = plan[0], plan[1], plan[2]
+        G = (n - 4 - 4 * n_wg) // (2 * n_wg)
+        desc = plan[4:4 + 4 * n_wg].reshape(n_wg, 4)
+        ej = plan[4 + 4 * n_wg:4 + 4 * n_wg + n_wg * G].reshape(n_wg, G)
+        eo = plan[4 + 4 * n_wg + n_wg * G:].reshape(n_wg, G)
+        assert nseg == -(-Cb // seg_cb) and seg_cb <= 128
+        seen = ej[ej >= 0]
+        assert sorted(seen.tolist()) == list(range(col.size))
+        assert ((ej >= 0) == (eo >= 0)).all()
+        row_of = np.repeat(np.arange(Rb), np.diff(off))
+        for w in range(n_wg):
+            row0, nrows, seg, nb = desc[w]
+            js = ej[w][ej[w] >= 0]
+            assert nb == js.size and 1 <= nrows <= 16
+            assert np.array_equal(eo[w][ej[w] >= 0] >> 16, row_of[js] - row0) and (row_of[js] - row0 < nrows).all()
+            assert np.array_equal(eo[w][ej[w] >= 0] & 0xffff, col[js] - seg * seg_cb) and (col[js] // seg_cb == seg).all()

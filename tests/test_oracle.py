@@ -342,3 +342,32 @@ def test_golden_mlp_slice_pins_swiglu_and_gating():
         _, hc, yc = c_oracle.mlp_bf16(z["x_bits"], gu, dn, 704, gates=None if g is None else g.astype(np.float32))
         assert np.abs(O.bf16_from_bits(hc) - O.bf16_from_bits(z[hk])).max() <= 2 ** -7 * np.abs(O.bf16_from_bits(z[hk])).max()
         assert np.abs(O.bf16_from_bits(yc) - O.bf16_from_bits(z[yk])).max() <= 1e-2 * np.abs(O.bf16_from_bits(z[yk])).max()
+
+
+# ---- backward products ------------------------------------------------------------------------------
+
+def test_backward_products_against_dense_matmul_and_adjoint_identity():
+    """dds_dx and sdd_at_b reduce to dense matmuls (+ gather of the kept blocks), and satisfy the adjoint
+    identities of y = x W^T: <dY, y> = <dY W, x> = <dW, blocks of W>.  A transposed operand, a swapped row/column
+    index or a block stored transposed fails one of these."""
+    rng = np.random.default_rng(5)
+    Rb, Cb, M = 5, 7, 37
+    mask = rng.random((Rb, Cb)) < 0.5
+    mask[np.arange(Rb), rng.integers(0, Cb, Rb)] = True
+    r, c = np.nonzero(mask)
+    nnz = r.size
+    codes = rng.integers(-1, 2, (nnz, 16, 16)).astype(np.int8)
+    scales = O.bf16_round(rng.uniform(0.01, 0.1, nnz).astype(np.float32))
+    x = O.bf16_round(rng.standard_normal((M, Cb * 16)).astype(np.float32))
+    dy = O.bf16_round(rng.standard_normal((M, Rb * 16)).astype(np.float32))
+    W = O.to_dense(O.effective_blocks(codes, scales), r, c, (Rb * 16, Cb * 16)).astype(np.float64)
+    dx = O.dds_dx(dy, codes, scales, r, c, (Rb * 16, Cb * 16), round_out=False)
+    np.testing.assert_allclose(dx, dy.astype(np.float64) @ W, rtol=1e-6, atol=1e-6)
+    dw = O.sdd_at_b(dy, x, r, c, round_out=False)
+    full = dy.astype(np.float64).T @ x.astype(np.float64)                   # dense dW [out, in]
+    for j in range(nnz):
+        np.testing.assert_allclose(dw[j], full[r[j] * 16:(r[j] + 1) * 16, c[j] * 16:(c[j] + 1) * 16], rtol=1e-6, atol=1e-5)
+    y = x.astype(np.float64) @ W.T
+    lhs = float((dy * y).sum())
+    np.testing.assert_allclose(float((dx.astype(np.float64) * x).sum()), lhs, rtol=1e-5)
+    np.testing.assert_allclose(float((dw.astype(np.float64) * O.effective_blocks(codes, scales)).sum()), lhs, rtol=1e-5)
