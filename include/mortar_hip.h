@@ -320,11 +320,12 @@ int mortar_requantize(const mortar_bcsr_t *W, const void *values, int32_t values
  *     int32 words needed; otherwise fills plan_out (plan_words = its capacity) and returns the words used;
  *     plan_out[0] = n_wg.  Upload the plan to the device.
  *   mortar_sdd_bf16: plan device int32; a bf16 [M, lda >= Rb*16], b bf16 [M, ldb >= Cb*16], 16-byte aligned with
- *     leading dimensions multiples of 8; acc device fp32 [nnz*256] workspace (token ranges are combined in it with
- *     atomic adds, so the last fp32 bit of a sum can differ between runs); out device bf16 [nnz,16,16], 16-byte
- *     aligned.  M = 0 gives zeros. */
+ *     leading dimensions multiples of 8; acc device workspace of mortar_sdd_workspace_bytes(n_wg, nnz, M) bytes,
+ *     16-byte aligned (every token range writes its fp32 sums to a slab of its own, and a last pass adds the slabs in
+ *     a fixed order: results are reproducible); out device bf16 [nnz,16,16], 16-byte aligned.  M = 0 gives zeros. */
 int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb, int32_t *plan_out,
                              int64_t plan_words);
+int64_t mortar_sdd_workspace_bytes(int32_t n_wg, int32_t nnz, int64_t M);
 int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t Rb, int32_t Cb, int32_t nnz, const uint16_t *a,
                     int64_t lda, const uint16_t *b, int64_t ldb, int64_t M, float *acc, uint16_t *out, void *stream);
 

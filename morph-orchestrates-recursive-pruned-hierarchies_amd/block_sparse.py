@@ -31,6 +31,32 @@ def _stk_transpose(size, data, row_indices, column_indices, offsets):
     return column_indices_t, offsets_t, block_offsets_t
 
 
+class _MortarLinearFn(torch.autograd.Function):
+    """y = x W^T on the carved topology with the reference's backward (morph/sparse/stk/backend/custom_ops.py:99-136):
+    dx = dy W through the W^T pack, d(mortar_data) = dy^T x restricted to the kept blocks."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, data: Tensor, layer: "CMSBlockLinear") -> Tensor:
+        W = layer.mortar_pack()
+        ctx.layer = layer
+        ctx.save_for_backward(x)
+        ctx.data_dtype = data.dtype
+        return ops.gemv(x, W) if 0 < x.shape[0] <= 64 else ops.spmm(x, W)
+
+    @staticmethod
+    def backward(ctx, dy: Tensor):
+        (x,) = ctx.saved_tensors
+        layer = ctx.layer
+        dy = dy if dy.dtype == torch.bfloat16 else dy.to(torch.bfloat16)
+        dy = dy.contiguous()
+        dx = ddata = None
+        if ctx.needs_input_grad[0]:
+            dx = ops.spmm(dy, layer.mortar_pack_t())
+        if ctx.needs_input_grad[1]:
+            ddata = ops.sdd(dy, x, layer.mortar_pack()).to(ctx.data_dtype)
+        return dx, ddata, None
+
+
 class CMSBlockLinear(nn.Module):
     def __init__(self, in_features: int, out_features: int, tile_size: int = 16, density: float = 1.0,
                  bias: bool = True, score_ema_alpha: float = 0.95, device=None, dtype=None) -> None:
@@ -48,6 +74,7 @@ class CMSBlockLinear(nn.Module):
         self._dense_mode, self._mortar, self._mortar_blocking = True, False, 0
         self._values_ternary_mode, self._values_threshold = False, 0.5
         self._pack: MortarPack | None = None
+        self._pack_key = self._pack_t_key = None
 
     # ------------------------------------------------------------------ masks / carve
 
@@ -140,33 +167,69 @@ class CMSBlockLinear(nn.Module):
         return d + (scale * q - d).detach()
 
     def mortar_pack(self) -> MortarPack:
-        """Device weight format for the HIP kernels, built once (topology and values are frozen at deploy)."""
-        if self._pack is not None:
-            return self._pack
+        """Device weight format for the HIP kernels.  A deployed layer (mortar_packed / mortar_scale) is packed once
+        on the host.  A layer in values-ternary QAT keeps its topology packed once and has the values ternarised and
+        encoded on the device whenever ``mortar_data`` changed (one launch instead of the reference's per-forward
+        torch ternarisation, block_sparse.py:909-919)."""
         if not self._mortar:
             raise RuntimeError("mortar_pack() requires a carved layer")
         if self._mortar_blocking != 16:
             raise ValueError(f"the gfx950 MORTAR runtime executes carve(blocking=16); this layer was carved at {self._mortar_blocking}")
         if "mortar_packed" in self._buffers:
-            packed, scale = self.mortar_packed, self.mortar_scale
-        elif self._values_ternary_mode:
-            q, scale = _ternary_quantize(self.mortar_data.data, self._values_threshold)
-            packed = pack_ternary_codes(q)
-        else:
+            if self._pack is None:
+                self._pack = MortarPack(self.mortar_packed, self.mortar_scale, self.mortar_column_indices, self.mortar_offsets,
+                                        self.out_features, self.in_features, self.mortar_offsets.device)
+            return self._pack
+        if not self._values_ternary_mode:
             raise RuntimeError("carved layer holds non-ternary values: call pack_mortar_ternary() or "
                                "enable_values_ternary() first (the MORTAR runtime executes ternary blocks only)")
-        self._pack = MortarPack(packed, scale, self.mortar_column_indices, self.mortar_offsets,
-                                self.out_features, self.in_features, self.mortar_offsets.device)
+        d = self.mortar_data
+        if not d.is_cuda:
+            if self._pack is None:        # host path (no GPU): pack once from the current values
+                q, scale = _ternary_quantize(d.data, self._values_threshold)
+                self._pack = MortarPack(pack_ternary_codes(q), scale, self.mortar_column_indices, self.mortar_offsets,
+                                        self.out_features, self.in_features, d.device)
+            return self._pack
+        if self._pack is None:
+            self._pack = MortarPack(None, None, self.mortar_column_indices, self.mortar_offsets, self.out_features,
+                                    self.in_features, d.device)
+            self._pack_key = self._pack_t_key = None
+        key = (d.data_ptr(), d._version)
+        if self._pack_key != key:
+            self._pack.requantize(self._values(), threshold=self._values_threshold, sync=False)
+            self._pack_key = key
         return self._pack
+
+    def mortar_pack_t(self) -> MortarPack:
+        """The pack of W^T for the dX product (QAT layers on the GPU), refreshed like ``mortar_pack``."""
+        if "mortar_packed" in self._buffers or not self.mortar_data.is_cuda:
+            raise RuntimeError("mortar_pack_t(): the backward needs a QAT layer (mortar_data) on the GPU")
+        t = self.mortar_pack().transposed()
+        if self._pack_t_key != self._pack_key:
+            t.requantize(self._values(), threshold=self._values_threshold, transpose=True, sync=False)
+            self._pack_t_key = self._pack_key
+        return t
+
+    def _values(self) -> Tensor:
+        d = self.mortar_data.detach()
+        if d.dtype not in (torch.bfloat16, torch.float32):
+            d = d.float()
+        return d.contiguous()
 
     def _forward_mortar(self, x: Tensor) -> Tensor:
         """Carved forward y = x @ W_sparse^T (+bias).  Reference: block_sparse.py:921-970 (flatten leading
-        dims, bf16 operands, fp32 accumulate, output in the activation dtype; no M padding is needed)."""
+        dims, bf16 operands, fp32 accumulate, output in the activation dtype; no M padding is needed).  With autograd
+        on a QAT layer the backward runs dX through the W^T pack and dW through the topology-restricted product
+        (reference: custom_ops.py:99-136), the gradient passing straight through the ternarisation into mortar_data."""
         lead = x.shape[:-1]
         x2 = x.reshape(-1, self.in_features)
         xb = x2 if x2.dtype == torch.bfloat16 else x2.to(torch.bfloat16)
-        W = self.mortar_pack()
-        y = ops.gemv(xb, W) if 0 < xb.shape[0] <= 64 else ops.spmm(xb, W)
+        trainable = "mortar_packed" not in self._buffers and self._values_ternary_mode and xb.is_cuda
+        if trainable and torch.is_grad_enabled() and (xb.requires_grad or self.mortar_data.requires_grad):
+            y = _MortarLinearFn.apply(xb, self.mortar_data, self)
+        else:
+            W = self.mortar_pack()
+            y = ops.gemv(xb, W) if 0 < xb.shape[0] <= 64 else ops.spmm(xb, W)
         if y.dtype != x.dtype:
             y = y.to(x.dtype)
         if self.bias is not None:

@@ -5,17 +5,21 @@
 // bf16 operands, fp32 accumulation, output in the operand dtype.
 //
 // Shape of the work: the contraction runs over tokens, so both MFMA operands need 8 tokens of ONE feature per lane
-// while memory holds 16 features of ONE token per 32 bytes.  The tiles are staged row-major (straight 16-byte
-// copies) and read back with the transposing LDS load (ds_read_b64_tr_b16): 16 lanes hand in the addresses of 4
-// token rows x 4 chunks of 4 features and each lane gets 4 tokens of one feature.  A workgroup keeps the fp32 tiles
-// of up to WAVES*NB blocks of a few consecutive block-rows in registers and walks the tokens in steps of 32; per
-// step it stages the 32 x (columns of its K segment) slice of b once and the slice of a for its rows.  Workgroups
-// that share a token range run on the same XCD (the range index is the low part of the workgroup index), so the
-// slice of b is fetched from HBM about once per XCD and served from L2 after that.  Token ranges are combined with
-// fp32 atomic adds into a workspace; a last pass rounds to bf16.
+// while memory holds 16 features of ONE token per 32 bytes.  The slices are staged row-major with direct
+// global->LDS loads (whole 128-byte lines: 4 block-columns of 8 tokens per instruction) and read back with the
+// transposing LDS load (ds_read_b64_tr_b16): 16 lanes hand in the addresses of 4 token rows x 4 pieces of 4
+// features and each lane gets 4 tokens of one feature.  A workgroup keeps the fp32 tiles of up to WAVES*NB blocks of
+// a few consecutive block-rows in registers and walks the tokens in steps of 32; per step it stages the
+// 32 x (columns of its K segment) slice of b once and the slice of a for its rows, into one of two buffers: the
+// loads of the next step are in flight while the current one multiplies.  Workgroups that share a token range run on the same XCD (the range index
+// is the low part of the workgroup index), so a slice of b is fetched from HBM about once per XCD and served from
+// L2 after that.  Every token range writes its fp32 sums to its own slab of the workspace; a last pass adds the
+// slabs in a fixed order and rounds to bf16, so results are reproducible.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <climits>
+#include <cstdint>
 #include <vector>
 
 #include "mortar_internal.h"
@@ -25,9 +29,13 @@ namespace {
 constexpr int SDD_WAVES = 16;
 constexpr int SDD_NB = 22;                       // blocks per wavefront (4 accumulator registers each)
 constexpr int SDD_G = SDD_WAVES * SDD_NB;        // blocks per workgroup
-constexpr int SDD_RMAX = 16;                     // block-rows per workgroup (slice of a in LDS)
-constexpr int SDD_SEG = 128;                     // block-columns per K segment (slice of b in LDS)
-constexpr int SDD_XS = 1024 + 32;                // bytes per (block-column, 32 tokens) tile: 32 B per token + skew
+constexpr int SDD_RMAX = 32;                     // block-rows per workgroup (slice of a in LDS)
+constexpr int SDD_SEG = 44;                      // block-columns per K segment (slice of b in LDS)
+constexpr int SDD_TARGET_WGS = 256;              // workgroups wanted in flight (one per CU: two slice buffers each)
+constexpr int SDD_NQ = SDD_SEG / 4;              // quads of block-columns per segment
+constexpr int SDD_CS = 1024 + 32;                // LDS bytes per chunk = 8 tokens x 128 bytes (a quad's line) + skew
+constexpr int SDD_QS = 4 * SDD_CS;               // LDS bytes per quad: 32 tokens
+constexpr int SDD_BUF = (SDD_NQ + SDD_RMAX / 4) * SDD_QS;    // one buffer: the slice of b, then the slice of a
 constexpr int SDD_STEP = 32;                     // tokens per step = K of one MFMA
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -41,7 +49,7 @@ struct SddArgs {
     int64_t lda, ldb, M;
     float *acc;
     uint16_t *out;
-    int32_t Cb, seg_cb, tsplit, steps_per_split, nsteps;
+    int32_t Cb, tsplit, steps_per_split, nsteps, nnz;
 };
 
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
@@ -50,16 +58,29 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
     return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
 }
 
-// 8 tokens of one feature: tokens 4g .. 4g+3 and 16+4g .. 16+4g+3 of the 32-token tile at `tile` (LDS byte address of
-// a [32 tokens][16 features] bf16 tile), feature = lane & 15, g = lane >> 4.  `off` = this lane's chunk address.
+// 8 tokens of one feature (= lane & 15) of the block-column (or block-row) whose first token sits at LDS byte `tile`:
+// group g = lane >> 4 gets tokens {8r + g} and {8r + 4 + g}, r = 0..3 - one token of each 8-token chunk per read, which
+// spreads the 32 lanes served together over all banks.  Both operands use the same order, so the contraction is
+// unchanged.  `off` = this lane's row/piece address inside the quad.
 __device__ __forceinline__ bf16x8 read_tr(const char *smem, int tile, int off) {
     typedef __attribute__((address_space(3))) s16x4 *lds_ptr;
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(smem + tile + off));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(smem + tile + off + 16 * 32));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(smem + tile + off + 4 * 128));
     union { s16x4 h[2]; bf16x8 v; } u;
     u.h[0] = lo;
     u.h[1] = hi;
     return u.v;
+}
+
+// Asynchronous 16-byte-per-lane copy global -> LDS: lane l's 16 bytes land at lds_base + 16 * l.  Written as inline
+// assembly so that the compiler does not make the LDS reads of the other buffer wait for it; the caller waits with
+// s_waitcnt vmcnt(0) and a barrier before the destination is read.
+__device__ __forceinline__ void load_to_lds_async(const void *gsrc, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gsrc) : "memory", "m0");
+}
+
+__device__ __forceinline__ uint32_t lds_addr(const char *p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
 }
 
 __global__ __launch_bounds__(SDD_WAVES * 64) void sdd_kernel(SddArgs p) {
@@ -70,70 +91,93 @@ __global__ __launch_bounds__(SDD_WAVES * 64) void sdd_kernel(SddArgs p) {
     const int n_wg = p.plan[0];
     const int32_t *desc = p.plan + 4 + wg * 4;
     const int row0 = desc[0], nrows = desc[1], seg = desc[2];
-    const int c0 = seg * p.seg_cb;
-    const int ncb = min(p.seg_cb, p.Cb - c0);
-    // this wavefront's blocks: block index (-1 = none) and (row slot << 16 | column in the segment) (-1 = none)
+    const int seg_cb = p.plan[1];
+    const int c0 = seg * seg_cb;
+    const int ncb = min(seg_cb, p.Cb - c0);
+    const int nq = (ncb + 3) >> 2, nrq = (nrows + 3) >> 2;          // quads of block-columns / block-rows
+    // this wavefront's blocks: block index (-1 = none) and (row slot << 20 | LDS byte offset of the column's tile);
+    // the second list stays in scalar registers for the whole kernel
     const int32_t *ent_j = p.plan + 4 + n_wg * 4 + (int64_t)(wg * SDD_WAVES + wave) * SDD_NB;
     const int32_t *ent_o = ent_j + (int64_t)n_wg * SDD_G;
+    int eo[SDD_NB];
+#pragma unroll
+    for (int b = 0; b < SDD_NB; ++b) eo[b] = __builtin_amdgcn_readfirstlane(ent_o[b]);
+    uint32_t new_row = 1u;                // bit b: slot b is in another block-row than slot b - 1 (reload the a operand)
+#pragma unroll
+    for (int b = 1; b < SDD_NB; ++b) new_row |= (uint32_t)((eo[b] >> 20) != (eo[b - 1] >> 20)) << b;
+    new_row = __builtin_amdgcn_readfirstlane(new_row);
     f32x4 acc[SDD_NB];
 #pragma unroll
     for (int b = 0; b < SDD_NB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const int a_base = SDD_SEG * SDD_XS;                                     // slice of a behind the slice of b
-    const int tr_off = (4 * (lane >> 4) + ((lane & 15) >> 2)) * 32 + (lane & 3) * 8;
+    const int tr_off = ((lane & 15) >> 2) * SDD_CS + (lane >> 4) * 128 + (lane & 3) * 8;
+    // staging role of this lane inside one instruction: token 8c + (lane >> 3), 16-byte piece lane & 7 of the 128-byte line
+    const int st_tok = lane >> 3, st_piece = lane & 7;
     const int s_begin = ts * p.steps_per_split, s_end = min(p.nsteps, s_begin + p.steps_per_split);
-    for (int s = s_begin; s < s_end; ++s) {
+
+    // Stage the slices of step s into buffer `buf` with direct global->LDS loads (asynchronous, no registers held).
+    // One wavefront instruction moves 8 tokens x one 128-byte line (4 block-columns, or 4 block-rows of a) into 1 KB
+    // of contiguous LDS.  Rows past M are not loaded; in the one partial step they are cleared with plain stores
+    // (disjoint addresses from the loads).
+    auto stage = [&](int s, int buf) {
         const int64_t t0 = (int64_t)s * SDD_STEP;
-        __syncthreads();                                                      // previous step's reads are done
-        // slice of b: 32 tokens x ncb block-columns; a wavefront copies whole token rows, 16 bytes per lane
-        for (int tok = wave; tok < SDD_STEP; tok += SDD_WAVES) {
-            const bool live = t0 + tok < p.M;
-            const uint16_t *src = p.b + (t0 + tok) * p.ldb + (int64_t)c0 * 16;
-            for (int ch = lane; ch < ncb * 2; ch += 64) {
-                u32x4 v = {0u, 0u, 0u, 0u};
-                if (live) v = *reinterpret_cast<const u32x4 *>(src + ch * 8);
-                *reinterpret_cast<u32x4 *>(smem + (ch >> 1) * SDD_XS + tok * 32 + (ch & 1) * 16) = v;
+        char *dst = smem + buf * SDD_BUF;
+        const bool partial = t0 + SDD_STEP > p.M;
+        for (int i = wave; i < (nq + nrq) * 4; i += SDD_WAVES) {
+            const int q = i >> 2, c = i & 3;
+            const int64_t t = t0 + 8 * c + st_tok;
+            const int qq = q < nq ? q : SDD_NQ + q - nq;
+            if (partial && t >= p.M)
+                *reinterpret_cast<u32x4 *>(dst + qq * SDD_QS + c * SDD_CS + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+            if (q < nq) {
+                if (t < p.M && 4 * q + (st_piece >> 1) < ncb)
+                    load_to_lds_async(p.b + t * p.ldb + (int64_t)(c0 + 4 * q) * 16 + st_piece * 8,
+                                      __builtin_amdgcn_readfirstlane(lds_addr(dst + qq * SDD_QS + c * SDD_CS)));
+            } else {
+                if (t < p.M && 4 * (q - nq) + (st_piece >> 1) < nrows)
+                    load_to_lds_async(p.a + t * p.lda + (int64_t)(row0 + 4 * (q - nq)) * 16 + st_piece * 8,
+                                      __builtin_amdgcn_readfirstlane(lds_addr(dst + qq * SDD_QS + c * SDD_CS)));
             }
         }
-        // slice of a: 32 tokens x nrows block-rows
-        for (int idx = tid; idx < SDD_STEP * SDD_RMAX * 2; idx += SDD_WAVES * 64) {
-            const int tok = idx >> 5, rs = (idx >> 1) & (SDD_RMAX - 1), half = idx & 1;
-            if (rs < nrows) {
-                u32x4 v = {0u, 0u, 0u, 0u};
-                if (t0 + tok < p.M)
-                    v = *reinterpret_cast<const u32x4 *>(p.a + (t0 + tok) * p.lda + (int64_t)(row0 + rs) * 16 + half * 8);
-                *reinterpret_cast<u32x4 *>(smem + a_base + rs * SDD_XS + tok * 32 + half * 16) = v;
-            }
-        }
-        __syncthreads();
-        // the entries are read again every step (scalar loads) instead of living in registers across the loop
-        const int32_t *eo = ent_o;
-        asm volatile("" : "+s"(eo));
-        int rs_prev = -1;
+    };
+
+    if (s_begin < s_end) stage(s_begin, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    int buf = 0;
+    for (int s = s_begin; s < s_end; ++s) {
+        if (s + 1 < s_end) stage(s + 1, buf ^ 1);            // in flight while this step multiplies
+        const char *cur = smem + buf * SDD_BUF;
+        // re-materialise the flag word every step: otherwise the 22 loop-invariant tests are hoisted as 22 lane masks
+        uint32_t nr = new_row;
+        asm volatile("" : "+s"(nr));
+        nr = __builtin_amdgcn_readfirstlane(nr);
         bf16x8 A = {};
+        bf16x8 Bn = read_tr(cur, eo[0] & 0xfffff, tr_off);
 #pragma unroll
         for (int b = 0; b < SDD_NB; ++b) {
-            const int e = eo[b];
-            if (e >= 0) {
-                const int rs = e >> 16, cr = e & 0xffff;
-                if (rs != rs_prev) {
-                    A = read_tr(smem, a_base + rs * SDD_XS, tr_off);
-                    rs_prev = rs;
-                }
-                const bf16x8 B = read_tr(smem, cr * SDD_XS, tr_off);
-                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, B, acc[b], 0, 0, 0);
+            if (nr & (1u << b)) {                 // (an empty slot repeats a valid tile: its sum is never stored)
+                const int rs = eo[b] >> 20;
+                A = read_tr(cur, SDD_NQ * SDD_QS + (rs >> 2) * SDD_QS + (rs & 3) * 32, tr_off);
             }
+            const bf16x8 B = Bn;
+            if (b + 1 < SDD_NB) Bn = read_tr(cur, eo[b + 1] & 0xfffff, tr_off);
+            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, B, acc[b], 0, 0, 0);
         }
+        __builtin_amdgcn_s_waitcnt(0);                       // the next step's slices have landed
+        __syncthreads();                                     // ... for every wavefront, and this buffer is free again
+        buf ^= 1;
     }
     // accumulator register r of lane (column = lane & 15, g = lane >> 4) is out[4g + r][column]
     const int oc = lane & 15, og = lane >> 4;
+    float *part = p.acc + (int64_t)ts * p.nnz * 256;
 #pragma unroll
     for (int b = 0; b < SDD_NB; ++b) {
-        const int j = ent_j[b];
+        const int j = __builtin_amdgcn_readfirstlane(ent_j[b]);
         if (j >= 0) {
             const int64_t base = (int64_t)j * 256 + (4 * og) * 16 + oc;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                if (p.tsplit > 1) atomicAdd(p.acc + base + r * 16, acc[b][r]);
+                if (p.tsplit > 1) part[base + r * 16] = acc[b][r];
                 else p.out[base + r * 16] = f32_to_bf16(acc[b][r]);
             }
         }
@@ -145,10 +189,12 @@ __global__ __launch_bounds__(256) void sdd_zero_kernel(float *acc, int64_t n4) {
     if (i < n4) reinterpret_cast<f32x4 *>(acc)[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
-__global__ __launch_bounds__(256) void sdd_round_kernel(const float *acc, uint16_t *out, int64_t n4) {
+// out = bf16(sum over the token ranges, in range order)
+__global__ __launch_bounds__(256) void sdd_round_kernel(const float *acc, uint16_t *out, int64_t n4, int tsplit) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n4) {
-        const f32x4 v = reinterpret_cast<const f32x4 *>(acc)[i];
+        f32x4 v = reinterpret_cast<const f32x4 *>(acc)[i];
+        for (int t = 1; t < tsplit; ++t) v += reinterpret_cast<const f32x4 *>(acc)[i + (int64_t)t * n4];
         uint2 o;
         o.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
         o.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
@@ -159,14 +205,14 @@ __global__ __launch_bounds__(256) void sdd_round_kernel(const float *acc, uint16
 }  // namespace
 
 // Plan: {n_wg, seg_cb, nseg, 0}, then per workgroup {first row, rows, segment, blocks}, then per (workgroup, wavefront,
-// slot) the block index or -1, then per (workgroup, wavefront, slot) (row - first row) << 16 | (column - segment start)
-// or -1.
+// slot) the block index or -1, then per (workgroup, wavefront, slot) (row - first row) << 20 | LDS byte offset of the
+// tile of (column - segment start); an empty slot repeats the workgroup's last block there.
 extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
                                         int32_t *plan_out, int64_t plan_words) {
     const int rc = mortar_check_bcsr_host(row_ptr, col, Rb, Cb);
     if (rc) return rc;
     const int nseg = (Cb + SDD_SEG - 1) / SDD_SEG;
-    const int seg_cb = (Cb + nseg - 1) / nseg;
+    const int seg_cb = ((Cb + nseg - 1) / nseg + 3) & ~3;          // whole 128-byte lines
     struct Wg { int row0, nrows, seg; std::vector<int32_t> j, o; };
     std::vector<Wg> wgs;
     for (int sg = 0; sg < nseg; ++sg) {
@@ -187,7 +233,8 @@ extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *c
             cur.nrows = r - cur.row0 + 1;
             for (int j = lo; j < hi; ++j) {
                 cur.j.push_back(j);
-                cur.o.push_back(((r - cur.row0) << 16) | (col[j] - sg * seg_cb));
+                const int cr = col[j] - sg * seg_cb;
+                cur.o.push_back(((r - cur.row0) << 20) | ((cr >> 2) * SDD_QS + (cr & 3) * 32));
             }
         }
         flush();
@@ -205,10 +252,33 @@ extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *c
         for (int i = 0; i < SDD_G; ++i) {
             const bool ok = i < (int)wgs[w].j.size();
             ent_j[w * SDD_G + i] = ok ? wgs[w].j[i] : -1;
-            ent_o[w * SDD_G + i] = ok ? wgs[w].o[i] : -1;
+            ent_o[w * SDD_G + i] = ok ? wgs[w].o[i] : wgs[w].o.back();
         }
     }
     return words;
+}
+
+// Token ranges for M tokens over n_wg row groups.  One workgroup runs per CU, so the launch takes
+// ceil(n_wg * ranges / CUs) rounds of ceil(steps / ranges) steps; every extra range also adds one slab of fp32 sums
+// to write and read back, priced here at about six steps.  The cheapest count of ranges wins.
+static void sdd_split(int32_t n_wg, int64_t M, int &nsteps, int &steps_per_split, int &tsplit) {
+    nsteps = (int)((M + SDD_STEP - 1) / SDD_STEP);
+    int best = 1;
+    int64_t best_cost = INT64_MAX;
+    for (int t = 1; t <= std::min(nsteps, 16); ++t) {
+        const int64_t rounds = ((int64_t)n_wg * t + SDD_TARGET_WGS - 1) / SDD_TARGET_WGS;
+        const int64_t cost = rounds * ((nsteps + t - 1) / t + 2) + (t > 1 ? 6 * t : 0);
+        if (cost < best_cost) { best_cost = cost; best = t; }
+    }
+    steps_per_split = std::max(1, (nsteps + best - 1) / best);
+    tsplit = std::max(1, (nsteps + steps_per_split - 1) / steps_per_split);
+}
+
+extern "C" int64_t mortar_sdd_workspace_bytes(int32_t n_wg, int32_t nnz, int64_t M) {
+    if (n_wg <= 0 || nnz <= 0 || M < 0) return mortar_fail(MORTAR_ERR_ARG, "sdd_workspace_bytes: bad argument");
+    int nsteps, sps, tsplit;
+    sdd_split(n_wg, M, nsteps, sps, tsplit);
+    return (int64_t)tsplit * nnz * 256 * (int64_t)sizeof(float);
 }
 
 extern "C" int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t Rb, int32_t Cb, int32_t nnz,
@@ -217,38 +287,32 @@ extern "C" int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t Rb, in
     if (!plan || !out || !acc || (M > 0 && (!a || !b))) return mortar_fail(MORTAR_ERR_ARG, "sdd: null pointer");
     if (n_wg <= 0 || Rb <= 0 || Cb <= 0 || nnz <= 0 || M < 0) return mortar_fail(MORTAR_ERR_ARG, "sdd: bad shape");
     if (reinterpret_cast<uintptr_t>(out) & 15) return mortar_fail(MORTAR_ERR_ARG, "sdd: out must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
     if (M == 0) {                                          // no tokens: the gradient is zero
-        hipLaunchKernelGGL(sdd_zero_kernel, dim3((unsigned)(((int64_t)nnz * 32 + 255) / 256)), dim3(256), 0,
-                           static_cast<hipStream_t>(stream), reinterpret_cast<float *>(out), (int64_t)nnz * 32);
+        hipLaunchKernelGGL(sdd_zero_kernel, dim3((unsigned)(((int64_t)nnz * 32 + 255) / 256)), dim3(256), 0, st,
+                           reinterpret_cast<float *>(out), (int64_t)nnz * 32);
         return MORTAR_OK;
     }
     if (lda < (int64_t)Rb * 16 || ldb < (int64_t)Cb * 16 || (lda & 7) || (ldb & 7) ||
         (reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15) ||
-        (reinterpret_cast<uintptr_t>(acc) & 15) || (reinterpret_cast<uintptr_t>(out) & 15))
+        (reinterpret_cast<uintptr_t>(acc) & 15))
         return mortar_fail(MORTAR_ERR_ARG, "sdd: operands need 16-byte aligned rows (leading dimensions multiples of 8)");
-    hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t n4 = (int64_t)nnz * 64;
-    const int nseg = (Cb + SDD_SEG - 1) / SDD_SEG;
     SddArgs p;
     p.plan = plan; p.a = a; p.b = b; p.lda = lda; p.ldb = ldb; p.M = M; p.acc = acc; p.out = out;
-    p.Cb = Cb; p.seg_cb = (Cb + nseg - 1) / nseg;
-    p.nsteps = (int)((M + SDD_STEP - 1) / SDD_STEP);
-    int tsplit = std::max(1, std::min(p.nsteps, (256 + n_wg - 1) / n_wg));
-    p.steps_per_split = (p.nsteps + tsplit - 1) / tsplit;
-    p.tsplit = (p.nsteps + p.steps_per_split - 1) / p.steps_per_split;
+    p.Cb = Cb; p.nnz = nnz;
+    sdd_split(n_wg, M, p.nsteps, p.steps_per_split, p.tsplit);
     static bool configured = false;
-    const int smem = (SDD_SEG + SDD_RMAX) * SDD_XS;
+    const int smem = 2 * SDD_BUF;
     if (!configured) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sdd_kernel),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
         configured = true;
     }
-    if (p.tsplit > 1)
-        hipLaunchKernelGGL(sdd_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st, acc, n4);
     hipLaunchKernelGGL(sdd_kernel, dim3((unsigned)(n_wg * p.tsplit)), dim3(SDD_WAVES * 64), smem, st, p);
     if (p.tsplit > 1)
-        hipLaunchKernelGGL(sdd_round_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st, acc, out, n4);
+        hipLaunchKernelGGL(sdd_round_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st, acc, out, n4, p.tsplit);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "sdd: %s", hipGetErrorString(e));
     return MORTAR_OK;

@@ -74,17 +74,28 @@ class _SwiGLUMortar(nn.Module):
     def _carved(self) -> bool:
         return self.gate_up._cms._mortar and self.down._cms._mortar
 
+    def _wants_grad(self, x: Tensor) -> bool:
+        """Autograd is recording and something upstream or the QAT block values need a gradient: the MLP then runs
+        layer by layer (carved linear -> SwiGLU in torch -> carved linear) so that every step has a backward."""
+        if not torch.is_grad_enabled():
+            return False
+        if x.requires_grad:
+            return True
+        return any(isinstance(getattr(m._cms, "mortar_data", None), torch.nn.Parameter) and m._cms.mortar_data.requires_grad
+                   and "mortar_packed" not in m._cms._buffers for m in (self.gate_up, self.down))
+
     def forward(self, x: Tensor, iter_idx: int = 0, gates: Tensor | None = None, norm: tuple | None = None) -> Tensor:
         """x [..., d_model] -> [..., d_model].  ``gates`` overrides the router output (fp32 [N, n_clusters]);
         it exists so that a caller which already evaluated the router (or holds seeded logits) can feed it.
         ``norm`` = (weight or None, eps): x is the activation BEFORE the block's RMSNorm (norm_mlp) and the norm is
         applied here, inside the gate_up launch when the matrix allows it; same result as mlp(rmsnorm(x))."""
+        train = self._carved() and self._wants_grad(x)
         if norm is not None:
-            fused = (self._carved() and x.is_cuda and (self.router is None or gates is not None)
+            fused = (self._carved() and x.is_cuda and not train and (self.router is None or gates is not None)
                      and ops.norm_fusable(self.gate_up._cms.mortar_pack()))
             if not fused:
                 nw, eps = norm
-                if self._carved() and x.is_cuda:
+                if self._carved() and x.is_cuda and not train:
                     x = ops.rmsnorm(x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16), nw, eps)
                 else:
                     xn = (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype)
@@ -92,7 +103,7 @@ class _SwiGLUMortar(nn.Module):
                 norm = None
             elif norm[0] is not None and norm[0].dtype != torch.bfloat16:
                 norm = (norm[0].to(torch.bfloat16), norm[1])
-        if not self._carved():
+        if not self._carved() or train:
             gu = self.gate_up(x)
             gate, up = gu.chunk(2, dim=-1)
             h = F.silu(gate) * up

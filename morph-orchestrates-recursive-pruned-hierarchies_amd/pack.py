@@ -147,7 +147,7 @@ class MortarPack:
     """
 
     def __init__(self, packed, scale, col, offsets, out_features: int, in_features: int, device,
-                 prefill_stream: bool = True, scale_after_sum: bool = True):
+                 prefill_stream: bool = True, scale_after_sum: bool = True, allow_empty_rows: bool = False):
         if out_features % BLK or in_features % BLK:
             raise ValueError(f"[{out_features},{in_features}] not divisible by blocking {BLK}")
         self.out_features, self.in_features = int(out_features), int(in_features)
@@ -159,7 +159,7 @@ class MortarPack:
         self.nnz = int(self.h_offsets[-1])
         if self.h_col.size != self.nnz:
             raise ValueError(f"column_indices has {self.h_col.size} entries, offsets say {self.nnz}")
-        if (np.diff(self.h_offsets) <= 0).any():
+        if (np.diff(self.h_offsets) <= 0).any() and not allow_empty_rows:       # the reference's carve refuses these
             raise RuntimeError("carved matrix has a block-row with zero kept blocks")
         self.device = torch.device(device)
         if packed is None:
@@ -252,10 +252,9 @@ class MortarPack:
         the reference's stk_dds(..., transpose_b=False)."""
         if self._transposed is None:
             off_t, col_t, src = transpose_topology(self.h_offsets, self.h_col, self.Rb, self.Cb)
-            if (np.diff(off_t) <= 0).any():
-                raise RuntimeError("carved matrix has a block-column with zero kept blocks: W^T cannot be packed")
             t = MortarPack(None, None, col_t, off_t, self.in_features, self.out_features, self.device,
-                           prefill_stream=self.codes4_o is not None, scale_after_sum=self.scale_after_sum)
+                           prefill_stream=self.codes4_o is not None, scale_after_sum=self.scale_after_sum,
+                           allow_empty_rows=True)        # a block-column of W without blocks: that slice of dX is 0
             t.src_block = torch.from_numpy(src).to(self.device)
             self._transposed = t
         return self._transposed

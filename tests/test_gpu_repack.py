@@ -97,10 +97,11 @@ def test_requantize_rejects_bad_input(dev):
 
 @pytest.mark.parametrize("per_block", [False, True])
 @pytest.mark.parametrize("M", [3, 200])
-def test_transposed_pack_gives_the_dx_product(dev, per_block, M):
-    """dX = dY @ W through the W^T pack (the reference's dds with the transposed metadata, transpose_b=False)."""
-    shape = (16 * 20, 16 * 12)
-    m = synth.synth_matrix(shape[0], shape[1], 0.3, seed=31, zipf_s=1.2)
+@pytest.mark.parametrize("shape,density", [((16 * 20, 16 * 12), 0.3), ((16 * 3, 16 * 40), 0.1)])
+def test_transposed_pack_gives_the_dx_product(dev, per_block, M, shape, density):
+    """dX = dY @ W through the W^T pack (the reference's dds with the transposed metadata, transpose_b=False).  The
+    second shape has block-columns without any block: those slices of dX are zero."""
+    m = synth.synth_matrix(shape[0], shape[1], density, seed=31, zipf_s=1.2)
     nnz = m["col_idx"].size
     vt, v = _values(nnz, 32, torch.bfloat16)
     W = MortarPack(None, None, m["col_idx"], m["offsets"], shape[0], shape[1], dev)
@@ -187,3 +188,87 @@ def test_sdd_edge_cases(dev):
     got = to_np(ops.sdd(a[:, 64:], b[:, :96], W))
     ref = O.sdd_at_b(to_np(a[:, 64:]), to_np(b[:, :96]), m["row_idx"], m["col_idx"])
     assert_close_bf16(got, ref, "strided")
+
+
+# ---------------------------------------------------------------------------------------------- training step
+
+def _qat_layer(out_f, in_f, density, seed, dev, dtype=torch.float32):
+    from mortar_amd.block_sparse import CMSBlockLinear
+    g = torch.Generator().manual_seed(seed)
+    lin = CMSBlockLinear(in_f, out_f, bias=False, dtype=dtype)
+    with torch.no_grad():
+        lin.weight.copy_(torch.randn(out_f, in_f, generator=g) * 0.05)
+    mask = torch.rand(out_f // 16, in_f // 16, generator=g) < density
+    mask[torch.arange(out_f // 16), torch.randint(0, in_f // 16, (out_f // 16,), generator=g)] = True
+    mask[torch.randint(0, out_f // 16, (in_f // 16,), generator=g), torch.arange(in_f // 16)] = True   # no empty column
+    lin.set_block_mask(mask, 16)
+    lin.carve(16)
+    lin.enable_values_ternary(0.5)
+    return lin.to(dev)
+
+
+def _effective_dense(lin):
+    """scale * q scattered to [out, in] in float64, with the scale rounded to bf16 as the kernels (and the reference's
+    bf16 autocast) apply it."""
+    d = lin.mortar_data.detach().float().cpu().numpy()
+    q, s = O.ternary_quantize(d, lin._values_threshold)
+    blocks = q.astype(np.float32) * O.bf16_round(np.float32(s))
+    return O.to_dense(blocks, lin.mortar_row_indices.cpu().numpy(), lin.mortar_column_indices.cpu().numpy(),
+                      (lin.out_features, lin.in_features)).astype(np.float64)
+
+
+@pytest.mark.parametrize("M", [8, 300])
+def test_qat_layer_forward_backward(dev, M):
+    """A carved layer in values-ternary QAT: forward through the device-side re-pack, dX through the W^T pack, the
+    gradient of mortar_data through the topology-restricted product (straight-through), then a second step after the
+    values changed in place (the packs must follow)."""
+    lin = _qat_layer(16 * 10, 16 * 7, 0.4, 61, dev)
+    for step in range(2):
+        W = _effective_dense(lin)
+        x = synth.synth_x(M, lin.in_features, seed=62 + step)
+        dy = synth.synth_x(M, lin.out_features, seed=64 + step)
+        xt = to_dev(x, dev).requires_grad_(True)
+        y = lin(xt)
+        y.backward(to_dev(dy, dev))
+        xb, dyb = O.bf16_round(x).astype(np.float64), O.bf16_round(dy).astype(np.float64)
+        assert_close_bf16(to_np(y), (xb @ W.T).astype(np.float32), f"y step {step}")
+        assert_close_bf16(to_np(xt.grad), (dyb @ W).astype(np.float32), f"dx step {step}")
+        ref_dw = O.sdd_at_b(O.bf16_round(dy), O.bf16_round(x), lin.mortar_row_indices.cpu().numpy(),
+                            lin.mortar_column_indices.cpu().numpy())
+        assert lin.mortar_data.grad.shape == lin.mortar_data.shape and lin.mortar_data.grad.dtype == lin.mortar_data.dtype
+        assert_close_bf16(to_np(lin.mortar_data.grad), ref_dw, f"d mortar_data step {step}")
+        with torch.no_grad():                      # an optimiser step: same storage, new version
+            lin.mortar_data.add_(lin.mortar_data.grad, alpha=-0.05)
+            lin.mortar_data.grad = None
+
+
+def test_qat_mlp_trains_layer_by_layer(dev):
+    """The SwiGLU MLP with QAT layers and autograd on: same value as the fused inference path, gradients reach the
+    input and both block-value tensors."""
+    from mortar_amd.mlp import _SwiGLUMortar
+    d_model, d_ff = 16 * 6, 16 * 10
+    mlp = _SwiGLUMortar(d_model, d_ff)
+    mlp.gate_up._cms = _qat_layer(2 * d_ff, d_model, 0.5, 71, dev)
+    mlp.down._cms = _qat_layer(d_model, d_ff, 0.5, 72, dev)
+    mlp = mlp.to(dev)
+    x = to_dev(synth.synth_x(50, d_model, seed=73), dev)
+    with torch.no_grad():
+        y_inf = mlp(x)
+    xg = x.clone().requires_grad_(True)
+    y = mlp(xg)
+    assert_close_bf16(to_np(y), to_np(y_inf), "train path vs fused path", ulps=8)
+    y.float().pow(2).sum().backward()
+    for name, g in (("x", xg.grad), ("gate_up", mlp.gate_up._cms.mortar_data.grad), ("down", mlp.down._cms.mortar_data.grad)):
+        assert g is not None and torch.isfinite(g.float()).all() and float(g.float().abs().max()) > 0, name
+    # against a dense torch twin with the same effective weights (fp32 autograd)
+    Wg = torch.from_numpy(_effective_dense(mlp.gate_up._cms)).float().to(dev)
+    Wd = torch.from_numpy(_effective_dense(mlp.down._cms)).float().to(dev)
+    xr = x.float().clone().requires_grad_(True)
+    gu = xr @ Wg.T
+    h = torch.nn.functional.silu(gu[:, :d_ff]) * gu[:, d_ff:]
+    yr = h @ Wd.T
+    yr.pow(2).sum().backward()
+    # five bf16 roundings lie between the two chains: compare in the large (max error 3e-2 of the largest entry, cosine)
+    got, ref = to_np(xg.grad).astype(np.float64), to_np(xr.grad).astype(np.float64)
+    assert np.abs(got - ref).max() <= 3e-2 * np.abs(ref).max()
+    assert (got * ref).sum() / np.sqrt((got * got).sum() * (ref * ref).sum()) > 0.9995
