@@ -316,6 +316,37 @@ def main() -> None:
                                "note": "RMSNorm before every MLP, applied while gate_up stages x (no separate launch); rows follow Zipf(1.2) clipped to 5-60 %"}
         del specs, packs4
 
+    if not args.no_extras:
+        # ---- training side (values-ternary QAT): device re-pack of W and W^T, dX through the W^T pack, dW on the
+        # topology, for both matrices at the headline shapes (4096 tokens) ------------------------------------------
+        from mortar_amd.pack import MortarPack
+        bw = {}
+        tot = 0.0
+        for name, Wf in (("gate_up", Wgu), ("down", Wdn)):
+            m = spec[name]
+            Wq = MortarPack(None, None, m["col_idx"], m["offsets"], Wf.out_features, Wf.in_features, dev)
+            vals = (torch.randn(Wf.nnz, 16, 16, device=dev) * 0.05).to(torch.bfloat16)
+            sc = Wq.requantize(vals)
+            Wt = Wq.transposed()
+            Wt.requantize(vals, scale=sc, transpose=True)
+            xin = torch.randn(TOKENS, Wf.in_features, device=dev).to(torch.bfloat16)
+            dy = torch.randn(TOKENS, Wf.out_features, device=dev).to(torch.bfloat16)
+            dx = torch.empty_like(xin)
+            dw = torch.empty(Wf.nnz, 16, 16, dtype=torch.bfloat16, device=dev)
+            fl = 2.0 * TOKENS * 256 * Wf.nnz
+            t_rq = event_time_ms(lambda: Wt.requantize(vals, scale=Wq.requantize(vals, sync=False), transpose=True, sync=False), 10)
+            t_dx = event_time_ms(lambda: ops.spmm(dy, Wt, out=dx), 10)
+            t_dw = event_time_ms(lambda: ops.sdd(dy, xin, Wq, out=dw), 10)
+            bw[name] = {"repack_w_and_wt_us": t_rq * 1e3, "dx_us": t_dx * 1e3, "dx_tflops": fl / (t_dx * 1e-3) / 1e12,
+                        "dw_us": t_dw * 1e3, "dw_tflops": fl / (t_dw * 1e-3) / 1e12}
+            tot += t_rq + t_dx + t_dw
+            del Wq, Wt, vals, xin, dy, dx, dw
+        bw["backward_ms_per_mlp"] = tot
+        bw["backward_over_forward"] = tot / (ms_gu + ms_dn)
+        bw["note"] = ("matrix products of the MLP's backward only (the SwiGLU derivative is elementwise torch); dW sums "
+                      "fp32 over 4096 tokens and rounds to bf16")
+        out["training_backward"] = bw
+
     # A plain device-to-device copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE counters when this
     # command runs under `rocprofv3 --pmc` (counter KiB per byte copied), and a practical HBM bandwidth figure.
     cal_src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).fill_(1)

@@ -289,7 +289,7 @@ int mortar_rmsnorm_bf16(const uint16_t *x, int64_t M, int32_t d, int64_t ldx, co
  * when present, codes4_o) in place; the topology arrays are not touched.  One launch (two with scale_mode 0)
  * replaces the reference's per-forward torch ternarisation of mortar_data (block_sparse.py:909-919) and its
  * deploy pack (deploy_quant.py:81-95, 344-374) followed by a host re-pack.
- *   values     device [nnz,16,16], bf16 (values_f32 = 0) or fp32 (1): the reference's mortar_data
+ *   values     device [nnz,16,16], bf16 (values_f32 = 0) or fp32 (1), 16-byte aligned: the reference's mortar_data
  *   pos        device int32 [nnz] from mortar_octet_positions_host
  *   src_block  device int32 [nnz] or NULL: block j of W takes the values of block src_block[j] (NULL: block j)
  *   transpose  != 0: the source block is read transposed.  src_block + transpose fill the W^T pack of

@@ -196,7 +196,7 @@ class CMSBlockLinear(nn.Module):
             self._pack_key = self._pack_t_key = None
         key = (d.data_ptr(), d._version)
         if self._pack_key != key:
-            self._pack.requantize(self._values(), threshold=self._values_threshold, sync=False)
+            self._pack_scale = self._pack.requantize(self._values(), threshold=self._values_threshold, sync=False)
             self._pack_key = key
         return self._pack
 
@@ -206,7 +206,8 @@ class CMSBlockLinear(nn.Module):
             raise RuntimeError("mortar_pack_t(): the backward needs a QAT layer (mortar_data) on the GPU")
         t = self.mortar_pack().transposed()
         if self._pack_t_key != self._pack_key:
-            t.requantize(self._values(), threshold=self._values_threshold, transpose=True, sync=False)
+            t.requantize(self._values(), threshold=self._values_threshold, scale=self._pack_scale, transpose=True,
+                         sync=False)              # the scale W was packed with: no second reduction over the values
             self._pack_t_key = self._pack_key
         return t
 

@@ -25,12 +25,26 @@ __device__ __forceinline__ double wave_sum(double x) {
     return x;
 }
 
-// sum |w| over all values -> partial[blockIdx] (fixed order: the result does not depend on timing)
+// sum |w| over all values -> partial[blockIdx] (fixed order: the result does not depend on timing).  n is a multiple
+// of 256 (whole blocks) and the array is 16-byte aligned, so every thread reads 16-byte pieces.
 __global__ __launch_bounds__(256) void abs_sum_kernel(const void *values, int64_t n, int f32, double *partial) {
     __shared__ double wsum[4];
     double s = 0.0;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)PARTIALS * 256)
-        s += (double)fabsf(load_val(values, i, f32 != 0));
+    const int per = f32 ? 4 : 8;                                     // values per 16-byte piece
+    const uint4 *v = reinterpret_cast<const uint4 *>(values);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n / per; i += (int64_t)PARTIALS * 256) {
+        const uint4 q = v[i];
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (f32) {
+                s += (double)fabsf(__uint_as_float(w[e]));
+            } else {
+                s += (double)fabsf(__uint_as_float(w[e] << 16));
+                s += (double)fabsf(__uint_as_float(w[e] & 0xffff0000u));
+            }
+        }
+    }
     s = wave_sum(s);
     if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = s;
     __syncthreads();
@@ -131,6 +145,7 @@ extern "C" int mortar_requantize(const mortar_bcsr_t *W, const void *values, int
     if (scale_mode >= 2 && !scale_in) return mortar_fail(MORTAR_ERR_ARG, "requantize: scale_mode %d needs scale_in", scale_mode);
     if (scale_mode == 0 && !workspace) return mortar_fail(MORTAR_ERR_ARG, "requantize: scale_mode 0 needs the workspace");
     if (!(threshold >= 0.f)) return mortar_fail(MORTAR_ERR_ARG, "requantize: threshold must be >= 0");
+    if (reinterpret_cast<uintptr_t>(values) & 15) return mortar_fail(MORTAR_ERR_ARG, "requantize: values must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (status) hipLaunchKernelGGL(clear_status_kernel, dim3(1), dim3(64), 0, st, status);
     if (scale_mode == 0)
