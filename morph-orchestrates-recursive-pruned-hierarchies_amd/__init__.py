@@ -9,9 +9,9 @@ from .mlp import _KwargSequential, _make_swiglu, _SwiGLUMortar        # noqa: F4
 from .pack import MortarPack                                          # noqa: F401
 from .routing import TileRouter                                       # noqa: F401
 from .sparsity import MortarLinear                                    # noqa: F401
-from .stk import stk_dds                                              # noqa: F401
+from .stk import stk_dds, stk_sdd_at_b                                # noqa: F401
 
 __all__ = ["CMSBlockLinear", "MortarLinear", "_SwiGLUMortar", "_KwargSequential", "_make_swiglu", "TileRouter",
-           "MortarPack", "MortarDecodeMLP", "stk_dds", "mortar_gemv", "mortar_pack_strips", "looped_core_forward",
+           "MortarPack", "MortarDecodeMLP", "stk_dds", "stk_sdd_at_b", "mortar_gemv", "mortar_pack_strips", "looped_core_forward",
            "pack_mortar_ternary", "pack_ternary_codes", "unpack_ternary", "shrink_mlp_to_mortar_ternary",
            "ops", "pack", "synth"]

@@ -272,3 +272,23 @@ def test_qat_mlp_trains_layer_by_layer(dev):
     got, ref = to_np(xg.grad).astype(np.float64), to_np(xr.grad).astype(np.float64)
     assert np.abs(got - ref).max() <= 3e-2 * np.abs(ref).max()
     assert (got * ref).sum() / np.sqrt((got * got).sum() * (ref * ref).sum()) > 0.9995
+
+
+def test_stk_dds_operator_autograd(dev):
+    """The custom op's registered backward: dlhs through the other orientation, ddata through stk_sdd_at_b."""
+    import mortar_amd
+    m = synth.synth_matrix(16 * 8, 16 * 6, 0.5, seed=81)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    data = t(O.effective_blocks(m["codes"], m["scales"])).to(torch.bfloat16).requires_grad_(True)
+    dense = O.to_dense(data.detach().float().cpu().numpy(), m["row_idx"], m["col_idx"], (128, 96)).astype(np.float64)
+    z32, z16 = torch.zeros(1, dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int16, device=dev)
+    args = (t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32)
+    x, dy = synth.synth_x(70, 96, seed=82), synth.synth_x(70, 128, seed=83)
+    xt = to_dev(x, dev).requires_grad_(True)
+    y = mortar_amd.stk_dds(xt, data, *args, 96, 128, True)
+    y.backward(to_dev(dy, dev))
+    assert_close_bf16(to_np(xt.grad), (O.bf16_round(dy) @ dense).astype(np.float32), "dlhs")
+    assert data.grad.shape == data.shape and data.grad.dtype == torch.bfloat16
+    assert_close_bf16(to_np(data.grad), O.sdd_at_b(O.bf16_round(dy), O.bf16_round(x), m["row_idx"], m["col_idx"]), "ddata")
+    direct = mortar_amd.stk_sdd_at_b(to_dev(dy, dev), to_dev(x, dev), data.detach(), *args[:3])
+    assert torch.equal(direct, data.grad)

@@ -373,3 +373,20 @@ def test_sdd_plan_partitions_the_blocks():
             tile = (off // 4224) * 4 + (off % 4224) // 32
             assert ((off % 4224) % 32 == 0).all() and (off % 4224 < 128).all() and (tile < seg_cb).all() and ((eo[w] >> 20) < nrows).all()
             assert np.array_equal(tile[ej[w] >= 0], col[js] - seg * seg_cb) and (col[js] // seg_cb == seg).all()
+
+
+def test_operator_fake_implementations_trace_without_a_gpu():
+    """stk_dds / stk_sdd_at_b carry fake (meta) implementations, as the reference's custom ops do
+    (custom_ops.py:59-65, 93-96): shapes and dtypes propagate under FakeTensorMode with no device present."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    with FakeTensorMode():
+        lhs = torch.empty(40, 96, dtype=torch.bfloat16, device="cuda")
+        data = torch.empty(10, 16, 16, dtype=torch.bfloat16, device="cuda")
+        off = torch.empty(9, dtype=torch.int32, device="cuda")
+        idx = torch.empty(10, dtype=torch.int16, device="cuda")
+        y = mortar_amd.stk_dds(lhs, data, off, idx, idx, off, idx, off, 96, 128, True)
+        assert tuple(y.shape) == (40, 128) and y.dtype == torch.bfloat16
+        dx = mortar_amd.stk_dds(y, data, off, idx, idx, off, idx, off, 128, 96, False)
+        assert tuple(dx.shape) == (40, 96)
+        dw = mortar_amd.stk_sdd_at_b(y, lhs, data, off, idx, idx)
+        assert tuple(dw.shape) == (10, 16, 16) and dw.dtype == torch.bfloat16
