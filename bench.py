@@ -341,10 +341,29 @@ def main() -> None:
                         "dw_us": t_dw * 1e3, "dw_tflops": fl / (t_dw * 1e-3) / 1e12}
             tot += t_rq + t_dx + t_dw
             del Wq, Wt, vals, xin, dy, dx, dw
+        # the whole MLP as a module in values-ternary QAT: forward + backward of one training step (re-pack of both
+        # matrices and their transposes, 3 SpMMs forward-type, 2 dW products, SwiGLU and its derivative)
+        qmlp = synth.qat_mlp_module(spec, dev)
+        xq = x.clone().requires_grad_(True)
+        gy = torch.randn(TOKENS, D_MODEL, device=dev).to(torch.bfloat16)
+
+        def train_step():
+            for p_ in qmlp.parameters():
+                p_.grad = None
+            xq.grad = None
+            qmlp(xq).backward(gy)
+            with torch.no_grad():                       # stand-in for the optimiser: the values change every step
+                qmlp.gate_up._cms.mortar_data.add_(1e-6)
+                qmlp.down._cms.mortar_data.add_(1e-6)
+        t_train = event_time_ms(train_step, 5, 2)
+        bw["qat_train_step_ms"] = t_train
+        bw["qat_train_tokens_per_s"] = TOKENS / (t_train * 1e-3)
+        del qmlp, xq, gy
         bw["backward_ms_per_mlp"] = tot
         bw["backward_over_forward"] = tot / (ms_gu + ms_dn)
-        bw["note"] = ("matrix products of the MLP's backward only (the SwiGLU derivative is elementwise torch); dW sums "
-                      "fp32 over 4096 tokens and rounds to bf16")
+        bw["note"] = ("per-matrix figures are the backward's matrix products; qat_train_step is forward + backward of the "
+                      "MLP module with trainable block values (re-pack, SpMMs, SwiGLU and its derivative, dW), "
+                      "4096 tokens; dW sums fp32 over the tokens and rounds to bf16")
         out["training_backward"] = bw
 
     # A plain device-to-device copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE counters when this

@@ -310,6 +310,17 @@ int mortar_requantize(const mortar_bcsr_t *W, const void *values, int32_t values
                       const int32_t *src_block, int32_t transpose, int32_t scale_mode, float threshold,
                       const float *scale_in, float *scale_out, int32_t *status, void *workspace, void *stream);
 
+/* ---- SwiGLU between the two matrices, training form ------------------------------------------------ */
+
+/* h = bf16(bf16(silu(gate)) * up) from a stored gate_up output gu [M, 2*d_ff] (gate = columns [0, d_ff), up =
+ * [d_ff, 2*d_ff)), and its derivative dgu [M, 2*d_ff] from gu and dh [M, d_ff]: the eager path of
+ * _SwiGLUMortar.forward (morph/model/transformer.py:411-413: gu.chunk(2), F.silu(gate) * up) and what torch autograd
+ * derives from it, each in one launch.  Inference uses the fused epilogue of mortar_gateup_swiglu_bf16 instead; training
+ * keeps gu for the backward.  All bf16, d_ff and leading dimensions multiples of 8, rows 16-byte aligned. */
+int mortar_swiglu_bf16(const uint16_t *gu, int64_t ldg, int64_t M, int32_t d_ff, uint16_t *h, int64_t ldh, void *stream);
+int mortar_swiglu_backward_bf16(const uint16_t *gu, int64_t ldg, const uint16_t *dh, int64_t ldh, int64_t M, int32_t d_ff,
+                                uint16_t *dgu, int64_t ldo, void *stream);
+
 /* ---- weight gradient on the topology ------------------------------------------------------------ */
 
 /* out[j] = a[:, 16 rows of block j]^T @ b[:, 16 columns of block j] for every kept block: the dW product of the

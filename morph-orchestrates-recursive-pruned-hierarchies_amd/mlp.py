@@ -44,6 +44,40 @@ def _make_swiglu(d_model: int, d_ff: int, dropout: float) -> nn.Module:
     return mlp
 
 
+class _SwiGLUMortarFn(torch.autograd.Function):
+    """The carved MLP as one differentiable op for QAT training: y = down(silu(gate) * up), gate_up kept for the
+    backward.  Forward: SpMM, SwiGLU, SpMM.  Backward (reference: torch autograd over transformer.py:411-431 with the
+    stk backward, custom_ops.py:99-136): dh through down's W^T pack, dW_down on the topology, the SwiGLU derivative in
+    one launch, dx through gate_up's W^T pack, dW_gate_up on the topology."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, data_gu: Tensor, data_dn: Tensor, mlp: "_SwiGLUMortar") -> Tensor:
+        cg, cd = mlp.gate_up._cms, mlp.down._cms
+        gu = ops.spmm(x, cg.mortar_pack())
+        h = ops.swiglu(gu)
+        y = ops.spmm(h, cd.mortar_pack())
+        ctx.mlp = mlp
+        ctx.dtypes = (data_gu.dtype, data_dn.dtype)
+        ctx.save_for_backward(x, gu, h)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy: Tensor):
+        x, gu, h = ctx.saved_tensors
+        cg, cd = ctx.mlp.gate_up._cms, ctx.mlp.down._cms
+        dy = (dy if dy.dtype == torch.bfloat16 else dy.to(torch.bfloat16)).contiguous()
+        need_x, need_gu, need_dn = ctx.needs_input_grad[:3]
+        d_dn = ops.sdd(dy, h, cd.mortar_pack()).to(ctx.dtypes[1]) if need_dn else None
+        dx = d_gu = None
+        if need_x or need_gu:
+            dgu = ops.swiglu_backward(gu, ops.spmm(dy, cd.mortar_pack_t()))
+            if need_gu:
+                d_gu = ops.sdd(dgu, x, cg.mortar_pack()).to(ctx.dtypes[0])
+            if need_x:
+                dx = ops.spmm(dgu, cg.mortar_pack_t())
+        return dx, d_gu, d_dn, None
+
+
 class _SwiGLUMortar(nn.Module):
     def __init__(self, d_model: int, d_ff: int):
         super().__init__()
@@ -103,6 +137,14 @@ class _SwiGLUMortar(nn.Module):
                 norm = None
             elif norm[0] is not None and norm[0].dtype != torch.bfloat16:
                 norm = (norm[0].to(torch.bfloat16), norm[1])
+        if (train and x.is_cuda and self.router is None and gates is None and norm is None
+                and all(m._cms._values_ternary_mode and "mortar_packed" not in m._cms._buffers and m._cms.bias is None
+                        for m in (self.gate_up, self.down))):
+            lead = x.shape[:-1]
+            x2 = x.reshape(-1, self.d_model)
+            xb = x2 if x2.dtype == torch.bfloat16 else x2.to(torch.bfloat16)
+            y = _SwiGLUMortarFn.apply(xb, self.gate_up._cms.mortar_data, self.down._cms.mortar_data, self)
+            return (y if y.dtype == x.dtype else y.to(x.dtype)).reshape(*lead, self.d_model)
         if not self._carved() or train:
             gu = self.gate_up(x)
             gate, up = gu.chunk(2, dim=-1)

@@ -195,6 +195,29 @@ def route_flags(gates: Tensor, d_ff: int, row_act: Tensor | None = None, col_act
     return row_act, col_act
 
 
+def swiglu(gu: Tensor, out: Tensor | None = None) -> Tensor:
+    """h = silu(gate) * up from a stored gate_up output gu [M, 2*d_ff] (training form; inference fuses this into gate_up)."""
+    gu = _bf16_2d(gu, "swiglu")
+    M, d_ff = gu.shape[0], gu.shape[1] // 2
+    if gu.shape[1] % 16:
+        raise ValueError("swiglu: gate_up width must be a multiple of 16")
+    h = out if out is not None else torch.empty((M, d_ff), dtype=torch.bfloat16, device=gu.device)
+    _lib.check(_lib.lib().mortar_swiglu_bf16(_p(gu), gu.stride(0), M, d_ff, _p(h), h.stride(0), _stream(gu)), "mortar_swiglu_bf16")
+    return h
+
+
+def swiglu_backward(gu: Tensor, dh: Tensor) -> Tensor:
+    """d(gate_up output) [M, 2*d_ff] from the stored gate_up output and dh [M, d_ff]."""
+    gu, dh = _bf16_2d(gu, "swiglu_backward"), _bf16_2d(dh, "swiglu_backward")
+    M, d_ff = gu.shape[0], gu.shape[1] // 2
+    if gu.shape[1] % 16 or tuple(dh.shape) != (M, d_ff):
+        raise ValueError(f"swiglu_backward: gu {tuple(gu.shape)} / dh {tuple(dh.shape)} do not match")
+    dgu = torch.empty_like(gu)
+    _lib.check(_lib.lib().mortar_swiglu_backward_bf16(_p(gu), gu.stride(0), _p(dh), dh.stride(0), M, d_ff, _p(dgu),
+                                                      dgu.stride(0), _stream(gu)), "mortar_swiglu_backward_bf16")
+    return dgu
+
+
 def sdd(a: Tensor, b: Tensor, W: MortarPack, out: Tensor | None = None) -> Tensor:
     """Weight gradient on W's topology: out[j] = a[:, rows of block j]^T @ b[:, columns of block j], bf16 [nnz,16,16]
     (reference stk_sdd_at_b; for y = x W^T pass a = dY [M, out_features], b = x [M, in_features])."""

@@ -94,6 +94,31 @@ def carved_state(mat: dict, prefix: str = "") -> dict:
             prefix + "mortar_ternary": torch.tensor([0.0, 0.5])}
 
 
+def qat_state(mat: dict, prefix: str = "", seed: int = 0) -> dict:
+    """state_dict entries of a carved layer in values-ternary QAT (bf16 mortar_data, not packed) on a synthetic
+    topology: smooth values N(0, 0.05), the reference's key set (block_sparse.py:783-799)."""
+    from .block_sparse import _stk_transpose
+    rows, cols = torch.from_numpy(mat["row_idx"]), torch.from_numpy(mat["col_idx"])
+    offs = torch.from_numpy(mat["offsets"])
+    ct, ot, bt = _stk_transpose(mat["shape"], torch.empty(0, BLK, BLK), rows, cols, offs)
+    g = torch.Generator().manual_seed(seed)
+    data = (torch.randn(rows.numel(), BLK, BLK, generator=g) * 0.05).to(torch.bfloat16)
+    return {prefix + "mortar_data": data, prefix + "mortar_row_indices": rows, prefix + "mortar_column_indices": cols,
+            prefix + "mortar_offsets": offs, prefix + "mortar_column_indices_t": ct, prefix + "mortar_offsets_t": ot,
+            prefix + "mortar_block_offsets_t": bt, prefix + "mortar_ternary": torch.tensor([1.0, 0.5])}
+
+
+def qat_mlp_module(spec: dict, device, seed: int = 0):
+    """A carved _SwiGLUMortar in values-ternary QAT (trainable bf16 block values) over the synthetic topologies."""
+    from .mlp import _SwiGLUMortar
+    with torch.device("meta"):
+        mlp = _SwiGLUMortar(spec["d_model"], spec["d_ff"])
+    mlp = mlp.to_empty(device="cpu")
+    sd = {**qat_state(spec["gate_up"], "gate_up._cms.", seed), **qat_state(spec["down"], "down._cms.", seed + 1)}
+    mlp.load_state_dict(sd, strict=True)
+    return mlp.to(device)
+
+
 def mlp_module(spec: dict, device):
     """A carved, packed _SwiGLUMortar holding the synthetic matrices, loaded through load_state_dict."""
     from .mlp import _SwiGLUMortar

@@ -15,6 +15,7 @@ reference checkout).  How each function is pinned (no reference import is needed
   dds_dx / sdd_at_b        (backward) reduce to dense float64 matmuls + a gather of the
                            kept blocks; the adjoint identity <dY, x W^T> = <dY W, x> = <dW, W>
   swiglu_mlp               textbook x*sigmoid(x) + the above
+  swiglu / swiglu_backward the same closed form; the derivative by central differences
   remoe_gates              brute force on tiny inputs incl. ties; invariants
   route_flags              closed form
   rmsnorm                  closed form
@@ -236,6 +237,28 @@ def dense_linear(x: np.ndarray, codes, scales, row_idx, col_idx, shape, blk=16) 
 def silu(x: np.ndarray) -> np.ndarray:
     x = x.astype(np.float32)
     return (x / (np.float32(1.0) + np.exp(-x, dtype=np.float32))).astype(np.float32)
+
+
+def swiglu(gu: np.ndarray) -> np.ndarray:
+    """h = bf16(bf16(silu(gate)) * up), gate = gu[:, :d_ff], up = gu[:, d_ff:]  (transformer.py:411-413, the bf16
+    tensors the eager path materialises).  gu float32 array of bf16-representable values."""
+    d_ff = gu.shape[1] // 2
+    g, u = gu[:, :d_ff].astype(np.float64), gu[:, d_ff:].astype(np.float64)
+    s = bf16_round((g / (1.0 + np.exp(-g))).astype(np.float32)).astype(np.float64)
+    return bf16_round((s * u).astype(np.float32))
+
+
+def swiglu_backward(gu: np.ndarray, dh: np.ndarray, round_out: bool = True) -> np.ndarray:
+    """d gu from dh for h = silu(gate) * up: d_up = dh * silu(g); d_gate = dh * up * sig(g) * (1 + g * (1 - sig(g)))
+    (what torch autograd derives for transformer.py:411-413).  With round_out the bf16 tensors of that graph are
+    rounded where they appear (silu(g), dh * up, the two results); without, plain float64 calculus."""
+    d_ff = gu.shape[1] // 2
+    g, u, d = gu[:, :d_ff].astype(np.float64), gu[:, d_ff:].astype(np.float64), dh.astype(np.float64)
+    sg = 1.0 / (1.0 + np.exp(-g))
+    r = (lambda a: bf16_round(a.astype(np.float32)).astype(np.float64)) if round_out else (lambda a: a)
+    d_up = r(d * r(g * sg))
+    d_gate = r(r(d * u) * (sg * (1.0 + g * (1.0 - sg))))
+    return np.concatenate([d_gate, d_up], axis=1).astype(np.float32)
 
 
 def swiglu_mlp(x, gate_up: dict, down: dict, gates: np.ndarray | None = None,

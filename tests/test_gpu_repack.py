@@ -292,3 +292,55 @@ def test_stk_dds_operator_autograd(dev):
     assert_close_bf16(to_np(data.grad), O.sdd_at_b(O.bf16_round(dy), O.bf16_round(x), m["row_idx"], m["col_idx"]), "ddata")
     direct = mortar_amd.stk_sdd_at_b(to_dev(dy, dev), to_dev(x, dev), data.detach(), *args[:3])
     assert torch.equal(direct, data.grad)
+
+
+@pytest.mark.parametrize("M,d_ff", [(1, 16), (70, 16 * 10), (300, 16 * 352)])
+def test_swiglu_training_kernels(dev, M, d_ff):
+    """The stand-alone SwiGLU and its derivative against the oracle (bf16 tensors rounded where the eager graph has them)."""
+    gu = synth.synth_x(M, 2 * d_ff, seed=91) * 2.0
+    dh = synth.synth_x(M, d_ff, seed=92)
+    gt, dt = to_dev(gu, dev), to_dev(dh, dev)
+    gb, db = O.bf16_round(gu), O.bf16_round(dh)
+    assert_close_bf16(to_np(ops.swiglu(gt)), O.swiglu(gb), "swiglu", ulps=2)
+    assert_close_bf16(to_np(ops.swiglu_backward(gt, dt)), O.swiglu_backward(gb, db), "swiglu backward", ulps=3)
+    # the fused gate_up epilogue and the stand-alone kernel round alike: same bits from the same gate_up output
+    wide = torch.zeros(M, 2 * d_ff + 32, dtype=torch.bfloat16, device=dev)
+    wide[:, 8:8 + 2 * d_ff] = gt
+    assert torch.equal(ops.swiglu(wide[:, 8:8 + 2 * d_ff]), ops.swiglu(gt))
+    with pytest.raises(ValueError):
+        ops.swiglu_backward(gt, dt[:, :-8])
+
+
+def test_qat_mlp_single_op_training_step(dev):
+    """The whole MLP as one autograd op (no router): value equals the fused inference path bit for bit where the
+    rounding points agree, and all three gradients match the layer-by-layer path."""
+    from mortar_amd.mlp import _SwiGLUMortar
+    d_model, d_ff = 16 * 6, 16 * 10
+    mlp = _SwiGLUMortar(d_model, d_ff)
+    mlp.gate_up._cms = _qat_layer(2 * d_ff, d_model, 0.5, 71, dev)
+    mlp.down._cms = _qat_layer(d_model, d_ff, 0.5, 72, dev)
+    mlp = mlp.to(dev)
+    x = to_dev(synth.synth_x(90, d_model, seed=73), dev)
+    dy = to_dev(synth.synth_x(90, d_model, seed=74), dev)
+    with torch.no_grad():
+        y_inf = mlp(x)
+    xg = x.clone().requires_grad_(True)
+    y = mlp(xg)
+    fns, node = [], y.grad_fn
+    while node is not None and len(fns) < 4:
+        fns.append(type(node).__name__)
+        node = node.next_functions[0][0] if node.next_functions else None
+    assert any("SwiGLUMortarFn" in f for f in fns), fns
+    assert_close_bf16(to_np(y), to_np(y_inf), "single-op forward vs fused inference", ulps=4)
+    y.backward(dy)
+    got = [xg.grad.clone(), mlp.gate_up._cms.mortar_data.grad.clone(), mlp.down._cms.mortar_data.grad.clone()]
+    for p in (mlp.gate_up._cms.mortar_data, mlp.down._cms.mortar_data):
+        p.grad = None
+    # layer by layer (carved linear -> torch SwiGLU -> carved linear), forced by a dummy gate of ones
+    xr = x.clone().requires_grad_(True)
+    gu = mlp.gate_up(xr)
+    h = torch.nn.functional.silu(gu[:, :d_ff]) * gu[:, d_ff:]
+    mlp.down(h).backward(dy)
+    ref = [xr.grad, mlp.gate_up._cms.mortar_data.grad, mlp.down._cms.mortar_data.grad]
+    for name, a, b in zip(("dx", "d gate_up", "d down"), got, ref):
+        assert_close_bf16(to_np(a), to_np(b), name, ulps=6)

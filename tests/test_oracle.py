@@ -371,3 +371,21 @@ def test_backward_products_against_dense_matmul_and_adjoint_identity():
     lhs = float((dy * y).sum())
     np.testing.assert_allclose(float((dx.astype(np.float64) * x).sum()), lhs, rtol=1e-5)
     np.testing.assert_allclose(float((dw.astype(np.float64) * O.effective_blocks(codes, scales)).sum()), lhs, rtol=1e-5)
+
+
+def test_swiglu_backward_against_central_differences():
+    """The unrounded derivative equals the numerical gradient of sum(w * silu(g) * u); the forward equals silu * up."""
+    rng = np.random.default_rng(9)
+    gu = rng.standard_normal((5, 32)) * 2.0
+    w = rng.standard_normal((5, 16))
+    f = lambda z: float((w * (z[:, :16] / (1.0 + np.exp(-z[:, :16]))) * z[:, 16:]).sum())
+    num = np.zeros_like(gu)
+    for i in range(gu.shape[0]):
+        for j in range(gu.shape[1]):
+            e = np.zeros_like(gu); e[i, j] = 1e-6
+            num[i, j] = (f(gu + e) - f(gu - e)) / 2e-6
+    got = O.swiglu_backward(gu.astype(np.float64), w, round_out=False)
+    np.testing.assert_allclose(got, num, rtol=2e-5, atol=1e-6)      # float32 output of the oracle
+    gb = O.bf16_round(gu.astype(np.float32))
+    h = O.swiglu(gb)
+    np.testing.assert_allclose(h, O.silu(gb[:, :16]) * gb[:, 16:], rtol=2 ** -6, atol=1e-6)
