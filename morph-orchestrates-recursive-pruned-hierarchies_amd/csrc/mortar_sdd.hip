@@ -37,6 +37,9 @@ constexpr int SDD_CS = 1024 + 32;                // LDS bytes per chunk = 8 toke
 constexpr int SDD_QS = 4 * SDD_CS;               // LDS bytes per quad: 32 tokens
 constexpr int SDD_BUF = (SDD_NQ + SDD_RMAX / 4) * SDD_QS;    // one buffer: the slice of b, then the slice of a
 constexpr int SDD_STEP = 32;                     // tokens per step = K of one MFMA
+#ifndef SDD_PF
+#define SDD_PF 1
+#endif
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -74,9 +77,10 @@ __device__ __forceinline__ bf16x8 read_tr(const char *smem, int tile, int off) {
 
 // Asynchronous 16-byte-per-lane copy global -> LDS: lane l's 16 bytes land at lds_base + 16 * l.  Written as inline
 // assembly so that the compiler does not make the LDS reads of the other buffer wait for it; the caller waits with
-// s_waitcnt vmcnt(0) and a barrier before the destination is read.
+// s_waitcnt vmcnt(0) and a barrier before the destination is read.  (One wait state separates the write of M0 from
+// its use as the LDS base.)
 __device__ __forceinline__ void load_to_lds_async(const void *gsrc, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gsrc) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gsrc) : "memory", "m0");
 }
 
 __device__ __forceinline__ uint32_t lds_addr(const char *p) {
@@ -152,15 +156,18 @@ __global__ __launch_bounds__(SDD_WAVES * 64) void sdd_kernel(SddArgs p) {
         asm volatile("" : "+s"(nr));
         nr = __builtin_amdgcn_readfirstlane(nr);
         bf16x8 A = {};
-        bf16x8 Bn = read_tr(cur, eo[0] & 0xfffff, tr_off);
+        // the b operand is fetched SDD_PF blocks ahead of its MFMA
+        bf16x8 Bq[SDD_PF];
+#pragma unroll
+        for (int k = 0; k < SDD_PF; ++k) Bq[k] = read_tr(cur, eo[k] & 0xfffff, tr_off);
 #pragma unroll
         for (int b = 0; b < SDD_NB; ++b) {
             if (nr & (1u << b)) {                 // (an empty slot repeats a valid tile: its sum is never stored)
                 const int rs = eo[b] >> 20;
                 A = read_tr(cur, SDD_NQ * SDD_QS + (rs >> 2) * SDD_QS + (rs & 3) * 32, tr_off);
             }
-            const bf16x8 B = Bn;
-            if (b + 1 < SDD_NB) Bn = read_tr(cur, eo[b + 1] & 0xfffff, tr_off);
+            const bf16x8 B = Bq[b % SDD_PF];
+            if (b + SDD_PF < SDD_NB) Bq[b % SDD_PF] = read_tr(cur, eo[b + SDD_PF] & 0xfffff, tr_off);
             acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, B, acc[b], 0, 0, 0);
         }
         __builtin_amdgcn_s_waitcnt(0);                       // the next step's slices have landed
