@@ -344,3 +344,33 @@ def test_qat_mlp_single_op_training_step(dev):
     ref = [xr.grad, mlp.gate_up._cms.mortar_data.grad, mlp.down._cms.mortar_data.grad]
     for name, a, b in zip(("dx", "d gate_up", "d down"), got, ref):
         assert_close_bf16(to_np(a), to_np(b), name, ulps=6)
+
+
+def test_full_size_backward_adjoint_identities(dev):
+    """Headline shapes (d_model 2048, d_ff 5632, 25 %, 4096 tokens): the oracle cannot run these in seconds, so the
+    backward is checked through the adjoint identities of y = x W^T, which hold for any size:
+    <dY, x W^T> = <dY W, x> = <dW, W>, with every product taken from the HIP path and the sums in float64."""
+    spec = synth.synth_mlp(2048, 5632, 0.25, seed=0)
+    M = 4096
+    for name in ("gate_up", "down"):
+        m = spec[name]
+        out_f, in_f = m["shape"]
+        nnz = m["col_idx"].size
+        W = MortarPack(None, None, m["col_idx"], m["offsets"], out_f, in_f, dev)
+        vals = (torch.randn(nnz, 16, 16, device=dev, generator=torch.Generator(device=dev).manual_seed(5)) * 0.05).to(torch.bfloat16)
+        s = W.requantize(vals, per_block=True)
+        Wt = W.transposed()
+        Wt.requantize(vals, per_block=True, transpose=True)
+        x = to_dev(synth.synth_x(M, in_f, seed=6), dev)
+        dy = to_dev(synth.synth_x(M, out_f, seed=7), dev)
+        y, dx, dw = ops.spmm(x, W), ops.spmm(dy, Wt), ops.sdd(dy, x, W)
+        codes = torch.from_numpy(decode_blocks(W.codes.cpu().numpy().view(np.uint32))).to(dev)
+        w_eff = codes.double() * s.to(torch.bfloat16).double()[:, None, None]
+        a = float((dy.double() * y.double()).sum())
+        b = float((dx.double() * x.double()).sum())
+        c = float((dw.double() * w_eff).sum())
+        scale = float(dy.double().pow(2).sum().sqrt() * y.double().pow(2).sum().sqrt())      # Cauchy-Schwarz size of the sum
+        assert abs(a - b) <= 2e-3 * scale and abs(a - c) <= 2e-3 * scale, (name, a, b, c, scale)
+        # and dW of the full-size launch equals dW of two half-batches added (linearity in the token dimension)
+        half = ops.sdd(dy[:2048], x[:2048], W).float() + ops.sdd(dy[2048:], x[2048:], W).float()
+        assert float((dw.float() - half).abs().max()) <= 2.0 ** -6 * float(dw.float().abs().max())
