@@ -147,6 +147,8 @@ def test_stk_dds_both_orientations(dev):
 # ---------------------------------------------------------------------------------------------- weight gradient
 
 @pytest.mark.parametrize("shape,density,zipf,M", [((16 * 4, 16 * 6), 1.0, None, 32), ((16 * 20, 16 * 12), 0.3, 1.2, 1),
+                                                   ((16 * 2, 16 * 1), 1.0, None, 33), ((16 * 3, 16 * 5), 0.6, None, 95),
+                                                   ((16 * 1, 16 * 90), 1.0, None, 64), ((16 * 130, 16 * 2), 0.5, None, 40),
                                                    ((16 * 20, 16 * 12), 0.3, 1.2, 77), ((16 * 40, 16 * 30), 0.25, None, 600),
                                                    ((16 * 6, 16 * 352), 0.25, 1.2, 200), ((16 * 70, 16 * 16), 0.1, None, 4096)])
 def test_sdd_weight_gradient(dev, shape, density, zipf, M):
