@@ -69,16 +69,28 @@ struct RequantArgs {
 
 // mode 0: one scale per matrix from the partial sums, 1: one per block, 2: scale_in[0], 3: scale_in[source block]
 __global__ __launch_bounds__(256) void requant_kernel(RequantArgs a) {
-    const int lane = threadIdx.x & 63;
-    const int j = blockIdx.x * 4 + (threadIdx.x >> 6);
+    __shared__ float tr[4][16][17];                     // per wavefront: one block, for the transposed read
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int j = blockIdx.x * 4 + wv;
     if (j >= a.nnz) return;
     const int src = a.src_block ? a.src_block[j] : j;
     const int n = lane >> 2, q = lane & 3;
+    // the lane's four consecutive values of row n of the source block, in one load
     float w[4];
+    if (a.f32) {
+        const float4 v = reinterpret_cast<const float4 *>(a.values)[(int64_t)src * 64 + lane];
+        w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    } else {
+        const uint2 v = reinterpret_cast<const uint2 *>(a.values)[(int64_t)src * 64 + lane];
+        w[0] = __uint_as_float(v.x << 16); w[1] = __uint_as_float(v.x & 0xffff0000u);
+        w[2] = __uint_as_float(v.y << 16); w[3] = __uint_as_float(v.y & 0xffff0000u);
+    }
+    if (a.transpose) {                                  // element (n, 4q + e) of the result is element (4q + e, n) of the source
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const int c = 4 * q + e;
-        w[e] = load_val(a.values, (int64_t)src * 256 + (a.transpose ? c * 16 + n : n * 16 + c), a.f32 != 0);
+        for (int e = 0; e < 4; ++e) tr[wv][n][4 * q + e] = w[e];
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = tr[wv][4 * q + e][n];
     }
     float s;
     if (a.mode == 0) {
