@@ -52,9 +52,35 @@ def mlp_slice():
                         h_routed_bits=O.bf16_bits(routed["h"]), y_routed_bits=O.bf16_bits(routed["y"]), **out)
 
 
+def train_slice():
+    """One QAT layer's training step: smooth block values (bf16) on a 20 x 12 block topology with Zipf rows, 77 tokens.
+    Expected: the ternarisation (codes, per-matrix and per-block scales), y = x W^T, dx = dy W, dW = dy^T x on the
+    topology, and the SwiGLU derivative of a 77 x (2 x 96) gate_up output."""
+    m = synth.synth_matrix(16 * 20, 16 * 12, 0.3, seed=31, zipf_s=1.2)
+    nnz = m["col_idx"].size
+    rng = np.random.Generator(np.random.PCG64(77))
+    vals = O.bf16_round((rng.standard_normal((nnz, 16, 16), dtype=np.float32) * 0.05).astype(np.float32))
+    x, dy = O.bf16_round(synth.synth_x(77, 16 * 12, seed=78)), O.bf16_round(synth.synth_x(77, 16 * 20, seed=79))
+    q, s = O.ternary_quantize(vals, 0.5)
+    qb, sb = O.ternary_quantize_per_block(vals, 0.5)
+    y = O.bcsr_spmm(x, q, np.float32(s), m["col_idx"], m["offsets"])
+    dx = O.dds_dx(dy, q, np.float32(s), m["row_idx"], m["col_idx"], m["shape"])
+    dw = O.sdd_at_b(dy, x, m["row_idx"], m["col_idx"])
+    gu = O.bf16_round(synth.synth_x(77, 192, seed=80) * 2.0)
+    dh = O.bf16_round(synth.synth_x(77, 96, seed=81))
+    np.savez_compressed(os.path.join(HERE, "train_slice.npz"), col_idx=m["col_idx"], offsets=m["offsets"],
+                        row_idx=m["row_idx"], shape=np.array(m["shape"], np.int64), values_bits=O.bf16_bits(vals),
+                        codes=q, scale_bits=np.float32(s).reshape(1).view(np.uint32), codes_per_block=qb,
+                        scale_per_block_bits=sb.view(np.uint32), x_bits=O.bf16_bits(x), dy_bits=O.bf16_bits(dy),
+                        y_bits=O.bf16_bits(y), dx_bits=O.bf16_bits(dx), dw_bits=O.bf16_bits(dw), gu_bits=O.bf16_bits(gu),
+                        dh_bits=O.bf16_bits(dh), h_bits=O.bf16_bits(O.swiglu(gu)),
+                        dgu_bits=O.bf16_bits(O.swiglu_backward(gu, dh)))
+
+
 if __name__ == "__main__":
     c0()
     mlp_slice()
+    train_slice()
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

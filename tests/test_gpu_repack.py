@@ -376,3 +376,32 @@ def test_full_size_backward_adjoint_identities(dev):
         # and dW of the full-size launch equals dW of two half-batches added (linearity in the token dimension)
         half = ops.sdd(dy[:2048], x[:2048], W).float() + ops.sdd(dy[2048:], x[2048:], W).float()
         assert float((dw.float() - half).abs().max()) <= 2.0 ** -6 * float(dw.float().abs().max())
+
+
+def test_training_golden_fixture(dev):
+    """The HIP training path against the committed vectors (tests/golden/train_slice.npz): device-side ternarisation,
+    forward, dX through the W^T pack, dW on the topology, SwiGLU and its derivative."""
+    import golden_util as G
+    z = G.load("train_slice.npz")
+    shape = tuple(int(v) for v in z["shape"])
+    bits = lambda name: torch.from_numpy(z[name].view(np.int16)).view(torch.bfloat16).to(dev)
+    vals, x, dy = bits("values_bits"), bits("x_bits"), bits("dy_bits")
+    W = MortarPack(None, None, z["col_idx"], z["offsets"], shape[0], shape[1], dev)
+    s = W.requantize(vals)
+    np.testing.assert_allclose(s.cpu().numpy(), z["scale_bits"].view(np.float32), rtol=4e-7, atol=0)
+    got = decode_blocks(W.codes.cpu().numpy().view(np.uint32))
+    v = O.bf16_from_bits(z["values_bits"])
+    off = np.abs(np.abs(v / z["scale_bits"].view(np.float32)[0]) - 0.5) > 1e-5          # away from the threshold itself
+    assert np.array_equal(got[off], z["codes"][off]) and (got != z["codes"]).mean() < 1e-5
+    Wb = MortarPack(None, None, z["col_idx"], z["offsets"], shape[0], shape[1], dev)
+    sb = Wb.requantize(vals, per_block=True)
+    np.testing.assert_allclose(sb.cpu().numpy(), z["scale_per_block_bits"].view(np.float32), rtol=4e-7, atol=0)
+    gotb = decode_blocks(Wb.codes.cpu().numpy().view(np.uint32))
+    assert (gotb != z["codes_per_block"]).mean() < 1e-5
+    Wt = W.transposed()
+    Wt.requantize(vals, scale=s, transpose=True)
+    assert_close_bf16(to_np(ops.spmm(x, W)), O.bf16_from_bits(z["y_bits"]), "y")
+    assert_close_bf16(to_np(ops.spmm(dy, Wt)), O.bf16_from_bits(z["dx_bits"]), "dx")
+    assert_close_bf16(to_np(ops.sdd(dy, x, W)), O.bf16_from_bits(z["dw_bits"]), "dW")
+    assert_close_bf16(to_np(ops.swiglu(bits("gu_bits"))), O.bf16_from_bits(z["h_bits"]), "h")
+    assert_close_bf16(to_np(ops.swiglu_backward(bits("gu_bits"), bits("dh_bits"))), O.bf16_from_bits(z["dgu_bits"]), "dgu", ulps=3)

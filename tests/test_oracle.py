@@ -389,3 +389,23 @@ def test_swiglu_backward_against_central_differences():
     gb = O.bf16_round(gu.astype(np.float32))
     h = O.swiglu(gb)
     np.testing.assert_allclose(h, O.silu(gb[:, :16]) * gb[:, 16:], rtol=2 ** -6, atol=1e-6)
+
+
+def test_training_fixture_matches_the_oracle():
+    """tests/golden/train_slice.npz (ternarisation, forward, dX, dW, SwiGLU and its derivative of one small layer) is
+    what the oracle computes today: guards both against drift."""
+    import golden_util as G
+    z = G.load("train_slice.npz")
+    vals = O.bf16_from_bits(z["values_bits"])
+    x, dy = O.bf16_from_bits(z["x_bits"]), O.bf16_from_bits(z["dy_bits"])
+    q, s = O.ternary_quantize(vals, 0.5)
+    assert np.array_equal(q, z["codes"]) and np.float32(s).view(np.uint32) == z["scale_bits"][0]
+    qb, sb = O.ternary_quantize_per_block(vals, 0.5)
+    assert np.array_equal(qb, z["codes_per_block"]) and np.array_equal(sb.view(np.uint32), z["scale_per_block_bits"])
+    shape = tuple(int(v) for v in z["shape"])
+    assert np.array_equal(O.bf16_bits(O.bcsr_spmm(x, q, np.float32(s), z["col_idx"], z["offsets"])), z["y_bits"])
+    assert np.array_equal(O.bf16_bits(O.dds_dx(dy, q, np.float32(s), z["row_idx"], z["col_idx"], shape)), z["dx_bits"])
+    assert np.array_equal(O.bf16_bits(O.sdd_at_b(dy, x, z["row_idx"], z["col_idx"])), z["dw_bits"])
+    gu, dh = O.bf16_from_bits(z["gu_bits"]), O.bf16_from_bits(z["dh_bits"])
+    assert np.array_equal(O.bf16_bits(O.swiglu(gu)), z["h_bits"])
+    assert np.array_equal(O.bf16_bits(O.swiglu_backward(gu, dh)), z["dgu_bits"])
