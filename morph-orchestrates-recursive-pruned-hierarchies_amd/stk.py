@@ -1,6 +1,6 @@
 """stk_dds / stk_sdd_at_b: the reference's sparse-backend operators (morph/sparse/stk/backend/custom_ops.py:35-136)
 served by the HIP kernels.  The MORTAR runtime executes ternary blocks, so ``data`` must be ternary-valued per
-block (+-s_j or 0); the packed form is cached per data tensor."""
+block (+-s_j or 0); the topology is packed once, the values are encoded on the device at every call."""
 from __future__ import annotations
 
 import torch
@@ -12,39 +12,42 @@ from .pack import MortarPack
 _cache: dict = {}
 
 
-def _pack_from_data(data: Tensor, offsets: Tensor, column_indices: Tensor, out_f: int, in_f: int) -> MortarPack:
-    """Pack of the stored matrix [out_f, in_f]: the topology is packed once per (offsets, column_indices) on the
-    host, the values are ternarised and encoded on the device whenever ``data`` changed."""
-    d = data.detach()
-    if d.dim() != 3 or d.shape[1] != 16 or d.shape[2] != 16:
-        raise ValueError(f"stk_dds: data must be [nnz, 16, 16] (carve(blocking=16)), got {tuple(data.shape)}")
-    tkey = (offsets.data_ptr(), column_indices.data_ptr(), int(d.shape[0]), out_f, in_f, str(d.device))
+def _topology(offsets: Tensor, column_indices: Tensor, nnz: int, out_f: int, in_f: int, device) -> MortarPack:
+    """The pack of a topology (all-zero values), built once per (offsets, column_indices) storage.  The entry keeps the
+    two index tensors alive, so their addresses cannot be handed to other tensors while it is cached."""
+    tkey = (offsets.data_ptr(), offsets._version, column_indices.data_ptr(), column_indices._version, nnz, out_f, in_f,
+            str(device))
     pack = _cache.get(tkey)
     if pack is None:
         if len(_cache) > 64:
             _cache.clear()
-        pack = MortarPack(None, None, column_indices, offsets, out_f, in_f, d.device)
-        pack._values_key = pack._t_values_key = None
+        pack = MortarPack(None, None, column_indices, offsets, out_f, in_f, device)
+        pack._checked = None
+        pack._keepalive = (offsets, column_indices)
         _cache[tkey] = pack
-    vkey = (d.data_ptr(), d._version)
-    if pack._values_key != vkey:
-        df = d if d.dtype in (torch.bfloat16, torch.float32) else d.float()
-        scale = df.abs().amax(dim=(1, 2)).float()
-        if not torch.equal(torch.sign(df.float()) * scale[:, None, None], df.float()):
-            raise ValueError("stk_dds: data is not ternary per block (+-s_j or 0); quantise it first")
-        pack._scale = scale
-        pack._values = df.contiguous()
-        pack.requantize(pack._values, scale=scale, threshold=0.5, sync=False)
-        pack._values_key = vkey
     return pack
 
 
-def _transposed_pack(pack: MortarPack) -> MortarPack:
-    t = pack.transposed()
-    if pack._t_values_key != pack._values_key:
-        t.requantize(pack._values, scale=pack._scale, threshold=0.5, transpose=True, sync=False)
-        pack._t_values_key = pack._values_key
-    return t
+def _pack_from_data(data: Tensor, offsets: Tensor, column_indices: Tensor, out_f: int, in_f: int,
+                    transposed: bool = False) -> MortarPack:
+    """Pack of the stored matrix [out_f, in_f] (or of its transpose): the topology is packed once on the host, the
+    values are encoded on the device on EVERY call (two small launches, no host synchronisation), so a data tensor
+    that changed - in place or by being replaced at the same address - is always honoured.  Only the check that the
+    data is ternary per block (it costs a synchronisation) is skipped while (storage, version) stay the same."""
+    d = data.detach()
+    if d.dim() != 3 or d.shape[1] != 16 or d.shape[2] != 16:
+        raise ValueError(f"stk_dds: data must be [nnz, 16, 16] (carve(blocking=16)), got {tuple(data.shape)}")
+    pack = _topology(offsets, column_indices, int(d.shape[0]), out_f, in_f, d.device)
+    df = (d if d.dtype in (torch.bfloat16, torch.float32) else d.float()).contiguous()
+    scale = df.abs().amax(dim=(1, 2)).float()
+    vkey = (d.data_ptr(), d._version, d.dtype)
+    if pack._checked != vkey:
+        if not torch.equal(torch.sign(df.float()) * scale[:, None, None], df.float()):
+            raise ValueError("stk_dds: data is not ternary per block (+-s_j or 0); quantise it first")
+        pack._checked = vkey
+    target = pack.transposed() if transposed else pack
+    target.requantize(df, scale=scale, threshold=0.5, transpose=transposed, sync=False)
+    return target
 
 
 def _check_meta(offsets: Tensor, row_indices: Tensor, column_indices: Tensor) -> None:
@@ -68,7 +71,7 @@ def stk_dds(lhs: Tensor, data: Tensor, offsets: Tensor, row_indices: Tensor, col
     if transpose_b:
         W = _pack_from_data(data, offsets, column_indices, shape1, shape0)
     else:
-        W = _transposed_pack(_pack_from_data(data, offsets, column_indices, shape0, shape1))
+        W = _pack_from_data(data, offsets, column_indices, shape0, shape1, transposed=True)
     x = lhs if lhs.dtype == torch.bfloat16 else lhs.to(torch.bfloat16)
     y = ops.spmm(x, W)
     return y if y.dtype == lhs.dtype else y.to(lhs.dtype)
@@ -88,14 +91,7 @@ def stk_sdd_at_b(a: Tensor, b: Tensor, data: Tensor, offsets: Tensor, row_indice
     _check_meta(offsets, row_indices, column_indices)
     if data.dim() != 3 or data.shape[1] != 16 or data.shape[2] != 16:
         raise ValueError(f"stk_sdd_at_b: data must be [nnz, 16, 16], got {tuple(data.shape)}")
-    tkey = (offsets.data_ptr(), column_indices.data_ptr(), int(data.shape[0]), a.shape[1], b.shape[1], str(a.device))
-    W = _cache.get(tkey)
-    if W is None:
-        if len(_cache) > 64:
-            _cache.clear()
-        W = MortarPack(None, None, column_indices, offsets, a.shape[1], b.shape[1], a.device)
-        W._values_key = W._t_values_key = None
-        _cache[tkey] = W
+    W = _topology(offsets, column_indices, int(data.shape[0]), a.shape[1], b.shape[1], a.device)
     ab = a if a.dtype == torch.bfloat16 else a.to(torch.bfloat16)
     bb = b if b.dtype == torch.bfloat16 else b.to(torch.bfloat16)
     out = ops.sdd(ab, bb, W)
