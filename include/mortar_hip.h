@@ -300,15 +300,23 @@ int mortar_rmsnorm_bf16(const uint16_t *x, int64_t M, int32_t d, int64_t ldx, co
  *   code = sign(w/s) where |w/s| > threshold (fp32 division, strict compare), else 0; means are summed in fp64
  *   in a fixed order.  The kernels multiply by bf16(s) (round to nearest even), as the reference's bf16 autocast does.
  *   scale_out  device fp32, [1] for modes 0 and 2, [nnz] for 1 and 3 (order of W's blocks), or NULL
- *   status     device int32 [1] or NULL: set to 0, then to 1 if bf16(s) of some block lies outside
- *              [2^-100, 2^100] (that block is zeroed; the host packer returns MORTAR_ERR_SCALE for it)
+ *   status     device int32 [2] or NULL.  Both words are set to 0 first (unless flags bit 0 is set), then
+ *              status[0] = 1 if bf16(s) of some block lies outside [2^-100, 2^100] (that block is zeroed; the host
+ *              packer returns MORTAR_ERR_SCALE for it), status[1] = 1 if the ternary check below fails
+ *   flags      bit 0: do not clear status first, so that it accumulates over several calls (a caller that reads it
+ *              only now and then still sees every failure)
+ *   ternary_tol  > 0 (scale_mode 2 or 3 only): the values are expected to be ternary already, 0 or +-s of the given
+ *              scale; status[1] = 1 if some value is neither, |v| <= tol * s or ||v| - s| <= tol * s.  This is how the
+ *              stk_dds operator states its restriction: the runtime multiplies ternary blocks only, and data that the
+ *              reference's stk_dds would multiply as arbitrary bf16 values is reported instead of silently quantised.
  *   workspace  device, mortar_requantize_workspace_bytes() bytes, 8-byte aligned; needed for scale_mode 0 only
  * mortar_bcsr_t.uniform_scale is host state: after modes 0 / 2 the caller may set it to bf16(s) to select the
  * scale-after-sum kernels, or leave it 0 (per-block kernels, always valid). */
 int64_t mortar_requantize_workspace_bytes(void);
 int mortar_requantize(const mortar_bcsr_t *W, const void *values, int32_t values_f32, const int32_t *pos,
                       const int32_t *src_block, int32_t transpose, int32_t scale_mode, float threshold,
-                      const float *scale_in, float *scale_out, int32_t *status, void *workspace, void *stream);
+                      const float *scale_in, float *scale_out, int32_t *status, int32_t flags, float ternary_tol,
+                      void *workspace, void *stream);
 
 /* ---- SwiGLU between the two matrices, training form ------------------------------------------------ */
 

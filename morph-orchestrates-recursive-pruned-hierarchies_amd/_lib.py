@@ -32,7 +32,8 @@ _SIGS = {
     "mortar_octet_positions_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp]),
     "mortar_transpose_topology_host": (C.c_int, [c_vp, c_vp, c_i32, c_i32, c_vp, c_vp, c_vp]),
     "mortar_requantize_workspace_bytes": (c_i64, []),
-    "mortar_requantize": (C.c_int, [c_vp, c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_f32, c_vp, c_vp, c_vp, c_vp, c_vp]),
+    "mortar_requantize": (C.c_int, [c_vp, c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_f32, c_vp, c_vp, c_vp, c_i32, c_f32,
+                                  c_vp, c_vp]),
     "mortar_swiglu_bf16": (C.c_int, [c_vp, c_i64, c_i64, c_i32, c_vp, c_i64, c_vp]),
     "mortar_swiglu_backward_bf16": (C.c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_i32, c_vp, c_i64, c_vp]),
     "mortar_sdd_plan_host": (c_i64, [c_vp, c_vp, c_i32, c_i32, c_vp, c_i64]),

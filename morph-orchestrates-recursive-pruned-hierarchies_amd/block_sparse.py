@@ -74,7 +74,8 @@ class CMSBlockLinear(nn.Module):
         self._dense_mode, self._mortar, self._mortar_blocking = True, False, 0
         self._values_ternary_mode, self._values_threshold = False, 0.5
         self._pack: MortarPack | None = None
-        self._pack_key = self._pack_t_key = None
+        self._pack_key = None
+        self._pack_gen, self._pack_t_gen = 0, -1
 
     # ------------------------------------------------------------------ masks / carve
 
@@ -193,22 +194,31 @@ class CMSBlockLinear(nn.Module):
         if self._pack is None:
             self._pack = MortarPack(None, None, self.mortar_column_indices, self.mortar_offsets, self.out_features,
                                     self.in_features, d.device)
-            self._pack_key = self._pack_t_key = None
+            self._pack_key = None
+            self._pack_gen, self._pack_t_gen = 0, -1
         key = (d.data_ptr(), d._version)
         if self._pack_key != key:
             self._pack_scale = self._pack.requantize(self._values(), threshold=self._values_threshold, sync=False)
             self._pack_key = key
+            self._pack_gen += 1
         return self._pack
+
+    def invalidate_pack(self) -> None:
+        """Forces the next mortar_pack() of a QAT layer to re-encode the values.  Writes through ``mortar_data.data``
+        (EMA swaps, manual re-initialisation, ``p.data.mul_``) do not advance the parameter's version counter, so the
+        (address, version) key alone would miss them; every training forward therefore calls this first (the re-encode
+        is two small launches and no synchronisation)."""
+        self._pack_key = None
 
     def mortar_pack_t(self) -> MortarPack:
         """The pack of W^T for the dX product (QAT layers on the GPU), refreshed like ``mortar_pack``."""
         if "mortar_packed" in self._buffers or not self.mortar_data.is_cuda:
             raise RuntimeError("mortar_pack_t(): the backward needs a QAT layer (mortar_data) on the GPU")
         t = self.mortar_pack().transposed()
-        if self._pack_t_key != self._pack_key:
+        if self._pack_t_gen != self._pack_gen:
             t.requantize(self._values(), threshold=self._values_threshold, scale=self._pack_scale, transpose=True,
                          sync=False)              # the scale W was packed with: no second reduction over the values
-            self._pack_t_key = self._pack_key
+            self._pack_t_gen = self._pack_gen
         return t
 
     def _values(self) -> Tensor:
@@ -226,6 +236,8 @@ class CMSBlockLinear(nn.Module):
         x2 = x.reshape(-1, self.in_features)
         xb = x2 if x2.dtype == torch.bfloat16 else x2.to(torch.bfloat16)
         trainable = "mortar_packed" not in self._buffers and self._values_ternary_mode and xb.is_cuda
+        if trainable and self.mortar_data.requires_grad:
+            self.invalidate_pack()            # trainable values may have been written through .data since the last call
         if trainable and torch.is_grad_enabled() and (xb.requires_grad or self.mortar_data.requires_grad):
             y = _MortarLinearFn.apply(xb, self.mortar_data, self)
         else:

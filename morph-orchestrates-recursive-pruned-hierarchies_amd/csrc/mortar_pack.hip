@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void abs_sum_kernel(const void *values, int64_
 }
 
 __global__ void clear_status_kernel(int32_t *status) {
-    if (threadIdx.x == 0) *status = 0;
+    if (threadIdx.x < 2) status[threadIdx.x] = 0;
 }
 
 struct RequantArgs {
@@ -65,6 +65,7 @@ struct RequantArgs {
     const double *partial;
     int32_t nnz, f32, transpose, mode;
     float threshold;
+    float ternary_tol;      // > 0: with a given scale, flag values that are neither 0 nor +-s within this relative bound
 };
 
 // mode 0: one scale per matrix from the partial sums, 1: one per block, 2: scale_in[0], 3: scale_in[source block]
@@ -109,11 +110,21 @@ __global__ __launch_bounds__(256) void requant_kernel(RequantArgs a) {
     if ((sb & 0x7fffu) != 0) {
         const uint32_t e8 = (sb >> 7) & 0xffu;
         if (e8 < 27 || e8 > 227) {
-            if (lane == 0 && a.status) *a.status = 1;
+            if (lane == 0 && a.status) a.status[0] = 1;
         } else {
             const uint32_t adj = sb - 0x0400u;
             sd = adj | (adj << 16);
         }
+    }
+    if (a.ternary_tol > 0.f && a.status) {
+        // every value must be 0 or +-s up to the bound (a bf16 cast of +-s(1 + rounding) may land one step beside bf16(s))
+        bool bad = false;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float m = fabsf(w[e]);
+            bad = bad || !(m <= a.ternary_tol * s || fabsf(m - s) <= a.ternary_tol * s);
+        }
+        if (bad) a.status[1] = 1;
     }
     uint32_t row = 0;
 #pragma unroll
@@ -148,8 +159,8 @@ extern "C" int64_t mortar_requantize_workspace_bytes(void) { return (int64_t)PAR
 
 extern "C" int mortar_requantize(const mortar_bcsr_t *W, const void *values, int32_t values_f32, const int32_t *pos,
                                  const int32_t *src_block, int32_t transpose, int32_t scale_mode, float threshold,
-                                 const float *scale_in, float *scale_out, int32_t *status, void *workspace,
-                                 void *stream) {
+                                 const float *scale_in, float *scale_out, int32_t *status, int32_t flags,
+                                 float ternary_tol, void *workspace, void *stream) {
     if (!W || !values || !pos) return mortar_fail(MORTAR_ERR_ARG, "requantize: null pointer");
     if (!W->codes || !W->sdup || !W->codes_o || !W->sd_o || W->nnz <= 0)
         return mortar_fail(MORTAR_ERR_ARG, "requantize: incomplete matrix");
@@ -157,9 +168,12 @@ extern "C" int mortar_requantize(const mortar_bcsr_t *W, const void *values, int
     if (scale_mode >= 2 && !scale_in) return mortar_fail(MORTAR_ERR_ARG, "requantize: scale_mode %d needs scale_in", scale_mode);
     if (scale_mode == 0 && !workspace) return mortar_fail(MORTAR_ERR_ARG, "requantize: scale_mode 0 needs the workspace");
     if (!(threshold >= 0.f)) return mortar_fail(MORTAR_ERR_ARG, "requantize: threshold must be >= 0");
+    if (flags & ~1) return mortar_fail(MORTAR_ERR_ARG, "requantize: unknown flags 0x%x", flags);
+    if (!(ternary_tol >= 0.f) || (ternary_tol > 0.f && (scale_mode < 2 || !status)))
+        return mortar_fail(MORTAR_ERR_ARG, "requantize: ternary_tol needs a given scale (scale_mode 2 or 3) and a status word");
     if (reinterpret_cast<uintptr_t>(values) & 15) return mortar_fail(MORTAR_ERR_ARG, "requantize: values must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (status) hipLaunchKernelGGL(clear_status_kernel, dim3(1), dim3(64), 0, st, status);
+    if (status && !(flags & 1)) hipLaunchKernelGGL(clear_status_kernel, dim3(1), dim3(64), 0, st, status);
     if (scale_mode == 0)
         hipLaunchKernelGGL(abs_sum_kernel, dim3(PARTIALS), dim3(256), 0, st, values, (int64_t)W->nnz * 256, values_f32,
                            static_cast<double *>(workspace));
@@ -181,6 +195,7 @@ extern "C" int mortar_requantize(const mortar_bcsr_t *W, const void *values, int
     a.transpose = transpose;
     a.mode = scale_mode;
     a.threshold = threshold;
+    a.ternary_tol = ternary_tol;
     hipLaunchKernelGGL(requant_kernel, dim3((W->nnz + 3) / 4), dim3(256), 0, st, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "requantize: %s", hipGetErrorString(e));

@@ -72,12 +72,17 @@ class MortarDecodeMLP:
 
 
 @torch.no_grad()
-def looped_core_forward(mlps, x: Tensor, n_iters: int, norm_weights=None, eps: float = 1e-6) -> Tensor:
+def looped_core_forward(mlps, x: Tensor, n_iters: int, norm_weights=None, eps: float = 1e-6, observer=None) -> Tensor:
     """Core-loop call pattern (morph/model/transformer.py:685-728,1146-1169) reduced to the MLP path:
     n_iters passes over the shared blocks, the same weights every pass, iter_idx = t forwarded to each MLP,
-    activations RMS-normalised before every MLP (mhc.py:249-250)."""
+    activations RMS-normalised before every MLP (mhc.py:249-250).  ``observer(t, i, x_in, x_out)``, when given, is
+    called after every MLP call with its input (before the norm) and output (diagnostics, the reference's
+    ``_capture_traj``)."""
     for t in range(n_iters):
         for i, m in enumerate(mlps):
             w = norm_weights[i] if norm_weights is not None else None
-            x = m(x, iter_idx=t, norm=(w, eps))
+            y = m(x, iter_idx=t, norm=(w, eps))
+            if observer is not None:
+                observer(t, i, x, y)
+            x = y
     return x

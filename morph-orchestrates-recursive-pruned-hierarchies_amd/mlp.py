@@ -53,6 +53,7 @@ class _SwiGLUMortarFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x: Tensor, data_gu: Tensor, data_dn: Tensor, mlp: "_SwiGLUMortar") -> Tensor:
         cg, cd = mlp.gate_up._cms, mlp.down._cms
+        cg.invalidate_pack(); cd.invalidate_pack()     # re-encode: .data writes do not advance the version counter
         gu = ops.spmm(x, cg.mortar_pack())
         h = ops.swiglu(gu)
         y = ops.spmm(h, cd.mortar_pack())
@@ -170,8 +171,9 @@ class _SwiGLUMortar(nn.Module):
             rx = x2.detach() if self._aux_detach_input else x2
             g3, aux = self.router(rx, iter_idx=iter_idx)
             self._last_aux_loss = aux
-            gates = g3.reshape(-1, g3.shape[-1]).float().contiguous()
-            active = self.router.last_active
+            gates = g3.detach().reshape(-1, g3.shape[-1]).float().contiguous()
+            # the mask is derived below from the gates of THIS call (active = gates > 0, routing.py:258), never from
+            # router state, which an earlier call of another shape may have left behind
         elif gates is not None:
             gates = gates.reshape(-1, gates.shape[-1]).float().contiguous()
         if gates is not None and self.d_ff % gates.shape[-1]:

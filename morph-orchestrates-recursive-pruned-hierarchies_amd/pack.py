@@ -190,6 +190,7 @@ class MortarPack:
         self._scheds: dict[int, torch.Tensor] = {}
         self._worklists: dict[tuple, tuple] = {}
         self._pos = self._ws = self._status = self.src_block = self._sdd = None
+        self._status_host = self._status_event = None
         self._transposed: "MortarPack | None" = None
         self.struct = self._make_struct()
         self.ref = C.byref(self.struct)
@@ -204,14 +205,18 @@ class MortarPack:
     # ---- device-side re-pack ----------------------------------------------------------------------------------
 
     def requantize(self, values: torch.Tensor, per_block: bool = False, threshold: float = 0.5,
-                   scale: torch.Tensor | None = None, transpose: bool = False, sync: bool = True) -> torch.Tensor:
+                   scale: torch.Tensor | None = None, transpose: bool = False, sync: bool = True,
+                   ternary_tol: float = 0.0) -> torch.Tensor:
         """Ternarise ``values`` [nnz,16,16] (bf16 or fp32, on this device) into this pack, in place, on the current
         stream: scale = mean|w| over the matrix (reference deploy_quant.py:81-95, block_sparse.py:909-919) or per
         block (``per_block``), or the given ``scale`` (fp32 [1] or [nnz], indexed like ``values``); code =
         sign(w/s) * (|w/s| > threshold).  A pack from ``transposed()`` reads the blocks of the original matrix
         (its ``src_block`` map) and pass ``transpose=True``.  Returns the scale tensor (fp32 [1] or [nnz], in this
         pack's block order).  ``sync=True`` waits, raises if a scale left the representable window, and selects the
-        scale-after-sum kernels for a one-scale matrix; ``sync=False`` only enqueues (per-block kernels)."""
+        scale-after-sum kernels for a one-scale matrix; ``sync=False`` only enqueues (per-block kernels) and lets the
+        device status word accumulate: ``poll_status()`` / ``raise_status()`` report it later.
+        ``ternary_tol`` > 0 (with a given ``scale``): values that are neither 0 nor +-scale within that relative bound
+        are reported as an error (the values are expected to be ternary already)."""
         if values.device != self.device or values.dtype not in (torch.bfloat16, torch.float32):
             raise ValueError("requantize: values must be bf16 or fp32 on the pack's device")
         if tuple(values.shape) != (self.nnz, BLK, BLK) or not values.is_contiguous():
@@ -220,7 +225,7 @@ class MortarPack:
         if self._pos is None:
             self._pos = torch.from_numpy(octet_positions(self.h_offsets, self.Rb, self.Cb, self.seg_cb, self.h_col)).to(self.device)
             self._ws = torch.empty(int(L.mortar_requantize_workspace_bytes()) // 8, dtype=torch.float64, device=self.device)
-            self._status = torch.zeros(1, dtype=torch.int32, device=self.device)
+            self._status = torch.zeros(2, dtype=torch.int32, device=self.device)
         if scale is not None:
             scale = scale.detach().to(device=self.device, dtype=torch.float32).reshape(-1).contiguous()
             if scale.numel() not in (1, self.nnz):
@@ -228,23 +233,70 @@ class MortarPack:
             mode = 2 if scale.numel() == 1 else 3
         else:
             mode = 1 if per_block else 0
+        if ternary_tol and scale is None:
+            raise ValueError("requantize: ternary_tol needs a given scale")
         out = torch.empty(1 if mode in (0, 2) else self.nnz, dtype=torch.float32, device=self.device)
         st = torch.cuda.current_stream(self.device).cuda_stream
+        # asynchronous calls leave the status words sticky (flags bit 0) so that a later poll still sees a failure
         _lib.check(L.mortar_requantize(self.ref, values.data_ptr(), int(values.dtype == torch.float32), self._pos.data_ptr(),
                                        self.src_block.data_ptr() if self.src_block is not None else None,
                                        int(bool(transpose)), mode, float(threshold),
                                        scale.data_ptr() if scale is not None else None, out.data_ptr(),
-                                       self._status.data_ptr(), self._ws.data_ptr(), st), "mortar_requantize")
+                                       self._status.data_ptr(), 0 if sync else 1, float(ternary_tol),
+                                       self._ws.data_ptr(), st), "mortar_requantize")
         us = 0.0
         if sync:
-            if int(self._status.item()):
-                raise ValueError("requantize: a block scale lies outside [2^-100, 2^100] (block zeroed)")
+            self.raise_status()
             if mode in (0, 2) and self.scale_after_sum:
                 us = float(out.to(torch.bfloat16).float().item())
+        elif ternary_tol:
+            self._post_status()
         if us != self.uniform_scale:
             self.uniform_scale = us
             self.struct.uniform_scale = us
         return out
+
+    # status of asynchronous re-packs: the device words are copied to pinned host memory behind every call; reading them
+    # costs no synchronisation once the copy has landed
+
+    def _post_status(self) -> None:
+        if torch.cuda.is_current_stream_capturing():       # a captured step keeps the words on the device only
+            return
+        if self._status_host is None:
+            self._status_host = torch.zeros(2, dtype=torch.int32, pin_memory=True)
+            self._status_event = torch.cuda.Event()
+        self._status_host.copy_(self._status, non_blocking=True)
+        self._status_event.record(torch.cuda.current_stream(self.device))
+
+    @staticmethod
+    def _status_error(flags) -> str | None:
+        if flags[1]:
+            return "values are not ternary per block (+-s_j or 0) for the given scale; quantise them first"
+        if flags[0]:
+            return "a block scale lies outside [2^-100, 2^100] (block zeroed)"
+        return None
+
+    def poll_status(self) -> str | None:
+        """Error text of an earlier asynchronous requantize whose status has reached the host, else None.  Never waits.
+        The device words are cleared once an error has been reported."""
+        if self._status_host is None or not self._status_event.query():
+            return None
+        msg = self._status_error(self._status_host.tolist())
+        if msg is not None:
+            self._status.zero_()
+            self._status_host.zero_()
+        return msg
+
+    def raise_status(self) -> None:
+        """Waits for the re-packs enqueued so far and raises ValueError if one of them reported an error."""
+        if self._status is None:
+            return
+        msg = self._status_error(self._status.tolist())
+        if msg is not None:
+            self._status.zero_()
+            if self._status_host is not None:
+                self._status_host.zero_()
+            raise ValueError("requantize: " + msg)
 
     def transposed(self) -> "MortarPack":
         """The pack of W^T [in, out] over the transposed topology (reference: stk matrix.py:107-125), all-zero until

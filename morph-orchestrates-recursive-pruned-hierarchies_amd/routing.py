@@ -44,7 +44,7 @@ class TileRouter(nn.Module):
         self.query_norm = nn.LayerNorm(d_model)
         self.register_buffer("group_load_ema", torch.ones(n_tile_groups) / n_tile_groups)
         self._load_ema_alpha = 0.99
-        self.last_active: Tensor | None = None      # uint8 [N, n] from the last inference call
+        self.last_active: Tensor | None = None      # uint8 [N, n] of the most recent forward / route call (diagnostics)
 
     def group_logits(self, x_flat: Tensor, iter_idx: int = 0) -> Tensor:
         """Steps 1-4 (reference routing.py:181-230): projected, normalised query -> product-key logits."""
@@ -104,6 +104,7 @@ class TileRouter(nn.Module):
                 gates = F.relu(logits)
             gates = gates * (k / gates.sum(dim=-1, keepdim=True).clamp(min=1e-6))
             active = (gates > 0)
+            self.last_active = active.detach().to(torch.uint8)
         else:
             gates, active = gates_from_logits(logits, k)
             self.last_active = active

@@ -22,32 +22,56 @@ def _topology(offsets: Tensor, column_indices: Tensor, nnz: int, out_f: int, in_
         if len(_cache) > 64:
             _cache.clear()
         pack = MortarPack(None, None, column_indices, offsets, out_f, in_f, device)
-        pack._checked = None
         pack._keepalive = (offsets, column_indices)
         _cache[tkey] = pack
     return pack
 
 
+# A bf16 cast of +-s (1 + fp32 rounding) may land one bf16 step beside bf16(s): accepted as ternary.
+_TERNARY_TOL = 2.0 ** -7
+
+
 def _pack_from_data(data: Tensor, offsets: Tensor, column_indices: Tensor, out_f: int, in_f: int,
                     transposed: bool = False) -> MortarPack:
     """Pack of the stored matrix [out_f, in_f] (or of its transpose): the topology is packed once on the host, the
-    values are encoded on the device on EVERY call (two small launches, no host synchronisation), so a data tensor
-    that changed - in place or by being replaced at the same address - is always honoured.  Only the check that the
-    data is ternary per block (it costs a synchronisation) is skipped while (storage, version) stay the same."""
+    values are encoded on the device on EVERY call (no host synchronisation), so a data tensor that changed - in
+    place or by being replaced at the same address - is always honoured.  The MORTAR runtime multiplies ternary
+    blocks only: the encode kernel checks that every value is 0 or +-s_j (s_j = the block's largest magnitude) and
+    raises a flag on the device otherwise.  The first call on a topology waits for that flag; later calls read it
+    without waiting, so a violation is reported by the first call that finds the flag on the host (at the latest by
+    ``stk_check()``)."""
     d = data.detach()
     if d.dim() != 3 or d.shape[1] != 16 or d.shape[2] != 16:
         raise ValueError(f"stk_dds: data must be [nnz, 16, 16] (carve(blocking=16)), got {tuple(data.shape)}")
     pack = _topology(offsets, column_indices, int(d.shape[0]), out_f, in_f, d.device)
+    target = pack.transposed() if transposed else pack
+    msg = target.poll_status()
+    if msg is not None:
+        raise ValueError("stk_dds (an earlier call): " + msg)
     df = (d if d.dtype in (torch.bfloat16, torch.float32) else d.float()).contiguous()
     scale = df.abs().amax(dim=(1, 2)).float()
-    vkey = (d.data_ptr(), d._version, d.dtype)
-    if pack._checked != vkey:
-        if not torch.equal(torch.sign(df.float()) * scale[:, None, None], df.float()):
-            raise ValueError("stk_dds: data is not ternary per block (+-s_j or 0); quantise it first")
-        pack._checked = vkey
-    target = pack.transposed() if transposed else pack
-    target.requantize(df, scale=scale, threshold=0.5, transpose=transposed, sync=False)
+    first = getattr(target, "_stk_checked", None) is None
+    target.requantize(df, scale=scale, threshold=0.5, transpose=transposed, sync=False, ternary_tol=_TERNARY_TOL)
+    if first:
+        try:
+            target.raise_status()
+        except ValueError as e:
+            raise ValueError("stk_dds: " + str(e).split(": ", 1)[-1]) from None
+        target._stk_checked = True
     return target
+
+
+def stk_check() -> None:
+    """Waits for the device and raises ValueError if any stk_dds call so far was handed data that is not ternary per
+    block.  Calls of stk_dds report such an error themselves once the device flag has reached the host; this is the
+    synchronous form for the end of a step or a test."""
+    for pack in list(_cache.values()):
+        for t in (pack, pack._transposed):
+            if t is not None:
+                try:
+                    t.raise_status()
+                except ValueError as e:
+                    raise ValueError("stk_dds: " + str(e).split(": ", 1)[-1]) from None
 
 
 def _check_meta(offsets: Tensor, row_indices: Tensor, column_indices: Tensor) -> None:

@@ -166,6 +166,37 @@ def test_mlp_with_gates_and_skip(dev):
     assert torch.equal(y2, y)
 
 
+def test_routed_module_mask_follows_the_call(dev):
+    """The carved routed forward takes its tile mask from the gates of the current call: a no-grad call with 128 rows
+    followed by a grad-enabled call with 32 other rows (router parameters trainable, weights packed) must route the
+    second call by its own gates, not by what the first call left in the router."""
+    d_model, d_ff, ncl = 256, 16 * 40, 40
+    spec = synth.synth_mlp(d_model, d_ff, 0.3, seed=33)
+    mlp = synth.mlp_module(spec, dev)
+    mlp.enable_routing(n_clusters=ncl, activation_ratio=0.25, n_iters=1)
+    torch.manual_seed(5)
+    with torch.no_grad():
+        mlp.router.group_bias.copy_(torch.randn(ncl, device=dev))
+    def oracle_for(x):
+        with torch.no_grad():
+            lg = mlp.router.group_logits(to_dev(x, dev), 0).float().cpu().numpy()
+        g_ref, a_ref = O.remoe_gates(lg, mlp.router.activation_k)
+        return O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=g_ref)["y"], a_ref
+    xa, xb = synth.synth_x(128, d_model, 34), synth.synth_x(32, d_model, 35)
+    with torch.no_grad():
+        ya = mlp(to_dev(xa, dev))
+    ref_a, act_a = oracle_for(xa)
+    assert_close_bf16(to_np(ya), ref_a, "no-grad call", ulps=8)
+    assert mlp.router.last_active.shape == (128, ncl)
+    assert any(p.requires_grad for p in mlp.router.parameters()) and torch.is_grad_enabled()
+    yb = mlp(to_dev(xb, dev))                                  # grad mode on, x and the packed weights need none
+    ref_b, act_b = oracle_for(xb)
+    assert not np.array_equal(act_a[:32], act_b)
+    assert_close_bf16(to_np(yb), ref_b, "grad-enabled call after a larger no-grad call", ulps=8)
+    assert mlp.router.last_active.shape == (32, ncl)
+    assert np.array_equal(mlp.router.last_active.cpu().numpy().astype(bool), act_b)
+
+
 @pytest.mark.parametrize("d_model,d_ff", [(256, 16 * 40), (2048, 16 * 24), (16 * 30, 16 * 352)])
 def test_prefill_code_streams_agree(dev, d_model, d_ff):
     """Prefill kernels over the 4-bit code stream and over the 2-bit one do the same arithmetic: identical bits
@@ -519,6 +550,66 @@ def test_looped_core_stack_small(dev):
     mlps = [synth.mlp_module(s, dev) for s in specs]
     y = mortar_amd.looped_core_forward(mlps, to_dev(x, dev), 3)
     assert_close_bf16(to_np(y), ref, "looped stack", ulps=64, max_rel=2e-2)
+
+
+def test_looped_core_stack_full_size(dev):
+    """benchmark config 4 at its own size: 8 shared blocks x 6 iterations, d_model 2048 / d_ff 5632, 4096 tokens,
+    Zipf(1.2) row lengths clipped to 5-60 %, RMSNorm (with a weight) folded into every gate_up launch.
+    Every one of the 48 MLP calls is checked on sampled rows against the oracle fed the HIP input of THAT call,
+    so the error of earlier calls does not compound into the comparison; the final output is checked for
+    finiteness and for the row RMS the oracle's last call predicts."""
+    d_model, d_ff, M, n_blocks, n_iters = 2048, 5632, 4096, 8, 6
+    specs = [synth.synth_mlp(d_model, d_ff, 0.25, seed=400 + i, zipf_s=1.2) for i in range(n_blocks)]
+    for s in specs:                                            # the rows really are uneven
+        cnt = np.diff(s["gate_up"]["offsets"])
+        assert cnt.min() <= 0.06 * 128 + 1 and cnt.max() >= 0.55 * 128
+    rng = np.random.default_rng(410)
+    norm_w = [O.bf16_round(rng.uniform(0.5, 1.5, d_model).astype(np.float32)) for _ in range(n_blocks)]
+    mlps = [synth.mlp_module(s, dev) for s in specs]
+    assert all(ops.norm_fusable(m.gate_up._cms.mortar_pack()) for m in mlps)
+    rows = np.array([0, 31, 32, 1000, 2047, 2048, 3333, 4095])
+    rows_t = torch.from_numpy(rows).to(dev)
+    seen = []
+    def observer(t, i, x_in, x_out):
+        seen.append((t, i, x_in[rows_t].float().cpu().numpy(), x_out[rows_t].float().cpu().numpy()))
+    x = synth.synth_x(M, d_model, 411)
+    y = mortar_amd.looped_core_forward(mlps, to_dev(x, dev), n_iters, norm_weights=[to_dev(w, dev) for w in norm_w],
+                                       observer=observer)
+    assert len(seen) == n_blocks * n_iters and [(t, i) for t, i, _, _ in seen] == \
+        [(t, i) for t in range(n_iters) for i in range(n_blocks)]
+    assert np.array_equal(seen[0][2], x[rows])
+    for k, (t, i, xin, yout) in enumerate(seen):
+        ref = O.swiglu_mlp(O.rmsnorm(xin, norm_w[i], 1e-6), specs[i]["gate_up"], specs[i]["down"])["y"]
+        assert_close_bf16(yout, ref, f"iteration {t} block {i}", ulps=8, max_rel=1e-2)
+        if k + 1 < len(seen):
+            assert np.array_equal(seen[k + 1][2], yout)                   # the next call reads this output unchanged
+    yn = to_np(y)
+    assert np.isfinite(yn).all() and np.array_equal(yn[rows], seen[-1][3])
+    rms = np.sqrt((yn.astype(np.float64) ** 2).mean(1))
+    assert rms.min() > 0 and rms.max() / np.median(rms) < 10 and rms.min() / np.median(rms) > 0.1
+
+
+def test_known_answers_on_the_device(dev):
+    """Hand-written cases of the three rules a loose test would let slip: the strict threshold of the ternary rule,
+    the place of eps in the RMSNorm, and the lo side of a straddling block in route_flags."""
+    # RMSNorm: x = (3, 4) * 2^-8 (bf16-exact) repeated: mean(x^2) = 12.5 * 2^-16, eps = 2^-16 -> y = x * 2^8 / sqrt(13.5)
+    x = np.tile(np.array([3.0, 4.0], np.float32) * 2.0 ** -8, (3, 64))
+    y = to_np(ops.rmsnorm(to_dev(x, dev), None, 2.0 ** -16))
+    want = O.bf16_round(np.tile(np.array([3.0, 4.0]) / np.sqrt(13.5), (3, 64)).astype(np.float32))
+    assert np.array_equal(y, want), (y[0, :2], want[0, :2])              # eps outside the root gives 0.664 / 0.886
+    assert np.array_equal(y, O.rmsnorm(x, None, 2.0 ** -16))
+    # the fused form (norm applied while gate_up stages x) sees the same eps
+    spec = synth.synth_mlp(128, 64, 0.5, seed=77)
+    Wgu = synth.to_pack(spec["gate_up"], dev)
+    xd = to_dev(x, dev)
+    assert torch.equal(ops.gateup_swiglu(xd, Wgu, norm=(None, 2.0 ** -16)), ops.gateup_swiglu(to_dev(want, dev), Wgu))
+    # route_flags, clusters of 8 (a 16-wide block spans lo = 2r and hi = 2r + 1): lo side alone, hi side alone
+    g = torch.zeros((3, 16), device=dev); g[0, 2] = 1.0; g[1, 3] = 0.5; g[2, 14] = 0.25
+    ract, cact = ops.route_flags(g, 128)
+    assert cact.cpu().tolist() == [[0, 1, 0, 0, 0, 0, 0, 0], [0, 1, 0, 0, 0, 0, 0, 0], [0, 0, 0, 0, 0, 0, 0, 1]]
+    assert ract.cpu().tolist() == [c + c for c in cact.cpu().tolist()]
+    gz = torch.zeros((1, 16), device=dev); gz[0, 2] = -1.0; gz[0, 5] = float("nan")
+    assert int(ops.route_flags(gz, 128)[1].sum()) == 0
 
 
 # ---------------------------------------------------------------------------------------------- full size, by properties

@@ -61,6 +61,32 @@ def test_requantize_equals_the_host_pack(dev, dtype, per_block, shape, seg):
     assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), ref, "spmm after requantize")
 
 
+def test_requantize_threshold_is_strict(dev):
+    """Known answers at the cut (deploy_quant.py:94, strict >): values exactly on threshold * mean|w| get code 0."""
+    m = dict(col_idx=np.array([0, 1], np.int16), offsets=np.array([0, 2], np.int32))
+    W = MortarPack(None, None, m["col_idx"], m["offsets"], 16, 32, dev)
+    for dtype in (torch.float32, torch.bfloat16):
+        v = np.full((2, 16, 16), 2.0, np.float32)
+        v[:, 0, :8] = 1.0; v[:, 1, :8] = -3.0                     # per block: mean|w| = (240*2 + 8 + 24) / 256 = 2 exactly
+        v[1] *= -0.5                                              # second block: mean 1, the entries -0.5 on the cut
+        vt = torch.from_numpy(v).to(dtype).to(dev)
+        s = W.requantize(vt, per_block=True, threshold=0.5).cpu().numpy()
+        assert s.tolist() == [2.0, 1.0]
+        q = decode_blocks(W.codes.cpu().numpy().view(np.uint32))
+        assert (q[0, 0, :8] == 0).all() and (q[0, 1, :8] == -1).all() and (q[0, 2:] == 1).all() and (q[0, 0, 8:] == 1).all()
+        assert (q[1, 0, :8] == 0).all() and (q[1, 1, :8] == 1).all() and (q[1, 2:] == -1).all()
+        assert np.array_equal(q, O.ternary_quantize_per_block(v)[0])
+        # per matrix: mean|w| = 1.5, cut at 0.75: |v| = 0.5 drops, 1.0 and above stay
+        s = W.requantize(vt, per_block=False, threshold=0.5).cpu().numpy()
+        assert s.tolist() == [1.5]
+        q = decode_blocks(W.codes.cpu().numpy().view(np.uint32))
+        assert (q[0, 0, :8] == 1).all() and (q[1, 0, :8] == 0).all() and np.array_equal(q, O.ternary_quantize(v)[0])
+    v = np.full((2, 16, 16), 4.0, np.float32); v[:, 0, :] = 2.0; v[:, 1, :] = 6.0          # mean|w| = 4 exactly
+    s = W.requantize(torch.from_numpy(v).to(dev), per_block=False, threshold=0.5).cpu().numpy()
+    q = decode_blocks(W.codes.cpu().numpy().view(np.uint32))
+    assert s.tolist() == [4.0] and (q[:, 0, :] == 0).all() and (q[:, 1:, :] == 1).all()
+
+
 def test_requantize_given_scales_and_refresh(dev):
     """Given scales (one or per block), a second refresh with other values, and the asynchronous form."""
     m = synth.synth_matrix(16 * 8, 16 * 24, 0.3, seed=21)
@@ -242,6 +268,67 @@ def test_qat_layer_forward_backward(dev, M):
         with torch.no_grad():                      # an optimiser step: same storage, new version
             lin.mortar_data.add_(lin.mortar_data.grad, alpha=-0.05)
             lin.mortar_data.grad = None
+
+
+def test_qat_pack_follows_writes_through_data(dev):
+    """Writes through ``mortar_data.data`` do not advance the parameter's version counter; the training forward re-encodes
+    the values on every call, so forward, dX and dW all see the new values."""
+    lin = _qat_layer(16 * 6, 16 * 5, 0.5, 66, dev)
+    x = synth.synth_x(40, lin.in_features, seed=67)
+    xt = to_dev(x, dev).requires_grad_(True)
+    y0 = lin(xt)
+    v0 = lin.mortar_data._version
+    lin.mortar_data.data.mul_(-1.0)
+    assert lin.mortar_data._version == v0                            # the write is invisible to the version key
+    y1 = lin(xt)
+    assert torch.equal(y1, -y0)
+    dy = to_dev(synth.synth_x(40, lin.out_features, seed=68), dev)
+    y1.backward(dy)
+    W = _effective_dense(lin)
+    assert_close_bf16(to_np(xt.grad), (O.bf16_round(to_np(dy)).astype(np.float64) @ W).astype(np.float32), "dx after .data write")
+    lin.mortar_data.data.mul_(-1.0)
+    with torch.no_grad():                                            # the inference path follows explicit invalidation
+        lin.invalidate_pack()
+        assert torch.equal(lin(xt.detach()), y0)
+
+
+def test_stk_dds_fp32_effective_data_and_non_ternary_report(dev):
+    """The reference's own caller in fp32: _mortar_effective_data() = d + (scale*q - d).detach() is +-s only to within an
+    fp32 ulp (several distinct magnitudes) and must be accepted; data that is not ternary is reported, by the first
+    call on a topology synchronously and by later calls through the device flag (stk_check waits for it)."""
+    import mortar_amd
+    from mortar_amd import stk
+    lin = _qat_layer(16 * 8, 16 * 6, 0.5, 86, dev)
+    eff = lin._mortar_effective_data().detach()
+    assert eff.dtype == torch.float32
+    mags = torch.unique(eff.abs()[eff != 0])
+    assert mags.numel() > 1 and float(mags.max() / mags.min()) < 1 + 1e-5      # really not bit-equal magnitudes
+    z32, z16 = torch.zeros(1, dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int16, device=dev)
+    args = (lin.mortar_offsets, lin.mortar_row_indices, lin.mortar_column_indices, z32, z16, z32)
+    x = synth.synth_x(30, lin.in_features, seed=87)
+    y = mortar_amd.stk_dds(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
+    assert_close_bf16(to_np(y), (O.bf16_round(x).astype(np.float64) @ _effective_dense(lin).T).astype(np.float32), "fp32 effective data")
+    yb = mortar_amd.stk_dds(to_dev(x, dev), eff.to(torch.bfloat16), *args, lin.in_features, lin.out_features, True)
+    assert torch.equal(y, yb)
+    stk.stk_check()                                                   # nothing to report so far
+    # same topology, later call, data that is NOT ternary: no wait in the call itself, the flag is raised on the device
+    bad = eff.clone(); bad[3, 2, 1] = 0.37 * float(mags[0])
+    mortar_amd.stk_dds(to_dev(x, dev), bad, *args, lin.in_features, lin.out_features, True)
+    with pytest.raises(ValueError, match="not ternary"):
+        stk.stk_check()
+    stk.stk_check()                                                   # reported once, then clean again
+    mortar_amd.stk_dds(to_dev(x, dev), bad, *args, lin.in_features, lin.out_features, True)
+    torch.cuda.synchronize()
+    with pytest.raises(ValueError, match="earlier call"):             # the next call finds the flag on the host
+        mortar_amd.stk_dds(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
+    y2 = mortar_amd.stk_dds(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
+    assert torch.equal(y2, y)
+    # a fresh topology sees the error in its first call
+    m = synth.synth_matrix(64, 64, 0.5, seed=88)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    with pytest.raises(ValueError, match="not ternary"):
+        mortar_amd.stk_dds(torch.zeros(4, 64, dtype=torch.bfloat16, device=dev), torch.randn(m["col_idx"].size, 16, 16, device=dev),
+                           t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32, 64, 64, True)
 
 
 def test_qat_mlp_trains_layer_by_layer(dev):

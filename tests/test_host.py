@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in mortar_hip.h but not exported"
     assert declared == set(_lib.EXPORTS)
-    assert _lib.lib().mortar_abi_version() == 4
+    assert _lib.lib().mortar_abi_version() == 5
 
 
 def test_encode_round_trip_and_bit_layout():

@@ -66,16 +66,34 @@ def test_transpose_meta_invariants():
 # ---- ternary / pack ----------------------------------------------------------------------------------
 
 def test_ternary_quantize_rule():
-    w = np.array([0.0, 0.49, 0.5, 0.51, -0.5, -0.51, 2.0, -3.0], dtype=np.float32)
-    w = w * np.float32(1.0) / np.abs(w).mean() * np.float32(1.0)            # mean|w| == 1 -> thresholds are |w| > 0.5
+    # known answers written out by hand (deploy_quant.py:91-94): sum|w| = 8 over 8 entries, so the scale is exactly
+    # 1.0 and the entries +-0.5 sit exactly ON the threshold 0.5 * mean|w|: the compare is strict, their code is 0
+    w = np.array([0.5, -0.5, 1.5, -1.5, 1.0, -1.0, 2.0, 0.0], dtype=np.float32)
     q, s = O.ternary_quantize(w)
-    wn = w / s
-    assert np.array_equal(q, (np.sign(wn) * (np.abs(wn) > 0.5)).astype(np.int8))
-    assert q[2 if abs(wn[2]) <= 0.5 else 0] == 0                             # strict >
+    assert s == np.float32(1.0)
+    assert q.tolist() == [0, 0, 1, -1, 1, -1, 1, 0]
+    # the same values times 4 (power of two: every quotient is exact): scale 4, entries +-2 on the threshold
+    q4, s4 = O.ternary_quantize(w * np.float32(4.0))
+    assert s4 == np.float32(4.0) and q4.tolist() == [0, 0, 1, -1, 1, -1, 1, 0]
+    # one ulp above the threshold is kept, one ulp below is dropped
+    w2 = w.copy(); w2[0] = np.nextafter(np.float32(0.5), np.float32(1)); w2[1] = -np.nextafter(np.float32(0.5), np.float32(0))
+    w2[7] = np.float32(8.0) - np.abs(w2[:7]).sum(dtype=np.float32)            # keeps sum|w| = 8 to within an ulp
+    q2, s2 = O.ternary_quantize(w2)
+    assert abs(float(s2) - 1.0) < 1e-6 and q2[:2].tolist() == [1, 0]
+    # a threshold other than the default moves the cut with it
+    assert O.ternary_quantize(w, threshold=1.0)[0].tolist() == [0, 0, 1, -1, 0, 0, 1, 0]
+    # the per-block form applies the same strict rule with each block's own mean
+    wb = np.zeros((2, 16, 16), np.float32)
+    wb[0] = 2.0; wb[0, 0, :8] = 1.0; wb[0, 1, :8] = -3.0     # mean|w| = (240*2 + 8 + 24) / 256 = 2.0: the 1.0s sit on the cut
+    wb[1] = -0.25; wb[1, 5, 5] = 0.125                       # mean = (255*0.25 + 0.125) / 256: 0.125 is just above half of it
+    qb, sb = O.ternary_quantize_per_block(wb)
+    assert sb[0] == np.float32(2.0) and (qb[0, 0, :8] == 0).all() and (qb[0, 1, :8] == -1).all() and (qb[0, 2:] == 1).all()
+    assert qb[1, 5, 5] == 1 and (qb[1].sum() == -255 + 1)
     # invariant of tests/test_lifecycle_tst_qat.py:100-105: every non-zero effective weight has one magnitude
     eff = q.astype(np.float32) * s
     assert len(np.unique(np.abs(eff[eff != 0]))) == 1
-    assert O.ternary_quantize(np.zeros(8, np.float32))[1] == np.float32(1e-8)  # clamp
+    assert O.ternary_quantize(np.zeros(8, np.float32))[1] == np.float32(1e-8)  # clamp (deploy_quant.py:91)
+    assert O.ternary_quantize_per_block(np.zeros((1, 16, 16), np.float32))[1][0] == np.float32(1e-6)  # block_sparse.py:397
 
 
 def test_ternary_per_block_is_per_tensor_on_each_block():
@@ -286,15 +304,46 @@ def test_route_flags_closed_form():
     ract, cact = O.route_flags(gates, 128, 16)
     assert cact.tolist() == [[0, 0, 1, 1, 0, 0, 0, 0], [0, 0, 0, 0, 0, 0, 1, 1]]
     assert ract.tolist() == [c + c for c in cact.tolist()]
-    g2 = np.zeros((1, 16), np.float32); g2[0, 3] = 1.0                           # clusters of 8: a block spans two
-    assert O.route_flags(g2, 128, 16)[1].tolist() == [[0, 1, 0, 0, 0, 0, 0, 0]]
+    # clusters of 8: block r spans clusters lo = 2r and hi = 2r + 1 (engine.py:384-413); either side alone turns it on
+    g_hi = np.zeros((1, 16), np.float32); g_hi[0, 3] = 1.0                       # hi side of block 1 only
+    assert O.route_flags(g_hi, 128, 16)[1].tolist() == [[0, 1, 0, 0, 0, 0, 0, 0]]
+    g_lo = np.zeros((1, 16), np.float32); g_lo[0, 2] = 1.0                       # lo side of block 1 only
+    assert O.route_flags(g_lo, 128, 16)[1].tolist() == [[0, 1, 0, 0, 0, 0, 0, 0]]
+    g_lo[0, 2] = 0.0; g_lo[0, 14] = 0.25                                         # lo side of the last block
+    rl, cl = O.route_flags(g_lo, 128, 16)
+    assert cl.tolist() == [[0, 0, 0, 0, 0, 0, 0, 1]] and rl.tolist() == [[0] * 7 + [1] + [0] * 7 + [1]]
+    # clusters of 24 over d_ff 96 (not a multiple of the block): block 1 = features 16..31 straddles clusters 0 | 1,
+    # block 4 = features 64..79 straddles 2 | 3
+    g24 = np.zeros((1, 4), np.float32); g24[0, 0] = 1.0
+    assert O.route_flags(g24, 96, 16)[1].tolist() == [[1, 1, 0, 0, 0, 0]]
+    g24[0, 0] = 0.0; g24[0, 3] = 1.0
+    assert O.route_flags(g24, 96, 16)[1].tolist() == [[0, 0, 0, 0, 1, 1]]
+    # a gate that is not positive does not count (strict > 0), NaN does not either
+    gz = np.zeros((1, 16), np.float32); gz[0, 2] = -1.0; gz[0, 5] = np.nan
+    assert O.route_flags(gz, 128, 16)[1].sum() == 0
 
 
 def test_rmsnorm_closed_form():
+    # known answers: x = (3, 4) * 1e-3, mean(x^2) = 12.5e-6, eps = 1e-6 -> x * rsqrt(13.5e-6): y = (sqrt(2/3), sqrt(32/27)).
+    # eps is as large as 8 % of the mean square here, so eps outside the root, a dropped eps or mean -> sum all miss.
+    x = np.array([[3e-3, 4e-3]], dtype=np.float32)
+    y = O.rmsnorm(x, None, 1e-6, bf16_out=False)
+    np.testing.assert_allclose(y[0], [0.816496580927726, 1.0886621079036347], rtol=2e-6)
+    # eps = 1 on x = (3, 4): the same numbers again (rsqrt(12.5 + 1) = rsqrt(13.5)), with eps >> rounding
+    y1 = O.rmsnorm(np.array([[3.0, 4.0]], np.float32), None, 1.0, bf16_out=False)
+    np.testing.assert_allclose(y1[0], [0.816496580927726, 1.0886621079036347], rtol=1e-6)
+    # eps = 0: unit mean square exactly
+    y0 = O.rmsnorm(np.array([[3.0, 4.0]], np.float32), None, 0.0, bf16_out=False)
+    np.testing.assert_allclose(y0[0], [3 / np.sqrt(12.5), 4 / np.sqrt(12.5)], rtol=1e-6)
+    # the weight multiplies after the cast to the activation dtype (attention.py:139-141): bf16(bf16(x r) w)
+    xb = O.bf16_round(np.array([[1.0, 2.0, 3.0, 4.0]], np.float32)); w = np.array([1.5, 1.0, 0.5, 3.0], np.float32)
+    r = 1.0 / np.sqrt(7.5 + 1e-6)
+    want = O.bf16_round(O.bf16_round((xb * np.float32(r)).astype(np.float32)) * w)
+    assert np.array_equal(O.rmsnorm(xb, w, 1e-6), want)
+    assert O.rmsnorm(xb, w, 1e-6)[0, 3] == O.bf16_round(np.float32(O.bf16_round(np.float32(4 * r)) * 3.0))
     x = xbf(4, 64, 60)
     y = O.rmsnorm(x, None, 1e-6, bf16_out=False)
     assert np.allclose((y.astype(np.float64) ** 2).mean(1), 1.0, atol=1e-4)
-    assert np.allclose(y, x / np.sqrt((x.astype(np.float64) ** 2).mean(1, keepdims=True) + 1e-6), rtol=1e-5)
     w = np.full(64, 2.0, np.float32)
     assert np.allclose(O.rmsnorm(x, w, bf16_out=False), 2 * y)
 
