@@ -265,6 +265,24 @@ int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_e
                      const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc,
                      void *stream);
 
+/* mortar_gemv_bf16 for callers that cannot allocate device memory or hand in a workspace: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and
+ * results (bit for bit) as mortar_gemv_bf16 minus `part`: the fp32 partial sums of split rows (nslots > 1) go to a
+ * buffer of MORTAR_GEMV_NOALLOC_MAX_FLOATS floats (4 MiB) that lives inside the library, one copy per GPU, held
+ * until the process ends.  nslots * B * Rb*16 floats beyond that size are refused with MORTAR_ERR_LIMIT.  The call
+ * allocates nothing, neither on the device nor on the host side of HIP.  All calls on one GPU share that GPU's buffer:
+ * calls that may overlap there (different streams, different threads) race on it and must be ordered by the caller;
+ * calls on one stream are ordered by the stream.  The first call on a device looks up the buffer's address
+ * (hipGetSymbolAddress): make one call outside a graph capture before capturing. */
+#define MORTAR_GEMV_NOALLOC_MAX_FLOATS (1 << 20)
+int64_t mortar_gemv_noalloc_max_floats(void);
+int mortar_gemv_bf16_noalloc(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_entries, int32_t nslots,
+                             const int32_t *row_slots, int32_t kseg, int32_t mode, const uint16_t *x, int32_t B,
+                             int64_t ldx, uint16_t *y, int64_t ldy,
+                             const float *gates, int32_t n_clusters, int64_t ldg,
+                             const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc,
+                             void *stream);
+
 /* ---- RMSNorm ---------------------------------------------------------------------------------- */
 
 /* mortar_gateup_swiglu_bf16 with the RMSNorm in front of the MLP (attention.RMSNorm, morph/model/attention.py:133-141,

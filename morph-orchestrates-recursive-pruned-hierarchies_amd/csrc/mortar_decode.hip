@@ -9,6 +9,8 @@
 // registers and contracts them with the staged activations in one 16x16x32 bf16 MFMA per 16 streams: the
 // matrix pipe does the 512 multiply-adds of a block pair in one issue slot, which keeps the vector ALU free
 // for the unpack -- the step that bounds this kernel when done with scalar FMAs.
+#include <mutex>
+
 #include "mortar_device.h"
 #include "mortar_internal.h"
 
@@ -189,32 +191,21 @@ int launch_gemv(const GemvParams &p, hipStream_t st) {
 
 }  // namespace
 
-extern "C" int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_entries,
-                                int32_t nslots, const int32_t *row_slots, int32_t kseg, int32_t mode,
-                                const uint16_t *x, int32_t B, int64_t ldx, uint16_t *y, int64_t ldy, float *part,
-                                const float *gates, int32_t n_clusters, int64_t ldg,
-                                const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc,
-                                void *stream) {
-    if (!W || !W->codes || !W->sdup || !W->col || !entries || !x || !y)
-        return mortar_fail(MORTAR_ERR_ARG, "gemv: null pointer");
-    if (B <= 0 || B > 64) return mortar_fail(MORTAR_ERR_LIMIT, "gemv: B=%d outside 1..64", B);
-    if (n_entries <= 0 || n_entries % 4 || n_entries > (int64_t)0x7fffffff) return mortar_fail(MORTAR_ERR_ARG, "gemv: entry count must be a positive multiple of 4");
-    if (mode != 0 && mode != 1) return mortar_fail(MORTAR_ERR_ARG, "gemv: mode must be 0 or 1");
-    if (mode == 1 && (W->Rb & 1)) return mortar_fail(MORTAR_ERR_ARG, "gemv: gate_up needs an even number of block-rows");
-    if (nslots < 1 || (nslots > 1 && (!part || !row_slots))) return mortar_fail(MORTAR_ERR_ARG, "gemv: nslots > 1 needs the partial workspace and row_slots");
-    if (kseg <= 0) return mortar_fail(MORTAR_ERR_ARG, "gemv: kseg must be positive");
-    const int64_t nout = mode == 0 ? (int64_t)W->Rb * 16 : (int64_t)W->Rb * 8;
-    if (ldx < (int64_t)W->Cb * 16 || ldx % 8 || ldy < nout || ldy % 4 ||
-        (reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(y) & 7))
-        return mortar_fail(MORTAR_ERR_ARG, "gemv: bad leading dimension or alignment");
+namespace {
+
+int gemv_run(const char *who, const mortar_bcsr_t *W, const int32_t *entries, int64_t n_entries, int32_t nslots,
+             const int32_t *row_slots, int32_t kseg, int32_t mode, const uint16_t *x, int32_t B, int64_t ldx,
+             uint16_t *y, int64_t ldy, float *part, const float *gates, int32_t n_clusters, int64_t ldg,
+             const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc, void *stream) {
     GemvParams p{};
+    const int64_t nout = mode == 0 ? (int64_t)W->Rb * 16 : (int64_t)W->Rb * 8;
     p.codes = W->codes; p.sdup = W->sdup; p.col = W->col; p.entries = entries; p.n_entries = (int)n_entries;
     p.nslots = nslots; p.kseg = kseg; p.mode = mode; p.Cb = W->Cb; p.N = W->Rb * 16;
     p.x = x; p.B = B; p.ldx = ldx; p.y = y; p.ldy = ldy; p.part = part;
     p.n_clusters = 1; p.cluster_size = 1 << 30;
     if (gates) {
         if (mode != 1 || n_clusters <= 0 || nout % n_clusters || (nout / n_clusters) % 4)
-            return mortar_fail(MORTAR_ERR_ARG, "gemv: gates need mode 1 and d_ff / n_clusters a whole multiple of 4");
+            return mortar_fail(MORTAR_ERR_ARG, "%s: gates need mode 1 and d_ff / n_clusters a whole multiple of 4", who);
         p.gates = gates; p.n_clusters = n_clusters; p.cluster_size = (int)(nout / n_clusters); p.ldg = ldg;
     }
     p.row_act = row_act; p.ldr = ldr; p.col_act = col_act; p.ldc = ldc;
@@ -228,4 +219,94 @@ extern "C" int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, 
         if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "combine launch: %s", hipGetErrorString(e));
     }
     return MORTAR_OK;
+}
+
+int gemv_check(const char *who, const mortar_bcsr_t *W, const int32_t *entries, int64_t n_entries, int32_t nslots,
+               const int32_t *row_slots, int32_t kseg, int32_t mode, const uint16_t *x, int32_t B, int64_t ldx,
+               const uint16_t *y, int64_t ldy) {
+    if (!W || !W->codes || !W->sdup || !W->col || !entries || !x || !y)
+        return mortar_fail(MORTAR_ERR_ARG, "%s: null pointer", who);
+    if (B <= 0 || B > 64) return mortar_fail(MORTAR_ERR_LIMIT, "%s: B=%d outside 1..64", who, B);
+    if (n_entries <= 0 || n_entries % 4 || n_entries > (int64_t)0x7fffffff) return mortar_fail(MORTAR_ERR_ARG, "%s: entry count must be a positive multiple of 4", who);
+    if (mode != 0 && mode != 1) return mortar_fail(MORTAR_ERR_ARG, "%s: mode must be 0 or 1", who);
+    if (mode == 1 && (W->Rb & 1)) return mortar_fail(MORTAR_ERR_ARG, "%s: gate_up needs an even number of block-rows", who);
+    if (nslots < 1 || (nslots > 1 && !row_slots)) return mortar_fail(MORTAR_ERR_ARG, "%s: nslots > 1 needs row_slots", who);
+    if (kseg <= 0) return mortar_fail(MORTAR_ERR_ARG, "%s: kseg must be positive", who);
+    const int64_t nout = mode == 0 ? (int64_t)W->Rb * 16 : (int64_t)W->Rb * 8;
+    if (ldx < (int64_t)W->Cb * 16 || ldx % 8 || ldy < nout || ldy % 4 ||
+        (reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(y) & 7))
+        return mortar_fail(MORTAR_ERR_ARG, "%s: bad leading dimension or alignment", who);
+    return MORTAR_OK;
+}
+
+}  // namespace
+
+extern "C" int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_entries,
+                                int32_t nslots, const int32_t *row_slots, int32_t kseg, int32_t mode,
+                                const uint16_t *x, int32_t B, int64_t ldx, uint16_t *y, int64_t ldy, float *part,
+                                const float *gates, int32_t n_clusters, int64_t ldg,
+                                const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc,
+                                void *stream) {
+    int rc = gemv_check("gemv", W, entries, n_entries, nslots, row_slots, kseg, mode, x, B, ldx, y, ldy);
+    if (rc) return rc;
+    if (nslots > 1 && !part) return mortar_fail(MORTAR_ERR_ARG, "gemv: nslots > 1 needs the partial workspace");
+    return gemv_run("gemv", W, entries, n_entries, nslots, row_slots, kseg, mode, x, B, ldx, y, ldy, part, gates,
+                    n_clusters, ldg, row_act, ldr, col_act, ldc, stream);
+}
+
+// ---- the same GEMV for callers that cannot allocate ------------------------------------------------------------
+// The partial sums of split rows go to this array inside the library instead of a caller workspace.  Every device
+// the library runs on holds its own copy at its own address; host code must use that address (looked up once per
+// device below), never the array's name, which in host code is only a stand-in for the symbol.
+namespace {
+
+constexpr int64_t NOALLOC_FLOATS = MORTAR_GEMV_NOALLOC_MAX_FLOATS;
+static __device__ __align__(256) float scratch[NOALLOC_FLOATS];
+
+constexpr int MAX_DEVICES = 64;
+float *scratch_addr[MAX_DEVICES];                 // per device, filled on the first call there
+std::mutex scratch_lock;
+
+int scratch_for_current_device(float **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "gemv_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= MAX_DEVICES) return mortar_fail(MORTAR_ERR_LIMIT, "gemv_noalloc: device ordinal %d not below %d", dev, MAX_DEVICES);
+    std::lock_guard<std::mutex> g(scratch_lock);
+    if (!scratch_addr[dev]) {
+        float *ptr = nullptr;
+        e = hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return mortar_fail(MORTAR_ERR_HIP, "gemv_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        scratch_addr[dev] = ptr;
+    }
+    *out = scratch_addr[dev];
+    return MORTAR_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t mortar_gemv_noalloc_max_floats(void) { return NOALLOC_FLOATS; }
+
+extern "C" int mortar_gemv_bf16_noalloc(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_entries,
+                                        int32_t nslots, const int32_t *row_slots, int32_t kseg, int32_t mode,
+                                        const uint16_t *x, int32_t B, int64_t ldx, uint16_t *y, int64_t ldy,
+                                        const float *gates, int32_t n_clusters, int64_t ldg,
+                                        const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc,
+                                        void *stream) {
+    int rc = gemv_check("gemv_noalloc", W, entries, n_entries, nslots, row_slots, kseg, mode, x, B, ldx, y, ldy);
+    if (rc) return rc;
+    float *part = nullptr;
+    if (nslots > 1) {
+        const int64_t need = (int64_t)nslots * B * W->Rb * 16;
+        if (need > NOALLOC_FLOATS)
+            return mortar_fail(MORTAR_ERR_LIMIT, "gemv_noalloc: nslots * B * out_features = %lld floats of partial sums exceed the "
+                               "built-in buffer of %lld (use mortar_gemv_bf16 with a workspace, fewer streams per call or a "
+                               "work list with fewer slots)", (long long)need, (long long)NOALLOC_FLOATS);
+        if ((rc = scratch_for_current_device(&part))) return rc;
+    }
+    // every slot the combine pass reads is written by the entries of this same call (skipped units write zeros), so
+    // nothing in the shared buffer has to be cleared first
+    return gemv_run("gemv_noalloc", W, entries, n_entries, nslots, row_slots, kseg, mode, x, B, ldx, y, ldy, part, gates,
+                    n_clusters, ldg, row_act, ldr, col_act, ldc, stream);
 }
