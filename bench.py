@@ -28,6 +28,8 @@ PEAK_BF16_TFLOPS, PEAK_HBM_GBS = 2500.0, 8000.0
 TRAFFIC_GATE_UP_BYTES = 41.58e6 + 50.54e6
 TRAFFIC_DOWN_BYTES = 60.34e6 + 16.78e6
 TRAFFIC_DECODE_STACK_BYTES = (262.95e6 + 4.56e6) + (162.10e6 + 1.81e6)   # gate_up + down launches, 160 layers, b = 1
+TRAFFIC_SOURCE = ("constant from profiles/bench_prefill_step_hbm_traffic_pmc.md and profiles/bench_all_legs_hbm_traffic_pmc.md "
+                  "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command); not measured in this run")
 
 
 def event_time_ms(fn, iters: int, warmup: int = 2) -> float:
@@ -45,9 +47,45 @@ def event_time_ms(fn, iters: int, warmup: int = 2) -> float:
     return a.elapsed_time(b) / iters
 
 
-def cpu_baseline(spec, sample_tokens: int) -> dict:
-    """The C restatement of the path (oracle, 'port') on the host cores over a bounded token sample."""
+def _dense_twin(spec, tokens: int, dtype, budget_s: float) -> dict:
+    """The reference's CPU-expressible form of the carved MLP (scatter the kept blocks into dense matrices, as
+    morph/sparse/stk/ops/matrix_ops.py:37-49 / morph/inference/engine.py:74-84 do, then torch.nn.functional.linear and
+    silu * up) timed through PyTorch on the host cores."""
     import numpy as np
+    import torch
+    import torch.nn.functional as F
+    from oracle import mortar_oracle as O
+    from mortar_amd import synth
+    d_model, d_ff = spec["d_model"], spec["d_ff"]
+    mats = []
+    for k in ("gate_up", "down"):
+        m = spec[k]
+        mats.append(torch.from_numpy(O.to_dense(O.effective_blocks(m["codes"], m["scales"]), m["row_idx"], m["col_idx"], m["shape"])).to(dtype))
+    x = torch.from_numpy(synth.synth_x(tokens, d_model, seed=999)).to(dtype)
+
+    def run():
+        gu = F.linear(x, mats[0])
+        return F.linear(F.silu(gu[:, :d_ff]) * gu[:, d_ff:], mats[1])
+    with torch.no_grad():
+        run()
+        t0 = time.perf_counter(); run(); t1 = time.perf_counter() - t0
+        reps = max(1, min(200, int(budget_s / max(t1, 1e-4))))
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            run()
+        dt = time.perf_counter() - t0
+    return {"value": reps * tokens / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{reps} passes over {tokens} tokens, d{d_model}/ff{d_ff}, dense-scatter weights + F.linear + silu*up in "
+                      f"{str(dtype).replace('torch.', '')} through PyTorch, {dt:.1f} s"}
+
+
+def cpu_baseline(spec, sample_tokens: int) -> dict:
+    """Host-core baselines on a bounded sample (reported only): the C restatement of the blockwise path (oracle,
+    'port'), and the reference's CPU-expressible twin - dense-scatter weights + torch.nn.functional.linear in fp32 and
+    bf16 - on the headline shape and on benchmark config 0's single 768 -> 2048 product."""
+    import numpy as np
+    import torch
+    import torch.nn.functional as F
     from oracle import c_oracle, mortar_oracle as O
     from mortar_amd import synth
     x = O.bf16_bits(synth.synth_x(sample_tokens, D_MODEL, seed=999))
@@ -55,14 +93,38 @@ def cpu_baseline(spec, sample_tokens: int) -> dict:
     t0 = time.perf_counter()
     c_oracle.mlp_bf16(x, spec["gate_up"], spec["down"], D_FF)
     t1 = time.perf_counter() - t0
-    reps = max(1, min(800, int(round(18.0 / max(t1, 1e-3)))))                # 10-20 s of CPU work in total
+    reps = max(1, min(800, int(round(10.0 / max(t1, 1e-3)))))                # about 10 s of CPU work
     t0 = time.perf_counter()
     for _ in range(reps):
         c_oracle.mlp_bf16(x, spec["gate_up"], spec["down"], D_FF)
     dt = time.perf_counter() - t0
-    return {"value": reps * sample_tokens / dt, "unit": "tokens/s", "cores": c_oracle.num_threads(), "kind": "port",
-            "sample": f"{reps} passes over {sample_tokens} tokens of the same d{D_MODEL}/ff{D_FF} MLP, blockwise C "
-                      f"BCSR restatement (OpenMP), {dt:.1f} s"}
+    res = {"value": reps * sample_tokens / dt, "unit": "tokens/s", "cores": c_oracle.num_threads(), "kind": "port",
+           "sample": f"{reps} passes over {sample_tokens} tokens of the same d{D_MODEL}/ff{D_FF} MLP, blockwise C "
+                     f"BCSR restatement (OpenMP), {dt:.1f} s"}
+    twin_tokens = min(sample_tokens, 1024)
+    res["dense_twin_fp32"] = _dense_twin(spec, twin_tokens, torch.float32, 5.0)
+    res["dense_twin_bf16"] = _dense_twin(spec, twin_tokens, torch.bfloat16, 5.0)
+    # benchmark config 0: one 768 -> 2048 product on 64 tokens, the reference's own CPU-runnable case
+    m0 = synth.synth_matrix(2048, 768, DENSITY, seed=100)
+    W0 = torch.from_numpy(O.to_dense(O.effective_blocks(m0["codes"], m0["scales"]), m0["row_idx"], m0["col_idx"], m0["shape"]))
+    x0 = torch.from_numpy(synth.synth_x(64, 768, seed=101))
+    c0 = {}
+    for name, dt_ in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        Wd, xd = W0.to(dt_), x0.to(dt_)
+        with torch.no_grad():
+            F.linear(xd, Wd)
+            n = 2000
+            t0 = time.perf_counter()
+            for _ in range(n):
+                F.linear(xd, Wd)
+            c0[name] = {"us_per_call": (time.perf_counter() - t0) / n * 1e6}
+    xb0 = O.bf16_bits(synth.synth_x(64, 768, seed=101))
+    t0 = time.perf_counter()
+    for _ in range(200):
+        c_oracle.bcsr_spmm_bf16(xb0, m0["codes"], m0["scales"], m0["col_idx"], m0["offsets"])
+    c0["blockwise_c_port"] = {"us_per_call": (time.perf_counter() - t0) / 200 * 1e6}
+    res["config0_single_spmm_64x768x2048"] = {"dense_linear": c0, "cores": torch.get_num_threads()}
+    return res
 
 
 def main() -> None:
@@ -120,10 +182,12 @@ def main() -> None:
         "roofline": {"bound": "mfma", "kernel": "mortar_resident_kernel<32 tokens, gate_up + SwiGLU>",
                      "achieved": flops_gu / (ms_gu * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops_gu / (ms_gu * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_GATE_UP_BYTES,
+                     "traffic_source": TRAFFIC_SOURCE,
                      "algorithmic_bytes": TOKENS * (D_MODEL + D_FF) * 2 + Wgu.weight_bytes, "ms": ms_gu},
         "roofline_down": {"bound": "mfma", "kernel": "mortar_segmented_kernel<32 tokens, plain> (down)",
                           "achieved": flops_dn / (ms_dn * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                           "frac": flops_dn / (ms_dn * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_DOWN_BYTES,
+                          "traffic_source": TRAFFIC_SOURCE,
                           "algorithmic_bytes": TOKENS * (D_MODEL + D_FF) * 2 + Wdn.weight_bytes, "ms": ms_dn},
     }
 
@@ -240,6 +304,8 @@ def main() -> None:
         out["roofline_decode"] = {"bound": "hbm", "kernel": "mortar_resident_kernel<4 tokens>, gate_up + down launches of 160 layers each, b=1",
                                   "achieved": stack["b1"]["algorithmic_GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                   "frac": stack["b1"]["frac_hbm"], "traffic": TRAFFIC_DECODE_STACK_BYTES,
+                                  "traffic_source": TRAFFIC_SOURCE,
+                                  "by_batch": {k: {"achieved": v["algorithmic_GBps"], "frac": v["frac_hbm"]} for k, v in stack.items()},
                                   "algorithmic_bytes": n_sets * (wbytes + (2 * D_MODEL + 2 * D_FF) * 2)}
         # ---- ReMoE-routed prefill (benchmark config 3) ----------------------------------------------------
         logits = torch.from_numpy(synth.synth_logits(TOKENS, N_CLUSTERS, seed=2)).to(dev)
@@ -297,24 +363,18 @@ def main() -> None:
         del x1, h1, y1
         # ---- benchmark config 4: 8 shared blocks x 6 iterations, Zipf(1.2) rows, RMS-normalised input ----------
         specs = [synth.synth_mlp(D_MODEL, D_FF, DENSITY, seed=20 + i, zipf_s=1.2) for i in range(8)]
-        packs4 = [(synth.to_pack(sp["gate_up"], dev), synth.to_pack(sp["down"], dev)) for sp in specs]
-        xs = [x, torch.empty_like(x)]
-
-        def looped():
-            cur = 0
-            for _ in range(6):
-                for g4, d4 in packs4:
-                    xn = ops.rmsnorm(xs[cur])
-                    ops.gateup_swiglu(xn, g4, out=h)
-                    ops.spmm(h, d4, out=xs[1 - cur] if cur == 0 else xs[1])
-                    cur = 1
-        t = event_time_ms(looped, 3, 1)
-        fl = 6 * sum(2.0 * TOKENS * 256 * (g4.nnz + d4.nnz) for g4, d4 in packs4)
+        mlps4 = [synth.mlp_module(sp, dev) for sp in specs]
+        fused_norm = all(ops.norm_fusable(m4.gate_up._cms.mortar_pack()) for m4 in mlps4)
+        t = event_time_ms(lambda: mortar_amd.looped_core_forward(mlps4, x, 6), 3, 1)
+        fl = 6 * sum(2.0 * TOKENS * 256 * (m4.gate_up._cms.mortar_pack().nnz + m4.down._cms.mortar_pack().nnz) for m4 in mlps4)
         out["looped_stack"] = {"ms": t, "mlp_calls": 48, "ms_per_mlp": t / 48, "tokens_per_s": TOKENS / (t * 1e-3),
                                "effective_tflops": fl / (t * 1e-3) / 1e12,
                                "frac_mfma": fl / (t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-                               "note": "RMSNorm before every MLP, applied while gate_up stages x (no separate launch); rows follow Zipf(1.2) clipped to 5-60 %"}
-        del specs, packs4
+                               "norm_fused_into_gate_up": bool(fused_norm),
+                               "note": "looped_core_forward over 8 carved MLP modules x 6 iterations: RMSNorm before every MLP, "
+                                       "applied while gate_up stages x when norm_fused_into_gate_up (no separate launch); two "
+                                       "launches per MLP; rows follow Zipf(1.2) clipped to 5-60 %"}
+        del specs, mlps4
 
     if not args.no_extras:
         # ---- training side (values-ternary QAT): device re-pack of W and W^T, dX through the W^T pack, dW on the

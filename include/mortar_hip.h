@@ -8,7 +8,10 @@
  *
  * Reference interfaces replaced (paths relative to the reference checkout):
  *   stk_dds(lhs, data, offsets, row_indices, column_indices, ..., shape0, shape1, True)
- *       morph/sparse/stk/backend/custom_ops.py:35-56 (forward use block_sparse.py:956-965)
+ *       morph/sparse/stk/backend/custom_ops.py:35-56 (forward use block_sparse.py:956-965).  Restriction: the
+ *       reference multiplies whatever bf16 values `data` holds; this runtime multiplies TERNARY blocks only
+ *       (every value of block j is 0 or +-s_j).  Other data is reported as an error (mortar_requantize,
+ *       ternary_tol), never multiplied approximately.
  *   _SwiGLUMortar.forward                      morph/model/transformer.py:402-431
  *   TileRouter.forward steps 5-8               morph/model/routing.py:232-284
  *   route_flags                                morph/kernels/triton/fused_decode_step.py:1913-1927
@@ -228,13 +231,13 @@ int mortar_router_bf16(const void *x, int32_t x_is_f32, int64_t B, int32_t d, in
 
 /* mortar_spmm_bf16 / mortar_gateup_swiglu_bf16 / mortar_spmm_bf16_masked serve decode batches directly: for
  * M <= 64 they run small-tile variants (4- or 16-token tiles, small workgroups) that read every weight block
- * from HBM once per launch.  That path replaces mortar_gemv of fused_decode_step.py:1701-1842 for the MLP pair.
+ * from HBM once per launch.  That path replaces mortar_gemv (fused_decode_step.py:1502-1547, kernels :1341-1459)
+ * for the MLP pair as the engine calls it (morph/inference/engine.py:980-986).
  *
  * Layer-batched form for M <= 16: ONE launch runs the same operation on n_layers independent
- * (matrix, input, output) triples of identical shape (Rb, Cb, seg_cb).  No counterpart in the reference,
- * whose decode megakernel walks its layers inside one persistent program (fused_decode_step.py:2104-2300);
- * this is the launch-level equivalent for callers that hold many weight sets (a stack of layers whose
- * inputs are known, several models, bandwidth measurement).
+ * (matrix, input, output) triples of identical shape (Rb, Cb, seg_cb).  No counterpart in the reference, which
+ * issues one mortar_gemv per matrix (morph/inference/engine.py:980-986); this is for callers that hold many weight
+ * sets whose inputs are known (several models, a stack probed for bandwidth).
  *   mortar_stack_table_bytes  bytes of device memory the parameter table needs
  *   mortar_stack_prepare      validates the layers, writes the table (synchronous host-to-device copy);
  *                             W: host array [n_layers] of descriptors with device pointers, x / y: host arrays

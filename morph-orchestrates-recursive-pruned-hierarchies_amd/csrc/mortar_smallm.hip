@@ -1,7 +1,7 @@
 // Small-M (decode, M <= 64) instantiations of the octet-stream SpMM kernels.
 //
 // Replaces the reference's decode GEMV over packed ternary strips (morph/kernels/triton/fused_decode_step.py:
-// 1701-1842, mortar_gemv) for batches of up to 64 rows: the batch is one token tile of 4 or 16 tokens (up to four
+// 1502-1547 mortar_gemv, kernels 1341-1459) for batches of up to 64 rows: the batch is one token tile of 4 or 16 tokens (up to four
 // 16-token tiles above 16 rows), so a weight block is read from HBM once per launch and the kernel is bound by
 // the weight stream.  Workgroups are small
 // (2 wavefronts) when one matrix has to cover the chip and 8 or 16 wavefronts when many layers share a launch.
