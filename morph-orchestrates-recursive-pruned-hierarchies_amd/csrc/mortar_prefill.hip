@@ -98,7 +98,7 @@ int dispatch(int kind, SpmmParams &p, const mortar_bcsr_t *W, hipStream_t st) {
 
 }  // namespace
 
-extern "C" int mortar_prefill_max_seg_cb(void) { return (LDS_BUDGET / 16 - LDS_PAD) / (2 * 33); }
+extern "C" int mortar_prefill_max_seg_cb(void) { return (LDS_BUDGET - LDS_PAD * 16) / (32 * 32); }
 
 extern "C" int mortar_route_tile(int32_t Cb, int64_t M) {
     if (M > 0 && M <= MORTAR_SMALLM_MAX) {

@@ -91,11 +91,14 @@ constexpr int CODE_2BIT = 0, CODE_4BIT = 1, CODE_UNIFORM = 2;
 constexpr int MORTAR_SMALLM_MAX = 64;    // rows up to which the small-tile (decode) instantiations are used
 constexpr int RES_GROUPS = 4;            // octets (4 block pairs each) loaded per batch
 constexpr int LDS_BUDGET = 156 * 1024;   // bytes of LDS a token tile may take
-constexpr int LDS_PAD = 16;              // 16-byte units past the tile that idle lanes of a narrow tile may read
+constexpr int LDS_PAD = 32;              // 16-byte units past the tile that idle lanes of a narrow tile may read
 
-// LDS bytes of a token tile of MT tokens and ncb block-columns (token stride MT + 1 keeps reads conflict-free).
-constexpr int tile_bytes(int mt, int ncb) { return (2 * ncb * (mt + 1) + LDS_PAD) * 16; }
-constexpr int LDS_EXTRA = 16;            // bytes after the tile: the resident kernel's unit counter
+// Tile layout in LDS: [block-column][token][column half] in 16-byte units, i.e. the 32 bytes (16 values) of one token
+// and block-column are adjacent and a block-column is a run of MT * 32 bytes.  The 32 lanes that fetch one block's MFMA
+// operand (16 tokens x 2 column halves) then read 512 contiguous bytes, which ds_read_b128 serves at full rate
+// (measured: 4.4 cycles per wave instruction, against 8.1 for any layout whose 16-lane windows are not aligned).
+constexpr int tile_bytes(int mt, int ncb) { return ncb * mt * 32 + LDS_PAD * 16; }
+constexpr int LDS_EXTRA = 16 + 256;      // bytes after the tile: the resident kernel's unit counter, per-row norm factors
 constexpr int NORM_MAX_CB = 128;         // block-columns up to which a row fits the registers of the staging wave
 
 // Lane k of every 16-lane row broadcast to the whole row (DPP row_newbcast); K must fold to a constant.
@@ -144,16 +147,16 @@ __device__ __forceinline__ void mortar_load_batch(const SpmmView &p, MortarBatch
 }
 
 // One row part: octets [g0, g1) (nb blocks) of the stream against the tile at `lx`.
-// `xo_base` is the lane's unit offset inside a block-column (column half, token) plus the segment's origin.
+// `xo_base` is the lane's byte offset inside a block-column (token, column half) plus the segment's origin.
 // `b` holds the part's first batch, loaded by the caller (mortar_load_batch at g0) where it suits it.
-template <int MSUB, int LDM, bool ROUTED, int CODE = 0>
+template <int MSUB, int MT, bool ROUTED, int CODE = 0>
 __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *lx, MortarBatch b, int g0, int g1,
                                                 int nb, uint32_t xo_base, const uint32_t (&tk)[MSUB], int nsub, int n,
                                                 int bsel, int hsel, f32x4_t (&acc)[MSUB]) {
     const unsigned char *lb = reinterpret_cast<const unsigned char *>(lx);
     for (int gq = g0; gq < g1; gq += RES_GROUPS) {
         if (gq != g0) mortar_load_batch<CODE>(p, b, gq, g1, n, bsel, hsel);
-        const uint32_t ccs = __umul24(b.ccv, (uint32_t)(2 * LDM * 16));   // byte offset of the block-column in the tile
+        const uint32_t ccs = __umul24(b.ccv, (uint32_t)(MT * 32));   // byte offset of the block-column in the tile
         const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;      // block pairs left in the row from this batch on
         // Activation operands are fetched two pairs ahead of the MFMAs that use them.  The only branches are
         // per octet (a whole octet past the end of the part is skipped) and, for prefill tiles, per half octet;
@@ -162,9 +165,9 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
         uint4 Bq[3][MSUB];
 #pragma unroll
         for (int d = 0; d < 2; ++d) {
-            const uint32_t xo = mortar_row_bcast(ccs, d) + xo_base * 16u;
+            const uint32_t xo = mortar_row_bcast(ccs, d) + xo_base;
 #pragma unroll
-            for (int ms = 0; ms < MSUB; ++ms) Bq[d][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 16u : ms * 256u));
+            for (int ms = 0; ms < MSUB; ++ms) Bq[d][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 32u : ms * 512u));
         }
 #pragma unroll
         for (int k = 0; k < RES_GROUPS; ++k) {
@@ -176,10 +179,10 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
                     const uint32_t nib = (CODE & CODE_4BIT) ? b.cw[k][t] : ((b.cw[k][t] << (2 * hsel)) & 0xCCCCCCCCu);
                     const u32x4_t A = (CODE & CODE_UNIFORM) ? mortar_nib4(nib) : mortar_scale4(nib, mortar_row_bcast(b.sdv, u));
                     if (u + 2 < NP) {
-                        const uint32_t xo = mortar_row_bcast(ccs, u + 2) + xo_base * 16u;
+                        const uint32_t xo = mortar_row_bcast(ccs, u + 2) + xo_base;
 #pragma unroll
                         for (int ms = 0; ms < MSUB; ++ms)
-                            Bq[(u + 2) % 3][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 16u : ms * 256u));
+                            Bq[(u + 2) % 3][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 32u : ms * 512u));
                     }
 #pragma unroll
                     for (int ms = 0; ms < MSUB; ++ms) {
@@ -195,97 +198,91 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
     }
 }
 
-// Stages x[m0 .. m0+MT, 16*c0 .. 16*(c0+ncb)] into the tile: unit (ch, row) <- 8 values of column half ch.
-// A wavefront takes whole rows (row = wave, wave + WAVES, ...), its lanes consecutive 16-byte units of the row,
-// so that addresses need no division: uniform row base + lane offset.  Rows past M are not staged: their LDS
-// units keep whatever they held and only feed accumulator columns that are never stored.
-// With MASKED, units of (token, input cluster) pairs that are off are zeroed.
-template <int MT, int WAVES, bool MASKED>
-__device__ __forceinline__ void mortar_stage_tile(const SpmmView &p, uint4 *lx, int m0, int c0, int ncb, int tid) {
-    // rows x 64-unit chunks in flight per lane: a small workgroup keeps up to 32 loads per lane in flight
-    constexpr int LDM = MT + 1, CU = 4, RU = MT / WAVES >= 8 ? 8 : (MT / WAVES >= 4 ? 4 : 2);
-    const int nch = 2 * ncb;
+// Stages x[m0 .. m0+MT, 16*c0 .. 16*(c0+ncb)] into the tile.  One wave instruction moves 16 rows x 64 bytes: the four
+// lanes of a quad read 64 contiguous bytes of one row (two block-columns), so global reads stay coalesced in 64-byte
+// pieces while the 16 lanes that the LDS serves together write 16 different bank groups (4 tokens x 4 units).
+// Rows past M are not staged: their LDS units keep whatever they held and only feed accumulator columns that are
+// never stored.  With MASKED, units of (token, input cluster) pairs that are off are zeroed.
+// NORM: the rows are scaled by their factor in `rs` (LDS, one float per tile row) and the weight, as rms_apply8 does.
+template <int MT, int WAVES, bool MASKED, bool NORM>
+__device__ __forceinline__ void mortar_stage_quads(const SpmmView &p, unsigned char *lb, int m0, int c0, int ncb, int tid,
+                                                   const float *rs) {
+    constexpr int RG = (MT + 15) / 16;                   // groups of 16 rows
+    constexpr int KC = RG >= 4 ? 2 : (RG == 2 ? 4 : 8);  // chunks in flight per wave: 8 loads per lane
+    const int nch = 2 * ncb;                             // 16-byte units per row
+    const int nck = (nch + 3) >> 2;                      // 64-byte chunks per row
     const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int rsub = lane >> 2, li = lane & 3;
     const MORTAR_GLOBAL char *xt = p.x + (int64_t)m0 * p.ldx * 2 + (int64_t)c0 * 32;
-    for (int r0 = wave; r0 <= rlast; r0 += WAVES * RU) {
-        for (int ch0 = 0; ch0 < nch; ch0 += 64 * CU) {
-            u32x4_t v[RU][CU];
+    const bool has_w = NORM && p.norm_w != nullptr;
+    for (int ck0 = wave; ck0 < nck; ck0 += WAVES * KC) {
+        u32x4_t v[KC][RG], wv[KC];
 #pragma unroll
-            for (int a = 0; a < RU; ++a) {
-                int row = r0 + a * WAVES;
+        for (int k = 0; k < KC; ++k) {
+            int u = (ck0 + k * WAVES) * 4 + li;
+            u = u < nch ? u : nch - 1;
+            if (NORM) wv[k] = has_w ? p.norm_w[c0 * 2 + u] : u32x4_t{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int rg = 0; rg < RG; ++rg) {
+                int row = rg * 16 + rsub;
                 row = row < rlast ? row : rlast;
-                const MORTAR_GLOBAL char *xr = xt + (int64_t)row * p.ldx * 2;
-#pragma unroll
-                for (int b = 0; b < CU; ++b) {
-                    int ch = ch0 + b * 64 + lane;
-                    ch = ch < nch ? ch : nch - 1;
-                    v[a][b] = *(const MORTAR_GLOBAL u32x4_t *)(xr + (uint32_t)ch * 16u);
-                    if (MASKED && p.active[(int64_t)(m0 + row) * p.n_clusters + (c0 * 16 + ch * 8) / p.cluster_size] == 0)
-                        v[a][b] = u32x4_t{0u, 0u, 0u, 0u};
-                }
+                v[k][rg] = *(const MORTAR_GLOBAL u32x4_t *)(xt + (int64_t)row * p.ldx * 2 + (uint32_t)u * 16u);
+                if (MASKED && p.active[(int64_t)(m0 + row) * p.n_clusters + (c0 * 16 + u * 8) / p.cluster_size] == 0)
+                    v[k][rg] = u32x4_t{0u, 0u, 0u, 0u};
             }
+        }
 #pragma unroll
-            for (int a = 0; a < RU; ++a) {
-                const int row = r0 + a * WAVES;
+        for (int k = 0; k < KC; ++k) {
+            const int u = (ck0 + k * WAVES) * 4 + li;
 #pragma unroll
-                for (int b = 0; b < CU; ++b) {
-                    const int ch = ch0 + b * 64 + lane;
-                    if (row <= rlast && ch < nch) reinterpret_cast<u32x4_t *>(lx)[ch * LDM + row] = v[a][b];
+            for (int rg = 0; rg < RG; ++rg) {
+                const int row = rg * 16 + rsub;
+                if (row <= rlast && u < nch) {
+                    u32x4_t o = v[k][rg];
+                    if (NORM) o = rms_apply8(o, rs[row], wv[k], has_w);
+                    *reinterpret_cast<u32x4_t *>(lb + (uint32_t)(u >> 1) * (uint32_t)(MT * 32) + row * 32 + (u & 1) * 16) = o;
                 }
             }
         }
     }
 }
 
-// The same staging with the rows RMS-normalised on the way (gate_up with the block's norm folded in): a wave holds
-// a whole row in registers (at most 256 units: the host admits the fused norm for ncb <= NORM_MAX_CB only), two
-// rows at a time, adds the squares, and writes bf16(bf16(x * r) * w).
+template <int MT, int WAVES, bool MASKED>
+__device__ __forceinline__ void mortar_stage_tile(const SpmmView &p, uint4 *lx, int m0, int c0, int ncb, int tid) {
+    mortar_stage_quads<MT, WAVES, MASKED, false>(p, reinterpret_cast<unsigned char *>(lx), m0, c0, ncb, tid, nullptr);
+}
+
+// The same staging with the rows RMS-normalised on the way (gate_up with the block's norm folded in).  First every
+// wave adds the squares of whole rows (lanes = consecutive 16-byte units, ascending, then the xor butterfly: the order
+// of the stand-alone RMSNorm kernel, so both give the same bits) and leaves the row factors in LDS at `rs`; after a
+// barrier the tile is staged as above with bf16(bf16(x * r) * w) applied (the second read of x hits the cache).
+// The host admits the fused norm for ncb <= NORM_MAX_CB only (a row is at most 256 units = 4 per lane).
 template <int MT, int WAVES>
-__device__ __forceinline__ void mortar_stage_tile_norm(const SpmmView &p, uint4 *lx, int m0, int ncb, int tid) {
-    constexpr int LDM = MT + 1, CU = 4, RU = 2;
+__device__ __forceinline__ void mortar_stage_tile_norm(const SpmmView &p, uint4 *lx, int m0, int ncb, int tid, float *rs) {
+    constexpr int CU = 4;
     const int nch = 2 * ncb;
     const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const MORTAR_GLOBAL char *xt = p.x + (int64_t)m0 * p.ldx * 2;
-    const bool has_w = p.norm_w != nullptr;
-    u32x4_t wv[CU];
+    for (int row = wave; row <= rlast; row += WAVES) {
+        const MORTAR_GLOBAL char *xr = xt + (int64_t)row * p.ldx * 2;
+        u32x4_t v[CU];
 #pragma unroll
-    for (int b = 0; b < CU; ++b) {
-        int ch = b * 64 + lane;
-        ch = ch < nch ? ch : nch - 1;
-        wv[b] = has_w ? p.norm_w[ch] : u32x4_t{0u, 0u, 0u, 0u};
-    }
-    for (int r0 = wave; r0 <= rlast; r0 += WAVES * RU) {
-        u32x4_t v[RU][CU];
-#pragma unroll
-        for (int a = 0; a < RU; ++a) {
-            int row = r0 + a * WAVES;
-            row = row < rlast ? row : rlast;
-            const MORTAR_GLOBAL char *xr = xt + (int64_t)row * p.ldx * 2;
-#pragma unroll
-            for (int b = 0; b < CU; ++b) {
-                int ch = b * 64 + lane;
-                ch = ch < nch ? ch : nch - 1;
-                v[a][b] = *(const MORTAR_GLOBAL u32x4_t *)(xr + (uint32_t)ch * 16u);
-            }
+        for (int b = 0; b < CU; ++b) {
+            int ch = b * 64 + lane;
+            ch = ch < nch ? ch : nch - 1;
+            v[b] = *(const MORTAR_GLOBAL u32x4_t *)(xr + (uint32_t)ch * 16u);
         }
+        float ss = 0.f;
 #pragma unroll
-        for (int a = 0; a < RU; ++a) {
-            const int row = r0 + a * WAVES;
-            float ss = 0.f;
-#pragma unroll
-            for (int b = 0; b < CU; ++b)
-                if (b * 64 + lane < nch) ss = rms_sumsq8(v[a][b], ss);
-            const float r = rms_scale(rms_wave_sum(ss), 8 * nch, p.norm_eps);
-#pragma unroll
-            for (int b = 0; b < CU; ++b) {
-                const int ch = b * 64 + lane;
-                if (row <= rlast && ch < nch)
-                    reinterpret_cast<u32x4_t *>(lx)[ch * LDM + row] = rms_apply8(v[a][b], r, wv[b], has_w);
-            }
-        }
+        for (int b = 0; b < CU; ++b)
+            if (b * 64 + lane < nch) ss = rms_sumsq8(v[b], ss);
+        const float r = rms_scale(rms_wave_sum(ss), 8 * nch, p.norm_eps);
+        if (lane == 0) rs[row] = r;
     }
+    __syncthreads();
+    mortar_stage_quads<MT, WAVES, false, true>(p, reinterpret_cast<unsigned char *>(lx), m0, 0, ncb, tid, rs);
 }
 
 // Epilogue of one row unit for the 16 tokens of sub-tile `ms`: the lane holds D[4g+v][token].
@@ -330,7 +327,7 @@ __device__ __forceinline__ u32x4_t mortar_part_desc(const SpmmView &p, int pos, 
 // ---------------------------------------------------------------------------------------------------------
 template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE, int CODE>
 __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmParams p0, const SpmmParams *table) {
-    constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1;
+    constexpr int MSUB = (MT + 15) / 16;
     const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint4 *lx = reinterpret_cast<uint4 *>(smem);
@@ -343,7 +340,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
     if (wg >= p.n_mtiles * p.n_split) return;
     const int mt = wg / p.n_split, sp = wg % p.n_split;
     const int m0 = mt * MT;
-    const uint32_t lane_xo = (uint32_t)(hsel * LDM + (ROUTED ? 0 : n));
+    const uint32_t lane_xo = (uint32_t)(hsel * 16 + (ROUTED ? 0 : n * 32));
     const bool has_gates = p.gates != nullptr;
 
     const int per = (p.n_units + p.n_split - 1) / p.n_split;
@@ -359,7 +356,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
     int pos = base + wave;
     u32x4_t d0 = mortar_part_desc<NACC>(p, pos, 0, 0);
 
-    if (NACC == 2 && p.norm) mortar_stage_tile_norm<MT, WAVES>(p, lx, m0, p.Cb, tid);      // gate_up may carry the norm
+    if (NACC == 2 && p.norm) mortar_stage_tile_norm<MT, WAVES>(p, lx, m0, p.Cb, tid, reinterpret_cast<float *>(next_unit + 4));      // gate_up may carry the norm
     else mortar_stage_tile<MT, WAVES, false>(p, lx, m0, 0, p.Cb, tid);
     __syncthreads();
 
@@ -397,7 +394,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
             for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
         for (int sg = 0; sg < p.nseg; ++sg) {
-            const uint32_t xo_base = lane_xo + (uint32_t)(sg * p.seg_cb) * (2 * LDM);
+            const uint32_t xo_base = lane_xo + (uint32_t)(sg * p.seg_cb) * (uint32_t)(MT * 32);
 #pragma unroll
             for (int a = 0; a < NACC; ++a) {
                 const bool last_part = sg + 1 == p.nseg && a + 1 == NACC;
@@ -409,7 +406,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
                 if (!skip && g0 < g1) {
                     MortarBatch b;
                     mortar_load_batch<CODE>(p, b, g0, g1, n, bsel, hsel);
-                    mortar_row_part<MSUB, LDM, ROUTED, CODE>(p, lx, b, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+                    mortar_row_part<MSUB, MT, ROUTED, CODE>(p, lx, b, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
                 }
                 d0 = d1;
             }
@@ -437,7 +434,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
 // ---------------------------------------------------------------------------------------------------------
 template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE, int CODE>
 __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const SpmmParams p0, const SpmmParams *table) {
-    constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1, NP = UPW * NACC;
+    constexpr int MSUB = (MT + 15) / 16, NP = UPW * NACC;
     const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint4 *lx = reinterpret_cast<uint4 *>(smem);
@@ -450,7 +447,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
     if (wg >= p.n_mtiles * p.n_split) return;
     const int mt = wg / p.n_split, sp = wg % p.n_split;
     const int m0 = mt * MT;
-    const uint32_t lane_xo = (uint32_t)(hsel * LDM + n);
+    const uint32_t lane_xo = (uint32_t)(hsel * 16 + n * 32);
     const bool has_gates = p.gates != nullptr;
 
     // this wave's units: schedule positions sp*per + wave + WAVES*k
@@ -496,7 +493,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
             if (g0[q] < g1[q]) {
                 MortarBatch b;
                 mortar_load_batch<CODE>(p, b, g0[q], g1[q], n, bsel, hsel);
-                mortar_row_part<MSUB, LDM, false, CODE>(p, lx, b, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
+                mortar_row_part<MSUB, MT, false, CODE>(p, lx, b, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
                                                   acc[q / NACC][q % NACC]);
             }
         }
@@ -525,7 +522,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
 // ---------------------------------------------------------------------------------------------------------
 template <int MT, int NACC, bool ROUTED, bool MASKED, int PW, int UW, int CODE>
 __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const SpmmParams p0) {
-    constexpr int MSUB = (MT + 15) / 16, LDM = MT + 1, WAVES = PW * UW;
+    constexpr int MSUB = (MT + 15) / 16, WAVES = PW * UW;
     const SpmmView p = mortar_view(p0);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint4 *lx = reinterpret_cast<uint4 *>(smem);
@@ -535,7 +532,7 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
     const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
     const int mt = blockIdx.x / p.n_split, sp = blockIdx.x % p.n_split;
     const int m0 = mt * MT;
-    const uint32_t lane_xo = (uint32_t)(hsel * LDM + (ROUTED ? 0 : n));
+    const uint32_t lane_xo = (uint32_t)(hsel * 16 + (ROUTED ? 0 : n * 32));
     const bool has_gates = p.gates != nullptr;
     const int ug = wave / PW, wq = wave % PW;            // unit slot in the workgroup, this wave's share of its parts
     const int pos = sp * UW + ug;
@@ -570,7 +567,7 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
     }
     const int nsub = ROUTED ? (cnt + 15) >> 4 : MSUB;
 
-    if (NACC == 2 && !MASKED && p.norm) mortar_stage_tile_norm<MT, WAVES>(p, lx, m0, p.Cb, tid);
+    if (NACC == 2 && !MASKED && p.norm) mortar_stage_tile_norm<MT, WAVES>(p, lx, m0, p.Cb, tid, reinterpret_cast<float *>(red));
     else mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, 0, p.Cb, tid);
     __syncthreads();
 
@@ -581,7 +578,7 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
         for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     if (!skip) {
         for (int sg = 0; sg < p.nseg; ++sg) {
-            const uint32_t xo_base = lane_xo + (uint32_t)(sg * p.seg_cb) * (2 * LDM);
+            const uint32_t xo_base = lane_xo + (uint32_t)(sg * p.seg_cb) * (uint32_t)(MT * 32);
 #pragma unroll
             for (int a = 0; a < NACC; ++a) {
                 const int q = sg * NACC + a;
@@ -592,7 +589,7 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
                 const int nb = __builtin_amdgcn_readfirstlane((int)dq[2]);
                 if (g0 >= g1) continue;
                 if (!is_first) mortar_load_batch<CODE>(p, first, g0, g1, n, bsel, hsel);
-                mortar_row_part<MSUB, LDM, ROUTED, CODE>(p, lx, first, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
+                mortar_row_part<MSUB, MT, ROUTED, CODE>(p, lx, first, g0, g1, nb, xo_base, tk, nsub, n, bsel, hsel, acc[a]);
             }
         }
     }

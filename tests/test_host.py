@@ -184,7 +184,7 @@ def test_unit_order_and_schedule():
 
 def test_tile_queries():
     L = _lib.lib()
-    assert L.mortar_prefill_max_seg_cb() == 151
+    assert L.mortar_prefill_max_seg_cb() == 155
     assert L.mortar_route_tile(128, 4096) == 32 and L.mortar_route_tile(48, 4096) == 64
     assert L.mortar_route_tile(128, 1) == 4 and L.mortar_route_tile(128, 16) == 16
     assert L.mortar_route_tile(352, 4096) == 0                                      # too wide for routed skipping
