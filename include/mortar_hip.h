@@ -184,6 +184,21 @@ int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *sched, const 
                             int64_t ldx, uint16_t *y, int64_t ldy, const uint8_t *active, int32_t n_clusters,
                             void *stream);
 
+/* `down` with the hyper-connection POST write fused into its epilogue, for decode batches (M <= 64): the MLP output
+ * y = x W^T never goes to memory.  Reference: engine._hc calls the MLP and then _hc_post_fwd_kernel
+ * (morph/inference/engine.py:996-1001, 1052-1060; morph/kernels/triton/fused_hyper_connection.py:927-970; wide carriers
+ * hc_post_wide, morph/kernels/triton/fused_decode_step.py:1725-1739):
+ *   out[t, i, :] = sum_j hres[t, i, j] * carrier[t, j, :] + hpost[t, i] * y[t, :] (+ term[t, :])
+ * fp32 arithmetic in that order; y enters rounded to bf16 (what mortar_spmm_bf16 would have stored).
+ *   carrier, out  [M, n_streams, Rb*16] contiguous, bf16 (carrier_f32 = 0; 8-byte aligned) or fp32 (1; 16-byte aligned);
+ *                 1 <= n_streams <= 4;  hres fp32 [M, n, n], hpost fp32 [M, n];  term [M, Rb*16] of the carrier's type or NULL
+ *   active / n_clusters  as mortar_spmm_bf16_masked (NULL: no input mask)
+ * MORTAR_ERR_LIMIT for M > 64: prefill-sized calls store y (mortar_spmm_bf16) and combine in a second pass. */
+int mortar_spmm_hc_post(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M, int64_t ldx,
+                        const void *carrier, int32_t carrier_f32, int32_t n_streams, const float *hres,
+                        const float *hpost, const void *term, void *out, const uint8_t *active, int32_t n_clusters,
+                        void *stream);
+
 /* Token tile of routed mortar_gateup_swiglu_bf16 for M rows against a matrix with Cb block-columns: the tile
  * size mortar_remoe_route must be called with.  4 for M <= 4, 16 for M <= 64, otherwise 32 or 64
  * depending on Cb; 0 when in_features is too wide for routed skipping (one LDS tile must hold a row of x). */

@@ -132,6 +132,37 @@ extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *sc
     return dispatch(3, p, W, static_cast<hipStream_t>(stream));
 }
 
+extern "C" int mortar_spmm_hc_post(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M, int64_t ldx,
+                                   const void *carrier, int32_t carrier_f32, int32_t n_streams, const float *hres,
+                                   const float *hpost, const void *term, void *out, const uint8_t *active,
+                                   int32_t n_clusters, void *stream) {
+    // the plain store is replaced, so y / ldy only have to pass the common checks
+    int rc = check_common(W, x, M, ldx, reinterpret_cast<const uint16_t *>(out), W ? (int64_t)W->Rb * 16 : 0, W ? (int64_t)W->Rb * 16 : 0);
+    if (rc) return rc;
+    if (M > MORTAR_SMALLM_MAX)
+        return mortar_fail(MORTAR_ERR_LIMIT, "spmm_hc_post: the fused POST write serves decode batches (M <= %d, got %lld); "
+                           "call mortar_spmm_bf16 and combine separately", MORTAR_SMALLM_MAX, (long long)M);
+    if (!carrier || !hres || !hpost || !out) return mortar_fail(MORTAR_ERR_ARG, "spmm_hc_post: null pointer");
+    if (n_streams < 1 || n_streams > 4) return mortar_fail(MORTAR_ERR_LIMIT, "spmm_hc_post: %d carrier streams outside 1..4", n_streams);
+    const uintptr_t al = carrier_f32 ? 15 : 7;
+    if ((reinterpret_cast<uintptr_t>(carrier) & al) || (reinterpret_cast<uintptr_t>(out) & al) || (reinterpret_cast<uintptr_t>(term) & al))
+        return mortar_fail(MORTAR_ERR_ARG, "spmm_hc_post: carrier, term and out must be %d-byte aligned", (int)al + 1);
+    SpmmParams p;
+    fill(p, W, sched, x, M, ldx, reinterpret_cast<uint16_t *>(out), (int64_t)W->Rb * 16);
+    p.n_units = W->Rb;
+    p.hc_h = carrier; p.hc_out = out; p.hc_res = hres; p.hc_post = hpost; p.hc_term = term; p.hc_n = n_streams; p.hc_f32 = carrier_f32 != 0;
+    int kind = 0;
+    if (active) {
+        if (n_clusters <= 0 || (W->Cb * 16) % n_clusters || ((W->Cb * 16) / n_clusters) % 8)
+            return mortar_fail(MORTAR_ERR_ARG, "spmm_hc_post: in_features/n_clusters must be a multiple of 8");
+        p.active = active; p.n_clusters = n_clusters; p.cluster_size = (W->Cb * 16) / n_clusters;
+        kind = 3;
+    }
+    rc = mortar_smallm_launch(kind, p, nullptr, 1, static_cast<hipStream_t>(stream));
+    if (rc < 0 && rc != MORTAR_ERR_HIP) return mortar_fail(MORTAR_ERR_LIMIT, "spmm_hc_post: shape has no small-tile kernel");
+    return rc;
+}
+
 namespace {
 int gateup_common(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M, int64_t ldx, bool norm,
                   const uint16_t *norm_w, float norm_eps, uint16_t *h, int64_t ldh, const float *gates,

@@ -39,6 +39,14 @@ struct SpmmParams {
     float uscale;             // CODE_UNIFORM kernels: half the matrix's (bf16-rounded) scale
     int pad_[2];
     const uint16_t *norm_w;   // bf16 [in_features] weight of that norm, or null for none
+    // hyper-connection POST write in place of the plain store (small tiles, plain products): out[t, i, :] =
+    // sum_j hc_res[t, i, j] * hc_h[t, j, :] + hc_post[t, i] * y[t, :] (+ hc_term[t, :]); null hc_h = plain store
+    const void *hc_h;         // carrier streams [M, hc_n, out_features], bf16 or fp32 (hc_f32)
+    void *hc_out;             // result, same shape and type as hc_h
+    const float *hc_res;      // [M, hc_n, hc_n]
+    const float *hc_post;     // [M, hc_n]
+    const void *hc_term;      // [M, out_features], type of hc_h, or null
+    int hc_n, hc_f32;
 };
 
 // Device-side view of the launch parameters: the pointers carry the global address space in their type, so
@@ -58,6 +66,10 @@ struct SpmmView {
     int n_units, Cb, M, n_clusters, cluster_size, n_mtiles, n_split, seg_cb, nseg, Rb, xcd_map, norm;
     float norm_eps, uscale;
     const MORTAR_GLOBAL u32x4_t *norm_w;
+    const MORTAR_GLOBAL char *hc_h, *hc_term;
+    MORTAR_GLOBAL char *hc_out;
+    const MORTAR_GLOBAL float *hc_res, *hc_post;
+    int hc_n, hc_f32;
 };
 static_assert(sizeof(SpmmParams) % 16 == 0, "table entries are copied in 16-byte words");
 // Entry i of a parameter table in device memory (uniform address: scalar loads).
@@ -80,6 +92,9 @@ __device__ __forceinline__ SpmmView mortar_view(const SpmmParams &q) {
     v.ldx = q.ldx; v.ldy = q.ldy; v.n_units = q.n_units; v.Cb = q.Cb; v.M = q.M; v.n_clusters = q.n_clusters;
     v.cluster_size = q.cluster_size; v.n_mtiles = q.n_mtiles; v.n_split = q.n_split; v.seg_cb = q.seg_cb; v.nseg = q.nseg; v.Rb = q.Rb; v.xcd_map = q.xcd_map;
     v.norm = q.norm; v.norm_eps = q.norm_eps; v.uscale = q.uscale; v.norm_w = (const MORTAR_GLOBAL u32x4_t *)q.norm_w;
+    v.hc_h = (const MORTAR_GLOBAL char *)q.hc_h; v.hc_term = (const MORTAR_GLOBAL char *)q.hc_term;
+    v.hc_out = (MORTAR_GLOBAL char *)q.hc_out; v.hc_res = (const MORTAR_GLOBAL float *)q.hc_res;
+    v.hc_post = (const MORTAR_GLOBAL float *)q.hc_post; v.hc_n = q.hc_n; v.hc_f32 = q.hc_f32;
     return v;
 }
 
@@ -207,25 +222,29 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
 template <int MT, int WAVES, bool MASKED, bool NORM>
 __device__ __forceinline__ void mortar_stage_quads(const SpmmView &p, unsigned char *lb, int m0, int c0, int ncb, int tid,
                                                    const float *rs) {
-    constexpr int RG = (MT + 15) / 16;                   // groups of 16 rows
-    constexpr int KC = RG >= 4 ? 2 : (RG == 2 ? 4 : 8);  // chunks in flight per wave: 8 loads per lane
+    // a wave instruction covers RPI rows x LPR consecutive 16-byte units: 16 rows x 64 bytes for the MFMA-sized
+    // tiles, 4 rows x 256 bytes for the narrow decode tiles (whose LDS write pattern does not matter)
+    constexpr int RPI = MT >= 16 ? 16 : 4, LPR = 64 / RPI;
+    constexpr int RG = (MT + RPI - 1) / RPI;             // row groups
+    constexpr int KC = RG >= 4 ? 2 : (RG == 2 ? 4 : 8);  // unit blocks in flight per wave: 8 loads per lane
     const int nch = 2 * ncb;                             // 16-byte units per row
-    const int nck = (nch + 3) >> 2;                      // 64-byte chunks per row
+    const int nck = (nch + LPR - 1) / LPR;               // blocks of LPR units per row
     const int rlast = (p.M - m0 < MT ? p.M - m0 : MT) - 1;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-    const int rsub = lane >> 2, li = lane & 3;
+    const int rsub = lane / LPR, li = lane % LPR;
     const MORTAR_GLOBAL char *xt = p.x + (int64_t)m0 * p.ldx * 2 + (int64_t)c0 * 32;
     const bool has_w = NORM && p.norm_w != nullptr;
     for (int ck0 = wave; ck0 < nck; ck0 += WAVES * KC) {
         u32x4_t v[KC][RG], wv[KC];
 #pragma unroll
         for (int k = 0; k < KC; ++k) {
-            int u = (ck0 + k * WAVES) * 4 + li;
+            if (ck0 + k * WAVES >= nck) break;           // uniform: nothing left for this wave
+            int u = (ck0 + k * WAVES) * LPR + li;
             u = u < nch ? u : nch - 1;
             if (NORM) wv[k] = has_w ? p.norm_w[c0 * 2 + u] : u32x4_t{0u, 0u, 0u, 0u};
 #pragma unroll
             for (int rg = 0; rg < RG; ++rg) {
-                int row = rg * 16 + rsub;
+                int row = rg * RPI + rsub;
                 row = row < rlast ? row : rlast;
                 v[k][rg] = *(const MORTAR_GLOBAL u32x4_t *)(xt + (int64_t)row * p.ldx * 2 + (uint32_t)u * 16u);
                 if (MASKED && p.active[(int64_t)(m0 + row) * p.n_clusters + (c0 * 16 + u * 8) / p.cluster_size] == 0)
@@ -234,10 +253,11 @@ __device__ __forceinline__ void mortar_stage_quads(const SpmmView &p, unsigned c
         }
 #pragma unroll
         for (int k = 0; k < KC; ++k) {
-            const int u = (ck0 + k * WAVES) * 4 + li;
+            if (ck0 + k * WAVES >= nck) break;
+            const int u = (ck0 + k * WAVES) * LPR + li;
 #pragma unroll
             for (int rg = 0; rg < RG; ++rg) {
-                const int row = rg * 16 + rsub;
+                const int row = rg * RPI + rsub;
                 if (row <= rlast && u < nch) {
                     u32x4_t o = v[k][rg];
                     if (NORM) o = rms_apply8(o, rs[row], wv[k], has_w);
@@ -285,8 +305,49 @@ __device__ __forceinline__ void mortar_stage_tile_norm(const SpmmView &p, uint4 
     mortar_stage_quads<MT, WAVES, false, true>(p, reinterpret_cast<unsigned char *>(lx), m0, 0, ncb, tid, rs);
 }
 
+// Four consecutive values of a carrier stream (bf16 or fp32 storage) as floats, and back.
+__device__ __forceinline__ f32x4_t mortar_load4(const MORTAR_GLOBAL char *base, int64_t elem, bool f32) {
+    if (f32) return *(const MORTAR_GLOBAL f32x4_t *)(base + elem * 4);
+    const u32x2_t u = *(const MORTAR_GLOBAL u32x2_t *)(base + elem * 2);
+    return f32x4_t{bf16_to_f32(u[0] & 0xffffu), bf16_to_f32(u[0] >> 16), bf16_to_f32(u[1] & 0xffffu), bf16_to_f32(u[1] >> 16)};
+}
+__device__ __forceinline__ void mortar_store4(MORTAR_GLOBAL char *base, int64_t elem, bool f32, f32x4_t v) {
+    if (f32) *(MORTAR_GLOBAL f32x4_t *)(base + elem * 4) = v;
+    else *(MORTAR_GLOBAL u32x2_t *)(base + elem * 2) = u32x2_t{bf16_pack2(v[0], v[1]), bf16_pack2(v[2], v[3])};
+}
+
+// Hyper-connection POST write for the four features a lane holds (reference: _hc_post_fwd_kernel,
+// morph/kernels/triton/fused_hyper_connection.py:927-970, called from engine._hc, morph/inference/engine.py:1052-1060;
+// wide form hc_post_wide, fused_decode_step.py:1725-1739): the MLP output y (rounded to bf16, the dtype the unfused
+// path hands over) never goes to memory; fp32 arithmetic in the reference's order (j ascending, then y, then term).
+template <int N>
+__device__ __forceinline__ void mortar_hc_post(const SpmmView &p, int tok, int f0, f32x4_t y) {
+    const int64_t C = (int64_t)p.Rb * 16;
+    const bool f32 = p.hc_f32 != 0;
+    f32x4_t h[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) h[j] = mortar_load4(p.hc_h, ((int64_t)tok * N + j) * C + f0, f32);
+    f32x4_t term = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (p.hc_term) term = mortar_load4(p.hc_term, (int64_t)tok * C + f0, f32);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        f32x4_t a = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const float hij = p.hc_res[((int64_t)tok * N + i) * N + j];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) a[v] = __builtin_fmaf(hij, h[j][v], a[v]);
+        }
+        const float pi = p.hc_post[(int64_t)tok * N + i];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) a[v] = __builtin_fmaf(pi, y[v], a[v]);
+        if (p.hc_term) a += term;
+        mortar_store4(p.hc_out, ((int64_t)tok * N + i) * C + f0, f32, a);
+    }
+}
+
 // Epilogue of one row unit for the 16 tokens of sub-tile `ms`: the lane holds D[4g+v][token].
-template <int NACC, int CODE = 0>
+template <int NACC, int CODE = 0, bool HC = false>
 __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, int tok, int g, bool has_gates,
                                                   f32x4_t a0, f32x4_t a1) {
     if (CODE & CODE_UNIFORM) {      // the blocks were multiplied as +-2: p.uscale is half the matrix's scale
@@ -296,6 +357,16 @@ __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, i
     u32x2_t pk;
     if (NACC == 1) {
         pk = u32x2_t{bf16_pack2(a0[0], a0[1]), bf16_pack2(a0[2], a0[3])};
+        if (HC && p.hc_h != nullptr) {
+            const f32x4_t y = {bf16_to_f32(pk[0] & 0xffffu), bf16_to_f32(pk[0] >> 16), bf16_to_f32(pk[1] & 0xffffu), bf16_to_f32(pk[1] >> 16)};
+            switch (p.hc_n) {
+                case 1: mortar_hc_post<1>(p, tok, unit * 16 + 4 * g, y); break;
+                case 2: mortar_hc_post<2>(p, tok, unit * 16 + 4 * g, y); break;
+                case 3: mortar_hc_post<3>(p, tok, unit * 16 + 4 * g, y); break;
+                default: mortar_hc_post<4>(p, tok, unit * 16 + 4 * g, y); break;
+            }
+            return;
+        }
     } else {
         float gv = 0.f;
         if (has_gates) gv = p.gates[(int64_t)tok * p.n_clusters + (unit * 16 + 4 * g) / p.cluster_size];
@@ -420,7 +491,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
             if (li >= (ROUTED ? cnt : MT)) continue;
             const int tok = m0 + (int)tk[ms];
             if (tok >= p.M) continue;
-            mortar_store_unit<NACC, CODE>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
+            mortar_store_unit<NACC, CODE, (MT <= 16 && NACC == 1 && !TABLE)>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
         }
     }
 }
@@ -508,7 +579,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
             if (li >= MT) continue;
             const int tok = m0 + li;
             if (tok >= p.M) continue;
-            mortar_store_unit<NACC, CODE>(p, units[k], tok, g, has_gates, acc[k][0][ms], acc[k][NACC - 1][ms]);
+            mortar_store_unit<NACC, CODE, (MT <= 16 && NACC == 1 && !TABLE)>(p, units[k], tok, g, has_gates, acc[k][0][ms], acc[k][NACC - 1][ms]);
         }
     }
 }
@@ -615,7 +686,7 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
         if (li >= (ROUTED ? cnt : MT)) continue;
         const int tok = m0 + (int)tk[ms];
         if (tok >= p.M) continue;
-        mortar_store_unit<NACC, CODE>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
+        mortar_store_unit<NACC, CODE, (MT <= 16 && NACC == 1)>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
     }
 }
 

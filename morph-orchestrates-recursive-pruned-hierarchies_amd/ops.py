@@ -67,6 +67,39 @@ def spmm(x: Tensor, W: MortarPack, out: Tensor | None = None, active: Tensor | N
     return y
 
 
+def spmm_hc_post(x: Tensor, W: MortarPack, carrier: Tensor, hres: Tensor, hpost: Tensor, term: Tensor | None = None,
+                 active: Tensor | None = None, out: Tensor | None = None) -> Tensor:
+    """`down` with the hyper-connection POST write in its epilogue (decode batches, M <= 64): returns
+    out[t, i] = sum_j hres[t, i, j] * carrier[t, j] + hpost[t, i] * (x W^T)[t] (+ term[t]); carrier / out [M, n, out_features]
+    in bf16 or fp32, hres fp32 [M, n, n], hpost fp32 [M, n], term [M, out_features] of the carrier's dtype.  The
+    reference runs the MLP, stores y, then launches _hc_post_fwd_kernel (engine.py:996-1001, 1052-1060)."""
+    x = _bf16_2d(x, "spmm_hc_post")
+    M = x.shape[0]
+    if x.shape[1] != W.in_features:
+        raise ValueError(f"spmm_hc_post: x has {x.shape[1]} features, matrix expects {W.in_features}")
+    if carrier.dtype not in (torch.bfloat16, torch.float32) or carrier.dim() != 3 or not carrier.is_contiguous():
+        raise TypeError("spmm_hc_post: carrier must be a contiguous bf16 or fp32 [M, n, out_features] tensor")
+    _need_gpu(carrier, "spmm_hc_post")
+    n = carrier.shape[1]
+    if carrier.shape[0] != M or carrier.shape[2] != W.out_features:
+        raise ValueError(f"spmm_hc_post: carrier is {tuple(carrier.shape)}, expected ({M}, n, {W.out_features})")
+    for name, t, shape in (("hres", hres, (M, n, n)), ("hpost", hpost, (M, n))):
+        if t.dtype != torch.float32 or tuple(t.shape) != shape or not t.is_contiguous():
+            raise TypeError(f"spmm_hc_post: {name} must be contiguous float32 {shape}")
+    if term is not None and (term.dtype != carrier.dtype or tuple(term.shape) != (M, W.out_features) or not term.is_contiguous()):
+        raise TypeError("spmm_hc_post: term must be contiguous [M, out_features] of the carrier's dtype")
+    res = out if out is not None else torch.empty_like(carrier)
+    if M == 0:
+        return res
+    if active is not None and (active.dtype != torch.uint8 or not active.is_contiguous()):
+        raise TypeError("spmm_hc_post: active must be a contiguous uint8 tensor")
+    rc = _lib.lib().mortar_spmm_hc_post(W.ref, _p(W.sched(1)), _p(x), M, x.stride(0), _p(carrier),
+                                        int(carrier.dtype == torch.float32), n, _p(hres), _p(hpost), _p(term), _p(res),
+                                        _p(active), active.shape[1] if active is not None else 0, _stream(x))
+    _lib.check(rc, "mortar_spmm_hc_post")
+    return res
+
+
 def norm_fusable(W: MortarPack) -> bool:
     """True if gateup_swiglu can apply the RMSNorm in front of the MLP while it stages x (in_features <= 2048)."""
     return bool(_lib.lib().mortar_norm_fusable(W.Cb)) and W.nseg == 1

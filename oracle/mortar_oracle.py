@@ -19,6 +19,8 @@ reference checkout).  How each function is pinned (no reference import is needed
   remoe_gates              brute force on tiny inputs incl. ties; invariants
   route_flags              closed form
   rmsnorm                  closed form
+  hc_post                  special cases with known results (identity mixing, pure pass-through of y, a
+                           permutation of the streams) + a hand-computed 2-stream case
   transpose_meta           order of blocks *inside one block-column* depends on the
                            reference's unstable argsort: PARITY UNPINNED for that
                            order (backward-only metadata, not on the forward path)
@@ -362,6 +364,21 @@ def route_flags(gates: np.ndarray, d_ff: int, blk: int = 16):
     hi = (r * blk + blk - 1) // cls
     col = ((gates[:, lo] > 0) | (gates[:, hi] > 0)).astype(np.int32)
     return np.concatenate([col, col], axis=1), col
+
+
+# --------------------------------------------------------------------------- hyper-connection POST
+
+
+def hc_post(hres: np.ndarray, hpost: np.ndarray, h: np.ndarray, y: np.ndarray, term: np.ndarray | None = None) -> np.ndarray:
+    """out[t, i, c] = sum_j Hres[t, i, j] * h[t, j, c] + Hpost_row[t, i] * y[t, c] (+ term[t, c]): the POST write of the
+    hyper-connection residual around the MLP (morph/kernels/triton/fused_hyper_connection.py:927-970; wide form
+    morph/kernels/triton/fused_decode_step.py:1725-1739; call site morph/inference/engine.py:996-1001, 1052-1060).
+    hres [T, n, n], hpost [T, n], h [T, n, C], y [T, C], term [T, C] or None -> float64 [T, n, C], unrounded."""
+    out = np.einsum("tij,tjc->tic", hres.astype(np.float64), h.astype(np.float64))
+    out = out + hpost.astype(np.float64)[:, :, None] * y.astype(np.float64)[:, None, :]
+    if term is not None:
+        out = out + term.astype(np.float64)[:, None, :]
+    return out
 
 
 # --------------------------------------------------------------------------- RMSNorm

@@ -486,6 +486,48 @@ def test_mortar_gemv_reference_signature(dev):
         mortar_amd.mortar_gemv(torch.from_numpy(x).to(dev), pk, swiglu_x=True)
 
 
+@pytest.mark.parametrize("B,n,f32", [(1, 4, True), (3, 4, False), (16, 2, True), (40, 4, False), (5, 1, True), (7, 3, False)])
+def test_down_with_hc_post_epilogue(dev, B, n, f32):
+    """`down` with the hyper-connection POST write in its epilogue against the oracle (y rounded to bf16, then the
+    float64 combination), for fp32 and bf16 carriers, with and without the inject term and the routed input mask."""
+    d_model, d_ff = 512, 16 * 96
+    m = synth.synth_matrix(d_model, d_ff, 0.25, seed=90)
+    W = synth.to_pack(m, dev)
+    rng = np.random.default_rng(91 + B)
+    x = synth.synth_x(B, d_ff, 92)
+    dt = torch.float32 if f32 else torch.bfloat16
+    rnd = (lambda a: a.astype(np.float32)) if f32 else (lambda a: O.bf16_round(a.astype(np.float32)))
+    h = rnd(rng.standard_normal((B, n, d_model)))
+    term = rnd(rng.standard_normal((B, d_model)))
+    hres = (rng.standard_normal((B, n, n)) * 0.5).astype(np.float32)
+    hpost = rng.standard_normal((B, n)).astype(np.float32)
+    T = lambda a, d=None: torch.from_numpy(a).to(dev).to(d) if d is not None else torch.from_numpy(a).to(dev)
+    y = oracle_spmm(x, m)                                                   # bf16-rounded, as the unfused path stores it
+    tol = dict(rtol=2e-6, atol=2e-6) if f32 else dict(rtol=2.0 ** -7, atol=1e-2)
+    for use_term in (False, True):
+        ref = O.hc_post(hres, hpost, h, y, term if use_term else None)
+        got = ops.spmm_hc_post(to_dev(x, dev), W, T(h, dt), T(hres), T(hpost), T(term, dt) if use_term else None)
+        assert got.dtype == dt and tuple(got.shape) == (B, n, d_model)
+        yk = to_np(ops.spmm(to_dev(x, dev), W))                             # the kernel's own y: same bits go into the POST
+        ref_k = O.hc_post(hres, hpost, h, yk, term if use_term else None)
+        np.testing.assert_allclose(got.float().cpu().numpy(), ref_k, **tol)
+        assert np.abs(got.float().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
+    # identity mixing and hpost = 0 returns the carrier bit for bit; hres = 0, hpost = 1 returns y in every stream
+    eye = torch.eye(n, device=dev).expand(B, n, n).contiguous()
+    out = ops.spmm_hc_post(to_dev(x, dev), W, T(h, dt), eye, torch.zeros(B, n, device=dev))
+    assert torch.equal(out, T(h, dt))
+    out = ops.spmm_hc_post(to_dev(x, dev), W, T(h, dt), torch.zeros(B, n, n, device=dev), torch.ones(B, n, device=dev))
+    assert torch.equal(out.float(), ops.spmm(to_dev(x, dev), W).float()[:, None, :].expand(B, n, d_model))
+    # routed: inactive input clusters read as zero, as in the masked product
+    act = torch.from_numpy((rng.random((B, 16)) < 0.5).astype(np.uint8)).to(dev)
+    ym = ops.spmm(to_dev(x, dev), W, active=act)
+    out = ops.spmm_hc_post(to_dev(x, dev), W, T(h, dt), torch.zeros(B, n, n, device=dev), torch.ones(B, n, device=dev), active=act)
+    assert torch.equal(out.float(), ym.float()[:, None, :].expand(B, n, d_model))
+    with pytest.raises(ValueError, match="decode batches"):
+        ops.spmm_hc_post(to_dev(synth.synth_x(65, d_ff, 1), dev), W, torch.zeros(65, n, d_model, device=dev),
+                         torch.zeros(65, n, n, device=dev), torch.zeros(65, n, device=dev))
+
+
 def test_rmsnorm(dev):
     x = O.bf16_round(synth.synth_x(37, 2048, 90) * 3)
     w = synth.synth_x(1, 2048, 91)[0]

@@ -348,6 +348,23 @@ def test_rmsnorm_closed_form():
     assert np.allclose(O.rmsnorm(x, w, bf16_out=False), 2 * y)
 
 
+def test_hc_post_known_cases():
+    rng = np.random.default_rng(81)
+    T, n, C = 3, 4, 8
+    h, y, term = rng.standard_normal((T, n, C)), rng.standard_normal((T, C)), rng.standard_normal((T, C))
+    eye = np.broadcast_to(np.eye(n), (T, n, n))
+    assert np.array_equal(O.hc_post(eye, np.zeros((T, n)), h, y), h)                       # identity mixing, y off: the carrier
+    assert np.array_equal(O.hc_post(np.zeros((T, n, n)), np.ones((T, n)), h, y), np.broadcast_to(y[:, None], (T, n, C)))
+    perm = np.zeros((T, n, n)); perm[:, np.arange(n), (np.arange(n) + 1) % n] = 1.0         # out[i] = h[i + 1]: rows index the OUTPUT
+    assert np.array_equal(O.hc_post(perm, np.zeros((T, n)), h, y), np.roll(h, -1, axis=1))
+    assert np.allclose(O.hc_post(eye, np.zeros((T, n)), h, y, term), h + term[:, None])    # the term is added to every stream once
+    # hand-computed: 2 streams, 1 channel: out0 = 2*10 + 3*20 + 0.5*4 = 82, out1 = -1*10 + 0*20 + 2*4 + 1 = -1
+    out = O.hc_post(np.array([[[2.0, 3.0], [-1.0, 0.0]]]), np.array([[0.5, 2.0]]), np.array([[[10.0], [20.0]]]), np.array([[4.0]]))
+    assert out.tolist() == [[[82.0], [-2.0]]]
+    out = O.hc_post(np.array([[[2.0, 3.0], [-1.0, 0.0]]]), np.array([[0.5, 2.0]]), np.array([[[10.0], [20.0]]]), np.array([[4.0]]), np.array([[1.0]]))
+    assert out.tolist() == [[[83.0], [-1.0]]]
+
+
 def test_bf16_round_matches_torch():
     import torch
     a = np.random.default_rng(70).standard_normal(10000).astype(np.float32) * 1e3
