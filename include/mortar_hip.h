@@ -283,6 +283,23 @@ int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_e
                      const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc,
                      void *stream);
 
+/* The same work-list GEMV in the reference engine's arithmetic (fused_decode_step.py:1335, 1341-1459, 1502-1547; the
+ * engine runs fp32, morph/inference/engine.py:156-160): fp32 activations in, exact +-x / 0 products, fp32 sums, the
+ * block's fp32 scale applied to the block sum (scale-after-sum; with scale_count = 1 the reference's one mortar_scale),
+ * SwiGLU as g * sigmoid(g) * u and gates in fp32, fp32 out.  Internally an fp32 activation is split exactly into three
+ * bf16 terms and a block is contracted with +-2 / 0 codes on the bf16 MFMA, so no product is rounded.
+ *   scale      device fp32 [scale_count], scale_count = 1 or nnz (NOT rounded to bf16)
+ *   swiglu_x   != 0: x is the gate_up output [B, 2 * in_features] and the input is silu(g) * u computed on load
+ *              (the reference's down call form, fused_decode_step.py:1410-1414)
+ *   x fp32 [B, ldx]; y fp32 [B, Rb*16] (mode 0) or [B, Rb*8] (mode 1), 16-byte aligned, ldy % 4 == 0
+ *   kseg       block-columns per K segment of the work list; 3 * 2 * kseg * (16 * ceil(B / 16) + 1) * 16 bytes of LDS
+ *   other arguments as mortar_gemv_bf16.  Agreement with a float64 evaluation: fp32 rounding of the sums only. */
+int mortar_gemv_f32(const mortar_bcsr_t *W, const float *scale, int64_t scale_count, const int32_t *entries,
+                    int64_t n_entries, int32_t nslots, const int32_t *row_slots, int32_t kseg, int32_t mode,
+                    int32_t swiglu_x, const float *x, int32_t B, int64_t ldx, float *y, int64_t ldy, float *part,
+                    const float *gates, int32_t n_clusters, int64_t ldg,
+                    const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc, void *stream);
+
 /* mortar_gemv_bf16 for callers that cannot allocate device memory or hand in a workspace: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and
  * results (bit for bit) as mortar_gemv_bf16 minus `part`: the fp32 partial sums of split rows (nslots > 1) go to a

@@ -254,6 +254,252 @@ extern "C" int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, 
                     n_clusters, ldg, row_act, ldr, col_act, ldc, stream);
 }
 
+// ---- the reference engine's arithmetic: fp32 activations, exact products, fp32 sums, scale after the block sum ------
+// (morph/kernels/triton/fused_decode_step.py:1335, 1341-1459; the engine runs fp32, morph/inference/engine.py:156-160).
+// An fp32 activation is split exactly into three bf16 terms x = hi + mid + lo (8 + 8 + 8 mantissa bits).  One MFMA
+// contracts ONE block against two of the terms at once: both K halves of the A operand hold the block's codes as
+// +-2 / 0 (exact in bf16), the B operand holds hi in the first 16 K slots and mid in the second; a second MFMA adds
+// the lo term.  Every product is exact, the fp32 accumulator of the matrix pipe takes the place of the reference's
+// fp32 sums, and the block's fp32 scale (times one half for the +-2) multiplies the block sum afterwards:
+// y = sum_j s_j * (C_j x_j), the per-block form of the reference's scale-after-sum.
+namespace {
+
+struct GemvF32Params {
+    const uint32_t *codes;
+    const int16_t *col;
+    const float *scale;       // fp32 [nnz], or [1] when scale_count == 1
+    const int32_t *entries;
+    int n_entries, nslots, kseg, mode, Cb, N, scale_count, swiglu_x;
+    const float *x;           // [B, ldx]; with swiglu_x the gate_up output [B, 2 * in_features]
+    int B;
+    int64_t ldx;
+    float *y;
+    int64_t ldy;
+    float *part;
+    const float *gates;
+    int n_clusters, cluster_size;
+    int64_t ldg;
+    const int32_t *row_act;
+    int64_t ldr;
+    const int32_t *col_act;
+    int64_t ldc;
+};
+
+template <int MSUB>
+__device__ __forceinline__ void run_blocks_f32(const GemvF32Params &p, int p0, int cnt, int c0, const uint4 *lx, int plane,
+                                               int zero_unit, const uint32_t *colflag, int n, int bsel, int hsel,
+                                               f32x4_t (&acc)[MSUB]) {
+    constexpr int LDB = 16 * MSUB + 1;
+    for (int q0 = 0; q0 < cnt; q0 += UN) {
+        uint32_t w[UN];
+        float sc[UN];
+        int c[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int q = q0 + u < cnt ? q0 + u : cnt - 1;
+            const int64_t j = p0 + q;
+            w[u] = p.codes[j * 16 + n];
+            sc[u] = 0.5f * p.scale[p.scale_count == 1 ? 0 : j];
+            c[u] = p.col[j] - c0;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            if (q0 + u < cnt) {
+                if (colflag && colflag[c[u]] == 0u) continue;                 // uniform: the whole wave reads the same flag
+                const u32x4_t A = mortar_nib4((w[u] << (2 * hsel)) & 0xCCCCCCCCu);
+                const uint32_t xo = (uint32_t)((c[u] * 2 + hsel) * LDB + n);
+#pragma unroll
+                for (int ms = 0; ms < MSUB; ++ms) {
+                    // K slots 0..15 (bsel 0): hi, then lo;  K slots 16..31 (bsel 1): mid, then zeros
+                    const uint4 b1 = lx[(bsel ? plane : 0) + xo + ms * 16];
+                    const uint4 b2 = bsel ? lx[zero_unit] : lx[2 * plane + xo + ms * 16];
+                    f32x4_t P = mortar_mfma(A, u32x4_t{b1.x, b1.y, b1.z, b1.w}, f32x4_t{0.f, 0.f, 0.f, 0.f});
+                    P = mortar_mfma(A, u32x4_t{b2.x, b2.y, b2.z, b2.w}, P);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[ms][v] = __builtin_fmaf(sc[u], P[v], acc[ms][v]);
+                }
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ float sigmoid_f32(float g) { return 1.0f / (1.0f + __expf(-g)); }
+
+template <int MSUB>
+__global__ void __launch_bounds__(256) mortar_gemv_f32_kernel(const GemvF32Params p) {
+    constexpr int LDB = 16 * MSUB + 1;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint4 *lx = reinterpret_cast<uint4 *>(smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, g = lane >> 4, bsel = g >> 1, hsel = g & 1;
+    const int32_t *e0p = p.entries + (int64_t)blockIdx.x * 4 * 8;
+    const int seg = __builtin_amdgcn_readfirstlane(e0p[7]);
+    const int c0 = seg * p.kseg;
+    const int ncb = (p.Cb - c0) < p.kseg ? (p.Cb - c0) : p.kseg;
+    const int nch = 2 * ncb;
+    const int plane = 2 * p.kseg * LDB;                         // 16-byte units per term plane
+    const int zero_unit = 3 * plane;                            // one all-zero unit
+    uint32_t *colflag = reinterpret_cast<uint32_t *>(smem + (size_t)(3 * plane + 1) * 16);
+    const int I = p.Cb * 16;
+
+    // stage the three bf16 terms of this K segment: unit (ch, tok) <- x[tok, c0*16 + ch*8 .. +8]
+    for (int it = tid; it < nch * p.B; it += 256) {
+        const int tok = it / nch, ch = it % nch;
+        const float *src = p.x + (int64_t)tok * p.ldx + (int64_t)c0 * 16 + ch * 8;
+        uint32_t hi[4], mid[4], lo[4];
+#pragma unroll
+        for (int k = 0; k < 8; k += 2) {
+            float v[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                float xv = src[k + e];
+                if (p.swiglu_x) xv = xv * sigmoid_f32(xv) * src[I + k + e];      // h = silu(g) * u on load, fp32
+                v[e] = xv;
+            }
+            const uint32_t h2 = bf16_pack2(v[0], v[1]);
+            const float r0 = v[0] - bf16_to_f32(h2 & 0xffffu), r1 = v[1] - bf16_to_f32(h2 >> 16);
+            const uint32_t m2 = bf16_pack2(r0, r1);
+            const float s0 = r0 - bf16_to_f32(m2 & 0xffffu), s1 = r1 - bf16_to_f32(m2 >> 16);
+            hi[k / 2] = h2; mid[k / 2] = m2; lo[k / 2] = bf16_pack2(s0, s1);
+        }
+        lx[ch * LDB + tok] = uint4{hi[0], hi[1], hi[2], hi[3]};
+        lx[plane + ch * LDB + tok] = uint4{mid[0], mid[1], mid[2], mid[3]};
+        lx[2 * plane + ch * LDB + tok] = uint4{lo[0], lo[1], lo[2], lo[3]};
+    }
+    if (tid == 0) lx[zero_unit] = uint4{0u, 0u, 0u, 0u};
+    if (p.col_act) {
+        for (int c = tid; c < ncb; c += 256) {
+            uint32_t f = 0;
+            for (int b = 0; b < p.B; ++b) f |= (uint32_t)(p.col_act[(int64_t)b * p.ldc + c0 + c] != 0);
+            colflag[c] = f;
+        }
+    }
+    __syncthreads();
+
+    const int32_t *ep = e0p + wave * 8;
+    const int rowA = __builtin_amdgcn_readfirstlane(ep[0]);
+    if (rowA < 0) return;
+    const int pA = __builtin_amdgcn_readfirstlane(ep[1]), cntA = __builtin_amdgcn_readfirstlane(ep[2]);
+    const int rowB = __builtin_amdgcn_readfirstlane(ep[3]);
+    const int pB = __builtin_amdgcn_readfirstlane(ep[4]), cntB = __builtin_amdgcn_readfirstlane(ep[5]);
+    const int slot = __builtin_amdgcn_readfirstlane(ep[6]);
+    bool unit_on = true;
+    if (p.row_act) {
+        int f = 0;
+        if (lane < p.B) f = p.row_act[(int64_t)lane * p.ldr + rowA] != 0;
+        unit_on = __builtin_amdgcn_readfirstlane(__ballot(f) != 0ull);
+    }
+    f32x4_t accA[MSUB], accB[MSUB];
+#pragma unroll
+    for (int ms = 0; ms < MSUB; ++ms) accA[ms] = accB[ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (unit_on) {
+        run_blocks_f32<MSUB>(p, pA, cntA, c0, lx, plane, zero_unit, p.col_act ? colflag : nullptr, n, bsel, hsel, accA);
+        if (rowB >= 0) run_blocks_f32<MSUB>(p, pB, cntB, c0, lx, plane, zero_unit, p.col_act ? colflag : nullptr, n, bsel, hsel, accB);
+    }
+#pragma unroll
+    for (int ms = 0; ms < MSUB; ++ms) {
+        const int tok = ms * 16 + n;
+        if (tok >= p.B) continue;
+        if (p.nslots > 1) {
+            float *pp = p.part + ((int64_t)slot * p.B + tok) * p.N;
+            *reinterpret_cast<f32x4_t *>(pp + rowA * 16 + 4 * g) = accA[ms];
+            if (rowB >= 0) *reinterpret_cast<f32x4_t *>(pp + rowB * 16 + 4 * g) = accB[ms];
+        } else {
+            const int e0 = rowA * 16 + 4 * g;
+            f32x4_t r = accA[ms];
+            if (p.mode == 1) {
+                const float gv = p.gates ? p.gates[(int64_t)tok * p.ldg + e0 / p.cluster_size] : 1.0f;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    r[v] = accA[ms][v] * sigmoid_f32(accA[ms][v]) * accB[ms][v];
+                    if (p.gates) r[v] *= gv;
+                }
+            }
+            *reinterpret_cast<f32x4_t *>(p.y + (int64_t)tok * p.ldy + e0) = r;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) mortar_combine_f32_kernel(const GemvF32Params p, const int32_t *row_slots) {
+    const int nout = p.mode == 0 ? p.N : p.N / 2;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)p.B * nout) return;
+    const int tok = (int)(i / nout), o = (int)(i % nout);
+    const int ns = row_slots[o >> 4];
+    float a = 0.f, b = 0.f;
+    for (int s = 0; s < ns; ++s) {
+        const float *pp = p.part + ((int64_t)s * p.B + tok) * p.N;
+        a += pp[o];
+        if (p.mode == 1) b += pp[nout + o];
+    }
+    float r = a;
+    if (p.mode == 1) {
+        r = a * sigmoid_f32(a) * b;
+        if (p.gates) r *= p.gates[(int64_t)tok * p.ldg + o / p.cluster_size];
+    }
+    p.y[(int64_t)tok * p.ldy + o] = r;
+}
+
+template <int MSUB>
+int launch_gemv_f32(const GemvF32Params &p, hipStream_t st) {
+    const size_t smem = ((size_t)3 * 2 * p.kseg * (16 * MSUB + 1) + 1) * 16 + (size_t)p.kseg * 4;
+    if (smem > 160 * 1024) return mortar_fail(MORTAR_ERR_LIMIT, "gemv_f32: K segment of %d block-columns needs %zu bytes of LDS", p.kseg, smem);
+    auto kern = mortar_gemv_f32_kernel<MSUB>;
+    static size_t attr_set = 0;
+    if (smem > attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        attr_set = smem;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p.n_entries / 4)), dim3(256), smem, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "gemv_f32 launch: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}
+
+}  // namespace
+
+extern "C" int mortar_gemv_f32(const mortar_bcsr_t *W, const float *scale, int64_t scale_count, const int32_t *entries,
+                               int64_t n_entries, int32_t nslots, const int32_t *row_slots, int32_t kseg, int32_t mode,
+                               int32_t swiglu_x, const float *x, int32_t B, int64_t ldx, float *y, int64_t ldy, float *part,
+                               const float *gates, int32_t n_clusters, int64_t ldg,
+                               const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc, void *stream) {
+    if (!W || !W->codes || !W->col || !scale || !entries || !x || !y) return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: null pointer");
+    if (scale_count != 1 && scale_count != W->nnz) return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: scale_count must be 1 or nnz");
+    if (B <= 0 || B > 64) return mortar_fail(MORTAR_ERR_LIMIT, "gemv_f32: B=%d outside 1..64", B);
+    if (n_entries <= 0 || n_entries % 4 || n_entries > (int64_t)0x7fffffff) return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: entry count must be a positive multiple of 4");
+    if (mode != 0 && mode != 1) return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: mode must be 0 or 1");
+    if (mode == 1 && (W->Rb & 1)) return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: gate_up needs an even number of block-rows");
+    if (nslots < 1 || (nslots > 1 && (!part || !row_slots))) return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: nslots > 1 needs the partial workspace and row_slots");
+    if (kseg <= 0) return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: kseg must be positive");
+    const int64_t nout = mode == 0 ? (int64_t)W->Rb * 16 : (int64_t)W->Rb * 8;
+    const int64_t need_x = (int64_t)W->Cb * 16 * (swiglu_x ? 2 : 1);
+    if (ldx < need_x || ldy < nout || ldy % 4 || (reinterpret_cast<uintptr_t>(x) & 3) || (reinterpret_cast<uintptr_t>(y) & 15))
+        return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: bad leading dimension or alignment (y 16-byte aligned, ldy %% 4 == 0)");
+    GemvF32Params p{};
+    p.codes = W->codes; p.col = W->col; p.scale = scale; p.scale_count = (int)scale_count; p.entries = entries;
+    p.n_entries = (int)n_entries; p.nslots = nslots; p.kseg = kseg; p.mode = mode; p.Cb = W->Cb; p.N = W->Rb * 16;
+    p.swiglu_x = swiglu_x != 0; p.x = x; p.B = B; p.ldx = ldx; p.y = y; p.ldy = ldy; p.part = part;
+    p.n_clusters = 1; p.cluster_size = 1 << 30;
+    if (gates) {
+        if (mode != 1 || n_clusters <= 0 || nout % n_clusters || (nout / n_clusters) % 4)
+            return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: gates need mode 1 and d_ff / n_clusters a whole multiple of 4");
+        p.gates = gates; p.n_clusters = n_clusters; p.cluster_size = (int)(nout / n_clusters); p.ldg = ldg;
+    }
+    p.row_act = row_act; p.ldr = ldr; p.col_act = col_act; p.ldc = ldc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int rc = B <= 16 ? launch_gemv_f32<1>(p, st) : (B <= 32 ? launch_gemv_f32<2>(p, st) : launch_gemv_f32<4>(p, st));
+    if (rc) return rc;
+    if (nslots > 1) {
+        const int64_t total = (int64_t)B * nout;
+        hipLaunchKernelGGL(mortar_combine_f32_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, p, row_slots);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "combine launch: %s", hipGetErrorString(e));
+    }
+    return MORTAR_OK;
+}
+
 // ---- the same GEMV for callers that cannot allocate ------------------------------------------------------------
 // The partial sums of split rows go to this array inside the library instead of a caller workspace.  Every device
 // the library runs on holds its own copy at its own address; host code must use that address (looked up once per

@@ -21,16 +21,18 @@ def mortar_pack_strips(cms) -> MortarPack:
 def mortar_gemv(x: Tensor, pack: MortarPack, swiglu_x: bool = False, swiglu_out: bool = False,
                 row_act: Tensor | None = None, col_act: Tensor | None = None, gates: Tensor | None = None,
                 cluster_size: int = 0) -> Tensor:
-    """x [B, I] row-contiguous -> [B, O], or [B, O/2] = silu(g)*u with swiglu_out (the gate_up call).
-    Same keywords as the reference; activations are bf16 on this path (fp32 input is rounded to bf16 and the
-    result returned as fp32, the reference engine's dtype)."""
-    if swiglu_x:
-        raise NotImplementedError("swiglu_x (SwiGLU on load) is superseded by swiglu_out on the gate_up call")
+    """x [B, I] row-contiguous -> [B, O], or [B, O/2] = silu(g)*u with swiglu_out (the gate_up call); with swiglu_x,
+    x is the packed gate_up output [B, 2I] and h = silu(g)*u is computed on load (the reference's down call form).
+    Same keywords as the reference (fused_decode_step.py:1502-1509).  float32 input runs the reference engine's
+    arithmetic (exact products, fp32 sums, fp32 scale after the block sum, fp32 out); bfloat16 input runs the bf16
+    activation path of this runtime (swiglu_x there goes through the fp32 kernel and is rounded to bf16 at the end)."""
     if gates is not None and cluster_size and (pack.out_features // 2) // gates.shape[-1] != cluster_size:
         raise ValueError("cluster_size does not match d_ff / n_clusters")
-    xb = x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16)
-    y = ops.gemv(xb, pack, swiglu_out=swiglu_out, gates=gates, row_act=row_act, col_act=col_act)
-    return y if x.dtype == torch.bfloat16 else y.to(x.dtype)
+    if x.dtype == torch.float32 or swiglu_x:
+        y = ops.gemv_f32(x.float(), pack, swiglu_x=swiglu_x, swiglu_out=swiglu_out, gates=gates, row_act=row_act, col_act=col_act)
+        return y if x.dtype == torch.float32 else y.to(x.dtype)
+    y = ops.gemv(x, pack, swiglu_out=swiglu_out, gates=gates, row_act=row_act, col_act=col_act)
+    return y
 
 
 class MortarDecodeMLP:

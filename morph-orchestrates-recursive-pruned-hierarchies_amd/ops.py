@@ -326,6 +326,52 @@ def gemv(x: Tensor, W: MortarPack, swiglu_out: bool = False, gates: Tensor | Non
     return y
 
 
+def gemv_f32(x: Tensor, W: MortarPack, swiglu_x: bool = False, swiglu_out: bool = False, gates: Tensor | None = None,
+             row_act: Tensor | None = None, col_act: Tensor | None = None, max_blocks: int | None = None,
+             out: Tensor | None = None) -> Tensor:
+    """Decode GEMV in the reference engine's arithmetic (fp32 activations, exact products, fp32 sums, fp32 scale after
+    the block sum, fp32 out): the reference's mortar_gemv (fused_decode_step.py:1502-1547).  ``swiglu_x``: x is the
+    gate_up output [B, 2 * in_features] and silu(g) * u is applied on load; ``swiglu_out``: W is gate_up and the result
+    is silu(g) * u [* gates]."""
+    _need_gpu(x, "gemv_f32")
+    if x.dtype != torch.float32 or x.dim() != 2:
+        raise TypeError("gemv_f32: expected a float32 [B, features] tensor")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    B = x.shape[0]
+    if not 1 <= B <= 64:
+        raise ValueError(f"gemv_f32: batch {B} outside 1..64")
+    need = W.in_features * (2 if swiglu_x else 1)
+    if x.shape[1] != need:
+        raise ValueError(f"gemv_f32: x has {x.shape[1]} features, expected {need}")
+    if W.scales_f32 is None:
+        raise ValueError("gemv_f32: the pack holds no scales yet (requantize it first)")
+    if swiglu_out and W.Rb % 2:
+        raise ValueError("gemv_f32: gate_up has an odd number of block-rows")
+    mt = 16 if B <= 16 else (32 if B <= 32 else 64)
+    kseg = max(2, min(W.Cb, (48 * 1024) // ((mt + 1) * 16) // 2))       # three term planes of at most 48 KiB each
+    ent, nslots, row_slots, _ = W.worklist(2 if swiglu_out else 1, kseg, max_blocks if max_blocks is not None else 1 << 20)
+    nout = W.out_features // 2 if swiglu_out else W.out_features
+    y = out if out is not None else torch.empty((B, nout), dtype=torch.float32, device=x.device)
+    part = torch.empty((nslots, B, W.out_features), dtype=torch.float32, device=x.device) if nslots > 1 else None
+    ncl, ldg = 0, 0
+    if gates is not None:
+        if gates.dtype != torch.float32 or gates.stride(1) != 1:
+            raise TypeError("gemv_f32: gates must be float32 with unit inner stride")
+        ncl, ldg = gates.shape[1], gates.stride(0)
+    for f in (row_act, col_act):
+        if f is not None and (f.dtype != torch.int32 or f.stride(1) != 1):
+            raise TypeError("gemv_f32: row_act / col_act must be int32 with unit inner stride")
+    sc = W.scales_f32
+    rc = _lib.lib().mortar_gemv_f32(
+        W.ref, _p(sc), sc.numel(), _p(ent), ent.shape[0], nslots, _p(row_slots), kseg, 1 if swiglu_out else 0,
+        1 if swiglu_x else 0, _p(x), B, x.stride(0), _p(y), y.stride(0), _p(part), _p(gates), ncl, ldg,
+        _p(row_act), row_act.stride(0) if row_act is not None else 0,
+        _p(col_act), col_act.stride(0) if col_act is not None else 0, _stream(x))
+    _lib.check(rc, "mortar_gemv_f32")
+    return y
+
+
 class LayerStack:
     """n layers of one shape (same Rb, Cb, K segments) whose small-M products run in ONE launch:
     y_l = x_l W_l^T, or with swiglu the fused silu(g)*u of gate_up W_l.  The inputs and outputs are fixed at

@@ -164,8 +164,12 @@ class MortarPack:
         self.device = torch.device(device)
         if packed is None:
             codes, sdup = np.zeros(self.nnz * 16, dtype=np.uint32), np.zeros(self.nnz, dtype=np.uint32)
+            self.scales_f32 = None
         else:
             codes, sdup = encode_blocks(packed, self.nnz, scale)
+            # the scales as given (fp32, not rounded to bf16): what the fp32 decode arithmetic multiplies by
+            sc = scale.detach().cpu().numpy() if isinstance(scale, torch.Tensor) else np.asarray(scale)
+            self.scales_f32 = torch.from_numpy(np.ascontiguousarray(sc, dtype=np.float32).reshape(-1)).to(self.device)
         validate_bcsr(self.h_offsets, self.h_col, self.Rb, self.Cb)
         us = C.c_float(0.0)
         _lib.check(_lib.lib().mortar_uniform_scale_host(_vp(sdup), self.nnz, C.byref(us)), "mortar_uniform_scale_host")
@@ -244,6 +248,7 @@ class MortarPack:
                                        scale.data_ptr() if scale is not None else None, out.data_ptr(),
                                        self._status.data_ptr(), 0 if sync else 1, float(ternary_tol),
                                        self._ws.data_ptr(), st), "mortar_requantize")
+        self.scales_f32 = out
         us = 0.0
         if sync:
             self.raise_status()
@@ -347,7 +352,7 @@ class MortarPack:
         """A second resident copy (own device buffers and schedules) of the same matrix."""
         import copy
         c = copy.copy(self)
-        for name in ("codes", "sdup", "col", "row_ptr", "row_desc", "codes_o", "sd_o", "col_o", "codes4_o"):
+        for name in ("codes", "sdup", "col", "row_ptr", "row_desc", "codes_o", "sd_o", "col_o", "codes4_o", "scales_f32"):
             if getattr(self, name) is not None:
                 setattr(c, name, getattr(self, name).clone())
         c._scheds = {k: v.clone() for k, v in self._scheds.items()}

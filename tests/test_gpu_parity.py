@@ -482,8 +482,62 @@ def test_mortar_gemv_reference_signature(dev):
     assert h.dtype == torch.float32
     ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
     assert_close_bf16(h.cpu().numpy(), ref["h"], "h", ulps=4)
-    with pytest.raises(NotImplementedError):
-        mortar_amd.mortar_gemv(torch.from_numpy(x).to(dev), pk, swiglu_x=True)
+    hb = mortar_amd.mortar_gemv(to_dev(x, dev), pk, swiglu_out=True)                   # bf16 in -> bf16 out
+    assert hb.dtype == torch.bfloat16
+    assert_close_bf16(to_np(hb), ref["h"], "h bf16", ulps=4)
+
+
+def _gemv_f32_tolerance(ref):
+    """fp32 sums of a few hundred exact products against float64: a few 1e-7 of the largest output (measured 2e-7)."""
+    return 3e-6 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("B", [1, 5, 16, 40])
+@pytest.mark.parametrize("per_tensor", [False, True])
+def test_mortar_gemv_fp32_arithmetic(dev, B, per_tensor):
+    """mortar_gemv with fp32 activations against the oracle's decode form (exact +-x / 0 products, fp32 scale after the
+    block sum, float64 sums): gate_up with SwiGLU (+ gates, row flags), then down, plain and with swiglu_x, with column
+    flags and with rows split into partial slots."""
+    d_model, d_ff, ncl = 512, 16 * 88, 22
+    spec = synth.synth_mlp(d_model, d_ff, 0.25, seed=95, zipf_s=1.2)
+    if per_tensor:
+        spec["gate_up"]["scales"] = spec["gate_up"]["scales"][:1] * 1.2345          # fp32 values that bf16 cannot hold
+        spec["down"]["scales"] = spec["down"]["scales"][:1] * 0.987
+    gu_m, dn_m = spec["gate_up"], spec["down"]
+    assert not np.array_equal(O.bf16_round(gu_m["scales"]), gu_m["scales"])
+    Wgu, Wdn = synth.to_pack(gu_m, dev), synth.to_pack(dn_m, dev)
+    rng = np.random.default_rng(96 + B)
+    x = rng.standard_normal((B, d_model)).astype(np.float32) * np.float32(1.37)          # full fp32 mantissas
+    xt = torch.from_numpy(x).to(dev)
+    gu = O.mortar_gemv(x, gu_m["codes"], gu_m["scales"], gu_m["col_idx"], gu_m["offsets"]).astype(np.float64)
+    got_gu = ops.gemv_f32(xt, Wgu).cpu().numpy()
+    assert np.abs(got_gu - gu).max() <= _gemv_f32_tolerance(gu)
+    assert np.abs(ops.gemv_f32(xt, Wgu, max_blocks=3).cpu().numpy() - gu).max() <= _gemv_f32_tolerance(gu)   # partial slots
+    # exactness beyond bf16: a bf16-rounded input gives a visibly different answer
+    gu_b = O.mortar_gemv(O.bf16_round(x), gu_m["codes"], gu_m["scales"], gu_m["col_idx"], gu_m["offsets"])
+    assert np.abs(gu_b - gu).max() > 100 * _gemv_f32_tolerance(gu)
+    g, u = gu[:, :d_ff], gu[:, d_ff:]
+    h_ref = g / (1.0 + np.exp(-g)) * u
+    h = ops.gemv_f32(xt, Wgu, swiglu_out=True)
+    assert h.dtype == torch.float32 and np.abs(h.cpu().numpy() - h_ref).max() <= _gemv_f32_tolerance(h_ref)
+    # gates + row flags (route_flags): gated SwiGLU, inactive clusters exactly zero
+    lg = torch.from_numpy(synth.synth_logits(B, ncl, 97)).to(dev)
+    gates, active = ops.remoe_gates(lg, 6)
+    ract, cact = ops.route_flags(gates, d_ff)
+    hg_ref = (h_ref.reshape(B, ncl, -1) * gates.cpu().numpy().astype(np.float64)[:, :, None]).reshape(B, d_ff)
+    hg = mortar_amd.mortar_gemv(xt, Wgu, swiglu_out=True, row_act=ract, gates=gates, cluster_size=d_ff // ncl)
+    assert np.abs(hg.cpu().numpy() - hg_ref).max() <= _gemv_f32_tolerance(h_ref)
+    off = np.repeat(~active.cpu().numpy().astype(bool), d_ff // ncl, axis=1)
+    assert (hg.cpu().numpy()[off] == 0).all()
+    # down: plain on h, with column flags on the gated h, and in the swiglu_x form on the raw gate_up output
+    y_ref = O.mortar_gemv(h.cpu().numpy(), dn_m["codes"], dn_m["scales"], dn_m["col_idx"], dn_m["offsets"]).astype(np.float64)
+    y = mortar_amd.mortar_gemv(h, Wdn)
+    assert np.abs(y.cpu().numpy() - y_ref).max() <= _gemv_f32_tolerance(y_ref)
+    yg_ref = O.mortar_gemv(hg.cpu().numpy(), dn_m["codes"], dn_m["scales"], dn_m["col_idx"], dn_m["offsets"])
+    yg = mortar_amd.mortar_gemv(hg, Wdn, col_act=cact)
+    assert np.abs(yg.cpu().numpy() - yg_ref).max() <= _gemv_f32_tolerance(yg_ref)
+    y2 = mortar_amd.mortar_gemv(torch.from_numpy(got_gu).to(dev), Wdn, swiglu_x=True)
+    assert np.abs(y2.cpu().numpy() - y_ref).max() <= 4 * _gemv_f32_tolerance(y_ref)
 
 
 @pytest.mark.parametrize("B,n,f32", [(1, 4, True), (3, 4, False), (16, 2, True), (40, 4, False), (5, 1, True), (7, 3, False)])
