@@ -229,7 +229,9 @@ int mortar_route_flags(const float *gates, int64_t B, int32_t n_clusters, int64_
  * (projection GEMV + one tail kernel, B == 1).
  *   qv = x Wq^T + iter_vec;  q = LayerNorm(qv; ln_w, ln_b, ln_eps);  sa = q[:d/2] Ka^T;  sb = q[d/2:] Kb^T
  *   logits[g] = sa[p / nsk] + sb[p % nsk] + bias[g],  p = g mod nsk^2   (nsk^2 == n: the 1:1 product map of
- *   fused_router.py; nsk^2 < n: the reference's wrap, routing.py:227-230; nsk^2 > n is refused: MORTAR_ERR_LIMIT)
+ *   fused_router.py; nsk^2 < n: the reference's wrap, routing.py:227-230)
+ *   nsk^2 > n: logits[g] = (g-th largest of the nsk^2 product scores) + bias[g], the reference's
+ *   topk(product_scores, n).values (routing.py:212-222; e.g. 352 groups under 19 x 19 keys); nsk^2 <= 2048
  *   gates / active as mortar_remoe_gates.
  * x: [B, d] bf16 (x_is_f32 = 0) or fp32 (1), row stride ldx; wq fp32 [d, d] row-major (query_proj.weight);
  * iter_vec fp32 [d] (iter_embed[it]) or NULL; ln_w, ln_b fp32 [d]; ka, kb fp32 [nsk, d/2]; bias fp32 [n].

@@ -147,7 +147,8 @@ __device__ __forceinline__ float block_sum256(float v, float *red) {      // red
 }
 
 // Launch 2, one workgroup per token: LayerNorm(qv) -> sub-key scores of the two query halves -> product-key logits
-// (+ group bias) -> gating tail.  P = nsk * nsk products map to the n groups one to one (P == n) or wrap (P < n).
+// (+ group bias) -> gating tail.  P = nsk * nsk products map to the n groups one to one (P == n), wrap (P < n), or are
+// ranked and the n largest kept (P > n).
 // PRE (d <= 2048, nsk <= 4): every parameter a thread needs (LayerNorm weights, its slices of the sub-keys, its
 // bias) is fetched into registers before the first reduction, so the kernel pays one memory round trip instead of
 // one per phase.
@@ -156,7 +157,7 @@ __global__ void __launch_bounds__(256) router_tail_kernel(const float *qv, int d
                                                            float ln_eps, const float *ka, const float *kb, int nsk,
                                                            const float *bias, int n, int k, float *logits_out,
                                                            float *gates, uint8_t *active) {
-    extern __shared__ __attribute__((aligned(16))) float sm[];       // qn[d] | s[2 * nsk] | logits[n] | red[4]
+    extern __shared__ __attribute__((aligned(16))) float sm[];       // qn[d] | s[2 * nsk] | logits[n] | red[4] | sort keys
     float *qn = sm, *sc = sm + d, *lg = sc + 2 * nsk, *red = lg + n;
     const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const float *q = qv + (int64_t)b * d;
@@ -238,11 +239,46 @@ __global__ void __launch_bounds__(256) router_tail_kernel(const float *qv, int d
     }
     __syncthreads();
     const int P = nsk * nsk;
-    for (int g = tid; g < n; g += 256) {
-        const int pr = g % P;
-        const float l = (sc[pr / nsk] + sc[nsk + pr % nsk]) + bias[g];
-        lg[g] = l;
-        if (logits_out) logits_out[(int64_t)b * n + g] = l;
+    if (P > n) {
+        // more product keys than groups: the group logits are the n largest product scores in descending order
+        // (torch.topk(product_scores, n).values, morph/model/routing.py:212-222).  Bitonic sort of order-preserving
+        // integer keys (NaN ranks above +inf, as torch.topk has it), padded with the smallest key.
+        uint32_t *sk = reinterpret_cast<uint32_t *>(red + 4);
+        int P2 = 1;
+        while (P2 < P) P2 <<= 1;
+        for (int i = tid; i < P2; i += 256) {
+            uint32_t key = 0u;
+            if (i < P) {
+                const uint32_t u = __float_as_uint(sc[i / nsk] + sc[nsk + i % nsk]);
+                key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+            }
+            sk[i] = key;
+        }
+        __syncthreads();
+        for (int k2 = 2; k2 <= P2; k2 <<= 1) {
+            for (int j = k2 >> 1; j > 0; j >>= 1) {
+                for (int t = tid; t < P2 / 2; t += 256) {
+                    const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1)), l = i | j;
+                    const uint32_t a = sk[i], c = sk[l];
+                    const bool desc = (i & k2) == 0;
+                    if (desc ? a < c : a > c) { sk[i] = c; sk[l] = a; }
+                }
+                __syncthreads();
+            }
+        }
+        for (int g = tid; g < n; g += 256) {
+            const uint32_t key = sk[g];
+            const float l = __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key) + bias[g];
+            lg[g] = l;
+            if (logits_out) logits_out[(int64_t)b * n + g] = l;
+        }
+    } else {
+        for (int g = tid; g < n; g += 256) {
+            const int pr = g % P;
+            const float l = (sc[pr / nsk] + sc[nsk + pr % nsk]) + bias[g];
+            lg[g] = l;
+            if (logits_out) logits_out[(int64_t)b * n + g] = l;
+        }
     }
     __syncthreads();
     if (wave == 0)
@@ -376,9 +412,8 @@ extern "C" int mortar_router_bf16(const void *x, int32_t x_is_f32, int64_t B, in
         return mortar_fail(MORTAR_ERR_ARG, "router: x, wq, ka and kb must be 16-byte aligned");
     if (n <= 0 || k <= 0 || nsk <= 0) return mortar_fail(MORTAR_ERR_ARG, "router: n, k, nsk must be positive");
     if (n > 64 * MAXPL_LIMIT) return mortar_fail(MORTAR_ERR_LIMIT, "router: n=%d exceeds %d clusters", n, 64 * MAXPL_LIMIT);
-    if ((int64_t)nsk * nsk > n)
-        return mortar_fail(MORTAR_ERR_LIMIT, "router: %d x %d product keys exceed the %d groups (the reference ranks the "
-                           "products with topk there; not served by the fused front end)", nsk, nsk, n);
+    if ((int64_t)nsk * nsk > 2048)
+        return mortar_fail(MORTAR_ERR_LIMIT, "router: %d x %d product keys exceed the 2048 the fused front end ranks", nsk, nsk);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 pg((unsigned)((d + 3) / 4)), blk(256);
 #define MORTAR_PROJ(TB, F) hipLaunchKernelGGL((router_project_kernel<TB, F>), pg, blk, 0, st, x, (int)B, d, ldx, wq, iter_vec, qv)
@@ -387,7 +422,9 @@ extern "C" int mortar_router_bf16(const void *x, int32_t x_is_f32, int64_t B, in
 #undef MORTAR_PROJ
     int rc = check_launch("router projection");
     if (rc) return rc;
-    const size_t smem = (size_t)(d + 2 * nsk + n + 4) * sizeof(float);
+    size_t sort_keys = 0;                          // nsk^2 > n: room for the product scores, padded to a power of two
+    if ((int64_t)nsk * nsk > n) { sort_keys = 1; while (sort_keys < (size_t)nsk * nsk) sort_keys <<= 1; }
+    const size_t smem = (size_t)(d + 2 * nsk + n + 4 + sort_keys) * sizeof(float);
     const dim3 tg((unsigned)B);
     const int npl = (n + 63) / 64;
     const bool pre = d <= 2048 && nsk <= 4;

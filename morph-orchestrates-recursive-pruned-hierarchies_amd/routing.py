@@ -68,7 +68,7 @@ class TileRouter(nn.Module):
         """Decode-sized inference calls on the GPU with fp32 router parameters go through the two-launch HIP router."""
         return (x_flat.is_cuda and 0 < x_flat.shape[0] <= ops.ROUTER_MAX_TOKENS and not torch.is_grad_enabled()
                 and x_flat.dtype in (torch.bfloat16, torch.float32) and self.query_proj.weight.dtype == torch.float32
-                and self.n_sub_keys * self.n_sub_keys <= self.n_tile_groups and self.d_model % 8 == 0
+                and self.n_sub_keys * self.n_sub_keys <= 2048 and self.d_model % 8 == 0
                 and self.n_tile_groups <= 1024)
 
     @torch.no_grad()

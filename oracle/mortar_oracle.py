@@ -316,7 +316,7 @@ def router_logits(x, wq, iter_vec, ln_w, ln_b, ln_eps, ka, kb, bias) -> np.ndarr
     """TileRouter.forward steps 1-4, morph/model/routing.py:181-230 (float64 here): q = LayerNorm(x Wq^T + iter_vec);
     sa = q[:, :d/2] Ka^T, sb = q[:, d/2:] Kb^T; product scores ps[a*nsk + b] = sa[a] + sb[b]; group logits = ps + bias
     when nsk^2 == n (:205-211), ps[g mod nsk^2] + bias when nsk^2 < n (:227-230).  LayerNorm uses the biased variance
-    (torch.nn.LayerNorm).  The nsk^2 > n branch (topk over products, :212-222) is not restated."""
+    (torch.nn.LayerNorm); with nsk^2 > n the group logits are the n largest product scores, descending (:212-222)."""
     x = np.asarray(x, np.float64)
     qv = x @ np.asarray(wq, np.float64).T
     if iter_vec is not None:
@@ -330,7 +330,8 @@ def router_logits(x, wq, iter_vec, ln_w, ln_b, ln_eps, ka, kb, bias) -> np.ndarr
     nsk = sa.shape[1]
     ps = (sa[:, :, None] + sb[:, None, :]).reshape(x.shape[0], nsk * nsk)
     n = np.asarray(bias).size
-    assert nsk * nsk <= n
+    if nsk * nsk > n:          # :212-222: the n largest product scores in descending order (torch.topk(...).values)
+        return np.sort(ps, axis=1)[:, ::-1][:, :n] + np.asarray(bias, np.float64)
     return ps[:, np.arange(n) % (nsk * nsk)] + np.asarray(bias, np.float64)
 
 

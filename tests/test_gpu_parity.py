@@ -288,7 +288,8 @@ def test_remoe_gates_ties_and_edges(dev):
 
 
 @pytest.mark.parametrize("B,d,nsk,n,xdt", [(1, 256, 4, 16, "bf16"), (5, 768, 4, 16, "bf16"), (16, 2048, 8, 64, "bf16"),
-                                          (3, 2048, 18, 352, "f32"), (64, 512, 4, 16, "f32"), (2, 264, 3, 9, "bf16")])
+                                          (3, 2048, 18, 352, "f32"), (64, 512, 4, 16, "f32"), (2, 264, 3, 9, "bf16"),
+                                          (2, 2048, 19, 352, "bf16"), (5, 256, 5, 20, "f32"), (1, 512, 33, 1024, "f32")])
 def test_fused_router_front_end(dev, B, d, nsk, n, xdt):
     """Two-launch decode router (projection; LayerNorm + product keys + gating tail) against the float64 oracle:
     logits to fp32 rounding, the active set exactly except where a logit sits within rounding of the threshold,
@@ -333,7 +334,7 @@ def test_fused_router_limits(dev):
     with pytest.raises(ValueError, match="1..64 tokens"):
         ops.router_fused(x, T(64, 64), None, T(64), T(64), 1e-5, T(4, 32), T(4, 32), T(16), 4)
     with pytest.raises(ValueError, match="product keys exceed"):
-        ops.router_fused(x[:2], T(64, 64), None, T(64), T(64), 1e-5, T(5, 32), T(5, 32), T(16), 4)
+        ops.router_fused(x[:2], T(64, 64), None, T(64), T(64), 1e-5, T(46, 32), T(46, 32), T(16), 4)
 
 
 def test_route_flags_exact(dev):

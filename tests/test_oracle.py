@@ -276,7 +276,7 @@ def test_router_logits_against_library_routines():
     reference's broadcast-add / wrap indexing (routing.py:205-230) written with torch indexing."""
     import torch
     rng = np.random.default_rng(52)
-    for d, nsk, n in ((64, 4, 16), (48, 3, 20), (32, 2, 4)):
+    for d, nsk, n in ((64, 4, 16), (48, 3, 20), (32, 2, 4), (64, 5, 20), (32, 19, 352)):
         x = rng.standard_normal((5, d)); wq = rng.standard_normal((d, d)) / np.sqrt(d); it = rng.standard_normal(d) * 0.1
         lw = 1 + 0.1 * rng.standard_normal(d); lb = 0.1 * rng.standard_normal(d)
         ka = rng.standard_normal((nsk, d // 2)); kb = rng.standard_normal((nsk, d // 2)); bias = rng.standard_normal(n)
@@ -285,7 +285,11 @@ def test_router_logits_against_library_routines():
         q = torch.nn.functional.layer_norm(torch.nn.functional.linear(t(x), t(wq)) + t(it), (d,), t(lw), t(lb), 1e-5)
         sa, sb = q[:, :d // 2] @ t(ka).T, q[:, d // 2:] @ t(kb).T
         ps = (sa.unsqueeze(2) + sb.unsqueeze(1)).reshape(5, nsk * nsk)
-        want = ps[:, torch.arange(n) % (nsk * nsk)] + t(bias).unsqueeze(0)
+        if nsk * nsk > n:                    # routing.py:212-222: topk over the products, values in descending order
+            want = ps.topk(n, dim=-1).values + t(bias).unsqueeze(0)
+            assert (np.diff(got - bias, axis=1) <= 0).all()
+        else:
+            want = ps[:, torch.arange(n) % (nsk * nsk)] + t(bias).unsqueeze(0)
         np.testing.assert_allclose(got, want.numpy(), rtol=1e-12, atol=1e-12)
         assert np.allclose(O.router_logits(x, wq, None, lw, lb, 1e-5, ka, kb, bias),
                            O.router_logits(x, wq, np.zeros(d), lw, lb, 1e-5, ka, kb, bias))
