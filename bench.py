@@ -317,8 +317,16 @@ def main() -> None:
             ops.spmm(h, Wdn, active=active, out=y)
         t = event_time_ms(routed, it)
         n_act = int(ops.remoe_gates(logits, TOP_K)[1].sum())
-        out["routed_prefill"] = {"ms": t, "tokens_per_s": TOKENS / (t * 1e-3),
-                                 "active_fraction": n_act / (TOKENS * N_CLUSTERS)}
+        act_frac = n_act / (TOKENS * N_CLUSTERS)
+        fl_active = (flops_gu + flops_dn) * act_frac          # products whose hidden cluster is active for the token
+        out["routed_prefill"] = {"ms": t, "tokens_per_s": TOKENS / (t * 1e-3), "active_fraction": act_frac,
+                                 "vs_unrouted": t / ms,
+                                 "roofline": {"bound": "mfma", "kernel": "remoe_gates + remoe_route + routed gate_up + masked down",
+                                              "achieved": fl_active / (t * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                              "frac": fl_active / (t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
+                                              "note": "FLOPs of active (token, cluster) pairs only; a cluster is one 16-neuron row unit, "
+                                                      "so a 32-token tile keeps about 8 active tokens per unit and the weight unpack, "
+                                                      "which bounds the kernel, is not reduced"}}
         # ---- the reference's own deploy format: ONE scale per matrix (pack_mortar_ternary), same shapes ----------
         spec_u = {k: dict(spec[k]) for k in ("gate_up", "down")}
         spec_u["gate_up"]["scales"], spec_u["down"]["scales"] = np.float32(0.05), np.float32(0.03)
