@@ -141,13 +141,17 @@ class MortarPack:
     ``scale_after_sum`` is on, the kernels scale the fp32 sums once instead of every block's weights
     (``uniform_scale``; about a third fewer vector instructions per block pair).
 
+    ``seg_cb`` sets the width of the stream's K segments in block-columns (default: the widest whose 32-token
+    activation tile fits LDS, ``mortar_prefill_max_seg_cb()``).
+
     ``packed=None`` builds the topology with all-zero blocks, to be filled on the device by ``requantize`` from
     block values (the reference's ``mortar_data``): the device-side pack used for QAT forwards and for the W^T
     pack of the dX product (``transposed()``).
     """
 
     def __init__(self, packed, scale, col, offsets, out_features: int, in_features: int, device,
-                 prefill_stream: bool = True, scale_after_sum: bool = True, allow_empty_rows: bool = False):
+                 prefill_stream: bool = True, scale_after_sum: bool = True, allow_empty_rows: bool = False,
+                 seg_cb: int | None = None):
         if out_features % BLK or in_features % BLK:
             raise ValueError(f"[{out_features},{in_features}] not divisible by blocking {BLK}")
         self.out_features, self.in_features = int(out_features), int(in_features)
@@ -181,8 +185,14 @@ class MortarPack:
         self.col = torch.from_numpy(self.h_col).to(dev)
         self.row_ptr = torch.from_numpy(self.h_offsets).to(dev)
         max_seg = int(_lib.lib().mortar_prefill_max_seg_cb())
-        nseg = -(-self.Cb // max_seg)
-        self.seg_cb = -(-self.Cb // nseg)
+        if seg_cb is not None:
+            if not 0 < seg_cb <= max_seg:
+                raise ValueError(f"seg_cb={seg_cb} outside 1..{max_seg}")
+            nseg = -(-self.Cb // seg_cb)
+            self.seg_cb = int(seg_cb)
+        else:
+            nseg = -(-self.Cb // max_seg)
+            self.seg_cb = -(-self.Cb // nseg)
         grp, codes_o, sd_o, col_o = octet_layout(self.h_offsets, self.Rb, self.Cb, self.seg_cb, codes, sdup, self.h_col)
         self.nseg = nseg
         self.h_row_desc = grp
