@@ -393,6 +393,9 @@ int mortar_swiglu_backward_bf16(const uint16_t *gu, int64_t ldg, const uint16_t 
  *   mortar_sdd_plan_host: the work partition for a topology (host, once).  plan_out = NULL returns the number of
  *     int32 words needed; otherwise fills plan_out (plan_words = its capacity) and returns the words used;
  *     plan_out[0] = n_wg.  Upload the plan to the device.
+ *   mortar_sdd_plan_max_groups_host: the largest number of row groups in one K segment of a (host) plan, the
+ *     max_groups argument of the launch (it sizes the grid: workgroup ids are laid out per XCD as (token range, row
+ *     group) x K segment so that the readers of one slice share an L2).
  *   mortar_sdd_bf16: plan device int32; a bf16 [M, lda >= Rb*16], b bf16 [M, ldb >= Cb*16], 16-byte aligned with
  *     leading dimensions multiples of 8; acc device workspace of mortar_sdd_workspace_bytes(n_wg, nnz, M) bytes,
  *     16-byte aligned (every token range writes its fp32 sums to a slab of its own, and a last pass adds the slabs in
@@ -400,8 +403,10 @@ int mortar_swiglu_backward_bf16(const uint16_t *gu, int64_t ldg, const uint16_t 
 int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb, int32_t *plan_out,
                              int64_t plan_words);
 int64_t mortar_sdd_workspace_bytes(int32_t n_wg, int32_t nnz, int64_t M);
-int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t Rb, int32_t Cb, int32_t nnz, const uint16_t *a,
-                    int64_t lda, const uint16_t *b, int64_t ldb, int64_t M, float *acc, uint16_t *out, void *stream);
+int32_t mortar_sdd_plan_max_groups_host(const int32_t *plan);
+int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t max_groups, int32_t Rb, int32_t Cb, int32_t nnz,
+                    const uint16_t *a, int64_t lda, const uint16_t *b, int64_t ldb, int64_t M, float *acc, uint16_t *out,
+                    void *stream);
 
 #ifdef __cplusplus
 }

@@ -11,10 +11,11 @@
 // features and each lane gets 4 tokens of one feature.  A workgroup keeps the fp32 tiles of up to WAVES*NB blocks of
 // a few consecutive block-rows in registers and walks the tokens in steps of 32; per step it stages the
 // 32 x (columns of its K segment) slice of b once and the slice of a for its rows, into one of two buffers: the
-// loads of the next step are in flight while the current one multiplies.  Workgroups that share a token range run on the same XCD (the range index
-// is the low part of the workgroup index), so a slice of b is fetched from HBM about once per XCD and served from
-// L2 after that.  Every token range writes its fp32 sums to its own slab of the workspace; a last pass adds the
-// slabs in a fixed order and rounds to bf16, so results are reproducible.
+// loads of the next step are in flight while the current one multiplies.  Workgroup ids are laid out per XCD (each
+// has its own L2) as runs of (token range, row group) pairs with the K segments of a pair side by side, so that a
+// slice of a is fetched from HBM once and a slice of b only by the XCDs that hold its token range.  Every token range
+// writes its fp32 sums to its own slab of the workspace; a last pass adds the slabs in a fixed order and rounds to
+// bf16, so results are reproducible.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -52,7 +53,7 @@ struct SddArgs {
     int64_t lda, ldb, M;
     float *acc;
     uint16_t *out;
-    int32_t Cb, tsplit, steps_per_split, nsteps, nnz;
+    int32_t Cb, tsplit, steps_per_split, nsteps, nnz, max_groups, pairs_per_xcd;
 };
 
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
@@ -91,8 +92,20 @@ __global__ __launch_bounds__(SDD_WAVES * 64) void sdd_kernel(SddArgs p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int ts = blockIdx.x % p.tsplit, wg = blockIdx.x / p.tsplit;
-    const int n_wg = p.plan[0];
+    // Workgroup -> (row group, K segment, token range).  Ids are dealt round-robin over the 8 XCDs, each with its own
+    // L2.  The (token range, row group) pairs are cut into 8 consecutive runs, one per XCD, and the K segments of a pair
+    // sit side by side: the slice of a is then fetched from HBM once (its nseg readers share an L2) and a slice of b
+    // only by the few XCDs that hold its token range.  Combinations that do not exist (a segment with fewer row groups)
+    // are idle ids.
+    const int n_wg = p.plan[0], nseg = p.plan[2];
+    const int32_t *seg_tab = p.plan + p.plan[3];                   // per segment: first workgroup, row groups
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int pl = slot / nseg, sgi = slot - pl * nseg;
+    const int pair = xcd * p.pairs_per_xcd + pl;
+    if (pl >= p.pairs_per_xcd || pair >= p.tsplit * p.max_groups) return;
+    const int ts = pair / p.max_groups, rg = pair - ts * p.max_groups;
+    if (rg >= seg_tab[2 * sgi + 1]) return;
+    const int wg = seg_tab[2 * sgi] + rg;
     const int32_t *desc = p.plan + 4 + wg * 4;
     const int row0 = desc[0], nrows = desc[1], seg = desc[2];
     const int seg_cb = p.plan[1];
@@ -211,9 +224,10 @@ __global__ __launch_bounds__(256) void sdd_round_kernel(const float *acc, uint16
 
 }  // namespace
 
-// Plan: {n_wg, seg_cb, nseg, 0}, then per workgroup {first row, rows, segment, blocks}, then per (workgroup, wavefront,
+// Plan: {n_wg, seg_cb, nseg, offset of the segment table}, then per workgroup {first row, rows, segment, blocks}, then per (workgroup, wavefront,
 // slot) the block index or -1, then per (workgroup, wavefront, slot) (row - first row) << 20 | LDS byte offset of the
-// tile of (column - segment start); an empty slot repeats the workgroup's last block there.
+// tile of (column - segment start); an empty slot repeats the workgroup's last block there; last the segment table:
+// per segment {its first workgroup, its number of row groups} (workgroups are stored segment by segment).
 extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
                                         int32_t *plan_out, int64_t plan_words) {
     const int rc = mortar_check_bcsr_host(row_ptr, col, Rb, Cb);
@@ -247,11 +261,18 @@ extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *c
         flush();
     }
     const int64_t n_wg = (int64_t)wgs.size();
-    const int64_t words = 4 + n_wg * 4 + n_wg * SDD_G * 2;
+    const int64_t tab = 4 + n_wg * 4 + n_wg * SDD_G * 2;          // word offset of the per-segment table
+    const int64_t words = tab + 2 * nseg;
+    if (tab > INT32_MAX) return mortar_fail(MORTAR_ERR_LIMIT, "sdd_plan: plan too large");
     if (!plan_out) return words;
     if (plan_words < words) return mortar_fail(MORTAR_ERR_ARG, "sdd_plan: buffer holds %lld words, need %lld",
                                                (long long)plan_words, (long long)words);
-    plan_out[0] = (int32_t)n_wg; plan_out[1] = seg_cb; plan_out[2] = nseg; plan_out[3] = 0;
+    plan_out[0] = (int32_t)n_wg; plan_out[1] = seg_cb; plan_out[2] = nseg; plan_out[3] = (int32_t)tab;
+    {   // workgroups are stored segment by segment: first workgroup and number of row groups of every segment
+        int32_t *st = plan_out + tab;
+        for (int sg = 0; sg < nseg; ++sg) { st[2 * sg] = 0; st[2 * sg + 1] = 0; }
+        for (int64_t w = n_wg - 1; w >= 0; --w) { st[2 * wgs[w].seg] = (int32_t)w; st[2 * wgs[w].seg + 1] += 1; }
+    }
     int32_t *ent_j = plan_out + 4 + n_wg * 4, *ent_o = ent_j + n_wg * SDD_G;
     for (int64_t w = 0; w < n_wg; ++w) {
         int32_t *d = plan_out + 4 + w * 4;
@@ -263,6 +284,13 @@ extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *c
         }
     }
     return words;
+}
+
+extern "C" int32_t mortar_sdd_plan_max_groups_host(const int32_t *plan) {
+    if (!plan || plan[0] <= 0 || plan[2] <= 0 || plan[3] <= 0) return mortar_fail(MORTAR_ERR_ARG, "sdd_plan_max_groups: not a plan");
+    int32_t mx = 0;
+    for (int sg = 0; sg < plan[2]; ++sg) mx = std::max(mx, plan[plan[3] + 2 * sg + 1]);
+    return mx;
 }
 
 // Token ranges for M tokens over n_wg row groups.  One workgroup runs per CU, so the launch takes
@@ -288,11 +316,12 @@ extern "C" int64_t mortar_sdd_workspace_bytes(int32_t n_wg, int32_t nnz, int64_t
     return (int64_t)tsplit * nnz * 256 * (int64_t)sizeof(float);
 }
 
-extern "C" int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t Rb, int32_t Cb, int32_t nnz,
+extern "C" int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t max_groups, int32_t Rb, int32_t Cb, int32_t nnz,
                                const uint16_t *a, int64_t lda, const uint16_t *b, int64_t ldb, int64_t M,
                                float *acc, uint16_t *out, void *stream) {
     if (!plan || !out || !acc || (M > 0 && (!a || !b))) return mortar_fail(MORTAR_ERR_ARG, "sdd: null pointer");
     if (n_wg <= 0 || Rb <= 0 || Cb <= 0 || nnz <= 0 || M < 0) return mortar_fail(MORTAR_ERR_ARG, "sdd: bad shape");
+    if (max_groups <= 0 || max_groups > n_wg) return mortar_fail(MORTAR_ERR_ARG, "sdd: max_groups=%d outside 1..n_wg", max_groups);
     if (reinterpret_cast<uintptr_t>(out) & 15) return mortar_fail(MORTAR_ERR_ARG, "sdd: out must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (M == 0) {                                          // no tokens: the gradient is zero
@@ -317,7 +346,10 @@ extern "C" int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t Rb, in
         if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
         configured = true;
     }
-    hipLaunchKernelGGL(sdd_kernel, dim3((unsigned)(n_wg * p.tsplit)), dim3(SDD_WAVES * 64), smem, st, p);
+    const int nseg = (Cb + SDD_SEG - 1) / SDD_SEG;
+    p.max_groups = max_groups;
+    p.pairs_per_xcd = (p.tsplit * max_groups + 7) / 8;
+    hipLaunchKernelGGL(sdd_kernel, dim3((unsigned)(8 * p.pairs_per_xcd * nseg)), dim3(SDD_WAVES * 64), smem, st, p);
     if (p.tsplit > 1)
         hipLaunchKernelGGL(sdd_round_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st, acc, out, n4, p.tsplit);
     const hipError_t e = hipGetLastError();

@@ -261,14 +261,14 @@ def sdd(a: Tensor, b: Tensor, W: MortarPack, out: Tensor | None = None) -> Tenso
         a = a.contiguous()
     if b.stride(0) % 8 or b.data_ptr() % 16:
         b = b.contiguous()
-    plan, n_wg = W.sdd_plan()
+    plan, n_wg, max_groups = W.sdd_plan()
     if out is None:
         out = torch.empty((W.nnz, BLK, BLK), dtype=torch.bfloat16, device=a.device)
     elif out.dtype != torch.bfloat16 or tuple(out.shape) != (W.nnz, BLK, BLK) or not out.is_contiguous():
         raise TypeError("sdd: out must be a contiguous bfloat16 [nnz, 16, 16] tensor")
     ws = _lib.check(_lib.lib().mortar_sdd_workspace_bytes(n_wg, W.nnz, a.shape[0]), "mortar_sdd_workspace_bytes")
     acc = torch.empty(ws // 4, dtype=torch.float32, device=a.device)
-    _lib.check(_lib.lib().mortar_sdd_bf16(_p(plan), n_wg, W.Rb, W.Cb, W.nnz, _p(a), a.stride(0), _p(b), b.stride(0),
+    _lib.check(_lib.lib().mortar_sdd_bf16(_p(plan), n_wg, max_groups, W.Rb, W.Cb, W.nnz, _p(a), a.stride(0), _p(b), b.stride(0),
                                           a.shape[0], _p(acc), _p(out), _stream(a)), "mortar_sdd_bf16")
     return out
 

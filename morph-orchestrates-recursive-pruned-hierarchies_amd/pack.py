@@ -326,8 +326,9 @@ class MortarPack:
             self._transposed = t
         return self._transposed
 
-    def sdd_plan(self) -> tuple[torch.Tensor, int]:
-        """(device plan, workgroups) of the weight-gradient kernel for this topology: see mortar_sdd_plan_host."""
+    def sdd_plan(self) -> tuple[torch.Tensor, int, int]:
+        """(device plan, workgroups, largest number of row groups in a K segment) of the weight-gradient kernel for this
+        topology: see mortar_sdd_plan_host."""
         if self._sdd is None:
             L = _lib.lib()
             n = _lib.check(L.mortar_sdd_plan_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, None, 0),
@@ -335,8 +336,9 @@ class MortarPack:
             plan = np.empty(n, dtype=np.int32)
             _lib.check(L.mortar_sdd_plan_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, _vp(plan), n),
                        "mortar_sdd_plan_host")
-            self._sdd = (torch.from_numpy(plan).to(self.device), int(plan[0]), plan)
-        return self._sdd[0], self._sdd[1]
+            mg = _lib.check(L.mortar_sdd_plan_max_groups_host(_vp(plan)), "mortar_sdd_plan_max_groups_host")
+            self._sdd = (torch.from_numpy(plan).to(self.device), int(plan[0]), plan, int(mg))
+        return self._sdd[0], self._sdd[1], self._sdd[3]
 
     def sched(self, rows_per_unit: int) -> torch.Tensor:
         """Device schedule (mortar_schedule_host over the balanced unit order) for plain (1) or gate/up (2) units."""

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in mortar_hip.h but not exported"
     assert declared == set(_lib.EXPORTS)
-    assert _lib.lib().mortar_abi_version() == 5
+    assert _lib.lib().mortar_abi_version() == 6
 
 
 def test_encode_round_trip_and_bit_layout():
@@ -354,11 +354,18 @@ def test_sdd_plan_partitions_the_blocks():
         plan = np.empty(n, np.int32)
         assert L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, vp(plan), n) == n
         assert L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, vp(plan), n - 1) < 0
-        n_wg, seg_cb, nseg = plan[0], plan[1], plan[2]
-        G = (n - 4 - 4 * n_wg) // (2 * n_wg)
+        n_wg, seg_cb, nseg, tab = plan[0], plan[1], plan[2], plan[3]
+        assert tab + 2 * nseg == n
+        G = (tab - 4 - 4 * n_wg) // (2 * n_wg)
         desc = plan[4:4 + 4 * n_wg].reshape(n_wg, 4)
         ej = plan[4 + 4 * n_wg:4 + 4 * n_wg + n_wg * G].reshape(n_wg, G)
-        eo = plan[4 + 4 * n_wg + n_wg * G:].reshape(n_wg, G)
+        eo = plan[4 + 4 * n_wg + n_wg * G:tab].reshape(n_wg, G)
+        # segment table: workgroups are stored segment by segment; {first workgroup, row groups} per segment
+        st = plan[tab:].reshape(nseg, 2)
+        for sg in range(nseg):
+            ws = np.nonzero(desc[:, 2] == sg)[0]
+            assert st[sg, 1] == ws.size and (ws.size == 0 or (st[sg, 0] == ws[0] and np.array_equal(ws, np.arange(ws[0], ws[0] + ws.size))))
+        assert L.mortar_sdd_plan_max_groups_host(vp(plan)) == st[:, 1].max()
         assert nseg >= -(-Cb // seg_cb) and seg_cb <= 44 and seg_cb % 4 == 0
         seen = ej[ej >= 0]
         assert sorted(seen.tolist()) == list(range(col.size))
