@@ -19,6 +19,12 @@ int check_common(const mortar_bcsr_t *W, const uint16_t *x, int64_t M, int64_t l
     if (W->Rb <= 0 || W->Cb <= 0 || W->nnz <= 0) return mortar_fail(MORTAR_ERR_ARG, "spmm: empty matrix");
     if (W->seg_cb <= 0 || tile_bytes(32, W->seg_cb < W->Cb ? W->seg_cb : W->Cb) > LDS_BUDGET)
         return mortar_fail(MORTAR_ERR_ARG, "spmm: seg_cb=%d does not fit LDS (max %d)", W->seg_cb, mortar_prefill_max_seg_cb());
+    {   // the kernels address the octet stream with 32-bit byte offsets (1 KiB of 4-bit codes per octet)
+        const int64_t nseg = (W->Cb + W->seg_cb - 1) / W->seg_cb;
+        if ((int64_t)W->nnz / 8 + (int64_t)W->Rb * nseg >= ((int64_t)1 << 22))
+            return mortar_fail(MORTAR_ERR_LIMIT, "spmm: octet stream of %d blocks in %d x %lld row parts exceeds 4 GiB",
+                               W->nnz, W->Rb, (long long)nseg);
+    }
     if (M <= 0 || M > (1 << 30)) return mortar_fail(MORTAR_ERR_ARG, "spmm: M=%lld out of range", (long long)M);
     if (ldx < (int64_t)W->Cb * 16 || ldx % 8) return mortar_fail(MORTAR_ERR_ARG, "spmm: ldx=%lld must be >= in_features and a multiple of 8", (long long)ldx);
     if (ldy < out_cols || ldy % 4) return mortar_fail(MORTAR_ERR_ARG, "spmm: ldy=%lld must be >= out_features and a multiple of 4", (long long)ldy);

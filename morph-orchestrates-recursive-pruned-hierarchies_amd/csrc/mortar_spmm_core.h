@@ -146,19 +146,25 @@ struct MortarBatch {
 // Loads the batch that starts at octet gq of a row part ending at octet g1 (octets past the end repeat the last).
 // FP4: the code stream is the 4-bit one (a lane's dword holds the 8 codes of its own column half, so the four
 // lane groups read four different 16-byte runs per octet instead of two).
+// gq and g1 are wave-uniform, so every address is (stream base, scalar byte offset of the octet, per-lane constant):
+// raw buffer loads take exactly these three and cost no address arithmetic on the vector ALU, which the kernels
+// are short of (the one vector instruction left is the clamp of the metadata octet at the end of a part).
 template <int CODE = 0>
 __device__ __forceinline__ void mortar_load_batch(const SpmmView &p, MortarBatch &b, int gq, int g1, int n, int bsel,
                                                   int hsel = 0) {
+    constexpr int OB = (CODE & CODE_4BIT) ? 1024 : 512;          // bytes of codes per octet
+    const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc((void *)p.codes_o, 0, -1, 0x00020000);
+    const int lane_c = (CODE & CODE_4BIT) ? ((bsel * 2 + hsel) * 16 + n) * 16 : (bsel * 16 + n) * 16;
 #pragma unroll
     for (int k = 0; k < RES_GROUPS; ++k) {
-        const uint32_t go = (uint32_t)(gq + k < g1 ? gq + k : g1 - 1);
-        const uint32_t gi = (CODE & CODE_4BIT) ? go * 4u + (uint32_t)(bsel * 2 + hsel) : go * 2u + (uint32_t)bsel;
-        b.cw[k] = p.codes_o[gi * 16u + n];
+        const int go = gq + k < g1 ? gq + k : g1 - 1;
+        b.cw[k] = __builtin_amdgcn_raw_buffer_load_b128(rc, lane_c, go * OB, 0);
     }
-    const int go = gq + (n >> 2);
-    const uint32_t mi = ((uint32_t)(go < g1 ? go : g1 - 1) * 2u + (uint32_t)bsel) * 4u + (uint32_t)(n & 3);
-    b.sdv = (CODE & CODE_UNIFORM) ? 0u : p.sd_dw[mi];
-    b.ccv = p.cc_dw[mi];
+    const uint32_t ko = (uint32_t)(n >> 2), last = (uint32_t)(g1 - 1 - gq);
+    const int lane_m = (int)((ko < last ? ko : last) * 32u) + (bsel * 4 + (n & 3)) * 4;
+    if (CODE & CODE_UNIFORM) b.sdv = 0u;
+    else b.sdv = __builtin_amdgcn_raw_buffer_load_b32(__builtin_amdgcn_make_buffer_rsrc((void *)p.sd_dw, 0, -1, 0x00020000), lane_m, gq * 32, 0);
+    b.ccv = __builtin_amdgcn_raw_buffer_load_b32(__builtin_amdgcn_make_buffer_rsrc((void *)p.cc_dw, 0, -1, 0x00020000), lane_m, gq * 32, 0);
 }
 
 // One row part: octets [g0, g1) (nb blocks) of the stream against the tile at `lx`.
