@@ -316,11 +316,16 @@ def main() -> None:
             ops.gateup_swiglu(x, Wgu, gates=gates, route=route, out=h)
             ops.spmm(h, Wdn, active=active, out=y)
         t = event_time_ms(routed, it)
-        n_act = int(ops.remoe_gates(logits, TOP_K)[1].sum())
+        act_now = ops.remoe_gates(logits, TOP_K)[1]
+        n_act = int(act_now.sum())
         act_frac = n_act / (TOKENS * N_CLUSTERS)
+        cnt_now = ops.remoe_route(act_now, ops.route_tile(Wgu, TOKENS))[0].to(torch.int64)
+        sub_exec = int(((cnt_now + 15) // 16).sum())             # 16-token MFMA sub-tiles the routed gate_up executes
         fl_active = (flops_gu + flops_dn) * act_frac          # products whose hidden cluster is active for the token
         out["routed_prefill"] = {"ms": t, "tokens_per_s": TOKENS / (t * 1e-3), "active_fraction": act_frac,
                                  "vs_unrouted": t / ms,
+                                 "gather_efficiency": n_act / (16.0 * sub_exec),          # active tokens per executed MFMA column
+                                 "mfma_subtiles_executed": sub_exec / float(cnt_now.numel() * (ops.route_tile(Wgu, TOKENS) // 16)),
                                  "roofline": {"bound": "mfma", "kernel": "remoe_gates + remoe_route + routed gate_up + masked down",
                                               "achieved": fl_active / (t * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                               "frac": fl_active / (t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
@@ -375,7 +380,27 @@ def main() -> None:
         fused_norm = all(ops.norm_fusable(m4.gate_up._cms.mortar_pack()) for m4 in mlps4)
         t = event_time_ms(lambda: mortar_amd.looped_core_forward(mlps4, x, 6), 3, 1)
         fl = 6 * sum(2.0 * TOKENS * 256 * (m4.gate_up._cms.mortar_pack().nnz + m4.down._cms.mortar_pack().nnz) for m4 in mlps4)
+        # static load balance of the Zipf rows: blocks per workgroup window of gate_up's schedule (units are then drawn
+        # dynamically by the 16 waves of a window) and blocks per wave of down's fixed assignment (4 units per wave)
+        def _balance(W, rpu, group):
+            from mortar_amd.pack import unit_order
+            nnz_row = np.diff(W.h_offsets).astype(np.int64)
+            per_unit = nnz_row.reshape(rpu, -1).sum(0)[unit_order(W.h_offsets, W.Rb, rpu)]
+            pad = (-per_unit.size) % group
+            work = np.concatenate([per_unit, np.zeros(pad, np.int64)]).reshape(-1, group)
+            return work
+        lb_gu, lb_dn = [], []
+        for m4 in mlps4:
+            Wg4, Wd4 = m4.gate_up._cms.mortar_pack(), m4.down._cms.mortar_pack()
+            n_split = max(1, 256 // (-(-TOKENS // 32)))
+            per = -(-(Wg4.Rb // 2) // n_split)
+            wg = _balance(Wg4, 2, per).sum(1)                               # one row of `work` = one workgroup window
+            lb_gu.append(float(wg.sum() / (wg.size * wg.max())))
+            wv = _balance(Wd4, 1, 64).reshape(-1, 4, 16).sum(1).reshape(-1)   # wave w of a 64-unit group takes units w, w+16, ...
+            lb_dn.append(float(wv.sum() / (wv.size * wv.max())))
         out["looped_stack"] = {"ms": t, "mlp_calls": 48, "ms_per_mlp": t / 48, "tokens_per_s": TOKENS / (t * 1e-3),
+                               "load_balance_efficiency": {"gate_up_workgroup_windows": min(lb_gu), "down_waves": min(lb_dn),
+                                                           "definition": "sum of blocks / (parts x blocks of the fullest part), worst of the 8 matrices"},
                                "effective_tflops": fl / (t * 1e-3) / 1e12,
                                "frac_mfma": fl / (t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
                                "norm_fused_into_gate_up": bool(fused_norm),
