@@ -25,9 +25,9 @@ PEAK_BF16_TFLOPS, PEAK_HBM_GBS = 2500.0, 8000.0
 # HBM-side bytes per launch (read + written) measured with `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` on this
 # workload and calibrated on a plain copy; the runs and factors are in profiles/bench_prefill_step_hbm_traffic_pmc.md
 # and profiles/bench_all_legs_hbm_traffic_pmc.md.  Not measured live: counters need the profiler.
-TRAFFIC_GATE_UP_BYTES = 41.62e6 + 50.88e6
-TRAFFIC_DOWN_BYTES = 60.33e6 + 16.78e6
-TRAFFIC_DECODE_STACK_BYTES = (263.01e6 + 4.56e6) + (162.17e6 + 1.85e6)   # gate_up + down launches, 160 layers, b = 1
+TRAFFIC_GATE_UP_BYTES = 41.58e6 + 51.22e6
+TRAFFIC_DOWN_BYTES = 60.31e6 + 16.78e6
+TRAFFIC_DECODE_STACK_BYTES = (263.03e6 + 4.55e6) + (162.14e6 + 1.84e6)   # gate_up + down launches, 160 layers, b = 1
 TRAFFIC_SOURCE = ("constant from profiles/bench_prefill_step_hbm_traffic_pmc.md and profiles/bench_all_legs_hbm_traffic_pmc.md "
                   "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command); not measured in this run")
 
@@ -168,8 +168,20 @@ def main() -> None:
     flops_gu = 2.0 * TOKENS * 256 * Wgu.nnz
     flops_dn = 2.0 * TOKENS * 256 * Wdn.nnz
     it = max(10, args.steps)
-    ms_gu = event_time_ms(lambda: ops.gateup_swiglu(x, Wgu, out=h), it)
-    ms_dn = event_time_ms(lambda: ops.spmm(h, Wdn, out=y), it)
+    # per-kernel durations inside the step sequence (gate_up and down alternating, as in the timed region): HIP events on
+    # the launch stream around every launch
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(it)]
+    step()
+    torch.cuda.synchronize()
+    for e in evs:
+        e[0].record()
+        ops.gateup_swiglu(x, Wgu, out=h)
+        e[1].record()
+        ops.spmm(h, Wdn, out=y)
+        e[2].record()
+    torch.cuda.synchronize()
+    ms_gu = sum(e[0].elapsed_time(e[1]) for e in evs) / it
+    ms_dn = sum(e[1].elapsed_time(e[2]) for e in evs) / it
     out = {
         "metric": "sparse-MLP prefill tokens/s @ d_model=2048, d_ff=5632, 25% block density, 4096 tokens",
         "value": TOKENS / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
