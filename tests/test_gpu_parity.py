@@ -222,6 +222,29 @@ def test_prefill_code_streams_agree(dev, d_model, d_ff):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("seg_cb", [7, 32, 64])
+@pytest.mark.parametrize("M", [5, 16, 100, 300])
+def test_narrow_k_segments(dev, seg_cb, M):
+    """A pack built with narrow K segments (MortarPack(seg_cb=...)) walks several segments per row in every kernel
+    family (prefill tiles run the K-segmented kernel also for gate_up, decode tiles walk the segments back to back):
+    same products as the oracle, and the padding blocks between a row's segments contribute nothing."""
+    from mortar_amd.pack import MortarPack
+    d_model, d_ff = 16 * 72, 16 * 40
+    spec = synth.synth_mlp(d_model, d_ff, 0.3, seed=71, zipf_s=1.2)
+    x = synth.synth_x(M, d_model, 72)
+    xd = to_dev(x, dev)
+    def pk(m):
+        return MortarPack(synth.flat_pack(m["codes"]), m["scales"], m["col_idx"], m["offsets"], m["shape"][0], m["shape"][1],
+                          dev, seg_cb=seg_cb)
+    Wgu, Wdn = pk(spec["gate_up"]), pk(spec["down"])
+    assert Wgu.nseg == -(-(d_model // 16) // seg_cb) and Wdn.nseg == -(-(d_ff // 16) // seg_cb)
+    ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
+    h = ops.gateup_swiglu(xd, Wgu)
+    assert_close_bf16(to_np(h), ref["h"], "h", ulps=8)
+    assert_close_bf16(to_np(ops.spmm(h, Wdn)), oracle_spmm(to_np(h), spec["down"]), "y", ulps=8)
+    assert_close_bf16(to_np(ops.spmm(xd, Wgu)), oracle_spmm(x, spec["gate_up"]), "gu", ulps=8)
+
+
 @pytest.mark.parametrize("d_model,d_ff,M", [(256, 16 * 40, 200), (2048, 16 * 24, 130), (16 * 30, 16 * 352, 100),
                                             (256, 16 * 40, 1), (2048, 16 * 24, 5), (16 * 30, 16 * 352, 16), (768, 2048, 40)])
 def test_one_scale_per_matrix(dev, d_model, d_ff, M):
