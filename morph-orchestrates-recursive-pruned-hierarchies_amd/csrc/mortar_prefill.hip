@@ -55,12 +55,13 @@ int resident_mt(int Cb) {
     return 0;
 }
 
-// prefill tiles: 16 wavefronts (4 per SIMD) for the 32-token tile, 8 for the 64-token tile (measured: a 96-token
-// tile of a narrow matrix leaves only two waves per SIMD and is slower)
+// prefill tiles: 16 wavefronts (4 per SIMD) for both tiles (the 64-token tile with 8 wavefronts was measured 18 % slower
+// on the base-width gate_up, although the 16-wave gate_up form spills six registers; a 96-token tile of a narrow
+// matrix leaves only two waves per SIMD and is slower still)
 template <int NACC, bool ROUTED, int CODE>
 int launch_resident_any(SpmmParams &p, hipStream_t st) {
     switch (resident_mt(p.Cb)) {
-        case 64: return mortar_launch_resident<64, NACC, ROUTED, 8, false, CODE>(p, nullptr, 1, st);
+        case 64: return mortar_launch_resident<64, NACC, ROUTED, 16, false, CODE>(p, nullptr, 1, st);
         default: return mortar_launch_resident<32, NACC, ROUTED, 16, false, CODE>(p, nullptr, 1, st);
     }
 }
