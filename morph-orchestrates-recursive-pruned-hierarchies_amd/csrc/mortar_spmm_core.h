@@ -196,7 +196,7 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const int u = 4 * k + t;
-                    if (MSUB >= 2 && t == 2 && u >= pairs) break;     // prefill tiles: the padded half of the last octet
+                    if (t == 2 && u >= pairs) break;                  // the padded half of the last octet
                     const uint32_t nib = (CODE & CODE_4BIT) ? b.cw[k][t] : ((b.cw[k][t] << (2 * hsel)) & 0xCCCCCCCCu);
                     const u32x4_t A = (CODE & CODE_UNIFORM) ? mortar_nib4(nib) : mortar_scale4(nib, mortar_row_bcast(b.sdv, u));
                     if (u + 2 < NP) {
