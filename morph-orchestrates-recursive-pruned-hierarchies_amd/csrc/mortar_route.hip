@@ -27,9 +27,20 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// Sum of a per-lane count over the wavefront with DPP adds only (quads, half rows, rows, then the row broadcasts): the
+// total arrives in the lanes of the last row and is read from lane 63.
+__device__ __forceinline__ int wave_count_total(uint32_t v) {
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false);    // quad_perm [1,0,3,2]
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false);    // quad_perm [2,3,0,1]
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, false);   // row_half_mirror
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, false);   // row_mirror
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1 and 3
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2 and 3
+    return __builtin_amdgcn_readlane((int)v, 63);
+}
+
 // Gating tail of one token on one wavefront.  The k-th largest logit is found exactly by an MSB-first radix
-// select on order-preserving keys: for each bit the wave counts (ballot + popcount) the keys >= the candidate
-// prefix.  Ties need no special care: the result is a VALUE, and the gate rule is `logit > kth`.
+// select on order-preserving keys: for each bit the wave counts the keys >= the candidate prefix.  Ties need no special care: the result is a VALUE, and the gate rule is `logit > kth`.
 // `lp` may point to global memory or LDS; gates / active are this token's output rows.
 template <int MAXPL>      // logits per lane this instantiation holds: n <= 64 * MAXPL
 __device__ __forceinline__ void remoe_gates_wave(const float *lp, int n, int k, float *gates, uint8_t *active, int lane) {
@@ -47,10 +58,12 @@ __device__ __forceinline__ void remoe_gates_wave(const float *lp, int n, int k, 
         uint32_t prefix = 0;
         for (int bit = 31; bit >= 0; --bit) {
             const uint32_t cand = prefix | (1u << bit);
-            int c = 0;
+            // counted on the vector ALU: a ballot + scalar popcount per key would queue on the one scalar ALU that the
+            // sixteen waves of a CU share
+            uint32_t own = 0;
 #pragma unroll
-            for (int i = 0; i < MAXPL; ++i) c += __popcll(__ballot(key[i] >= cand));     // padding keys are 0 < cand
-            if (c >= k) prefix = cand;
+            for (int i = 0; i < MAXPL; ++i) own += key[i] >= cand ? 1u : 0u;             // padding keys are 0 < cand
+            if (wave_count_total(own) >= k) prefix = cand;
         }
         kth = key_to_float(prefix);
     }
