@@ -170,13 +170,15 @@ __device__ __forceinline__ void mortar_load_batch(const SpmmView &p, MortarBatch
 // One row part: octets [g0, g1) (nb blocks) of the stream against the tile at `lx`.
 // `xo_base` is the lane's byte offset inside a block-column (token, column half) plus the segment's origin.
 // `b` holds the part's first batch, loaded by the caller (mortar_load_batch at g0) where it suits it.
-template <int MSUB, int MT, bool ROUTED, int CODE = 0>
+// FIRST_ONLY: only the batch in `b` (the part's first RES_GROUPS octets) is multiplied and no load is issued here, so
+// that a caller which keeps the next part's batch in flight gets a counted wait for `b` instead of a full one.
+template <int MSUB, int MT, bool ROUTED, int CODE = 0, bool FIRST_ONLY = false>
 __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *lx, MortarBatch b, int g0, int g1,
                                                 int nb, uint32_t xo_base, const uint32_t (&tk)[MSUB], int nsub, int n,
                                                 int bsel, int hsel, f32x4_t (&acc)[MSUB]) {
     const unsigned char *lb = reinterpret_cast<const unsigned char *>(lx);
-    for (int gq = g0; gq < g1; gq += RES_GROUPS) {
-        if (gq != g0) mortar_load_batch<CODE>(p, b, gq, g1, n, bsel, hsel);
+    for (int gq = g0; gq < (FIRST_ONLY ? g0 + 1 : g1); gq += RES_GROUPS) {
+        if (!FIRST_ONLY && gq != g0) mortar_load_batch<CODE>(p, b, gq, g1, n, bsel, hsel);
         const uint32_t ccs = __umul24(b.ccv, (uint32_t)(MT * 32));   // byte offset of the block-column in the tile
         const int pairs = ((nb - (gq - g0) * 8) + 1) >> 1;      // block pairs left in the row from this batch on
         // Activation operands are fetched two pairs ahead of the MFMAs that use them.  The only branches are
@@ -562,17 +564,33 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
 #pragma unroll
             for (int q = 0; q < NP; ++q) dn[q] = mortar_part_desc<NACC>(p, pos0 + WAVES * (q / NACC), sg + 1, q % NACC);
         }
+        // The first batch of every part is requested one part ahead (the first part's before the tile is staged), always
+        // and in a fixed order (an empty part reads octet 0), and a part's first batch is multiplied without a load in
+        // between: the wait for it then counts the loads issued since and never includes the newest ones.
+        constexpr int FIRST = 8 * RES_GROUPS;                      // blocks of a part's first batch
+        auto first_batch = [&](MortarBatch &bb, int q) {
+            const bool any = g0[q] < g1[q];
+            mortar_load_batch<CODE>(p, bb, any ? g0[q] : 0, any ? g1[q] : 1, n, bsel, hsel);
+        };
+        MortarBatch bq;
+        first_batch(bq, 0);
         if (sg > 0) __syncthreads();
         mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, c0, ncb, tid);
         __syncthreads();
 #pragma unroll
         for (int q = 0; q < NP; ++q) {
-            if (g0[q] < g1[q]) {
-                MortarBatch b;
-                mortar_load_batch<CODE>(p, b, g0[q], g1[q], n, bsel, hsel);
-                mortar_row_part<MSUB, MT, false, CODE>(p, lx, b, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
-                                                  acc[q / NACC][q % NACC]);
+            MortarBatch bn;
+            if (q + 1 < NP) first_batch(bn, q + 1);
+            const int nbq = g0[q] < g1[q] ? nb[q] : 0;
+            mortar_row_part<MSUB, MT, false, CODE, true>(p, lx, bq, g0[q], g1[q], nbq < FIRST ? nbq : FIRST, lane_xo, tk, MSUB,
+                                                         n, bsel, hsel, acc[q / NACC][q % NACC]);
+            if (nbq > FIRST) {                                      // the rest of a long part
+                MortarBatch bt;
+                mortar_load_batch<CODE>(p, bt, g0[q] + RES_GROUPS, g1[q], n, bsel, hsel);
+                mortar_row_part<MSUB, MT, false, CODE>(p, lx, bt, g0[q] + RES_GROUPS, g1[q], nbq - FIRST, lane_xo, tk, MSUB,
+                                                       n, bsel, hsel, acc[q / NACC][q % NACC]);
             }
+            if (q + 1 < NP) bq = bn;
         }
     }
 
