@@ -567,16 +567,30 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
         // The first batch of every part is requested one part ahead (the first part's before the tile is staged), always
         // and in a fixed order (an empty part reads octet 0), and a part's first batch is multiplied without a load in
         // between: the wait for it then counts the loads issued since and never includes the newest ones.
+        // (Prefill tiles only: the decode tiles of this kernel run many waves per SIMD on few registers.)
         constexpr int FIRST = 8 * RES_GROUPS;                      // blocks of a part's first batch
+        constexpr bool BATCH_AHEAD = MT >= 32;
         auto first_batch = [&](MortarBatch &bb, int q) {
             const bool any = g0[q] < g1[q];
             mortar_load_batch<CODE>(p, bb, any ? g0[q] : 0, any ? g1[q] : 1, n, bsel, hsel);
         };
         MortarBatch bq;
-        first_batch(bq, 0);
+        if (BATCH_AHEAD) first_batch(bq, 0);
         if (sg > 0) __syncthreads();
         mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, c0, ncb, tid);
         __syncthreads();
+        if (!BATCH_AHEAD) {
+#pragma unroll
+            for (int q = 0; q < NP; ++q) {
+                if (g0[q] < g1[q]) {
+                    MortarBatch b;
+                    mortar_load_batch<CODE>(p, b, g0[q], g1[q], n, bsel, hsel);
+                    mortar_row_part<MSUB, MT, false, CODE>(p, lx, b, g0[q], g1[q], nb[q], lane_xo, tk, MSUB, n, bsel, hsel,
+                                                           acc[q / NACC][q % NACC]);
+                }
+            }
+            continue;
+        }
 #pragma unroll
         for (int q = 0; q < NP; ++q) {
             MortarBatch bn;
