@@ -140,6 +140,18 @@ int mortar_prefill_max_seg_cb(void);
 int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_t rows_per_unit, int32_t group,
                            int32_t *order_out);
 
+/* Second pass over a unit order for matrices with several K segments (nseg > 1).  The K-segmented prefill
+ * kernel ends every segment with a workgroup barrier, so a workgroup waits in each segment for the wave whose
+ * units hold the most blocks IN THAT SEGMENT.  Within every window of waves * units_per_wave consecutive
+ * positions (one workgroup; wave w owns positions w, w + waves, ...) the units are dealt again so that the sum
+ * over the segments of the heaviest wave is small (greedy by heaviest segment, then pairwise exchanges).  Which
+ * units a window holds does not change.  The prefill kernels run waves = 16 with units_per_wave = 4 for plain
+ * units and 2 for gate/up units.  row_desc: host [nseg*Rb*4] from mortar_octet_layout_host.  order: host
+ * [n_units], in and out (start from mortar_unit_order_host).  A no-op for nseg == 1 or units_per_wave == 1.
+ * No counterpart in the reference, whose Triton grid has one program per output tile. */
+int mortar_unit_order_segments_host(const int32_t *row_desc, int32_t Rb, int32_t nseg, int32_t rows_per_unit,
+                                    int32_t waves, int32_t units_per_wave, int32_t *order);
+
 /* Part descriptors in schedule order, the form the kernels walk: for position pos, K segment sg and row a of
  * the unit, sched_out[((pos*nseg + sg)*rows_per_unit + a)*4 ..] = {first octet, end octet, blocks, unit}, taken
  * from row_desc (mortar_octet_layout_host) of row unit + a*n_units.  order: host [n_units] from

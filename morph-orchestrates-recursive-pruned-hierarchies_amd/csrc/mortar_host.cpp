@@ -280,6 +280,94 @@ extern "C" int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_
     return MORTAR_OK;
 }
 
+extern "C" int mortar_unit_order_segments_host(const int32_t *row_desc, int32_t Rb, int32_t nseg,
+                                               int32_t rows_per_unit, int32_t waves, int32_t units_per_wave,
+                                               int32_t *order) {
+    if (!row_desc || !order || Rb <= 0 || nseg <= 0 || waves <= 0 || units_per_wave <= 0 ||
+        (rows_per_unit != 1 && rows_per_unit != 2) || Rb % rows_per_unit)
+        return mortar_fail(MORTAR_ERR_ARG, "unit_order_segments: bad argument");
+    const int nu = Rb / rows_per_unit;
+    if (nseg == 1 || units_per_wave == 1) return MORTAR_OK;   // no barrier between parts / nothing to deal
+    // cost[u][s]: block pairs the kernel multiplies for unit u in segment s (parts run in half octets)
+    std::vector<int32_t> cost((size_t)nu * nseg);
+    for (int u = 0; u < nu; ++u) {
+        if (order[u] < 0 || order[u] >= nu) return mortar_fail(MORTAR_ERR_ARG, "unit_order_segments: order out of range");
+        for (int s = 0; s < nseg; ++s) {
+            int32_t c = 0;
+            for (int a = 0; a < rows_per_unit; ++a)
+                c += (row_desc[4 * ((int64_t)s * Rb + u + (int64_t)a * nu) + 2] + 3) / 4 * 2;
+            cost[(size_t)u * nseg + s] = c;
+        }
+    }
+    const int per = waves * units_per_wave;
+    std::vector<int64_t> load((size_t)waves * nseg);
+    std::vector<std::vector<int>> mem(waves);
+    // sum over the segments of the heaviest wave: what the barriers make the workgroup wait for
+    auto objective = [&]() {
+        int64_t t = 0;
+        for (int s = 0; s < nseg; ++s) {
+            int64_t m = 0;
+            for (int w = 0; w < waves; ++w) m = std::max(m, load[(size_t)w * nseg + s]);
+            t += m;
+        }
+        return t;
+    };
+    auto move = [&](int w, int u, int sign) {
+        for (int s = 0; s < nseg; ++s) load[(size_t)w * nseg + s] += sign * cost[(size_t)u * nseg + s];
+    };
+    for (int p0 = 0; p0 < nu; p0 += per) {
+        const int n = std::min(per, nu - p0);
+        std::vector<int> units(order + p0, order + p0 + n);
+        auto peak = [&](int u) { return *std::max_element(&cost[(size_t)u * nseg], &cost[(size_t)u * nseg] + nseg); };
+        std::stable_sort(units.begin(), units.end(), [&](int a, int b) { return peak(a) > peak(b); });
+        std::fill(load.begin(), load.end(), 0);
+        std::vector<int> cap(waves);
+        for (int w = 0; w < waves; ++w) {       // wave w owns the window's positions w, w + waves, ...
+            mem[w].clear();
+            cap[w] = w < n ? (n - w + waves - 1) / waves : 0;
+        }
+        for (int u : units) {                   // greedy: the wave whose heaviest segment stays lightest
+            int best = -1;
+            int64_t best_peak = 0, best_sum = 0;
+            for (int w = 0; w < waves; ++w) {
+                if ((int)mem[w].size() >= cap[w]) continue;
+                int64_t pk = 0, sm = 0;
+                for (int s = 0; s < nseg; ++s) {
+                    const int64_t v = load[(size_t)w * nseg + s] + cost[(size_t)u * nseg + s];
+                    pk = std::max(pk, v);
+                    sm += v;
+                }
+                if (best < 0 || pk < best_peak || (pk == best_peak && sm < best_sum)) best = w, best_peak = pk, best_sum = sm;
+            }
+            mem[best].push_back(u);
+            move(best, u, +1);
+        }
+        int64_t cur = objective();              // then exchanges of two units while one lowers the objective
+        for (int pass = 0; pass < 16; ++pass) {
+            bool improved = false;
+            for (int a = 0; a < waves; ++a)
+                for (int b = a + 1; b < waves; ++b)
+                    for (size_t i = 0; i < mem[a].size(); ++i)
+                        for (size_t j = 0; j < mem[b].size(); ++j) {
+                            const int ua = mem[a][i], ub = mem[b][j];
+                            move(a, ua, -1); move(a, ub, +1); move(b, ub, -1); move(b, ua, +1);
+                            const int64_t t = objective();
+                            if (t < cur) {
+                                cur = t;
+                                std::swap(mem[a][i], mem[b][j]);
+                                improved = true;
+                            } else {
+                                move(a, ub, -1); move(a, ua, +1); move(b, ua, -1); move(b, ub, +1);
+                            }
+                        }
+            if (!improved) break;
+        }
+        for (int w = 0; w < waves; ++w)
+            for (size_t k = 0; k < mem[w].size(); ++k) order[p0 + w + waves * (int)k] = mem[w][k];
+    }
+    return MORTAR_OK;
+}
+
 extern "C" int mortar_schedule_host(const int32_t *row_desc, int32_t Rb, int32_t nseg, int32_t rows_per_unit,
                                     const int32_t *order, int32_t *sched_out) {
     if (!row_desc || !sched_out || Rb <= 0 || nseg <= 0 || (rows_per_unit != 1 && rows_per_unit != 2) ||

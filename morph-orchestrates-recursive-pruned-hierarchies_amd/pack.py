@@ -16,6 +16,7 @@ from . import _lib
 
 BLK = 16
 SCHED_GROUP = 16      # wavefronts of a prefill workgroup: the group size of the row-unit order
+SCHED_UNITS_PER_WAVE = {1: 4, 2: 2}   # units a wave of the K-segmented prefill kernel owns, by rows per unit
 
 
 def _np(a, dtype):
@@ -103,6 +104,15 @@ def unit_order(offsets, Rb: int, rows_per_unit: int, group: int = SCHED_GROUP) -
     offsets = _np(offsets, np.int32)
     out = np.empty(Rb // rows_per_unit, dtype=np.int32)
     _lib.check(_lib.lib().mortar_unit_order_host(_vp(offsets), Rb, rows_per_unit, group, _vp(out)), "mortar_unit_order_host")
+    return out
+
+
+def unit_order_segments(row_desc, Rb: int, nseg: int, rows_per_unit: int, order: np.ndarray) -> np.ndarray:
+    """Re-deal every workgroup window of ``order`` so that no wave is the slowest in every K segment."""
+    row_desc, out = _np(row_desc, np.int32), _np(order, np.int32).copy()
+    _lib.check(_lib.lib().mortar_unit_order_segments_host(_vp(row_desc), Rb, nseg, rows_per_unit, SCHED_GROUP,
+                                                          SCHED_UNITS_PER_WAVE[rows_per_unit], _vp(out)),
+               "mortar_unit_order_segments_host")
     return out
 
 
@@ -344,6 +354,8 @@ class MortarPack:
         """Device schedule (mortar_schedule_host over the balanced unit order) for plain (1) or gate/up (2) units."""
         if rows_per_unit not in self._scheds:
             o = unit_order(self.h_offsets, self.Rb, rows_per_unit)
+            if self.nseg > 1:
+                o = unit_order_segments(self.h_row_desc, self.Rb, self.nseg, rows_per_unit, o)
             sc = schedule(self.h_row_desc, self.Rb, self.nseg, rows_per_unit, o)
             self._scheds[rows_per_unit] = torch.from_numpy(sc).to(self.device)
         return self._scheds[rows_per_unit]
