@@ -63,7 +63,8 @@ __device__ __forceinline__ uint32_t bf16_pack2(float lo, float hi) {
 }
 __device__ __forceinline__ uint32_t bf16_bits_rne(float f) { return bf16_pack2(f, 0.f) & 0xffffu; }
 __device__ __forceinline__ float bf16_to_f32(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
-__device__ __forceinline__ float bf16r(float f) { return __builtin_bit_cast(float, bf16_pack2(0.f, f) & 0xffff0000u); }
+// f rounded to bf16, as a float: the conversion of (0, f) leaves the bf16 of f in the high half and zeros below it.
+__device__ __forceinline__ float bf16r(float f) { return __builtin_bit_cast(float, bf16_pack2(0.f, f)); }
 
 // ---- RMSNorm pieces shared by the stand-alone kernel and the fused staging of gate_up, so that both round alike.
 // A row is handled by one wavefront in 16-byte units (8 bf16): a lane adds the squares of its units in ascending
@@ -107,23 +108,14 @@ __device__ __forceinline__ float silu_f32(float g) { return g * __builtin_amdgcn
 // bf16 where the reference materialises a bf16 tensor (gate_up output, silu, product, gated product).
 // `gate` is the router gate of these features (they lie in one cluster); pass has_gate = false for none.
 __device__ __forceinline__ u32x2_t swiglu_pack4(f32x4_t g, f32x4_t u, bool has_gate, float gate) {
+    // each value is rounded on its own (one conversion, no unpacking of a packed pair)
     float h[4];
 #pragma unroll
-    for (int v = 0; v < 4; v += 2) {
-        const uint32_t gp = bf16_pack2(g[v], g[v + 1]), up = bf16_pack2(u[v], u[v + 1]);
-        const float g0 = __builtin_bit_cast(float, gp << 16), g1 = __builtin_bit_cast(float, gp & 0xffff0000u);
-        const float u0 = __builtin_bit_cast(float, up << 16), u1 = __builtin_bit_cast(float, up & 0xffff0000u);
-        const uint32_t sp = bf16_pack2(silu_f32(g0), silu_f32(g1));
-        h[v] = __builtin_bit_cast(float, sp << 16) * u0;
-        h[v + 1] = __builtin_bit_cast(float, sp & 0xffff0000u) * u1;
-    }
+    for (int v = 0; v < 4; ++v) h[v] = bf16r(silu_f32(bf16r(g[v]))) * bf16r(u[v]);
     if (has_gate) {
         const float gb = bf16r(gate);
-        const uint32_t p0 = bf16_pack2(h[0], h[1]), p1 = bf16_pack2(h[2], h[3]);
-        h[0] = __builtin_bit_cast(float, p0 << 16) * gb;
-        h[1] = __builtin_bit_cast(float, p0 & 0xffff0000u) * gb;
-        h[2] = __builtin_bit_cast(float, p1 << 16) * gb;
-        h[3] = __builtin_bit_cast(float, p1 & 0xffff0000u) * gb;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) h[v] = bf16r(h[v]) * gb;
     }
     return u32x2_t{bf16_pack2(h[0], h[1]), bf16_pack2(h[2], h[3])};
 }
