@@ -355,8 +355,9 @@ __device__ __forceinline__ void mortar_hc_post(const SpmmView &p, int tok, int f
 }
 
 // Epilogue of one row unit for the 16 tokens of sub-tile `ms`: the lane holds D[4g+v][token].
+// `gv` is the router gate of the lane's four features for this token (read when has_gates).
 template <int NACC, int CODE = 0, bool HC = false>
-__device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, int tok, int g, bool has_gates,
+__device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, int tok, int g, bool has_gates, float gv,
                                                   f32x4_t a0, f32x4_t a1) {
     if (CODE & CODE_UNIFORM) {      // the blocks were multiplied as +-2: p.uscale is half the matrix's scale
         a0 *= p.uscale;
@@ -376,11 +377,34 @@ __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, i
             return;
         }
     } else {
-        float gv = 0.f;
-        if (has_gates) gv = p.gates[(int64_t)tok * p.n_clusters + (unit * 16 + 4 * g) / p.cluster_size];
         pk = swiglu_pack4(a0, a1, has_gates, gv);
     }
     *(MORTAR_GLOBAL u32x2_t *)(p.y + (int64_t)tok * p.ldy + unit * 16 + 4 * g) = pk;
+}
+
+// Epilogue of one row unit for all sub-tiles of the token tile.  tl[ms] is the tile row of the lane's token in
+// sub-tile ms, `cnt` the number of live rows per 16-row sub-tile set (MT, or the routed list length).  The cluster of
+// the lane's features is found once per unit and the gates of all sub-tiles are requested before the first SwiGLU.
+template <int MSUB, int NACC, int CODE, bool HC>
+__device__ __forceinline__ void mortar_store_tile(const SpmmView &p, int unit, int m0, const uint32_t (&tl)[MSUB], int cnt,
+                                                  int n, int g, bool has_gates, const f32x4_t (&a0)[MSUB],
+                                                  const f32x4_t (&a1)[MSUB]) {
+    float gv[MSUB];
+    bool ok[MSUB];
+#pragma unroll
+    for (int ms = 0; ms < MSUB; ++ms) {
+        ok[ms] = ms * 16 + n < cnt && m0 + (int)tl[ms] < p.M;
+        gv[ms] = 0.f;
+    }
+    if (NACC == 2 && has_gates) {
+        const int gcol = (unit * 16 + 4 * g) / p.cluster_size;
+#pragma unroll
+        for (int ms = 0; ms < MSUB; ++ms)
+            if (ok[ms]) gv[ms] = p.gates[(int64_t)(m0 + (int)tl[ms]) * p.n_clusters + gcol];
+    }
+#pragma unroll
+    for (int ms = 0; ms < MSUB; ++ms)
+        if (ok[ms]) mortar_store_unit<NACC, CODE, HC>(p, unit, m0 + (int)tl[ms], g, has_gates, gv[ms], a0[ms], a1[ms]);
 }
 
 // Part descriptor of schedule position `pos`, segment `sg`, row `a` of the unit: {g0, g1, nb, unit}.
@@ -493,14 +517,8 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
         pos = npos;
         if (skip) continue;
 
-#pragma unroll
-        for (int ms = 0; ms < MSUB; ++ms) {
-            const int li = ms * 16 + n;
-            if (li >= (ROUTED ? cnt : MT)) continue;
-            const int tok = m0 + (int)tk[ms];
-            if (tok >= p.M) continue;
-            mortar_store_unit<NACC, CODE, (MT <= 16 && NACC == 1 && !TABLE)>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
-        }
+        mortar_store_tile<MSUB, NACC, CODE, (MT <= 16 && NACC == 1 && !TABLE)>(p, unit, m0, tk, ROUTED ? cnt : MT, n, g, has_gates,
+                                                                               acc[0], acc[NACC - 1]);
     }
 }
 
@@ -608,17 +626,14 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
         }
     }
 
+    uint32_t tl[MSUB];
+#pragma unroll
+    for (int ms = 0; ms < MSUB; ++ms) tl[ms] = ms * 16 + n;
 #pragma unroll
     for (int k = 0; k < UPW; ++k) {
         if (units[k] < 0) continue;
-#pragma unroll
-        for (int ms = 0; ms < MSUB; ++ms) {
-            const int li = ms * 16 + n;
-            if (li >= MT) continue;
-            const int tok = m0 + li;
-            if (tok >= p.M) continue;
-            mortar_store_unit<NACC, CODE, (MT <= 16 && NACC == 1 && !TABLE)>(p, units[k], tok, g, has_gates, acc[k][0][ms], acc[k][NACC - 1][ms]);
-        }
+        mortar_store_tile<MSUB, NACC, CODE, (MT <= 16 && NACC == 1 && !TABLE)>(p, units[k], m0, tl, MT, n, g, has_gates, acc[k][0],
+                                                                               acc[k][NACC - 1]);
     }
 }
 
@@ -718,14 +733,8 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
                 for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] += red[(((wave + w) * NACC + a) * MSUB + ms) * 64 + lane];
     }
     if (skip) return;
-#pragma unroll
-    for (int ms = 0; ms < MSUB; ++ms) {
-        const int li = ms * 16 + n;
-        if (li >= (ROUTED ? cnt : MT)) continue;
-        const int tok = m0 + (int)tk[ms];
-        if (tok >= p.M) continue;
-        mortar_store_unit<NACC, CODE, (MT <= 16 && NACC == 1)>(p, unit, tok, g, has_gates, acc[0][ms], acc[NACC - 1][ms]);
-    }
+    mortar_store_tile<MSUB, NACC, CODE, (MT <= 16 && NACC == 1)>(p, unit, m0, tk, ROUTED ? cnt : MT, n, g, has_gates, acc[0],
+                                                                 acc[NACC - 1]);
 }
 
 // ---- launchers -------------------------------------------------------------------------------------------
