@@ -219,7 +219,7 @@ int gateup_common(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *
     if (tok_cnt || tok_list) {
         if (!tok_cnt || !tok_list || !gates) return mortar_fail(MORTAR_ERR_ARG, "gateup: routed mode needs gates, tok_cnt and tok_list");
         if (p.cluster_size % 16) return mortar_fail(MORTAR_ERR_ARG, "gateup: routed mode needs cluster_size %% 16 == 0");
-        if (p.nseg != 1 || mortar_route_tile(W->Cb, M) == 0)
+        if (mortar_route_tile(W->Cb, M) == 0)
             return mortar_fail(MORTAR_ERR_LIMIT, "gateup: routed mode needs in_features to fit one LDS tile "
                                "(mortar_route_tile() == 0: call without tok_cnt / tok_list)");
         p.tok_cnt = tok_cnt; p.tok_list = tok_list;

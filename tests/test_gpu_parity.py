@@ -245,6 +245,33 @@ def test_narrow_k_segments(dev, seg_cb, M):
     assert_close_bf16(to_np(ops.spmm(xd, Wgu)), oracle_spmm(x, spec["gate_up"]), "gu", ulps=8)
 
 
+@pytest.mark.parametrize("d_model,seg_cb,M", [(16 * 30, 20, 257), (16 * 200, None, 4), (2048, 32, 17), (16 * 78, 65, 63)])
+def test_routed_gate_up_over_several_k_segments(dev, d_model, seg_cb, M):
+    """Routed skipping whenever mortar_route_tile() names a tile, also for a matrix whose stream has several K segments
+    (a narrow seg_cb, or in_features wider than one prefill segment at a decode-sized M): exactly the active tiles are
+    written and they equal the dense gated call."""
+    from mortar_amd.pack import MortarPack
+    d_ff, ncl = 16 * 22, 22
+    spec = synth.synth_mlp(d_model, d_ff, 0.25, seed=91)
+    m = spec["gate_up"]
+    Wgu = MortarPack(synth.flat_pack(m["codes"]), m["scales"], m["col_idx"], m["offsets"], m["shape"][0], m["shape"][1], dev,
+                     seg_cb=seg_cb)
+    assert Wgu.nseg > 1
+    x = synth.synth_x(M, d_model, 92)
+    logits = synth.synth_logits(M, ncl, 93)
+    g_ref, act_ref = O.remoe_gates(logits, 7)
+    gates, active = ops.remoe_gates(torch.from_numpy(logits).to(dev), 7)
+    xd = to_dev(x, dev)
+    h_dense = ops.gateup_swiglu(xd, Wgu, gates=gates)
+    assert_close_bf16(to_np(h_dense), O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=g_ref)["h"], "h gated", ulps=8)
+    tile = ops.route_tile(Wgu, M)
+    assert tile > 0
+    h_skip = torch.full_like(h_dense, float("nan"))
+    ops.gateup_swiglu(xd, Wgu, gates=gates, route=ops.remoe_route(active, tile), out=h_skip)
+    hs, hd, on = to_np(h_skip), to_np(h_dense), np.repeat(act_ref, 16, axis=1)
+    assert np.array_equal(hs[on], hd[on]) and np.isnan(hs[~on]).all()
+
+
 @pytest.mark.parametrize("d_model,d_ff,M", [(256, 16 * 40, 200), (2048, 16 * 24, 130), (16 * 30, 16 * 352, 100),
                                             (256, 16 * 40, 1), (2048, 16 * 24, 5), (16 * 30, 16 * 352, 16), (768, 2048, 40)])
 def test_one_scale_per_matrix(dev, d_model, d_ff, M):
