@@ -690,17 +690,26 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
         }
     }
     const int nsub = ROUTED ? (cnt + 15) >> 4 : MSUB;
+    // Gated gate_up without token lists: a unit whose cluster is off for every token of the tile multiplies nothing
+    // (its accumulators stay zero and the epilogue stores the zeros the gates would have produced).  The gates are
+    // requested here and looked at after the tile is staged.
+    constexpr bool GATE_SKIP = NACC == 2 && !ROUTED && MT <= 16;
+    float gsk = 0.f;
+    if (GATE_SKIP && valid && has_gates && p.cluster_size % 16 == 0 && n < MT && m0 + n < p.M)
+        gsk = p.gates[(int64_t)(m0 + n) * p.n_clusters + (unit * 16) / p.cluster_size];
 
     if (NACC == 2 && !MASKED && p.norm) mortar_stage_tile_norm<MT, WAVES>(p, lx, m0, p.Cb, tid, reinterpret_cast<float *>(red));
     else mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, 0, p.Cb, tid);
     __syncthreads();
+    bool idle = skip;
+    if (GATE_SKIP && valid && has_gates && p.cluster_size % 16 == 0) idle = __ballot(gsk > 0.f) == 0ull;
 
     f32x4_t acc[NACC][MSUB];
 #pragma unroll
     for (int a = 0; a < NACC; ++a)
 #pragma unroll
         for (int ms = 0; ms < MSUB; ++ms) acc[a][ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    if (!skip) {
+    if (!idle) {
         for (int sg = 0; sg < p.nseg; ++sg) {
             const uint32_t xo_base = lane_xo + (uint32_t)(sg * p.seg_cb) * (uint32_t)(MT * 32);
 #pragma unroll

@@ -56,19 +56,10 @@ class MortarDecodeMLP:
             return self.mlp(x.reshape(B, -1).to(torch.bfloat16), iter_idx=self.iter_idx, gates=gates,
                             norm=(self.norm_weight, self.eps)).view(B, 1, -1)
         xn = ops.rmsnorm(x.reshape(B, -1).to(torch.bfloat16), self.norm_weight, self.eps)
-        active = None
         if gates is None and rt is not None:
-            gates, active = rt.route(xn, self.iter_idx)
-        tile = ops.route_tile(self.Mgu, B) if gates is not None and (self.d_ff // gates.shape[-1]) % 16 == 0 else 0
-        if tile:
-            # gather-skip: only (stream, block-row) tiles of active clusters are computed; `down` reads the
-            # hidden activations of inactive clusters as zero
-            gates = gates.contiguous()
-            if active is None:
-                active = (gates > 0).to(torch.uint8)
-            route = ops.remoe_route(active, tile)
-            h = ops.gateup_swiglu(xn, self.Mgu, gates=gates, route=route)
-            return ops.spmm(h, self.Mdown, active=active).view(B, 1, -1)
+            gates, _ = rt.route(xn, self.iter_idx)
+        # the gated gate_up kernel leaves out the units whose cluster is off for every stream of its tile (and stores
+        # their zeros), so `down` reads the hidden activations of inactive clusters as zero without a mask
         h = ops.gateup_swiglu(xn, self.Mgu, gates=gates.contiguous() if gates is not None else None)
         return ops.spmm(h, self.Mdown).view(B, 1, -1)
 

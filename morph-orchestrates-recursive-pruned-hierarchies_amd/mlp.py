@@ -179,9 +179,10 @@ class _SwiGLUMortar(nn.Module):
         if gates is not None and self.d_ff % gates.shape[-1]:
             raise ValueError("the carved MLP needs equal-size clusters (d_ff % n_clusters == 0)")
         N = xb.shape[0]
-        # one path for prefill and decode: the library picks 4- or 16-token tiles for decode-sized N
         cs = self.d_ff // gates.shape[-1] if gates is not None else 0
-        tile = ops.route_tile(Wgu, N) if (gates is not None and self.route_skip and cs % 16 == 0 and N > 0) else 0
+        # decode-sized batches need no token lists: the gated gate_up kernel itself leaves out units whose cluster is
+        # off for all tokens of its 4- or 16-token tile and stores their zeros
+        tile = ops.route_tile(Wgu, N) if (gates is not None and self.route_skip and cs % 16 == 0 and N > ops.DECODE_MAX_ROWS) else 0
         if tile:
             if active is None:
                 active = (gates > 0).to(torch.uint8)

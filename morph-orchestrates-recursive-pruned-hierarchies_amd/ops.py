@@ -162,6 +162,7 @@ def remoe_gates(logits: Tensor, k: int) -> tuple[Tensor, Tensor]:
 
 
 ROUTER_MAX_TOKENS = 64
+DECODE_MAX_ROWS = 64      # rows up to which a call runs on the 4- / 16-token decode tiles
 
 
 def router_fused(x: Tensor, wq: Tensor, iter_vec: Tensor | None, ln_w: Tensor, ln_b: Tensor, ln_eps: float,
