@@ -378,6 +378,28 @@ def test_fused_router_front_end(dev, B, d, nsk, n, xdt):
     np.testing.assert_allclose(lt.cpu().numpy(), ref, rtol=0, atol=2e-5 * max(1.0, np.abs(ref).max()))
 
 
+def test_decode_mlp_module_routes_with_its_own_router(dev):
+    """MortarDecodeMLP with a router attached (no token lists: the gated gate_up kernel leaves out inactive units
+    itself) equals the step-by-step composition rmsnorm -> route -> gated gate_up -> down, and the oracle."""
+    d_model, d_ff = 512, 16 * 64
+    spec = synth.synth_mlp(d_model, d_ff, 0.3, seed=77)
+    mlp = synth.mlp_module(spec, dev)
+    torch.manual_seed(5)
+    mlp.enable_routing(n_clusters=16, activation_ratio=0.5, n_sub_keys=4)
+    w = to_dev(O.bf16_round(1.0 + 0.1 * synth.synth_x(1, d_model, 78)[0]), dev)
+    dec = mortar_amd.MortarDecodeMLP(mlp, norm_weight=w, eps=1e-6)
+    for B in (1, 3, 16, 40):
+        x = to_dev(synth.synth_x(B, d_model, 79 + B) * 2.0, dev)
+        y = dec(x.reshape(B, 1, d_model))
+        xn = ops.rmsnorm(x, w, 1e-6)
+        gates, active = mlp.router.route(xn, 0)
+        assert 0 < int(active.sum()) < active.numel()
+        h = ops.gateup_swiglu(xn, dec.Mgu, gates=gates)
+        assert torch.equal(y.reshape(B, d_model), ops.spmm(h, dec.Mdown))
+        ref = O.swiglu_mlp(to_np(xn), spec["gate_up"], spec["down"], gates=gates.cpu().numpy())
+        assert_close_bf16(to_np(y).reshape(B, d_model), ref["y"], f"B={B}", ulps=8)
+
+
 def test_fused_router_limits(dev):
     T = lambda *s: torch.zeros(s, dtype=torch.float32, device=dev)
     x = torch.zeros((65, 64), dtype=torch.bfloat16, device=dev)
