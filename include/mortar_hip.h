@@ -185,7 +185,9 @@ int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *sched, const uint16_
  * Routed skipping (optional): tok_cnt/tok_list from mortar_remoe_route with tile = mortar_route_tile(Cb, M); when
  * given (requires cluster_size % 16 == 0 and mortar_route_tile != 0) only active (token, block-row) tiles are
  * computed and written; inactive entries of h are left untouched and must be masked by the consumer
- * (mortar_spmm_bf16_masked). */
+ * (mortar_spmm_bf16_masked).  Without the lists, calls of M <= 64 rows with gates and cluster_size % 16 == 0 still
+ * leave out every unit whose cluster has no positive gate among the tokens of its 4- or 16-token tile, and write
+ * zeros for it (the value the gates produce), so h is fully written. */
 int mortar_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M,
                               int64_t ldx, uint16_t *h, int64_t ldh, const float *gates, int32_t n_clusters,
                               const int32_t *tok_cnt, const uint8_t *tok_list, void *stream);
