@@ -486,11 +486,12 @@ def test_decode_gather_flags_worklist(dev):
     assert_close_bf16(to_np(y), ref["y"], "flagged decode", ulps=8)
 
 
-@pytest.mark.parametrize("B,n_layers", [(3, 5), (12, 5), (2, 300)])
-def test_layer_stack_matches_single_launches(dev, B, n_layers):
+@pytest.mark.parametrize("B,n_layers,d_model", [(3, 5, 256), (12, 5, 256), (2, 300, 256), (12, 300, 1024)])
+def test_layer_stack_matches_single_launches(dev, B, n_layers, d_model):
     """Layer-batched launch: n layers in one launch match n separate launches (to fp32 summation order: the
-    single-matrix launches split a row's K segments over several waves) and the oracle."""
-    d_model, d_ff = 256, 16 * 380                                                    # down is K-segmented
+    single-matrix launches split a row's K segments over several waves) and the oracle.  The last case has enough
+    workgroups for the K-segmented `down` kernel to give every wave two row units."""
+    d_ff = 16 * 380                                                                  # down is K-segmented
     specs = [synth.synth_mlp(d_model, d_ff, 0.25, seed=500 + i, zipf_s=1.2) for i in range(min(n_layers, 5))]
     packs = [(synth.to_pack(s["gate_up"], dev), synth.to_pack(s["down"], dev)) for s in specs]
     packs = [packs[i % len(packs)] for i in range(n_layers)]
