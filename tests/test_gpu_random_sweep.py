@@ -1,0 +1,148 @@
+"""Seeded random sweeps of the GPU entry points against the oracle: shapes, densities, row counts, K segment widths,
+scale modes and gating drawn at random (fixed seeds), so that combinations no hand-written case names are exercised.
+Each failing case prints its configuration.  The bars are those of test_gpu_parity.py."""
+import numpy as np
+import pytest
+import torch
+
+from mortar_amd import ops, synth
+from mortar_amd.pack import MortarPack, decode_blocks
+from oracle import mortar_oracle as O
+from util import assert_close_bf16, oracle_spmm, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _pack(m, dev, **kw):
+    return MortarPack(synth.flat_pack(m["codes"]), m["scales"], m["col_idx"], m["offsets"], m["shape"][0], m["shape"][1], dev, **kw)
+
+
+@pytest.mark.parametrize("seed", [101, 102])
+def test_random_mlp_shapes_prefill_and_decode_tiles(dev, seed):
+    """gate_up + SwiGLU, down, plain gate_up product, gated and list-routed gate_up, masked down."""
+    rng = np.random.default_rng(seed)
+    for it in range(40):
+        dm_b = int(rng.choice([1, 2, 3, 5, 8, 16, 30, 48, 77, 78, 128, 155, 156, 200]))
+        dff_b = int(rng.choice([1, 2, 4, 7, 16, 22, 40, 64, 130, 352]))
+        if dm_b * dff_b > 352 * 48:
+            dff_b = 22
+        cfg = dict(it=it, d_model=dm_b * 16, d_ff=dff_b * 16, dens=float(rng.choice([0.05, 0.1, 0.25, 0.5, 1.0])),
+                   zipf=None if rng.random() < 0.5 else 1.2,
+                   M=int(rng.choice([1, 2, 3, 4, 5, 8, 15, 16, 17, 31, 32, 33, 63, 64, 65, 96, 127, 129, 200, 257])),
+                   seg=None if rng.random() < 0.6 else int(rng.integers(1, 80)), uniform=bool(rng.random() < 0.25),
+                   stream4=bool(rng.random() < 0.7), seed=int(rng.integers(1, 10000)))
+        what = f"seed {seed} case {cfg}"
+        spec = synth.synth_mlp(cfg["d_model"], cfg["d_ff"], cfg["dens"], seed=cfg["seed"], zipf_s=cfg["zipf"])
+        if cfg["uniform"]:
+            spec["gate_up"]["scales"], spec["down"]["scales"] = np.float32(0.05), np.float32(0.03)
+        M = cfg["M"]
+        x = synth.synth_x(M, cfg["d_model"], cfg["seed"] + 1)
+        xd = to_dev(x, dev)
+        Wgu = _pack(spec["gate_up"], dev, seg_cb=cfg["seg"], prefill_stream=cfg["stream4"])
+        Wdn = _pack(spec["down"], dev, seg_cb=cfg["seg"], prefill_stream=cfg["stream4"])
+        ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
+        h = ops.gateup_swiglu(xd, Wgu)
+        assert_close_bf16(to_np(h), ref["h"], what + " h", ulps=8)
+        assert_close_bf16(to_np(ops.spmm(h, Wdn)), oracle_spmm(to_np(h), spec["down"]), what + " y", ulps=8)
+        assert_close_bf16(to_np(ops.spmm(xd, Wgu)), oracle_spmm(x, spec["gate_up"]), what + " gu", ulps=8)
+        ncl, k = dff_b, max(1, dff_b // 3)
+        logits = synth.synth_logits(M, ncl, cfg["seed"] + 2)
+        g_ref, act_ref = O.remoe_gates(logits, k)
+        gates, active = ops.remoe_gates(torch.from_numpy(logits).to(dev), k)
+        assert np.array_equal(active.cpu().numpy().astype(bool), act_ref), what
+        refg = O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=g_ref)
+        hg = ops.gateup_swiglu(xd, Wgu, gates=gates)
+        assert_close_bf16(to_np(hg), refg["h"], what + " h gated", ulps=8)
+        tile = ops.route_tile(Wgu, M)
+        if tile:
+            hs = torch.full_like(hg, float("nan"))
+            ops.gateup_swiglu(xd, Wgu, gates=gates, route=ops.remoe_route(active, tile), out=hs)
+            on = np.repeat(act_ref, 16, axis=1)
+            a, b = to_np(hs), to_np(hg)
+            assert np.array_equal(a[on], b[on]) and np.isnan(a[~on]).all(), what + " routed tiles"
+            ym = ops.spmm(hs, Wdn, active=active)
+        else:
+            ym = ops.spmm(hg, Wdn, active=active)
+        assert_close_bf16(to_np(ym), refg["y"], what + " y routed", ulps=16)
+
+
+@pytest.mark.parametrize("seed", [201, 202])
+def test_random_decode_entry_points(dev, seed):
+    """Small-tile launches, the work-list GEMV with gather flags and partial slots (bf16 and fp32 arithmetic), layer stacks."""
+    rng = np.random.default_rng(seed)
+    for it in range(60):
+        dm_b = int(rng.choice([1, 2, 3, 8, 16, 32, 48, 77, 128, 160, 200]))
+        ncl, cs_b = int(rng.choice([1, 2, 4, 8, 11, 22])), int(rng.choice([1, 1, 2, 4]))
+        dff_b = ncl * cs_b
+        cfg = dict(it=it, d_model=dm_b * 16, d_ff=dff_b * 16, ncl=ncl, dens=float(rng.choice([0.05, 0.1, 0.25, 0.5, 1.0])),
+                   zipf=None if rng.random() < 0.5 else 1.2, B=int(rng.choice([1, 2, 3, 4, 5, 8, 15, 16, 17, 31, 32, 33, 48, 64])),
+                   mb=None if rng.random() < 0.5 else int(rng.integers(1, 12)), uniform=bool(rng.random() < 0.25),
+                   seed=int(rng.integers(1, 10000)), n_layers=int(rng.choice([1, 2, 7])))
+        what = f"seed {seed} case {cfg}"
+        B, mb = cfg["B"], cfg["mb"]
+        spec = synth.synth_mlp(cfg["d_model"], cfg["d_ff"], cfg["dens"], seed=cfg["seed"], zipf_s=cfg["zipf"])
+        if cfg["uniform"]:
+            spec["gate_up"]["scales"], spec["down"]["scales"] = np.float32(0.05), np.float32(0.03)
+        x = synth.synth_x(B, cfg["d_model"], cfg["seed"] + 1)
+        xd = to_dev(x, dev)
+        Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+        g_ref, _ = O.remoe_gates(synth.synth_logits(B, ncl, cfg["seed"] + 2), max(1, ncl // 3))
+        gates = torch.from_numpy(g_ref).to(dev)
+        ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
+        refg = O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=g_ref)
+        h = ops.gemv(xd, Wgu, swiglu_out=True)
+        assert_close_bf16(to_np(h), ref["h"], what + " h", ulps=8)
+        assert_close_bf16(to_np(ops.gemv(h, Wdn)), oracle_spmm(to_np(h), spec["down"]), what + " y", ulps=8)
+        ract, cact = ops.route_flags(gates, cfg["d_ff"])
+        hg = ops.gemv(xd, Wgu, swiglu_out=True, gates=gates, row_act=ract, max_blocks=mb)
+        assert_close_bf16(to_np(hg), refg["h"], what + " h flagged", ulps=8)
+        assert_close_bf16(to_np(ops.gemv(hg, Wdn, col_act=cact, max_blocks=mb)), refg["y"], what + " y flagged", ulps=16)
+        assert_close_bf16(to_np(ops.gemv(xd, Wgu, swiglu_out=True, max_blocks=mb if mb else 5)), ref["h"], what + " h partial", ulps=8)
+        gm = spec["gate_up"]
+        sc = np.broadcast_to(gm["scales"], (int(gm["offsets"][-1]),)) if cfg["uniform"] else gm["scales"]
+        gu64 = O.mortar_gemv(x, gm["codes"], sc, gm["col_idx"], gm["offsets"]).astype(np.float64)
+        got = ops.gemv_f32(torch.from_numpy(x).to(dev), Wgu, max_blocks=mb).cpu().numpy()
+        assert np.abs(got - gu64).max() <= 3e-6 * max(np.abs(gu64).max(), 1e-30), what + " gemv_f32"
+        if B <= 16:
+            n = cfg["n_layers"]
+            hs = [torch.empty((B, cfg["d_ff"]), dtype=torch.bfloat16, device=dev) for _ in range(n)]
+            ys = [torch.empty((B, cfg["d_model"]), dtype=torch.bfloat16, device=dev) for _ in range(n)]
+            ops.LayerStack([Wgu] * n, [xd] * n, hs, swiglu=True).run()
+            ops.LayerStack([Wdn] * n, hs, ys, swiglu=False).run()
+            assert_close_bf16(to_np(hs[-1]), ref["h"], what + " stack h", ulps=8)
+            assert_close_bf16(to_np(ys[-1]), oracle_spmm(to_np(hs[-1]), spec["down"]), what + " stack y", ulps=8)
+
+
+@pytest.mark.parametrize("seed", [301])
+def test_random_backward_products(dev, seed):
+    """dW on the topology and dX through the transposed pack after a device re-pack."""
+    rng = np.random.default_rng(seed)
+    for it in range(60):
+        Rb = int(rng.choice([1, 2, 3, 7, 16, 31, 32, 33, 40, 64, 70, 128]))
+        Cb = int(rng.choice([1, 2, 5, 16, 43, 44, 45, 48, 88, 89, 128, 200, 352]))
+        if Rb * Cb > 128 * 128:
+            Rb = 16
+        cfg = dict(it=it, Rb=Rb, Cb=Cb, dens=float(rng.choice([0.03, 0.1, 0.25, 0.5, 1.0])), zipf=None if rng.random() < 0.5 else 1.2,
+                   M=int(rng.choice([1, 2, 15, 16, 17, 31, 33, 64, 100, 255, 256, 257, 511, 700])), per_block=bool(rng.random() < 0.5),
+                   seed=int(rng.integers(1, 10000)))
+        what = f"seed {seed} case {cfg}"
+        M = cfg["M"]
+        m = synth.synth_matrix(Rb * 16, Cb * 16, cfg["dens"], seed=cfg["seed"], zipf_s=cfg["zipf"])
+        a, b = synth.synth_x(M, Rb * 16, seed=cfg["seed"] + 1), synth.synth_x(M, Cb * 16, seed=cfg["seed"] + 2)
+        got = to_np(ops.sdd(to_dev(a, dev), to_dev(b, dev), synth.to_pack(m, dev)))
+        assert_close_bf16(got, O.sdd_at_b(O.bf16_round(a), O.bf16_round(b), m["row_idx"], m["col_idx"]), what + " dW")
+        nnz = m["col_idx"].size
+        g = np.random.Generator(np.random.PCG64(cfg["seed"] + 3))
+        v = g.standard_normal((nnz, 16, 16), dtype=np.float32) * g.uniform(0.01, 0.1, (nnz, 1, 1)).astype(np.float32)
+        vt = torch.from_numpy(v).to(torch.bfloat16).to(dev)
+        W = MortarPack(None, None, m["col_idx"], m["offsets"], Rb * 16, Cb * 16, dev)
+        s = W.requantize(vt, per_block=cfg["per_block"]).cpu().numpy()
+        Wt = W.transposed()
+        Wt.requantize(vt, per_block=cfg["per_block"], transpose=True)
+        cw = decode_blocks(W.codes.cpu().numpy().view(np.uint32))
+        dense = O.to_dense(cw.astype(np.float32) * O.bf16_round(np.broadcast_to(s, (nnz,)))[:, None, None], m["row_idx"], m["col_idx"],
+                           (Rb * 16, Cb * 16)).astype(np.float64)
+        assert_close_bf16(to_np(ops.spmm(to_dev(a, dev), Wt)), (O.bf16_round(a).astype(np.float64) @ dense).astype(np.float32),
+                          what + " dX", ulps=8)
+        assert_close_bf16(to_np(ops.spmm(to_dev(b, dev), W)), (O.bf16_round(b).astype(np.float64) @ dense.T).astype(np.float32),
+                          what + " y", ulps=8)
