@@ -787,12 +787,13 @@ inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
     const bool wide = (int64_t)layers * p.n_units >= 8 * 512;
     int upw = 1;
     if (MT <= 16 && wide) {
-        // up to 4 units per wave (fewer workgroups, each staging its tile once), but never so few workgroups that
-        // the launch cannot fill the chip's resident slots about once: a second, mostly empty round is what a
-        // count just above the slot count costs, and half-empty CUs what a count far below it costs
+        // up to 4 units per wave, 8 for the 16-token tile whose staging costs more (fewer workgroups, each staging
+        // its tile once), but never so few workgroups that the launch cannot fill the chip's resident slots about
+        // once: a second, mostly empty round is what a count just above the slot count costs, and half-empty CUs
+        // what a count far below it costs
         const int by_lds = (160 * 1024) / (tile_bytes(MT, p.Cb) + LDS_EXTRA), by_waves = 32 / WAVES;
         const int64_t slots = 256 * (int64_t)(by_lds < by_waves ? by_lds : by_waves);
-        for (upw = 4; upw > 1; --upw)
+        for (upw = MT == 16 ? 8 : 4; upw > 1; --upw)
             if ((int64_t)layers * p.n_mtiles * ((p.n_units + WAVES * upw - 1) / (WAVES * upw)) * 10 >= slots * 9) break;
     }
     const int target = MT <= 16 ? 256 * 12 : 256;
