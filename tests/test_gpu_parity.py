@@ -514,6 +514,19 @@ def test_layer_stack_matches_single_launches(dev, B, n_layers, d_model):
                        [torch.empty((17, d_ff), dtype=torch.bfloat16, device=dev)], swiglu=True)
 
 
+@pytest.mark.parametrize("B", [1, 4, 16])
+def test_decode_rows_wider_than_any_resident_tile(dev, B):
+    """in_features so wide (> 19904) that no 4-token tile of all K fits in LDS: gemv() takes the work-list kernel (K split
+    over workgroups, partial sums combined) and the plain SpMM entry point still gives the same product."""
+    m = synth.synth_matrix(16 * 6, 16 * 1300, 0.1, seed=64, zipf_s=1.2)
+    W = synth.to_pack(m, dev)
+    assert ops.route_tile(W, 1) == 0 and W.nseg > 8
+    x = synth.synth_x(B, 16 * 1300, 65)
+    ref = oracle_spmm(x, m)
+    assert_close_bf16(to_np(ops.gemv(to_dev(x, dev), W)), ref, "work-list", ulps=8)
+    assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), ref, "K-segmented SpMM", ulps=8)
+
+
 @pytest.mark.parametrize("max_blocks", [3, 8])
 def test_decode_split_rows_partials(dev, max_blocks):
     spec = synth.synth_mlp(512, 16 * 90, 0.3, seed=60, zipf_s=1.2)
