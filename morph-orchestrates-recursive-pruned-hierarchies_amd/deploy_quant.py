@@ -8,45 +8,49 @@ from torch import Tensor, nn
 __all__ = ["pack_ternary_codes", "unpack_ternary", "_ternary_quantize", "_ternary_quantize_per_block",
            "pack_mortar_ternary", "shrink_mlp_to_mortar_ternary"]
 
-_SHIFTS = torch.tensor([0, 2, 4, 6], dtype=torch.uint8)
+_CODES_PER_BYTE = 4
+_PLACE = (1, 4, 16, 64)          # value of a code in slot 0..3 of its byte (2 bits each, slot 0 lowest)
 
 
 def pack_ternary_codes(q: Tensor) -> Tensor:
-    """{-1,0,+1} -> uint8, 4 codes/byte, stored value = code + 1, little-endian in the byte, length padded
-    to a multiple of 4 with zeros.  Reference: deploy_quant.py:56-71."""
-    flat = q.reshape(-1)
-    pad = (-flat.numel()) % 4
-    u = (flat.to(torch.int16) + 1).to(torch.uint8)
-    if pad:
-        u = torch.cat([u, torch.zeros(pad, dtype=torch.uint8, device=u.device)])
-    u = u.view(-1, 4)
-    return (u[:, 0] | (u[:, 1] << 2) | (u[:, 2] << 4) | (u[:, 3] << 6)).contiguous()
+    """{-1,0,+1} -> uint8, 4 codes per byte: byte = sum of (code + 1) * 4**slot over its four slots, flat order, the tail
+    padded with stored value 0.  Same bytes as the reference's packer (deploy_quant.py:56-71)."""
+    stored = q.reshape(-1).to(torch.int32) + 1
+    n_bytes = -(-stored.numel() // _CODES_PER_BYTE)
+    slots = stored.new_zeros(n_bytes * _CODES_PER_BYTE)
+    slots[:stored.numel()] = stored
+    place = torch.tensor(_PLACE, dtype=torch.int32, device=stored.device)
+    return (slots.view(n_bytes, _CODES_PER_BYTE) * place).sum(dim=1).to(torch.uint8)
 
 
 def unpack_ternary(packed: Tensor, numel: int, dtype: torch.dtype) -> Tensor:
-    """Inverse of pack_ternary_codes.  Reference: deploy_quant.py:74-78."""
-    u = (packed.unsqueeze(-1) >> _SHIFTS.to(packed.device)) & 3
-    return u.reshape(-1)[:numel].to(dtype) - 1.0
+    """The first ``numel`` codes of a pack_ternary_codes buffer as {-1,0,+1} in ``dtype`` (deploy_quant.py:74-78)."""
+    b = packed.reshape(-1).to(torch.int32)
+    stored = torch.stack([(b // p) % 4 for p in _PLACE], dim=1).reshape(-1)[:numel]
+    return stored.to(dtype) - 1.0
+
+
+def _ternary_codes(w: Tensor, scale: Tensor, threshold: float) -> Tensor:
+    """sign(w / scale) where |w / scale| exceeds the threshold, else 0 (the quotient is formed first, as the reference
+    does, so that values at the threshold round the same way)."""
+    ratio = w / scale
+    return torch.where(ratio.abs() > threshold, torch.sign(ratio), torch.zeros_like(ratio)).to(torch.int8)
 
 
 def _ternary_quantize(w: Tensor, threshold: float = 0.5) -> tuple[Tensor, Tensor]:
-    """Per-tensor symmetric ternary: scale = mean|w| (clamp 1e-8), q = sign(w/s) * (|w/s| > threshold).
+    """Per-tensor symmetric ternary: scale = mean|w| (at least 1e-8), codes as _ternary_codes.
     Reference: deploy_quant.py:81-95; block_sparse.py:909-919."""
-    wf = w.detach().float()
-    scale = wf.abs().mean().clamp(min=1e-8)
-    wn = wf / scale
-    q = (torch.sign(wn) * (wn.abs() > threshold)).to(torch.int8)
-    return q, scale
+    w32 = w.detach().float()
+    scale = w32.abs().mean().clamp(min=1e-8)
+    return _ternary_codes(w32, scale, threshold), scale
 
 
 def _ternary_quantize_per_block(w: Tensor, threshold: float = 0.5) -> tuple[Tensor, Tensor]:
-    """The same rule with one scale per [blk, blk] block (mean|w| per block, clamp 1e-6), the per-tile form
+    """The same rule with one scale per [blk, blk] block (mean|w| per block, at least 1e-6), the per-tile form
     of block_sparse.py:341-349,393-401 applied to carved blocks.  w [nnz, blk, blk] -> (codes, scale [nnz])."""
-    wf = w.detach().float()
-    scale = wf.abs().mean(dim=(1, 2)).clamp(min=1e-6)
-    wn = wf / scale[:, None, None]
-    q = (torch.sign(wn) * (wn.abs() > threshold)).to(torch.int8)
-    return q, scale
+    w32 = w.detach().float()
+    scale = w32.abs().mean(dim=(1, 2)).clamp(min=1e-6)
+    return _ternary_codes(w32, scale[:, None, None], threshold), scale
 
 
 def pack_mortar_ternary(cms: nn.Module, threshold: float = 0.5, per_block: bool = False) -> dict:
