@@ -296,7 +296,7 @@ def main() -> None:
         out["decode_cold"] = cold
         # ---- decode, layer-batched: the 160 weight sets in TWO launches (gate_up stack, down stack) ---------
         stack = {}
-        for B in (1, 4, 16):
+        for B in (1, 4, 16, 64):
             xb = x[:B].contiguous()
             hs = [torch.empty((B, D_FF), dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
             ys = [torch.empty((B, D_MODEL), dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]

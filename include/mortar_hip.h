@@ -265,7 +265,7 @@ int mortar_router_bf16(const void *x, int32_t x_is_f32, int64_t B, int32_t d, in
  * from HBM once per launch.  That path replaces mortar_gemv (fused_decode_step.py:1502-1547, kernels :1341-1459)
  * for the MLP pair as the engine calls it (morph/inference/engine.py:980-986).
  *
- * Layer-batched form for M <= 16: ONE launch runs the same operation on n_layers independent
+ * Layer-batched form for M <= 64 (one to four 16-token tiles per layer): ONE launch runs the same operation on n_layers independent
  * (matrix, input, output) triples of identical shape (Rb, Cb, seg_cb).  No counterpart in the reference, which
  * issues one mortar_gemv per matrix (morph/inference/engine.py:980-986); this is for callers that hold many weight
  * sets whose inputs are known (several models, a stack probed for bandwidth).

@@ -240,7 +240,7 @@ extern "C" int mortar_stack_prepare(int32_t swiglu, int32_t n_layers, const mort
                                     int64_t M, int64_t ldx, int64_t ldy, void *table_dev, void *stream) {
     if (n_layers <= 0 || n_layers > 65535 || !W || !x || !y || !table_dev)
         return mortar_fail(MORTAR_ERR_ARG, "stack_prepare: bad arguments");
-    if (M > 16) return mortar_fail(MORTAR_ERR_LIMIT, "stack_prepare: layer-batched launches serve M <= 16 (got %lld)", (long long)M);
+    if (M > 64) return mortar_fail(MORTAR_ERR_LIMIT, "stack_prepare: layer-batched launches serve M <= 64 (got %lld)", (long long)M);
     std::vector<SpmmParams> tab((size_t)n_layers);
     for (int l = 0; l < n_layers; ++l) {
         if (W[l].Rb != W[0].Rb || W[l].Cb != W[0].Cb || W[l].seg_cb != W[0].seg_cb)
@@ -267,7 +267,7 @@ extern "C" int mortar_stack_prepare(int32_t swiglu, int32_t n_layers, const mort
 
 extern "C" int mortar_stack_run(int32_t swiglu, int32_t n_layers, const mortar_bcsr_t *W0, int64_t M,
                                 const void *table_dev, void *stream) {
-    if (n_layers <= 0 || n_layers > 65535 || !W0 || !table_dev || M <= 0 || M > 16)
+    if (n_layers <= 0 || n_layers > 65535 || !W0 || !table_dev || M <= 0 || M > 64)
         return mortar_fail(MORTAR_ERR_ARG, "stack_run: bad arguments");
     SpmmParams p;
     fill(p, W0, nullptr, nullptr, M, 0, nullptr, 0);

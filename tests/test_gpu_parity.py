@@ -486,7 +486,8 @@ def test_decode_gather_flags_worklist(dev):
     assert_close_bf16(to_np(y), ref["y"], "flagged decode", ulps=8)
 
 
-@pytest.mark.parametrize("B,n_layers,d_model", [(3, 5, 256), (12, 5, 256), (2, 300, 256), (12, 300, 1024)])
+@pytest.mark.parametrize("B,n_layers,d_model", [(3, 5, 256), (12, 5, 256), (2, 300, 256), (12, 300, 1024), (40, 5, 256),
+                                                  (64, 40, 1024)])
 def test_layer_stack_matches_single_launches(dev, B, n_layers, d_model):
     """Layer-batched launch: n layers in one launch match n separate launches (to fp32 summation order: the
     single-matrix launches split a row's K segments over several waves) and the oracle.  The last case has enough
@@ -510,8 +511,8 @@ def test_layer_stack_matches_single_launches(dev, B, n_layers, d_model):
     ref = O.swiglu_mlp(to_np(xs[1]), specs[1]["gate_up"], specs[1]["down"])
     assert_close_bf16(to_np(ys[1]), ref["y"], "stack vs oracle", ulps=8)
     with pytest.raises(ValueError):
-        ops.LayerStack([packs[0][0]], [to_dev(synth.synth_x(17, d_model, 1), dev)],
-                       [torch.empty((17, d_ff), dtype=torch.bfloat16, device=dev)], swiglu=True)
+        ops.LayerStack([packs[0][0]], [to_dev(synth.synth_x(65, d_model, 1), dev)],
+                       [torch.empty((65, d_ff), dtype=torch.bfloat16, device=dev)], swiglu=True)
 
 
 @pytest.mark.parametrize("B", [1, 4, 16])
