@@ -91,8 +91,29 @@ static int launch_partsplit(int kind, SpmmParams &p, hipStream_t st) {
     return -1;
 }
 
+// Layer-batched launches of 17..64 rows run the 32-token prefill tiles (one unpack feeds two MFMAs) when the shape has
+// one: 1 = resident tile, 2 = K-segmented (plain products only), 0 = none (16-token tiles serve the rows).  They keep
+// reading the 2-bit stream: the 4-bit one (two instructions less per block pair, twice the bytes) was measured no
+// faster for 160 layers at 32 and 64 rows.
+static int stack_tile32(int kind, const SpmmParams &p) {
+    // 17..32 and 49..64 rows: one or two 32-token tiles instead of two or four 16-token ones (33..48 rows would leave
+    // the second 32-token tile half empty: three 16-token tiles cost the same there)
+    if (p.M <= 16 || (p.M > 32 && p.M <= 48) || kind > 1) return 0;
+    if (p.nseg == 1 && fits(32, p.Cb)) return 1;
+    if (kind == 0 && p.nseg > 1 && fits(32, p.seg_cb)) return 2;
+    return 0;
+}
+
 template <int CODE>
 static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
+    if (table) {
+        switch (stack_tile32(kind, p)) {
+            case 1:
+                if (kind == 0) return mortar_launch_resident<32, 1, false, 16, true, CODE>(p, table, layers, st);
+                return mortar_launch_resident<32, 2, false, 16, true, CODE>(p, table, layers, st);
+            case 2: return mortar_launch_segmented<32, 1, false, 16, 4, true, CODE>(p, table, layers, st);
+        }
+    }
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
     if (t == 0) return -1;
     const bool resident = t > 0;
@@ -117,7 +138,12 @@ int mortar_smallm_launch(int kind, SpmmParams &p, const SpmmParams *table, int l
                            : smallm_launch_code<CODE_2BIT>(kind, p, table, layers, st);
 }
 
+
 int mortar_smallm_shape(int kind, SpmmParams &p, int layers) {
+    switch (stack_tile32(kind, p)) {       // table launches only: the choice of smallm_launch_code
+        case 1: mortar_resident_shape<32, 16>(p, layers); return MORTAR_OK;
+        case 2: mortar_segmented_shape<32, 16, 4>(p, layers); return MORTAR_OK;
+    }
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
     if (t == 0) return mortar_fail(MORTAR_ERR_LIMIT, "shape has no small-M kernel");
     const int w = pick_waves(t, p, layers);
