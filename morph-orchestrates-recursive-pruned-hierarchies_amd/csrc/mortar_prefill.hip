@@ -68,11 +68,24 @@ int launch_resident_any(SpmmParams &p, hipStream_t st) {
 
 constexpr int SEG_WAVES = 16, SEG_UPW = 4;
 
+// Row units per wave of the K-segmented plain product: 4 when the token tiles alone fill the chip; with fewer tiles
+// 2 or 1, so that more workgroups share a tile's rows (64 units per workgroup left 8 workgroups for 128 tokens).
+int segmented_upw(const SpmmParams &p) {
+    const int64_t tiles = (p.M + 31) / 32;
+    for (int upw = SEG_UPW; upw > 1; upw >>= 1)
+        if (tiles * ((p.n_units + SEG_WAVES * upw - 1) / (SEG_WAVES * upw)) >= 224) return upw;
+    return 1;
+}
+
 template <int CODE>
 int dispatch_prefill(int kind, SpmmParams &p, hipStream_t st) {
     switch (kind) {
         case 0:
             if (p.nseg == 1) return launch_resident_any<1, false, CODE>(p, st);
+            switch (segmented_upw(p)) {
+                case 1: return mortar_launch_segmented<32, 1, false, SEG_WAVES, 1, false, CODE>(p, nullptr, 1, st);
+                case 2: return mortar_launch_segmented<32, 1, false, SEG_WAVES, 2, false, CODE>(p, nullptr, 1, st);
+            }
             return mortar_launch_segmented<32, 1, false, SEG_WAVES, SEG_UPW, false, CODE>(p, nullptr, 1, st);
         case 1:
             if (p.nseg == 1) return launch_resident_any<2, false, CODE>(p, st);
@@ -80,6 +93,10 @@ int dispatch_prefill(int kind, SpmmParams &p, hipStream_t st) {
         case 2:
             return launch_resident_any<2, true, CODE>(p, st);
         default:
+            switch (segmented_upw(p)) {
+                case 1: return mortar_launch_segmented<32, 1, true, SEG_WAVES, 1, false, CODE>(p, nullptr, 1, st);
+                case 2: return mortar_launch_segmented<32, 1, true, SEG_WAVES, 2, false, CODE>(p, nullptr, 1, st);
+            }
             return mortar_launch_segmented<32, 1, true, SEG_WAVES, SEG_UPW, false, CODE>(p, nullptr, 1, st);
     }
 }

@@ -796,8 +796,10 @@ inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
         for (upw = MT == 16 ? 8 : 4; upw > 1; --upw)
             if ((int64_t)layers * p.n_mtiles * ((p.n_units + WAVES * upw - 1) / (WAVES * upw)) * 10 >= slots * 9) break;
     }
+    // prefill tiles: never more workgroups than CUs (one workgroup fills a CU's LDS, so 264 of them take two rounds
+    // where 252 take one)
     const int target = MT <= 16 ? 256 * 12 : 256;
-    int split = (target + layers * p.n_mtiles - 1) / (layers * p.n_mtiles);
+    int split = MT <= 16 ? (target + layers * p.n_mtiles - 1) / (layers * p.n_mtiles) : target / (layers * p.n_mtiles);
     const int max_split = (p.n_units + WAVES * upw - 1) / (WAVES * upw);
     split = split < 1 ? 1 : (split > max_split ? max_split : split);
     p.n_split = split;
