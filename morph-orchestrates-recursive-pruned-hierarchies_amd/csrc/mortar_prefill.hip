@@ -68,13 +68,20 @@ int launch_resident_any(SpmmParams &p, hipStream_t st) {
 
 constexpr int SEG_WAVES = 16, SEG_UPW = 4;
 
-// Row units per wave of the K-segmented plain product: 4 when the token tiles alone fill the chip; with fewer tiles
-// 2 or 1, so that more workgroups share a tile's rows (64 units per workgroup left 8 workgroups for 128 tokens).
+// Row units per wave of the K-segmented plain product: 4, 2 or 1.  Fewer units per wave mean more workgroups per token
+// tile (64 units per workgroup left 8 workgroups for 128 tokens) but every workgroup stages the tile's segments again,
+// and workgroups beyond the 256 CUs wait for a second round: take the choice with the least rounds x (staging + units),
+// staging weighing about three units.
 int segmented_upw(const SpmmParams &p) {
     const int64_t tiles = (p.M + 31) / 32;
-    for (int upw = SEG_UPW; upw > 1; upw >>= 1)
-        if (tiles * ((p.n_units + SEG_WAVES * upw - 1) / (SEG_WAVES * upw)) >= 224) return upw;
-    return 1;
+    int best = SEG_UPW;
+    int64_t best_cost = 0;
+    for (int upw = SEG_UPW; upw >= 1; upw >>= 1) {
+        const int64_t wgs = tiles * ((p.n_units + SEG_WAVES * upw - 1) / (SEG_WAVES * upw));
+        const int64_t cost = ((wgs + 255) / 256) * (3 + upw);
+        if (upw == SEG_UPW || cost < best_cost) { best = upw; best_cost = cost; }
+    }
+    return best;
 }
 
 template <int CODE>
