@@ -25,9 +25,9 @@ PEAK_BF16_TFLOPS, PEAK_HBM_GBS = 2500.0, 8000.0
 # HBM-side bytes per launch (read + written) measured with `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` on this
 # workload and calibrated on a plain copy; the runs and factors are in profiles/bench_prefill_step_hbm_traffic_pmc.md
 # and profiles/bench_all_legs_hbm_traffic_pmc.md.  Not measured live: counters need the profiler.
-TRAFFIC_GATE_UP_BYTES = 41.59e6 + 51.24e6
+TRAFFIC_GATE_UP_BYTES = 41.59e6 + 51.19e6
 TRAFFIC_DOWN_BYTES = 60.39e6 + 17.78e6
-TRAFFIC_DECODE_STACK_BYTES = (262.99e6 + 4.54e6) + (168.47e6 + 2.03e6)   # gate_up + down launches, 160 layers, b = 1
+TRAFFIC_DECODE_STACK_BYTES = (263.04e6 + 4.54e6) + (168.48e6 + 2.04e6)   # gate_up + down launches, 160 layers, b = 1
 TRAFFIC_SOURCE = ("constant from profiles/bench_prefill_step_hbm_traffic_pmc.md and profiles/bench_all_legs_hbm_traffic_pmc.md "
                   "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command); not measured in this run")
 
