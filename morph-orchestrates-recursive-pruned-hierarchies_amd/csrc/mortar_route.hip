@@ -430,8 +430,8 @@ extern "C" int mortar_router_bf16(const void *x, int32_t x_is_f32, int64_t B, in
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 pg((unsigned)((d + 3) / 4)), blk(256);
 #define MORTAR_PROJ(TB, F) hipLaunchKernelGGL((router_project_kernel<TB, F>), pg, blk, 0, st, x, (int)B, d, ldx, wq, iter_vec, qv)
-    if (x_is_f32) { if (B == 1) MORTAR_PROJ(1, true); else if (B <= 4) MORTAR_PROJ(4, true); else MORTAR_PROJ(8, true); }
-    else { if (B == 1) MORTAR_PROJ(1, false); else if (B <= 4) MORTAR_PROJ(4, false); else MORTAR_PROJ(8, false); }
+    if (x_is_f32) { if (B == 1) MORTAR_PROJ(1, true); else if (B <= 4) MORTAR_PROJ(4, true); else if (B <= 8) MORTAR_PROJ(8, true); else MORTAR_PROJ(16, true); }
+    else { if (B == 1) MORTAR_PROJ(1, false); else if (B <= 4) MORTAR_PROJ(4, false); else if (B <= 8) MORTAR_PROJ(8, false); else MORTAR_PROJ(16, false); }
 #undef MORTAR_PROJ
     int rc = check_launch("router projection");
     if (rc) return rc;
