@@ -404,23 +404,26 @@ int mortar_swiglu_backward_bf16(const uint16_t *gu, int64_t ldg, const uint16_t 
  * carved linear, the reference's stk_sdd_at_b(a, b, data, offsets, row_indices, column_indices) -> [nnz, blk, blk]
  * (morph/sparse/stk/backend/custom_ops.py:78-96; forward y = x W^T: a = dY [M, out], b = x [M, in]).  bf16 operands,
  * fp32 accumulation over the M tokens, bf16 result (round to nearest even).
- *   mortar_sdd_plan_host: the work partition for a topology (host, once).  plan_out = NULL returns the number of
- *     int32 words needed; otherwise fills plan_out (plan_words = its capacity) and returns the words used;
- *     plan_out[0] = n_wg.  Upload the plan to the device.
- *   mortar_sdd_plan_max_groups_host: the largest number of row groups in one K segment of a (host) plan, the
- *     max_groups argument of the launch (it sizes the grid: workgroup ids are laid out per XCD as (token range, row
- *     group) x K segment so that the readers of one slice share an L2).
- *   mortar_sdd_bf16: plan device int32; a bf16 [M, lda >= Rb*16], b bf16 [M, ldb >= Cb*16], 16-byte aligned with
- *     leading dimensions multiples of 8; acc device workspace of mortar_sdd_workspace_bytes(n_wg, nnz, M) bytes,
- *     16-byte aligned (every token range writes its fp32 sums to a slab of its own, and a last pass adds the slabs in
- *     a fixed order: results are reproducible); out device bf16 [nnz,16,16], 16-byte aligned.  M = 0 gives zeros. */
-int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb, int32_t *plan_out,
-                             int64_t plan_words);
-int64_t mortar_sdd_workspace_bytes(int32_t n_wg, int32_t nnz, int64_t M);
-int32_t mortar_sdd_plan_max_groups_host(const int32_t *plan);
-int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t max_groups, int32_t Rb, int32_t Cb, int32_t nnz,
-                    const uint16_t *a, int64_t lda, const uint16_t *b, int64_t ldb, int64_t M, float *acc, uint16_t *out,
-                    void *stream);
+ *   mortar_sdd_blocks_per_wave_host: how many kept blocks one wavefront of a workgroup accumulates (8, 10, ... 22;
+ *     a workgroup of 16 wavefronts owns 16 times as many blocks of a few consecutive block-rows of one K segment),
+ *     chosen for this topology at M tokens: smaller groups fill the chip with fewer token ranges, larger ones stage
+ *     fewer bytes per block.  Any built size gives the same results.
+ *   mortar_sdd_plan_host: the work partition for a topology and a group size (host, once per pair).  plan_out = NULL
+ *     returns the number of int32 words needed; otherwise fills plan_out (plan_words = its capacity) and returns the
+ *     words used; plan_out[0] = n_wg.  Upload the plan to the device.
+ *   mortar_sdd_bf16: plan device int32, with the n_wg and blocks_per_wave it was made for (workgroup ids are laid
+ *     out per XCD as runs of (token range, row group x K segment) so that the readers of one slice share an L2); a bf16
+ *     [M, lda >= Rb*16], b bf16 [M, ldb >= Cb*16], 16-byte aligned with leading dimensions multiples of 8; acc device
+ *     workspace of mortar_sdd_workspace_bytes(n_wg, nnz, blocks_per_wave, M) bytes, 16-byte aligned (every token range
+ *     writes its fp32 sums to a slab of its own, and a last pass adds the slabs in a fixed order: results are
+ *     reproducible); out device bf16 [nnz,16,16], 16-byte aligned.  M = 0 gives zeros. */
+int32_t mortar_sdd_blocks_per_wave_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb, int64_t M);
+int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb, int32_t blocks_per_wave,
+                             int32_t *plan_out, int64_t plan_words);
+int64_t mortar_sdd_workspace_bytes(int32_t n_wg, int32_t nnz, int32_t blocks_per_wave, int64_t M);
+int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t blocks_per_wave, int32_t Rb, int32_t Cb,
+                    int32_t nnz, const uint16_t *a, int64_t lda, const uint16_t *b, int64_t ldb, int64_t M, float *acc,
+                    uint16_t *out, void *stream);
 
 #ifdef __cplusplus
 }

@@ -36,9 +36,9 @@ _SIGS = {
                                   c_vp, c_vp]),
     "mortar_swiglu_bf16": (C.c_int, [c_vp, c_i64, c_i64, c_i32, c_vp, c_i64, c_vp]),
     "mortar_swiglu_backward_bf16": (C.c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_i32, c_vp, c_i64, c_vp]),
-    "mortar_sdd_plan_host": (c_i64, [c_vp, c_vp, c_i32, c_i32, c_vp, c_i64]),
-    "mortar_sdd_workspace_bytes": (c_i64, [c_i32, c_i32, c_i64]),
-    "mortar_sdd_plan_max_groups_host": (c_i32, [c_vp]),
+    "mortar_sdd_blocks_per_wave_host": (c_i32, [c_vp, c_vp, c_i32, c_i32, c_i64]),
+    "mortar_sdd_plan_host": (c_i64, [c_vp, c_vp, c_i32, c_i32, c_i32, c_vp, c_i64]),
+    "mortar_sdd_workspace_bytes": (c_i64, [c_i32, c_i32, c_i32, c_i64]),
     "mortar_sdd_bf16": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_i64, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp]),
     "mortar_prefill_max_seg_cb": (C.c_int, []),
     "mortar_validate_bcsr_host": (C.c_int, [c_vp, c_vp, c_i32, c_i32]),

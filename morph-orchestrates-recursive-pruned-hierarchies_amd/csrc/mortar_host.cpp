@@ -25,7 +25,7 @@ int mortar_fail(int code, const char *fmt, ...) {
 }
 
 extern "C" const char *mortar_last_error(void) { return g_err; }
-extern "C" int mortar_abi_version(void) { return 6; }
+extern "C" int mortar_abi_version(void) { return 7; }
 
 static inline uint16_t f32_to_bf16_bits(float f) {
     uint32_t u;

@@ -28,8 +28,8 @@
 namespace {
 
 constexpr int SDD_WAVES = 16;
-constexpr int SDD_NB = 22;                       // blocks per wavefront (4 accumulator registers each)
-constexpr int SDD_G = SDD_WAVES * SDD_NB;        // blocks per workgroup
+constexpr int SDD_NB_MAX = 22;                   // most blocks per wavefront (4 accumulator registers each)
+constexpr int SDD_NB_SIZES[] = {8, 10, 12, 14, 16, 18, 20, 22};      // the kernels that are built
 constexpr int SDD_RMAX = 32;                     // block-rows per workgroup (slice of a in LDS)
 constexpr int SDD_SEG = 44;                      // block-columns per K segment (slice of b in LDS)
 constexpr int SDD_TARGET_WGS = 256;              // workgroups wanted in flight (one per CU: two slice buffers each)
@@ -38,6 +38,7 @@ constexpr int SDD_CS = 1024 + 32;                // LDS bytes per chunk = 8 toke
 constexpr int SDD_QS = 4 * SDD_CS;               // LDS bytes per quad: 32 tokens
 constexpr int SDD_BUF = (SDD_NQ + SDD_RMAX / 4) * SDD_QS;    // one buffer: the slice of b, then the slice of a
 constexpr int SDD_STEP = 32;                     // tokens per step = K of one MFMA
+constexpr int SDD_SLAB_BLOCKS = 272;             // blocks of one fp32 slab (written, read back) that cost one unit
 #ifndef SDD_PF
 #define SDD_PF 1
 #endif
@@ -53,7 +54,7 @@ struct SddArgs {
     int64_t lda, ldb, M;
     float *acc;
     uint16_t *out;
-    int32_t Cb, tsplit, steps_per_split, nsteps, nnz, max_groups, pairs_per_xcd;
+    int32_t Cb, tsplit, steps_per_split, nsteps, nnz, per_xcd;
 };
 
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
@@ -88,24 +89,23 @@ __device__ __forceinline__ uint32_t lds_addr(const char *p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
 }
 
+template <int SDD_NB>
 __global__ __launch_bounds__(SDD_WAVES * 64) void sdd_kernel(SddArgs p) {
+    constexpr int SDD_G = SDD_WAVES * SDD_NB;        // blocks per workgroup
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Workgroup -> (row group, K segment, token range).  Ids are dealt round-robin over the 8 XCDs, each with its own
-    // L2.  The (token range, row group) pairs are cut into 8 consecutive runs, one per XCD, and the K segments of a pair
-    // sit side by side: the slice of a is then fetched from HBM once (its nseg readers share an L2) and a slice of b
-    // only by the few XCDs that hold its token range.  Combinations that do not exist (a segment with fewer row groups)
-    // are idle ids.
-    const int n_wg = p.plan[0], nseg = p.plan[2];
-    const int32_t *seg_tab = p.plan + p.plan[3];                   // per segment: first workgroup, row groups
+    // Workgroup -> (token range, row group, K segment).  Ids are dealt round-robin over the 8 XCDs, each with its own
+    // L2.  The (token range, workgroup) items, workgroups in the plan's order (row groups of about the same rows side by
+    // side over the K segments), are cut into 8 equal runs, one per XCD: the slice of a is then fetched from HBM once
+    // (its nseg readers share an L2) and a slice of b only by the few XCDs that hold its token range.
+    const int n_wg = p.plan[0];
+    const int32_t *order = p.plan + p.plan[3];
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int pl = slot / nseg, sgi = slot - pl * nseg;
-    const int pair = xcd * p.pairs_per_xcd + pl;
-    if (pl >= p.pairs_per_xcd || pair >= p.tsplit * p.max_groups) return;
-    const int ts = pair / p.max_groups, rg = pair - ts * p.max_groups;
-    if (rg >= seg_tab[2 * sgi + 1]) return;
-    const int wg = seg_tab[2 * sgi] + rg;
+    const int item = xcd * p.per_xcd + slot;
+    if (slot >= p.per_xcd || item >= p.tsplit * n_wg) return;
+    const int ts = item / n_wg;
+    const int wg = order[item - ts * n_wg];
     const int32_t *desc = p.plan + 4 + wg * 4;
     const int row0 = desc[0], nrows = desc[1], seg = desc[2];
     const int seg_cb = p.plan[1];
@@ -224,23 +224,27 @@ __global__ __launch_bounds__(256) void sdd_round_kernel(const float *acc, uint16
 
 }  // namespace
 
-// Plan: {n_wg, seg_cb, nseg, offset of the segment table}, then per workgroup {first row, rows, segment, blocks}, then per (workgroup, wavefront,
-// slot) the block index or -1, then per (workgroup, wavefront, slot) (row - first row) << 20 | LDS byte offset of the
-// tile of (column - segment start); an empty slot repeats the workgroup's last block there; last the segment table:
-// per segment {its first workgroup, its number of row groups} (workgroups are stored segment by segment).
-extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
-                                        int32_t *plan_out, int64_t plan_words) {
-    const int rc = mortar_check_bcsr_host(row_ptr, col, Rb, Cb);
-    if (rc) return rc;
-    const int nseg = (Cb + SDD_SEG - 1) / SDD_SEG;
-    const int seg_cb = ((Cb + nseg - 1) / nseg + 3) & ~3;          // whole 128-byte lines
-    struct Wg { int row0, nrows, seg; std::vector<int32_t> j, o; };
-    std::vector<Wg> wgs;
+// Workgroups of a plan with `nb` blocks per wavefront: per K segment, runs of consecutive block-rows holding at most
+// 16 * nb blocks of the segment and at most SDD_RMAX rows.
+struct SddGroup { int row0, nrows, seg; std::vector<int32_t> j, o; };
+
+static bool sdd_nb_built(int nb) {
+    for (int v : SDD_NB_SIZES) if (v == nb) return true;
+    return false;
+}
+
+static void sdd_groups(const int32_t *row_ptr, const int16_t *col, int Rb, int Cb, int nb, bool fill,
+                       std::vector<SddGroup> &wgs, int &nseg, int &seg_cb) {
+    const int G = SDD_WAVES * nb;
+    nseg = (Cb + SDD_SEG - 1) / SDD_SEG;
+    seg_cb = ((Cb + nseg - 1) / nseg + 3) & ~3;                    // whole 128-byte lines
     for (int sg = 0; sg < nseg; ++sg) {
-        Wg cur{0, 0, sg, {}, {}};
+        SddGroup cur{0, 0, sg, {}, {}};
+        int held = 0;
         auto flush = [&]() {
-            if (!cur.j.empty()) wgs.push_back(cur);
-            cur = Wg{0, 0, sg, {}, {}};
+            if (held) wgs.push_back(cur);
+            cur = SddGroup{0, 0, sg, {}, {}};
+            held = 0;
         };
         for (int r = 0; r < Rb; ++r) {
             int lo = row_ptr[r];
@@ -249,9 +253,11 @@ extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *c
             int hi = lo;
             while (hi < e && col[hi] < (sg + 1) * seg_cb) ++hi;
             if (hi == lo) continue;
-            if (!cur.j.empty() && ((int)cur.j.size() + (hi - lo) > SDD_G || r - cur.row0 + 1 > SDD_RMAX)) flush();
-            if (cur.j.empty()) cur.row0 = r;
+            if (held && (held + (hi - lo) > G || r - cur.row0 + 1 > SDD_RMAX)) flush();
+            if (!held) cur.row0 = r;
             cur.nrows = r - cur.row0 + 1;
+            held += hi - lo;
+            if (!fill) continue;
             for (int j = lo; j < hi; ++j) {
                 cur.j.push_back(j);
                 const int cr = col[j] - sg * seg_cb;
@@ -260,18 +266,81 @@ extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *c
         }
         flush();
     }
+}
+
+// Token ranges for M tokens over the n_wg workgroups of a plan with nb blocks per wavefront.  One workgroup runs per
+// CU and the (range, workgroup) items are dealt evenly over the XCDs, so the launch takes
+// ceil(items per XCD / CUs per XCD) rounds of ceil(steps / ranges) + 1 steps, a step costing nb + 7 units (one per
+// block and wavefront, plus staging and the barrier); every extra range adds one slab of fp32 sums to write and to
+// read back, priced per block.  The constants are a fit to launch times over group sizes, range counts and 1024 to
+// 16384 tokens (4.5 % rms).  Returns the cost of the cheapest count of ranges.
+static int64_t sdd_split(int32_t n_wg, int32_t nnz, int nb, int64_t M, int &nsteps, int &steps_per_split, int &tsplit) {
+    nsteps = (int)((M + SDD_STEP - 1) / SDD_STEP);
+    int best = 1;
+    int64_t best_cost = INT64_MAX;
+    for (int t = 1; t <= std::min(nsteps, 16); ++t) {
+        const int sps = (nsteps + t - 1) / t, tt = (nsteps + sps - 1) / sps;
+        const int64_t per_xcd = ((int64_t)n_wg * tt + 7) / 8;
+        const int64_t rounds = (per_xcd + SDD_TARGET_WGS / 8 - 1) / (SDD_TARGET_WGS / 8);
+        const int64_t cost = rounds * (sps + 1) * (nb + 7) + (tt > 1 ? (int64_t)tt * nnz / SDD_SLAB_BLOCKS : 0);
+        if (cost < best_cost) { best_cost = cost; best = t; }
+    }
+    steps_per_split = std::max(1, (nsteps + best - 1) / best);
+    tsplit = std::max(1, (nsteps + steps_per_split - 1) / steps_per_split);
+    return best_cost;
+}
+
+// Blocks per wavefront for this topology at M tokens: the built size whose plan is cheapest by sdd_split's measure.
+// Fewer blocks per workgroup mean more row groups, which fill the chip with fewer token ranges (fewer slabs), at the
+// price of more staged bytes per block.
+extern "C" int32_t mortar_sdd_blocks_per_wave_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb, int64_t M) {
+    const int rc = mortar_check_bcsr_host(row_ptr, col, Rb, Cb);
+    if (rc) return rc;
+    if (M < 0) return mortar_fail(MORTAR_ERR_ARG, "sdd_blocks_per_wave: M < 0");
+    int best = SDD_NB_MAX;
+    int64_t best_cost = INT64_MAX;
+    for (int nb : SDD_NB_SIZES) {
+        std::vector<SddGroup> wgs;
+        int nseg, seg_cb, nsteps, sps, tsplit;
+        sdd_groups(row_ptr, col, Rb, Cb, nb, false, wgs, nseg, seg_cb);
+        const int64_t cost = sdd_split((int32_t)wgs.size(), row_ptr[Rb], nb, M, nsteps, sps, tsplit);
+        if (cost <= best_cost) { best_cost = cost; best = nb; }      // ties: the larger group (fewer staged bytes)
+    }
+    return best;
+}
+
+// Plan: {n_wg, seg_cb, nseg, offset of the launch order}, then per workgroup {first row, rows, segment, blocks}, then
+// per (workgroup, wavefront, slot) the block index or -1, then per (workgroup, wavefront, slot)
+// (row - first row) << 20 | LDS byte offset of the tile of (column - segment start); an empty slot repeats the
+// workgroup's last block there; last the launch order: the workgroups (stored segment by segment) sorted by their
+// position inside the segment, then by segment, so that row groups of about the same rows are neighbours.
+extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb,
+                                        int32_t blocks_per_wave, int32_t *plan_out, int64_t plan_words) {
+    const int rc = mortar_check_bcsr_host(row_ptr, col, Rb, Cb);
+    if (rc) return rc;
+    if (!sdd_nb_built(blocks_per_wave))
+        return mortar_fail(MORTAR_ERR_ARG, "sdd_plan: blocks_per_wave=%d is not a built size (8, 10, ... 22)", blocks_per_wave);
+    const int SDD_G = SDD_WAVES * blocks_per_wave;
+    std::vector<SddGroup> wgs;
+    int nseg, seg_cb;
+    sdd_groups(row_ptr, col, Rb, Cb, blocks_per_wave, true, wgs, nseg, seg_cb);
     const int64_t n_wg = (int64_t)wgs.size();
     const int64_t tab = 4 + n_wg * 4 + n_wg * SDD_G * 2;          // word offset of the per-segment table
-    const int64_t words = tab + 2 * nseg;
+    const int64_t words = tab + n_wg;
     if (tab > INT32_MAX) return mortar_fail(MORTAR_ERR_LIMIT, "sdd_plan: plan too large");
     if (!plan_out) return words;
     if (plan_words < words) return mortar_fail(MORTAR_ERR_ARG, "sdd_plan: buffer holds %lld words, need %lld",
                                                (long long)plan_words, (long long)words);
     plan_out[0] = (int32_t)n_wg; plan_out[1] = seg_cb; plan_out[2] = nseg; plan_out[3] = (int32_t)tab;
-    {   // workgroups are stored segment by segment: first workgroup and number of row groups of every segment
-        int32_t *st = plan_out + tab;
-        for (int sg = 0; sg < nseg; ++sg) { st[2 * sg] = 0; st[2 * sg + 1] = 0; }
-        for (int64_t w = n_wg - 1; w >= 0; --w) { st[2 * wgs[w].seg] = (int32_t)w; st[2 * wgs[w].seg + 1] += 1; }
+    {
+        std::vector<int> first(nseg + 1, 0);                       // first workgroup of every segment
+        for (int64_t w = 0; w < n_wg; ++w) first[wgs[w].seg + 1] = (int)w + 1;
+        for (int sg = 0; sg < nseg; ++sg) first[sg + 1] = std::max(first[sg + 1], first[sg]);
+        int32_t *order = plan_out + tab;
+        int64_t n = 0;
+        for (int k = 0; n < n_wg; ++k)
+            for (int sg = 0; sg < nseg; ++sg)
+                if (first[sg] + k < first[sg + 1]) order[n++] = first[sg] + k;
     }
     int32_t *ent_j = plan_out + 4 + n_wg * 4, *ent_o = ent_j + n_wg * SDD_G;
     for (int64_t w = 0; w < n_wg; ++w) {
@@ -286,42 +355,36 @@ extern "C" int64_t mortar_sdd_plan_host(const int32_t *row_ptr, const int16_t *c
     return words;
 }
 
-extern "C" int32_t mortar_sdd_plan_max_groups_host(const int32_t *plan) {
-    if (!plan || plan[0] <= 0 || plan[2] <= 0 || plan[3] <= 0) return mortar_fail(MORTAR_ERR_ARG, "sdd_plan_max_groups: not a plan");
-    int32_t mx = 0;
-    for (int sg = 0; sg < plan[2]; ++sg) mx = std::max(mx, plan[plan[3] + 2 * sg + 1]);
-    return mx;
-}
-
-// Token ranges for M tokens over n_wg row groups.  One workgroup runs per CU, so the launch takes
-// ceil(n_wg * ranges / CUs) rounds of ceil(steps / ranges) steps; every extra range also adds one slab of fp32 sums
-// to write and read back, priced here at about six steps.  The cheapest count of ranges wins.
-static void sdd_split(int32_t n_wg, int64_t M, int &nsteps, int &steps_per_split, int &tsplit) {
-    nsteps = (int)((M + SDD_STEP - 1) / SDD_STEP);
-    int best = 1;
-    int64_t best_cost = INT64_MAX;
-    for (int t = 1; t <= std::min(nsteps, 16); ++t) {
-        const int64_t rounds = ((int64_t)n_wg * t + SDD_TARGET_WGS - 1) / SDD_TARGET_WGS;
-        const int64_t cost = rounds * ((nsteps + t - 1) / t + 2) + (t > 1 ? 6 * t : 0);
-        if (cost < best_cost) { best_cost = cost; best = t; }
-    }
-    steps_per_split = std::max(1, (nsteps + best - 1) / best);
-    tsplit = std::max(1, (nsteps + steps_per_split - 1) / steps_per_split);
-}
-
-extern "C" int64_t mortar_sdd_workspace_bytes(int32_t n_wg, int32_t nnz, int64_t M) {
-    if (n_wg <= 0 || nnz <= 0 || M < 0) return mortar_fail(MORTAR_ERR_ARG, "sdd_workspace_bytes: bad argument");
+extern "C" int64_t mortar_sdd_workspace_bytes(int32_t n_wg, int32_t nnz, int32_t blocks_per_wave, int64_t M) {
+    if (n_wg <= 0 || nnz <= 0 || M < 0 || !sdd_nb_built(blocks_per_wave))
+        return mortar_fail(MORTAR_ERR_ARG, "sdd_workspace_bytes: bad argument");
     int nsteps, sps, tsplit;
-    sdd_split(n_wg, M, nsteps, sps, tsplit);
+    sdd_split(n_wg, nnz, blocks_per_wave, M, nsteps, sps, tsplit);
     return (int64_t)tsplit * nnz * 256 * (int64_t)sizeof(float);
 }
 
-extern "C" int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t max_groups, int32_t Rb, int32_t Cb, int32_t nnz,
+template <int NB>
+static hipError_t sdd_launch(const SddArgs &p, hipStream_t st) {
+    static bool configured = false;
+    const int smem = 2 * SDD_BUF;
+    if (!configured) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sdd_kernel<NB>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    hipLaunchKernelGGL(sdd_kernel<NB>, dim3((unsigned)(8 * p.per_xcd)), dim3(SDD_WAVES * 64), smem, st, p);
+    return hipSuccess;
+}
+
+extern "C" int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t blocks_per_wave,
+                               int32_t Rb, int32_t Cb, int32_t nnz,
                                const uint16_t *a, int64_t lda, const uint16_t *b, int64_t ldb, int64_t M,
                                float *acc, uint16_t *out, void *stream) {
     if (!plan || !out || !acc || (M > 0 && (!a || !b))) return mortar_fail(MORTAR_ERR_ARG, "sdd: null pointer");
     if (n_wg <= 0 || Rb <= 0 || Cb <= 0 || nnz <= 0 || M < 0) return mortar_fail(MORTAR_ERR_ARG, "sdd: bad shape");
-    if (max_groups <= 0 || max_groups > n_wg) return mortar_fail(MORTAR_ERR_ARG, "sdd: max_groups=%d outside 1..n_wg", max_groups);
+    if (!sdd_nb_built(blocks_per_wave))
+        return mortar_fail(MORTAR_ERR_ARG, "sdd: blocks_per_wave=%d is not a built size (8, 10, ... 22)", blocks_per_wave);
     if (reinterpret_cast<uintptr_t>(out) & 15) return mortar_fail(MORTAR_ERR_ARG, "sdd: out must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (M == 0) {                                          // no tokens: the gradient is zero
@@ -337,22 +400,23 @@ extern "C" int mortar_sdd_bf16(const int32_t *plan, int32_t n_wg, int32_t max_gr
     SddArgs p;
     p.plan = plan; p.a = a; p.b = b; p.lda = lda; p.ldb = ldb; p.M = M; p.acc = acc; p.out = out;
     p.Cb = Cb; p.nnz = nnz;
-    sdd_split(n_wg, M, p.nsteps, p.steps_per_split, p.tsplit);
-    static bool configured = false;
-    const int smem = 2 * SDD_BUF;
-    if (!configured) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sdd_kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-        configured = true;
+    sdd_split(n_wg, nnz, blocks_per_wave, M, p.nsteps, p.steps_per_split, p.tsplit);
+    p.per_xcd = (p.tsplit * n_wg + 7) / 8;
+    hipError_t e = hipSuccess;
+    switch (blocks_per_wave) {
+        case 8: e = sdd_launch<8>(p, st); break;
+        case 10: e = sdd_launch<10>(p, st); break;
+        case 12: e = sdd_launch<12>(p, st); break;
+        case 14: e = sdd_launch<14>(p, st); break;
+        case 16: e = sdd_launch<16>(p, st); break;
+        case 18: e = sdd_launch<18>(p, st); break;
+        case 20: e = sdd_launch<20>(p, st); break;
+        default: e = sdd_launch<22>(p, st); break;
     }
-    const int nseg = (Cb + SDD_SEG - 1) / SDD_SEG;
-    p.max_groups = max_groups;
-    p.pairs_per_xcd = (p.tsplit * max_groups + 7) / 8;
-    hipLaunchKernelGGL(sdd_kernel, dim3((unsigned)(8 * p.pairs_per_xcd * nseg)), dim3(SDD_WAVES * 64), smem, st, p);
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     if (p.tsplit > 1)
         hipLaunchKernelGGL(sdd_round_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st, acc, out, n4, p.tsplit);
-    const hipError_t e = hipGetLastError();
+    e = hipGetLastError();
     if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "sdd: %s", hipGetErrorString(e));
     return MORTAR_OK;
 }

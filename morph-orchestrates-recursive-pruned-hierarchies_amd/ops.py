@@ -252,9 +252,10 @@ def swiglu_backward(gu: Tensor, dh: Tensor) -> Tensor:
     return dgu
 
 
-def sdd(a: Tensor, b: Tensor, W: MortarPack, out: Tensor | None = None) -> Tensor:
+def sdd(a: Tensor, b: Tensor, W: MortarPack, out: Tensor | None = None, blocks_per_wave: int | None = None) -> Tensor:
     """Weight gradient on W's topology: out[j] = a[:, rows of block j]^T @ b[:, columns of block j], bf16 [nnz,16,16]
-    (reference stk_sdd_at_b; for y = x W^T pass a = dY [M, out_features], b = x [M, in_features])."""
+    (reference stk_sdd_at_b; for y = x W^T pass a = dY [M, out_features], b = x [M, in_features]).
+    `blocks_per_wave` picks the kernel's group size instead of the library's choice for this topology and M."""
     a, b = _bf16_2d(a, "sdd"), _bf16_2d(b, "sdd")
     if a.shape[0] != b.shape[0] or a.shape[1] != W.out_features or b.shape[1] != W.in_features:
         raise ValueError(f"sdd: a {tuple(a.shape)} / b {tuple(b.shape)} do not match the matrix [{W.out_features}, {W.in_features}]")
@@ -262,14 +263,14 @@ def sdd(a: Tensor, b: Tensor, W: MortarPack, out: Tensor | None = None) -> Tenso
         a = a.contiguous()
     if b.stride(0) % 8 or b.data_ptr() % 16:
         b = b.contiguous()
-    plan, n_wg, max_groups = W.sdd_plan()
+    plan, n_wg, nb = W.sdd_plan(a.shape[0], blocks_per_wave)
     if out is None:
         out = torch.empty((W.nnz, BLK, BLK), dtype=torch.bfloat16, device=a.device)
     elif out.dtype != torch.bfloat16 or tuple(out.shape) != (W.nnz, BLK, BLK) or not out.is_contiguous():
         raise TypeError("sdd: out must be a contiguous bfloat16 [nnz, 16, 16] tensor")
-    ws = _lib.check(_lib.lib().mortar_sdd_workspace_bytes(n_wg, W.nnz, a.shape[0]), "mortar_sdd_workspace_bytes")
+    ws = _lib.check(_lib.lib().mortar_sdd_workspace_bytes(n_wg, W.nnz, nb, a.shape[0]), "mortar_sdd_workspace_bytes")
     acc = torch.empty(ws // 4, dtype=torch.float32, device=a.device)
-    _lib.check(_lib.lib().mortar_sdd_bf16(_p(plan), n_wg, max_groups, W.Rb, W.Cb, W.nnz, _p(a), a.stride(0), _p(b), b.stride(0),
+    _lib.check(_lib.lib().mortar_sdd_bf16(_p(plan), n_wg, nb, W.Rb, W.Cb, W.nnz, _p(a), a.stride(0), _p(b), b.stride(0),
                                           a.shape[0], _p(acc), _p(out), _stream(a)), "mortar_sdd_bf16")
     return out
 

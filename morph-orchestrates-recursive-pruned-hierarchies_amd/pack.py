@@ -336,19 +336,26 @@ class MortarPack:
             self._transposed = t
         return self._transposed
 
-    def sdd_plan(self) -> tuple[torch.Tensor, int, int]:
-        """(device plan, workgroups, largest number of row groups in a K segment) of the weight-gradient kernel for this
-        topology: see mortar_sdd_plan_host."""
+    def sdd_plan(self, M: int, blocks_per_wave: int | None = None) -> tuple[torch.Tensor, int, int]:
+        """(device plan, workgroups, blocks per wavefront) of the weight-gradient kernel for this topology at M tokens:
+        see mortar_sdd_blocks_per_wave_host and mortar_sdd_plan_host.  One plan per group size is kept;
+        `blocks_per_wave` overrides the choice (any built size gives the same gradient)."""
+        L = _lib.lib()
         if self._sdd is None:
-            L = _lib.lib()
-            n = _lib.check(L.mortar_sdd_plan_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, None, 0),
+            self._sdd = {}
+        nb = blocks_per_wave if blocks_per_wave is not None else self._sdd.get(("M", M))
+        if nb is None:
+            nb = _lib.check(L.mortar_sdd_blocks_per_wave_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, M),
+                            "mortar_sdd_blocks_per_wave_host")
+            self._sdd[("M", M)] = nb
+        if nb not in self._sdd:
+            n = _lib.check(L.mortar_sdd_plan_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, nb, None, 0),
                            "mortar_sdd_plan_host")
             plan = np.empty(n, dtype=np.int32)
-            _lib.check(L.mortar_sdd_plan_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, _vp(plan), n),
+            _lib.check(L.mortar_sdd_plan_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, nb, _vp(plan), n),
                        "mortar_sdd_plan_host")
-            mg = _lib.check(L.mortar_sdd_plan_max_groups_host(_vp(plan)), "mortar_sdd_plan_max_groups_host")
-            self._sdd = (torch.from_numpy(plan).to(self.device), int(plan[0]), plan, int(mg))
-        return self._sdd[0], self._sdd[1], self._sdd[3]
+            self._sdd[nb] = (torch.from_numpy(plan).to(self.device), int(plan[0]))
+        return (*self._sdd[nb], nb)
 
     def sched(self, rows_per_unit: int) -> torch.Tensor:
         """Device schedule (mortar_schedule_host over the balanced unit order) for plain (1) or gate/up (2) units."""

@@ -187,6 +187,30 @@ def test_sdd_weight_gradient(dev, shape, density, zipf, M):
     assert_close_bf16(got, ref, f"dW {shape} M={M}")
 
 
+_GROUP_SIZE_CASE = {}
+
+
+def _group_size_case(M):
+    """One ragged topology over three K segments with its operands and the oracle's gradient, computed once."""
+    if M not in _GROUP_SIZE_CASE:
+        m = synth.synth_matrix(16 * 200, 16 * 100, 0.3, seed=61, zipf_s=1.2)
+        a, b = synth.synth_x(M, 16 * 200, seed=62 + M), synth.synth_x(M, 16 * 100, seed=63 + M)
+        _GROUP_SIZE_CASE[M] = (m, a, b, O.sdd_at_b(O.bf16_round(a), O.bf16_round(b), m["row_idx"], m["col_idx"]))
+    return _GROUP_SIZE_CASE[M]
+
+
+@pytest.mark.parametrize("blocks_per_wave", [8, 10, 12, 14, 16, 18, 20, 22])
+def test_sdd_every_group_size(dev, blocks_per_wave):
+    """Each built group size (blocks per wavefront) against the oracle, on ragged rows over several K segments and
+    several token ranges, and on a token count that ends inside a step."""
+    for M in (600, 37):
+        m, a, b, ref = _group_size_case(M)
+        got = to_np(ops.sdd(to_dev(a, dev), to_dev(b, dev), synth.to_pack(m, dev), blocks_per_wave=blocks_per_wave))
+        assert_close_bf16(got, ref, f"dW group size {blocks_per_wave} M={M}")
+    with pytest.raises(ValueError):
+        ops.sdd(to_dev(a, dev), to_dev(b, dev), synth.to_pack(m, dev), blocks_per_wave=9)
+
+
 def test_sdd_exact_positions(dev):
     """One-hot operands: a single token with a single 1 in a and in b gives a single 1 in exactly one block element."""
     m = synth.synth_matrix(16 * 3, 16 * 5, 1.0, seed=1)

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in mortar_hip.h but not exported"
     assert declared == set(_lib.EXPORTS)
-    assert _lib.lib().mortar_abi_version() == 6
+    assert _lib.lib().mortar_abi_version() == 7
 
 
 def test_encode_round_trip_and_bit_layout():
@@ -381,27 +381,31 @@ def test_sdd_plan_partitions_the_blocks():
     """Every kept block appears exactly once, inside its workgroup's row window and K segment."""
     from mortar_amd import synth
     L = _lib.lib()
-    for shape in ((16 * 40, 16 * 30), (16 * 9, 16 * 352), (16 * 704, 16 * 128)):
+    for shape, nbw in (((16 * 40, 16 * 30), 22), ((16 * 9, 16 * 352), 8), ((16 * 704, 16 * 128), 22), ((16 * 704, 16 * 128), 12)):
         m = synth.synth_matrix(shape[0], shape[1], 0.25, seed=9, zipf_s=1.2)
         Rb, Cb = shape[0] // 16, shape[1] // 16
         off, col = np.ascontiguousarray(m["offsets"], np.int32), np.ascontiguousarray(m["col_idx"], np.int16)
         vp = lambda a: a.ctypes.data_as(C.c_void_p)
-        n = L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, None, 0)
+        n = L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, nbw, None, 0)
         plan = np.empty(n, np.int32)
-        assert L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, vp(plan), n) == n
-        assert L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, vp(plan), n - 1) < 0
+        assert L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, nbw, vp(plan), n) == n
+        assert L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, nbw, vp(plan), n - 1) < 0
+        assert L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, 9, None, 0) < 0        # not a built group size
         n_wg, seg_cb, nseg, tab = plan[0], plan[1], plan[2], plan[3]
-        assert tab + 2 * nseg == n
+        assert tab + n_wg == n
         G = (tab - 4 - 4 * n_wg) // (2 * n_wg)
+        assert G == 16 * nbw
         desc = plan[4:4 + 4 * n_wg].reshape(n_wg, 4)
         ej = plan[4 + 4 * n_wg:4 + 4 * n_wg + n_wg * G].reshape(n_wg, G)
         eo = plan[4 + 4 * n_wg + n_wg * G:tab].reshape(n_wg, G)
-        # segment table: workgroups are stored segment by segment; {first workgroup, row groups} per segment
-        st = plan[tab:].reshape(nseg, 2)
-        for sg in range(nseg):
-            ws = np.nonzero(desc[:, 2] == sg)[0]
-            assert st[sg, 1] == ws.size and (ws.size == 0 or (st[sg, 0] == ws[0] and np.array_equal(ws, np.arange(ws[0], ws[0] + ws.size))))
-        assert L.mortar_sdd_plan_max_groups_host(vp(plan)) == st[:, 1].max()
+        # workgroups are stored segment by segment; the launch order lists every workgroup once, by its position
+        # inside the segment first (row groups of about the same rows side by side), then by segment
+        assert (np.diff(desc[:, 2]) >= 0).all()
+        order = plan[tab:]
+        assert sorted(order.tolist()) == list(range(n_wg))
+        first = np.searchsorted(desc[:, 2], np.arange(nseg))
+        key = [(w - first[desc[w, 2]], desc[w, 2]) for w in order]
+        assert key == sorted(key)
         assert nseg >= -(-Cb // seg_cb) and seg_cb <= 44 and seg_cb % 4 == 0
         seen = ej[ej >= 0]
         assert sorted(seen.tolist()) == list(range(col.size))
@@ -416,6 +420,30 @@ def test_sdd_plan_partitions_the_blocks():
             tile = (off // 4224) * 4 + (off % 4224) // 32
             assert ((off % 4224) % 32 == 0).all() and (off % 4224 < 128).all() and (tile < seg_cb).all() and ((eo[w] >> 20) < nrows).all()
             assert np.array_equal(tile[ej[w] >= 0], col[js] - seg * seg_cb) and (col[js] // seg_cb == seg).all()
+
+
+def test_sdd_blocks_per_wave_is_a_built_size_and_fills_the_chip():
+    """The chosen group size is one of the built kernels; at the headline shapes and 4096 tokens its plan has a count
+    of token ranges that puts 200 to 256 workgroups on the 256 CUs (one per CU, one round)."""
+    from mortar_amd import synth
+    L = _lib.lib()
+    vp = lambda a: a.ctypes.data_as(C.c_void_p)
+    for shape, M in (((11264, 2048), 4096), ((2048, 5632), 4096), ((64, 96), 7), ((11264, 2048), 0), ((2048, 5632), 16384)):
+        m = synth.synth_matrix(shape[0], shape[1], 0.25, seed=3)
+        Rb, Cb = shape[0] // 16, shape[1] // 16
+        off, col = np.ascontiguousarray(m["offsets"], np.int32), np.ascontiguousarray(m["col_idx"], np.int16)
+        nbw = L.mortar_sdd_blocks_per_wave_host(vp(off), vp(col), Rb, Cb, M)
+        assert nbw in (8, 10, 12, 14, 16, 18, 20, 22)
+        n = L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, nbw, None, 0)
+        plan = np.empty(n, np.int32)
+        assert L.mortar_sdd_plan_host(vp(off), vp(col), Rb, Cb, nbw, vp(plan), n) == n
+        ws = L.mortar_sdd_workspace_bytes(int(plan[0]), col.size, nbw, M)
+        ranges = ws // (col.size * 1024)
+        assert ws == ranges * col.size * 1024 and 1 <= ranges <= 16
+        if M >= 4096:
+            assert 200 <= ranges * plan[0] <= 256, (shape, M, nbw, ranges, plan[0])
+    assert L.mortar_sdd_blocks_per_wave_host(vp(off), vp(col), Rb, Cb, -1) < 0
+    assert L.mortar_sdd_workspace_bytes(4, 16, 9, 64) < 0
 
 
 def test_operator_fake_implementations_trace_without_a_gpu():
