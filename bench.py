@@ -368,6 +368,29 @@ def main() -> None:
                                    "decode_stack_b1_frac_hbm": b_s / (t_s * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                    "note": "blocks multiplied as +-2 / 0, fp32 sums scaled once (scale-after-sum, as the "
                                            "reference's decode kernel); the headline uses per-block scales"}
+        # the reference engine's own decode arithmetic on that format: fp32 activations in and out, exact products,
+        # fp32 scale after the sums (mortar_gemv with fp32 x); 32 MLPs (gate_up + SwiGLU, then down) per graph replay
+        f32dec = {}
+        for B in (1, 16):
+            xf = x[:B].float().contiguous()
+            hf = torch.empty((B, D_FF), dtype=torch.float32, device=dev)
+            yf = torch.empty((B, D_MODEL), dtype=torch.float32, device=dev)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    ops.gemv_f32(xf, Ugu, swiglu_out=True, out=hf)
+                    ops.gemv_f32(hf, Udn, out=yf)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(32):
+                    ops.gemv_f32(xf, Ugu, swiglu_out=True, out=hf)
+                    ops.gemv_f32(hf, Udn, out=yf)
+            t_f = event_time_ms(graph.replay, 20, 3) / 32
+            f32dec[f"b{B}"] = {"us_per_mlp_graph": t_f * 1e3, "tokens_per_s": B / (t_f * 1e-3)}
+            del graph
+        out["per_tensor_scale"]["decode_fp32_arithmetic"] = f32dec
         del up, dn, hs, ys, upacks, Ugu, Udn
 
     if not args.no_extras:

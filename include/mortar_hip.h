@@ -309,11 +309,21 @@ int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_e
  *              (the reference's down call form, fused_decode_step.py:1410-1414)
  *   x fp32 [B, ldx]; y fp32 [B, Rb*16] (mode 0) or [B, Rb*8] (mode 1), 16-byte aligned, ldy % 4 == 0
  *   kseg       block-columns per K segment of the work list; 3 * 2 * kseg * (16 * ceil(B / 16) + 1) * 16 bytes of LDS
- *   other arguments as mortar_gemv_bf16.  Agreement with a float64 evaluation: fp32 rounding of the sums only. */
-int mortar_gemv_f32(const mortar_bcsr_t *W, const float *scale, int64_t scale_count, const int32_t *entries,
+ *   sched      the plain-product schedule of the pack (mortar_schedule_host with one row per unit, device), or NULL
+ *   part       device workspace of part_bytes >= mortar_gemv_f32_workspace_bytes(W, B, nslots) bytes, 16-byte aligned
+ *              (may be NULL when nslots == 1; then only the work-list kernel runs)
+ *   other arguments as mortar_gemv_bf16.  Agreement with a float64 evaluation: fp32 rounding of the sums only.
+ * With one scale (scale_count = 1, the reference's format), no flags, a schedule and the workspace, the product runs on
+ * the bandwidth-bound SpMM kernels instead of the work list: the three bf16 terms of the B rows become 3 * B bf16 rows,
+ * the one-scale SpMM kernels contract them with the +-2 / 0 blocks and keep the fp32 sums unrounded, and a last pass
+ * adds the three sums of a row and applies the scale and the epilogue - the same exact products and fp32 sums, in
+ * another order of addition (2 to 3 times faster at the headline shapes). */
+int64_t mortar_gemv_f32_workspace_bytes(const mortar_bcsr_t *W, int32_t B, int32_t nslots);
+int mortar_gemv_f32(const mortar_bcsr_t *W, const float *scale, int64_t scale_count, const int32_t *sched,
+                    const int32_t *entries,
                     int64_t n_entries, int32_t nslots, const int32_t *row_slots, int32_t kseg, int32_t mode,
                     int32_t swiglu_x, const float *x, int32_t B, int64_t ldx, float *y, int64_t ldy, float *part,
-                    const float *gates, int32_t n_clusters, int64_t ldg,
+                    int64_t part_bytes, const float *gates, int32_t n_clusters, int64_t ldg,
                     const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc, void *stream);
 
 /* mortar_gemv_bf16 for callers that cannot allocate device memory or hand in a workspace: code under HIP graph capture,

@@ -66,8 +66,9 @@ _SIGS = {
                                    c_vp, c_vp, c_i32, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp]),
     "mortar_rmsnorm_bf16": (C.c_int, [c_vp, c_i64, c_i32, c_i64, c_vp, c_f32, c_vp, c_i64, c_vp]),
     "mortar_spmm_hc_post": (C.c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_vp]),
-    "mortar_gemv_f32": (C.c_int, [c_vp, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_i32, c_i32, c_i32, c_vp, c_i32, c_i64, c_vp, c_i64,
-                                  c_vp, c_vp, c_i32, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp]),
+    "mortar_gemv_f32_workspace_bytes": (c_i64, [c_vp, c_i32, c_i32]),
+    "mortar_gemv_f32": (C.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_i32, c_vp, c_i32, c_i32, c_i32, c_vp, c_i32, c_i64, c_vp, c_i64,
+                                  c_vp, c_i64, c_vp, c_i32, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp]),
     "mortar_gemv_noalloc_max_floats": (c_i64, []),
     "mortar_gemv_bf16_noalloc": (C.c_int, [c_vp, c_vp, c_i64, c_i32, c_vp, c_i32, c_i32, c_vp, c_i32, c_i64, c_vp, c_i64,
                                            c_vp, c_i32, c_i64, c_vp, c_i64, c_vp, c_i64, c_vp]),

@@ -458,12 +458,103 @@ int launch_gemv_f32(const GemvF32Params &p, hipStream_t st) {
     return MORTAR_OK;
 }
 
+// ---- one scale for the whole matrix, no flags: the product runs on the bandwidth-bound SpMM kernels ----------------
+// The three bf16 terms of every activation row become three rows of a bf16 matrix [3B, in_features] (hi rows, then
+// mid, then lo); the SpMM kernels for matrices with one scale contract them with the +-2 / 0 blocks (every product
+// exact, fp32 sums in the matrix pipe) and store the sums unrounded; a last kernel adds the three sums of a row, applies
+// the fp32 scale once (the reference's scale-after-sum) and the SwiGLU / gate epilogue.  Same arithmetic as the
+// work-list kernel above up to the order of the fp32 additions.
+
+// thread = 8 consecutive features of one row: x (or silu(g) * u of a gate_up output) -> 16 bytes of each term row
+__global__ void __launch_bounds__(256) gemv_f32_split_kernel(const float *x, int B, int K, int64_t ldx, int swiglu_x,
+                                                             uint16_t *xs) {
+    const int nch = K / 8;
+    const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (it >= (int64_t)B * nch) return;
+    const int tok = (int)(it / nch), ch = (int)(it % nch);
+    const float4 *src = reinterpret_cast<const float4 *>(x + (int64_t)tok * ldx + ch * 8);
+    float4 q[2] = {src[0], src[1]};
+    if (swiglu_x) {
+        const float4 u0 = src[K / 4], u1 = src[K / 4 + 1];
+        q[0] = float4{q[0].x * sigmoid_f32(q[0].x) * u0.x, q[0].y * sigmoid_f32(q[0].y) * u0.y,
+                      q[0].z * sigmoid_f32(q[0].z) * u0.z, q[0].w * sigmoid_f32(q[0].w) * u0.w};
+        q[1] = float4{q[1].x * sigmoid_f32(q[1].x) * u1.x, q[1].y * sigmoid_f32(q[1].y) * u1.y,
+                      q[1].z * sigmoid_f32(q[1].z) * u1.z, q[1].w * sigmoid_f32(q[1].w) * u1.w};
+    }
+    const float xv[8] = {q[0].x, q[0].y, q[0].z, q[0].w, q[1].x, q[1].y, q[1].z, q[1].w};
+    uint32_t hi[4], mid[4], lo[4];
+#pragma unroll
+    for (int k = 0; k < 8; k += 2) {
+        const float v[2] = {xv[k], xv[k + 1]};
+        const uint32_t h2 = bf16_pack2(v[0], v[1]);
+        const float r0 = v[0] - bf16_to_f32(h2 & 0xffffu), r1 = v[1] - bf16_to_f32(h2 >> 16);
+        const uint32_t m2 = bf16_pack2(r0, r1);
+        const float s0 = r0 - bf16_to_f32(m2 & 0xffffu), s1 = r1 - bf16_to_f32(m2 >> 16);
+        hi[k / 2] = h2; mid[k / 2] = m2; lo[k / 2] = bf16_pack2(s0, s1);
+    }
+    uint4 *dst = reinterpret_cast<uint4 *>(xs + (int64_t)tok * K + ch * 8);
+    const int64_t plane = (int64_t)B * K / 8;                    // 16-byte units per term
+    dst[0] = uint4{hi[0], hi[1], hi[2], hi[3]};
+    dst[plane] = uint4{mid[0], mid[1], mid[2], mid[3]};
+    dst[2 * plane] = uint4{lo[0], lo[1], lo[2], lo[3]};
+}
+
+// y3 [3B, N]: the sums of the hi, mid and lo rows.  y = scale * ((hi + mid) + lo), then the epilogue of the mode.
+__global__ void __launch_bounds__(256) gemv_f32_combine3_kernel(const float *y3, const float *scale, int B, int N, int mode,
+                                                                const float *gates, int cluster_size, int64_t ldg,
+                                                                float *y, int64_t ldy) {
+    const int nout = mode == 0 ? N : N / 2;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)B * nout) return;
+    const int tok = (int)(i / nout), o = (int)(i % nout);
+    const float s = scale[0];
+    const float *r0 = y3 + (int64_t)tok * N, *r1 = r0 + (int64_t)B * N, *r2 = r1 + (int64_t)B * N;
+    const float a = s * ((r0[o] + r1[o]) + r2[o]);
+    float r = a;
+    if (mode == 1) {
+        const float b = s * ((r0[nout + o] + r1[nout + o]) + r2[nout + o]);
+        r = a * sigmoid_f32(a) * b;
+        if (gates) r *= gates[(int64_t)tok * ldg + o / cluster_size];
+    }
+    y[(int64_t)tok * ldy + o] = r;
+}
+
+int64_t gemv_f32_fast_bytes(const mortar_bcsr_t *W, int B) {
+    return (int64_t)3 * B * ((int64_t)W->Rb * 16 * 4 + (int64_t)W->Cb * 16 * 2);
+}
+
+// Returns MORTAR_NO_KERNEL when the SpMM kernels cannot serve the shape (the caller then runs the work-list kernel).
+int gemv_f32_fast(const mortar_bcsr_t *W, const int32_t *sched, const GemvF32Params &p, void *ws, hipStream_t st) {
+    const int K = W->Cb * 16, N = W->Rb * 16;
+    float *y3 = reinterpret_cast<float *>(ws);
+    uint16_t *xs = reinterpret_cast<uint16_t *>(y3 + (int64_t)3 * p.B * N);
+    const int64_t nsplit = (int64_t)p.B * (K / 8);
+    hipLaunchKernelGGL(gemv_f32_split_kernel, dim3((unsigned)((nsplit + 255) / 256)), dim3(256), 0, st, p.x, p.B, K, p.ldx,
+                       p.swiglu_x, xs);
+    const int rc = mortar_spmm_codes_f32(W, sched, xs, 3 * p.B, K, y3, N, st);
+    if (rc) return rc;
+    const int64_t total = (int64_t)p.B * (p.mode == 0 ? N : N / 2);
+    hipLaunchKernelGGL(gemv_f32_combine3_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, y3, p.scale, p.B, N,
+                       p.mode, p.gates, p.cluster_size, p.ldg, p.y, p.ldy);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "gemv_f32 launch: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}
+
 }  // namespace
 
-extern "C" int mortar_gemv_f32(const mortar_bcsr_t *W, const float *scale, int64_t scale_count, const int32_t *entries,
+extern "C" int64_t mortar_gemv_f32_workspace_bytes(const mortar_bcsr_t *W, int32_t B, int32_t nslots) {
+    if (!W || W->Rb <= 0 || W->Cb <= 0 || B <= 0 || B > 64 || nslots < 1)
+        return mortar_fail(MORTAR_ERR_ARG, "gemv_f32_workspace_bytes: bad argument");
+    const int64_t slots = nslots > 1 ? (int64_t)nslots * B * W->Rb * 16 * 4 : 0, fast = gemv_f32_fast_bytes(W, B);
+    return slots > fast ? slots : fast;
+}
+
+extern "C" int mortar_gemv_f32(const mortar_bcsr_t *W, const float *scale, int64_t scale_count, const int32_t *sched,
+                               const int32_t *entries,
                                int64_t n_entries, int32_t nslots, const int32_t *row_slots, int32_t kseg, int32_t mode,
                                int32_t swiglu_x, const float *x, int32_t B, int64_t ldx, float *y, int64_t ldy, float *part,
-                               const float *gates, int32_t n_clusters, int64_t ldg,
+                               int64_t part_bytes, const float *gates, int32_t n_clusters, int64_t ldg,
                                const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc, void *stream) {
     if (!W || !W->codes || !W->col || !scale || !entries || !x || !y) return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: null pointer");
     if (scale_count != 1 && scale_count != W->nnz) return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: scale_count must be 1 or nnz");
@@ -489,6 +580,14 @@ extern "C" int mortar_gemv_f32(const mortar_bcsr_t *W, const float *scale, int64
     }
     p.row_act = row_act; p.ldr = ldr; p.col_act = col_act; p.ldc = ldc;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (nslots > 1 && part_bytes < (int64_t)nslots * B * W->Rb * 16 * 4)
+        return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: the partial workspace holds %lld bytes, need %lld", (long long)part_bytes,
+                           (long long)nslots * B * W->Rb * 16 * 4);
+    if (scale_count == 1 && sched && !row_act && !col_act && W->codes_o && part && !(reinterpret_cast<uintptr_t>(part) & 15) &&
+        part_bytes >= gemv_f32_fast_bytes(W, B) && ldx % 4 == 0 && !(reinterpret_cast<uintptr_t>(x) & 15)) {
+        const int rc = gemv_f32_fast(W, sched, p, part, st);
+        if (rc != MORTAR_NO_KERNEL) return rc;
+    }
     int rc = B <= 16 ? launch_gemv_f32<1>(p, st) : (B <= 32 ? launch_gemv_f32<2>(p, st) : launch_gemv_f32<4>(p, st));
     if (rc) return rc;
     if (nslots > 1) {

@@ -149,6 +149,26 @@ extern "C" int mortar_spmm_bf16(const mortar_bcsr_t *W, const int32_t *sched, co
     return dispatch(0, p, W, static_cast<hipStream_t>(stream));
 }
 
+int mortar_spmm_codes_f32(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M, int64_t ldx,
+                          float *y32, int64_t ldy, void *stream) {
+    int rc = check_common(W, x, M, ldx, reinterpret_cast<const uint16_t *>(y32), ldy, W ? (int64_t)W->Rb * 16 : 0);
+    if (rc) return rc;
+    if (reinterpret_cast<uintptr_t>(y32) & 15) return mortar_fail(MORTAR_ERR_ARG, "spmm: the fp32 output must be 16-byte aligned");
+    SpmmParams p;
+    fill(p, W, sched, x, M, ldx, nullptr, ldy);
+    p.n_units = W->Rb;
+    p.y32 = y32;
+    p.uscale = 0.5f;                       // the kernels multiply the blocks as +-2 / 0
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (M <= MORTAR_SMALLM_MAX) {
+        rc = mortar_smallm_launch(0, p, nullptr, 1, st);
+        if (rc >= 0) return rc;
+    }
+    if (!W->codes4_o) return MORTAR_NO_KERNEL;      // prefill-sized tiles multiply +-2 / 0 blocks only from the 4-bit stream
+    p.codes_o = reinterpret_cast<const u32x4_t *>(W->codes4_o);
+    return dispatch_prefill<CODE_4BIT | CODE_UNIFORM>(0, p, st);
+}
+
 extern "C" int mortar_spmm_bf16_masked(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *x, int64_t M,
                                        int64_t ldx, uint16_t *y, int64_t ldy, const uint8_t *active,
                                        int32_t n_clusters, void *stream) {

@@ -37,7 +37,7 @@ struct SpmmParams {
     int norm;                 // 1: rows of x are RMS-normalised while they are staged (single-segment tiles only)
     float norm_eps;
     float uscale;             // CODE_UNIFORM kernels: half the matrix's (bf16-rounded) scale
-    int pad_[2];
+    float *y32;               // plain products: unrounded fp32 output [M, ldy] in place of the bf16 store, or null
     const uint16_t *norm_w;   // bf16 [in_features] weight of that norm, or null for none
     // hyper-connection POST write in place of the plain store (small tiles, plain products): out[t, i, :] =
     // sum_j hc_res[t, i, j] * hc_h[t, j, :] + hc_post[t, i] * y[t, :] (+ hc_term[t, :]); null hc_h = plain store
@@ -58,6 +58,7 @@ struct SpmmView {
     const MORTAR_GLOBAL uint32_t *sd_dw, *cc_dw;      // scale patterns / block-columns of the octet stream as dwords
     const MORTAR_GLOBAL char *x;
     MORTAR_GLOBAL uint16_t *y;
+    MORTAR_GLOBAL float *y32;
     const MORTAR_GLOBAL float *gates;
     const MORTAR_GLOBAL uint8_t *active;
     const MORTAR_GLOBAL int32_t *tok_cnt;
@@ -86,7 +87,7 @@ __device__ __forceinline__ SpmmView mortar_view(const SpmmParams &q) {
     v.row_desc = (const MORTAR_GLOBAL u32x4_t *)q.row_desc; v.codes_o = (const MORTAR_GLOBAL u32x4_t *)q.codes_o;
     v.sched = (const MORTAR_GLOBAL u32x4_t *)q.sched;
     v.sd_dw = (const MORTAR_GLOBAL uint32_t *)q.sd_o; v.cc_dw = (const MORTAR_GLOBAL uint32_t *)q.col_o;
-    v.x = (const MORTAR_GLOBAL char *)q.x; v.y = (MORTAR_GLOBAL uint16_t *)q.y;
+    v.x = (const MORTAR_GLOBAL char *)q.x; v.y = (MORTAR_GLOBAL uint16_t *)q.y; v.y32 = (MORTAR_GLOBAL float *)q.y32;
     v.gates = (const MORTAR_GLOBAL float *)q.gates; v.active = (const MORTAR_GLOBAL uint8_t *)q.active;
     v.tok_cnt = (const MORTAR_GLOBAL int32_t *)q.tok_cnt; v.tok_list = (const MORTAR_GLOBAL uint8_t *)q.tok_list;
     v.ldx = q.ldx; v.ldy = q.ldy; v.n_units = q.n_units; v.Cb = q.Cb; v.M = q.M; v.n_clusters = q.n_clusters;
@@ -365,6 +366,10 @@ __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, i
     }
     u32x2_t pk;
     if (NACC == 1) {
+        if (p.y32 != nullptr) {      // the fp32 sums as they are (the three-term fp32 decode product adds them up later)
+            *(MORTAR_GLOBAL f32x4_t *)(p.y32 + (int64_t)tok * p.ldy + unit * 16 + 4 * g) = a0;
+            return;
+        }
         pk = u32x2_t{bf16_pack2(a0[0], a0[1]), bf16_pack2(a0[2], a0[3])};
         if (HC && p.hc_h != nullptr) {
             const f32x4_t y = {bf16_to_f32(pk[0] & 0xffffu), bf16_to_f32(pk[0] >> 16), bf16_to_f32(pk[1] & 0xffffu), bf16_to_f32(pk[1] >> 16)};

@@ -357,7 +357,15 @@ def gemv_f32(x: Tensor, W: MortarPack, swiglu_x: bool = False, swiglu_out: bool 
     ent, nslots, row_slots, _ = W.worklist(2 if swiglu_out else 1, kseg, max_blocks if max_blocks is not None else 1 << 20)
     nout = W.out_features // 2 if swiglu_out else W.out_features
     y = out if out is not None else torch.empty((B, nout), dtype=torch.float32, device=x.device)
-    part = torch.empty((nslots, B, W.out_features), dtype=torch.float32, device=x.device) if nslots > 1 else None
+    sc = W.scales_f32
+    sc_one = sc.numel() == 1
+    L = _lib.lib()
+    # one scale, no flags, no explicit split: the SpMM kernels run the product
+    fast = sc_one and row_act is None and col_act is None and max_blocks is None
+    ws = _lib.check(L.mortar_gemv_f32_workspace_bytes(W.ref, B, nslots), "mortar_gemv_f32_workspace_bytes")
+    part = torch.empty(ws // 4, dtype=torch.float32, device=x.device) if (nslots > 1 or fast) else None
+    if fast and ((B > 1 and x.stride(0) % 4) or x.data_ptr() % 16):       # the split kernel reads 16-byte words
+        x = x.clone(memory_format=torch.contiguous_format)
     ncl, ldg = 0, 0
     if gates is not None:
         if gates.dtype != torch.float32 or gates.stride(1) != 1:
@@ -366,10 +374,10 @@ def gemv_f32(x: Tensor, W: MortarPack, swiglu_x: bool = False, swiglu_out: bool 
     for f in (row_act, col_act):
         if f is not None and (f.dtype != torch.int32 or f.stride(1) != 1):
             raise TypeError("gemv_f32: row_act / col_act must be int32 with unit inner stride")
-    sc = W.scales_f32
-    rc = _lib.lib().mortar_gemv_f32(
-        W.ref, _p(sc), sc.numel(), _p(ent), ent.shape[0], nslots, _p(row_slots), kseg, 1 if swiglu_out else 0,
-        1 if swiglu_x else 0, _p(x), B, x.stride(0), _p(y), y.stride(0), _p(part), _p(gates), ncl, ldg,
+    rc = L.mortar_gemv_f32(
+        W.ref, _p(sc), sc.numel(), _p(W.sched(1)) if fast else None, _p(ent), ent.shape[0], nslots, _p(row_slots), kseg,
+        1 if swiglu_out else 0, 1 if swiglu_x else 0, _p(x), B, x.stride(0) if B > 1 else x.shape[1], _p(y), y.stride(0), _p(part),
+        part.numel() * 4 if part is not None else 0, _p(gates), ncl, ldg,
         _p(row_act), row_act.stride(0) if row_act is not None else 0,
         _p(col_act), col_act.stride(0) if col_act is not None else 0, _stream(x))
     _lib.check(rc, "mortar_gemv_f32")

@@ -628,6 +628,43 @@ def test_mortar_gemv_fp32_arithmetic(dev, B, per_tensor):
     assert np.abs(y2.cpu().numpy() - y_ref).max() <= 4 * _gemv_f32_tolerance(y_ref)
 
 
+@pytest.mark.parametrize("B", [1, 3, 16, 22, 64])
+def test_mortar_gemv_fp32_one_scale_runs_on_the_spmm_kernels(dev, B):
+    """One scale per matrix and no flags: the fp32 product runs as 3 * B bf16 term rows through the SpMM kernels (one
+    4-token tile, 16-token tiles, the 32-token prefill tiles at 3 * 64 rows, one and several K segments).  Checked against
+    the oracle's float64 sums and against the work-list kernel (forced with an explicit split), incl. gates without
+    flags and the swiglu_x form."""
+    d_model, d_ff, ncl = 512, 16 * 200, 25
+    spec = synth.synth_mlp(d_model, d_ff, 0.25, seed=195, zipf_s=1.2)
+    spec["gate_up"]["scales"] = spec["gate_up"]["scales"][:1] * 1.2345               # fp32 values that bf16 cannot hold
+    spec["down"]["scales"] = spec["down"]["scales"][:1] * 0.987
+    gu_m, dn_m = spec["gate_up"], spec["down"]
+    Wgu, Wdn = synth.to_pack(gu_m, dev), synth.to_pack(dn_m, dev)
+    assert Wdn.nseg > 1 and Wgu.scales_f32.numel() == 1
+    rng = np.random.default_rng(196 + B)
+    x = rng.standard_normal((B, d_model)).astype(np.float32) * np.float32(1.37)
+    xt = torch.from_numpy(x).to(dev)
+    gu = O.mortar_gemv(x, gu_m["codes"], gu_m["scales"], gu_m["col_idx"], gu_m["offsets"]).astype(np.float64)
+    fast, slow = ops.gemv_f32(xt, Wgu).cpu().numpy(), ops.gemv_f32(xt, Wgu, max_blocks=1 << 20).cpu().numpy()
+    assert np.abs(fast - gu).max() <= _gemv_f32_tolerance(gu) and np.abs(slow - gu).max() <= _gemv_f32_tolerance(gu)
+    # a strided fp32 view (rows of a wider buffer, not 16-byte aligned) gives the same values
+    wide = torch.zeros(B, d_model + 3, device=dev); wide[:, 1:d_model + 1] = xt
+    assert np.array_equal(ops.gemv_f32(wide[:, 1:d_model + 1], Wgu).cpu().numpy(), fast)
+    g, u = gu[:, :d_ff], gu[:, d_ff:]
+    h_ref = g / (1.0 + np.exp(-g)) * u
+    gates = ops.remoe_gates(torch.from_numpy(synth.synth_logits(B, ncl, 197)).to(dev), 7)[0]
+    hg_ref = (h_ref.reshape(B, ncl, -1) * gates.cpu().numpy().astype(np.float64)[:, :, None]).reshape(B, d_ff)
+    hg = ops.gemv_f32(xt, Wgu, swiglu_out=True, gates=gates)
+    assert np.abs(hg.cpu().numpy() - hg_ref).max() <= _gemv_f32_tolerance(h_ref)
+    h = ops.gemv_f32(xt, Wgu, swiglu_out=True)
+    assert np.abs(h.cpu().numpy() - h_ref).max() <= _gemv_f32_tolerance(h_ref)
+    y_ref = O.mortar_gemv(h.cpu().numpy(), dn_m["codes"], dn_m["scales"], dn_m["col_idx"], dn_m["offsets"]).astype(np.float64)
+    for y in (ops.gemv_f32(h, Wdn), ops.gemv_f32(h, Wdn, max_blocks=1 << 20)):
+        assert np.abs(y.cpu().numpy() - y_ref).max() <= _gemv_f32_tolerance(y_ref)
+    y2 = ops.gemv_f32(torch.from_numpy(fast).to(dev), Wdn, swiglu_x=True)
+    assert np.abs(y2.cpu().numpy() - y_ref).max() <= 4 * _gemv_f32_tolerance(y_ref)
+
+
 @pytest.mark.parametrize("B,n,f32", [(1, 4, True), (3, 4, False), (16, 2, True), (40, 4, False), (5, 1, True), (7, 3, False)])
 def test_down_with_hc_post_epilogue(dev, B, n, f32):
     """`down` with the hyper-connection POST write in its epilogue against the oracle (y rounded to bf16, then the
