@@ -214,6 +214,14 @@ def test_unit_order_segments(rpu, Rb, zipf):
     assert after <= before
     if zipf == 0.0:
         assert after < 0.97 * before                                                # uniform rows: > 3 % less waiting
+    # a kernel that gives a wave half as many units runs each half of a full window as its own workgroup: the halves
+    # hold the same number of executed block pairs to within a few units (the greedy alone would put a wave's heaviest
+    # units all in the first half)
+    pairs = (desc.reshape(nseg, Rb, 4)[:, :, 2] + 3) // 4 * 2
+    ucost = (pairs[:, :nu] + (pairs[:, nu:] if rpu == 2 else 0)).sum(axis=0)
+    for p0 in range(0, nu - per + 1, per):
+        first, second = ucost[o2[p0:p0 + per // 2]].sum(), ucost[o2[p0 + per // 2:p0 + per]].sum()
+        assert abs(int(first) - int(second)) <= 0.03 * (first + second), (p0, first, second)
     one = P.unit_order_segments(desc[:Rb * 4], Rb, 1, rpu, o)                       # a single segment: untouched
     assert np.array_equal(one, o)
 
