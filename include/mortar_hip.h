@@ -136,8 +136,13 @@ int mortar_prefill_max_seg_cb(void);
 /* Row-unit order for uneven nnz: units sorted by descending block count and dealt into groups of `group`
  * consecutive positions with similar totals (longest-processing-time first); use group = 16, the number of
  * wavefronts of a prefill workgroup.  rows_per_unit = 1 (plain) or 2 (gate row u and up row u + Rb/2).
+ * Every group lists its units heaviest first; with snake != 0 the odd groups are reversed.  Use snake = 1 for
+ * matrices with several K segments (their prefill kernel gives wave w the positions w, w + group, ... of its window:
+ * without the reversal wave 0 would collect the heaviest unit of every group) and snake = 0 for single-segment
+ * matrices, whose kernels let the waves of a workgroup draw positions one after another (the last draws of a window
+ * should be its lightest units).
  * order_out host [n_units]: the unit at each schedule position.  Uniform rows keep the natural order. */
-int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_t rows_per_unit, int32_t group,
+int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_t rows_per_unit, int32_t group, int32_t snake,
                            int32_t *order_out);
 
 /* Second pass over a unit order for matrices with several K segments (nseg > 1).  The K-segmented prefill

@@ -43,7 +43,7 @@ _SIGS = {
     "mortar_prefill_max_seg_cb": (C.c_int, []),
     "mortar_validate_bcsr_host": (C.c_int, [c_vp, c_vp, c_i32, c_i32]),
     "mortar_schedule_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp]),
-    "mortar_unit_order_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp]),
+    "mortar_unit_order_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp]),
     "mortar_unit_order_segments_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
     "mortar_decode_worklist_host": (c_i64, [c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp]),
     "mortar_spmm_bf16": (C.c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_i64, c_vp]),

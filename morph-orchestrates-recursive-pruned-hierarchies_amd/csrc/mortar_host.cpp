@@ -239,7 +239,7 @@ extern "C" int mortar_fp4_stream_host(const uint32_t *codes_o, int64_t ngroups, 
 }
 
 extern "C" int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_t rows_per_unit,
-                                      int32_t group, int32_t *order_out) {
+                                      int32_t group, int32_t snake, int32_t *order_out) {
     if (!row_ptr || !order_out || Rb <= 0 || group <= 0 || (rows_per_unit != 1 && rows_per_unit != 2) ||
         Rb % rows_per_unit)
         return mortar_fail(MORTAR_ERR_ARG, "unit_order: bad argument");
@@ -270,13 +270,14 @@ extern "C" int mortar_unit_order_host(const int32_t *row_ptr, int32_t Rb, int32_
         members[best].push_back(u);
         load[best] += cost[u];
     }
-    // Wave w of a workgroup takes the positions w, w + group, ... of its window: every group hands one unit
-    // to each wave.  Members are in descending cost; odd groups are reversed so that no wave collects the
-    // heaviest unit of every group.
+    // Members are in descending cost.  Where wave w of a workgroup takes the positions w, w + group, ... of its
+    // window (every group hands one unit to each wave) the odd groups are reversed so that no wave collects the
+    // heaviest unit of every group; where the waves draw positions one after another every group stays heaviest
+    // first, so that a window ends with light units (ragged gate_up, 160 layers at one row: 91 -> 84 us).
     int o = 0;
     for (int g = 0; g < ng; ++g) {
         const int n = (int)members[g].size();
-        for (int i = 0; i < n; ++i) order_out[o++] = members[g][(g & 1) ? n - 1 - i : i];
+        for (int i = 0; i < n; ++i) order_out[o++] = members[g][(snake && (g & 1)) ? n - 1 - i : i];
     }
     return MORTAR_OK;
 }

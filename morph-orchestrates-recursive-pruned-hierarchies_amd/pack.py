@@ -100,10 +100,13 @@ def transpose_topology(offsets, col, Rb: int, Cb: int):
     return off_t, col_t, src
 
 
-def unit_order(offsets, Rb: int, rows_per_unit: int, group: int = SCHED_GROUP) -> np.ndarray:
+def unit_order(offsets, Rb: int, rows_per_unit: int, group: int = SCHED_GROUP, snake: bool = True) -> np.ndarray:
+    """Row units by schedule position (mortar_unit_order_host): ``snake`` reverses the odd groups, for the kernels
+    that give wave w the positions w, w + group, ... of a window (matrices with several K segments)."""
     offsets = _np(offsets, np.int32)
     out = np.empty(Rb // rows_per_unit, dtype=np.int32)
-    _lib.check(_lib.lib().mortar_unit_order_host(_vp(offsets), Rb, rows_per_unit, group, _vp(out)), "mortar_unit_order_host")
+    _lib.check(_lib.lib().mortar_unit_order_host(_vp(offsets), Rb, rows_per_unit, group, 1 if snake else 0, _vp(out)),
+               "mortar_unit_order_host")
     return out
 
 
@@ -360,7 +363,7 @@ class MortarPack:
     def sched(self, rows_per_unit: int) -> torch.Tensor:
         """Device schedule (mortar_schedule_host over the balanced unit order) for plain (1) or gate/up (2) units."""
         if rows_per_unit not in self._scheds:
-            o = unit_order(self.h_offsets, self.Rb, rows_per_unit)
+            o = unit_order(self.h_offsets, self.Rb, rows_per_unit, snake=self.nseg > 1)
             if self.nseg > 1:
                 o = unit_order_segments(self.h_row_desc, self.Rb, self.nseg, rows_per_unit, o)
             sc = schedule(self.h_row_desc, self.Rb, self.nseg, rows_per_unit, o)

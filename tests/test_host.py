@@ -167,6 +167,12 @@ def test_unit_order_and_schedule():
         loads = [cost[o[g:g + group]].sum() for g in range(0, nu, group)]
         naive = [cost[g:g + group].sum() for g in range(0, nu, group)]
         assert max(loads) <= max(naive)
+        # groups hold the same units either way; without the snake every group is heaviest first, with it the odd
+        # groups are reversed
+        flat = P.unit_order(m["offsets"], 64, rpu, snake=False)
+        for gi, g in enumerate(range(0, nu, group)):
+            assert (np.diff(cost[flat[g:g + group]]) <= 0).all()
+            assert flat[g:g + group].tolist() == (o[g:g + group][::-1] if gi % 2 else o[g:g + group]).tolist()
         sc = P.schedule(desc, 64, 3, rpu, o)                                            # [nu, nseg, rpu, 4]
         d3 = desc.reshape(3, 64, 4)
         for pos in (0, 1, nu - 1):
