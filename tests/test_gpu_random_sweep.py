@@ -129,8 +129,11 @@ def test_random_backward_products(dev, seed):
         M = cfg["M"]
         m = synth.synth_matrix(Rb * 16, Cb * 16, cfg["dens"], seed=cfg["seed"], zipf_s=cfg["zipf"])
         a, b = synth.synth_x(M, Rb * 16, seed=cfg["seed"] + 1), synth.synth_x(M, Cb * 16, seed=cfg["seed"] + 2)
-        got = to_np(ops.sdd(to_dev(a, dev), to_dev(b, dev), synth.to_pack(m, dev)))
-        assert_close_bf16(got, O.sdd_at_b(O.bf16_round(a), O.bf16_round(b), m["row_idx"], m["col_idx"]), what + " dW")
+        ref_dw = O.sdd_at_b(O.bf16_round(a), O.bf16_round(b), m["row_idx"], m["col_idx"])
+        Wd = synth.to_pack(m, dev)
+        assert_close_bf16(to_np(ops.sdd(to_dev(a, dev), to_dev(b, dev), Wd)), ref_dw, what + " dW")
+        nbw = int(np.random.default_rng(cfg["seed"] + 9).choice([8, 10, 12, 14, 16, 18, 20, 22]))      # any built group size
+        assert_close_bf16(to_np(ops.sdd(to_dev(a, dev), to_dev(b, dev), Wd, blocks_per_wave=nbw)), ref_dw, what + f" dW group size {nbw}")
         nnz = m["col_idx"].size
         g = np.random.Generator(np.random.PCG64(cfg["seed"] + 3))
         v = g.standard_normal((nnz, 16, 16), dtype=np.float32) * g.uniform(0.01, 0.1, (nnz, 1, 1)).astype(np.float32)
@@ -146,3 +149,27 @@ def test_random_backward_products(dev, seed):
                           what + " dX", ulps=8)
         assert_close_bf16(to_np(ops.spmm(to_dev(b, dev), W)), (O.bf16_round(b).astype(np.float64) @ dense.T).astype(np.float32),
                           what + " y", ulps=8)
+
+
+@pytest.mark.parametrize("seed", [401])
+def test_random_fp32_decode_products(dev, seed):
+    """mortar_gemv in fp32 arithmetic on random shapes with one scale per matrix (the SpMM-kernel form: 3 * B term rows
+    through 4-, 8-, 16-token and prefill tiles, one or several K segments, with and without the 4-bit stream) and with a
+    scale per block (the work-list kernel), against the oracle's float64 sums."""
+    rng = np.random.default_rng(seed)
+    for it in range(40):
+        Rb = int(rng.choice([1, 2, 7, 16, 33, 64, 128, 200]))
+        Cb = int(rng.choice([1, 2, 5, 16, 48, 96, 128, 155, 156, 352]))
+        cfg = dict(it=it, Rb=Rb, Cb=Cb, dens=float(rng.choice([0.1, 0.25, 0.5, 1.0])), zipf=None if rng.random() < 0.5 else 1.2,
+                   B=int(rng.choice([1, 2, 4, 5, 6, 16, 21, 22, 43, 64])), one=bool(rng.random() < 0.7),
+                   seg=None if rng.random() < 0.6 else int(rng.integers(1, 80)), stream4=bool(rng.random() < 0.6),
+                   seed=int(rng.integers(1, 10000)))
+        what = f"seed {seed} case {cfg}"
+        m = synth.synth_matrix(Rb * 16, Cb * 16, cfg["dens"], seed=cfg["seed"], zipf_s=cfg["zipf"])
+        if cfg["one"]:
+            m["scales"] = m["scales"][:1] * np.float32(1.2345)
+        W = _pack(m, dev, seg_cb=cfg["seg"], prefill_stream=cfg["stream4"])
+        x = (np.random.default_rng(cfg["seed"] + 1).standard_normal((cfg["B"], Cb * 16)) * 1.37).astype(np.float32)
+        ref = O.mortar_gemv(x, m["codes"], m["scales"], m["col_idx"], m["offsets"]).astype(np.float64)
+        got = ops.gemv_f32(torch.from_numpy(x).to(dev), W).cpu().numpy()
+        assert np.abs(got - ref).max() <= 3e-6 * max(np.abs(ref).max(), 1e-30), what
