@@ -350,6 +350,8 @@ class MortarPack:
         if nb is None:
             nb = _lib.check(L.mortar_sdd_blocks_per_wave_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, M),
                             "mortar_sdd_blocks_per_wave_host")
+            if len(self._sdd) > 256:                        # many token counts seen: keep the plans, forget the choices
+                self._sdd = {k: v for k, v in self._sdd.items() if not isinstance(k, tuple)}
             self._sdd[("M", M)] = nb
         if nb not in self._sdd:
             n = _lib.check(L.mortar_sdd_plan_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, nb, None, 0),
