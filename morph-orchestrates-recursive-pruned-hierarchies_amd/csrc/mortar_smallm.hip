@@ -114,6 +114,13 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
             case 2: return mortar_launch_segmented<32, 1, false, 16, 4, true, CODE>(p, table, layers, st);
         }
     }
+    if (!table && p.M > MORTAR_SMALLM_MAX) {      // 65..128 rows: only the part-split form of a K-segmented plain product
+        if (p.M <= MORTAR_PARTSPLIT_MAX && (kind == 0 || kind == 3) && p.nseg > 1 && fits(8, p.Cb)) {
+            const int rc = launch_partsplit<8, CODE>(kind, p, st);
+            if (rc >= 0) return rc;
+        }
+        return -1;
+    }
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
     if (t == 0) return -1;
     const bool resident = t > 0;

@@ -105,6 +105,7 @@ __device__ __forceinline__ SpmmView mortar_view(const SpmmParams &q) {
 constexpr int CODE_2BIT = 0, CODE_4BIT = 1, CODE_UNIFORM = 2;
 
 constexpr int MORTAR_SMALLM_MAX = 64;    // rows up to which the small-tile (decode) instantiations are used
+constexpr int MORTAR_PARTSPLIT_MAX = 128; // rows up to which a plain product over several K segments runs 8-token tiles of all K
 constexpr int RES_GROUPS = 4;            // octets (4 block pairs each) loaded per batch
 constexpr int LDS_BUDGET = 156 * 1024;   // bytes of LDS a token tile may take
 constexpr int LDS_PAD = 32;              // 16-byte units past the tile that idle lanes of a narrow tile may read

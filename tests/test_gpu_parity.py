@@ -528,6 +528,22 @@ def test_decode_rows_wider_than_any_resident_tile(dev, B):
     assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), ref, "K-segmented SpMM", ulps=8)
 
 
+@pytest.mark.parametrize("M", [65, 100, 128, 129])
+def test_plain_product_over_k_segments_at_65_to_128_rows(dev, M):
+    """65..128 rows of a matrix with several K segments run 8-token tiles of all K (a row's parts on different waves);
+    one more row goes to the 32-token tiles: same product, plain and with the routed input mask, ragged rows."""
+    d_ff, ncl = 16 * 352, 352
+    m = synth.synth_matrix(16 * 40, d_ff, 0.25, seed=66, zipf_s=1.2)
+    W = synth.to_pack(m, dev)
+    assert W.nseg > 1
+    x = synth.synth_x(M, d_ff, 67)
+    assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), oracle_spmm(x, m), f"M={M}", ulps=8)
+    act = O.remoe_gates(synth.synth_logits(M, ncl, 68), 88)[1]
+    xm = x * np.repeat(act, d_ff // ncl, axis=1)
+    got = ops.spmm(to_dev(x, dev), W, active=torch.from_numpy(act.astype(np.uint8)).to(dev))
+    assert_close_bf16(to_np(got), oracle_spmm(xm, m), f"masked M={M}", ulps=8)
+
+
 @pytest.mark.parametrize("max_blocks", [3, 8])
 def test_decode_split_rows_partials(dev, max_blocks):
     spec = synth.synth_mlp(512, 16 * 90, 0.3, seed=60, zipf_s=1.2)
