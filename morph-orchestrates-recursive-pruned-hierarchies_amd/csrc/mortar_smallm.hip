@@ -114,11 +114,20 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
             case 2: return mortar_launch_segmented<32, 1, false, 16, 4, true, CODE>(p, table, layers, st);
         }
     }
-    if (!table && p.M > MORTAR_SMALLM_MAX) {      // 65..128 rows: only the part-split form of a K-segmented plain product
-        if (p.M <= MORTAR_PARTSPLIT_MAX && (kind == 0 || kind == 3) && p.nseg > 1 && fits(8, p.Cb)) {
+    if (!table && p.M > MORTAR_SMALLM_MAX) {
+        // 65 rows and more: only a plain product over several K segments, whose 32-token prefill tiles walk the segments
+        // one after another in few workgroups, has faster small-tile forms, as long as these fit one round of
+        // workgroups: 8-token tiles of all K with a row's parts on different waves up to 128 rows (`down`: 10.7 against
+        // 13.3 us), else 16-token K-segmented tiles with 8 waves (256 rows: 11.1 against 13.7 us) or 16 waves (384 rows:
+        // 12.8 against 14.0 us).
+        if ((kind != 0 && kind != 3) || p.nseg <= 1) return -1;
+        if (p.M <= MORTAR_PARTSPLIT_MAX && fits(8, p.Cb)) {
             const int rc = launch_partsplit<8, CODE>(kind, p, st);
             if (rc >= 0) return rc;
         }
+        const int64_t tiles = (p.M + 15) / 16;
+        if (tiles * ((p.n_units + 7) / 8) <= 256) return launch_kind<16, 8, CODE>(kind, false, p, nullptr, 1, st);
+        if (tiles * ((p.n_units + 15) / 16) <= 256) return launch_kind<16, 16, CODE>(kind, false, p, nullptr, 1, st);
         return -1;
     }
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
@@ -138,6 +147,9 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
         if (w == 16) return launch_kind<4, 16, CODE>(kind, true, p, table, layers, st);
         return w == 8 ? launch_kind<4, 8, CODE>(kind, true, p, table, layers, st) : launch_kind<4, 2, CODE>(kind, true, p, table, layers, st);
     }
+    // one matrix whose rows are too wide for an 8-token tile of all K: K-segmented 16-token tiles with 8 waves, which
+    // stage a segment four times faster than 2-wave workgroups (4096 x 11008 at 5..64 rows: 13 against 20 us; 16 waves 15 us)
+    if (!table && !resident) return launch_kind<16, 8, CODE>(kind, resident, p, table, layers, st);
     if (w == 16) return launch_kind<16, 16, CODE>(kind, resident, p, table, layers, st);
     return w == 8 ? launch_kind<16, 8, CODE>(kind, resident, p, table, layers, st) : launch_kind<16, 2, CODE>(kind, resident, p, table, layers, st);
 }
