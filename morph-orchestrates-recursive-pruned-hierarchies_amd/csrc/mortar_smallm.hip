@@ -131,13 +131,34 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
         return -1;
     }
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
-    if (t == 0) return -1;
+    // One matrix whose 16-token tile of all K leaves no room for the partial sums of the part-split form, or (gate_up)
+    // does not fit at all: 8-token tiles up to 32 rows, else 4-token tiles up to 8 rows - the weights are then read
+    // from L2 once per tile, which beats one 2-wave workgroup per CU staging 130 KB or the 32-token prefill tiles
+    // (gate_up [22016, 4096] at 12.5 %: 5.6 us at 5..8 rows, 9.6 at 16, 13.9 at 32, against 17..19 us; [43648, 8192]
+    // with 4-token tiles: 16 against 22.5 us at 5..8 rows, but 34 against 23 us at 16).
+    auto narrow_tiles = [&]() {
+        int rc = -1;
+        if (p.M <= 32) rc = launch_partsplit<8, CODE>(kind, p, st);
+        if (rc < 0 && p.M <= 8 && fits(4, p.Cb)) rc = launch_partsplit<4, CODE>(kind, p, st);
+        return rc;
+    };
+    if (t == 0) {
+        if (!table && layers == 1 && kind == 1 && p.M <= MORTAR_SMALLM_MAX) {
+            const int rc = narrow_tiles();
+            if (rc >= 0) return rc;
+        }
+        return -1;
+    }
     const bool resident = t > 0;
     const int w = pick_waves(t, p, layers);
     if (!table && layers == 1 && w == 2) {      // one matrix over the whole chip: latency form
         int rc = -1;
-        if (resident) rc = t == 4 ? launch_partsplit<4, CODE>(kind, p, st) : launch_partsplit<16, CODE>(kind, p, st);
-        else if (fits(8, p.Cb)) rc = launch_partsplit<8, CODE>(kind, p, st);      // 8-token tiles of all K instead of K segments
+        if (resident) {
+            rc = t == 4 ? launch_partsplit<4, CODE>(kind, p, st) : launch_partsplit<16, CODE>(kind, p, st);
+            if (rc < 0 && t == 16 && kind != 2 && tile_bytes(16, p.Cb) + 16 * 2 * 1024 > 160 * 1024) rc = narrow_tiles();
+        } else if (fits(8, p.Cb)) {
+            rc = launch_partsplit<8, CODE>(kind, p, st);      // 8-token tiles of all K instead of K segments
+        }
         if (rc >= 0) return rc;
         // no part-split form (a plain product whose rows are one part each): above one 16-token tile the 32-token
         // prefill tiles of the caller are faster than 2-wave workgroups per 16-token tile (48 rows: 7.5 against 15.5 us)

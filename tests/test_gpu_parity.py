@@ -528,6 +528,25 @@ def test_decode_rows_wider_than_any_resident_tile(dev, B):
     assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), ref, "K-segmented SpMM", ulps=8)
 
 
+@pytest.mark.parametrize("d_model,rows", [(4096, (5, 8, 9, 16, 24, 32, 33)), (5120, (5, 16, 32, 40)), (8192, (3, 5, 8, 9, 16))])
+def test_gate_up_of_wide_models_at_decode_batches(dev, d_model, rows):
+    """gate_up + SwiGLU for d_model 4096 / 5120 / 8192 at 3..40 rows: a 16-token tile of all K leaves no room for the
+    part-split form's partial sums (or does not fit at all), so 8-token tiles (up to 32 rows) or 4-token tiles (up to 8
+    rows) run, several per launch; beyond those the wider tiles.  Plain, gated, and the plain gate_up product."""
+    d_ff, ncl = 16 * 24, 24
+    spec = synth.synth_mlp(d_model, d_ff, 0.25, seed=77, zipf_s=1.2)
+    Wgu = synth.to_pack(spec["gate_up"], dev)
+    for M in rows:
+        x = synth.synth_x(M, d_model, 78 + M)
+        g_ref = O.remoe_gates(synth.synth_logits(M, ncl, 79), 9)[0]
+        ref, refg = O.swiglu_mlp(x, spec["gate_up"], spec["down"]), O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=g_ref)
+        xd = to_dev(x, dev)
+        assert_close_bf16(to_np(ops.gateup_swiglu(xd, Wgu)), ref["h"], f"h d_model={d_model} M={M}", ulps=8)
+        hg = ops.gateup_swiglu(xd, Wgu, gates=torch.from_numpy(g_ref).to(dev))
+        assert_close_bf16(to_np(hg), refg["h"], f"gated h d_model={d_model} M={M}", ulps=8)
+        assert_close_bf16(to_np(ops.spmm(xd, Wgu)), oracle_spmm(x, spec["gate_up"]), f"gu d_model={d_model} M={M}", ulps=8)
+
+
 @pytest.mark.parametrize("M", [65, 100, 128, 129])
 def test_plain_product_over_k_segments_at_65_to_128_rows(dev, M):
     """65..128 rows of a matrix with several K segments run 8-token tiles of all K (a row's parts on different waves);
