@@ -68,12 +68,16 @@ static int pick_waves(int t, const SpmmParams &p, int layers) {
     return bytes > 40 * 1024 ? 16 : 8;
 }
 
-// Part-split launch for one matrix: PW waves per unit, PW = 4, 3 or 2 dividing the unit's part count.
+// Part-split launch for one matrix: PW waves per unit, PW = 4, 3 or 2, dividing the unit's part count where one does.
 template <int MT, int CODE>
 static int launch_partsplit(int kind, SpmmParams &p, hipStream_t st) {
     const int nacc = (kind == 0 || kind == 3) ? 1 : 2, nparts = p.nseg * nacc;
-    const int pw = nparts % 4 == 0 ? 4 : (nparts % 3 == 0 ? 3 : (nparts % 2 == 0 ? 2 : 0));
-    if (pw == 0 || tile_bytes(MT, p.Cb) + 16 * 2 * 1024 > 160 * 1024) return -1;
+    // a part count no wave count divides (5, 7, 11 ... K segments): the waves of a unit take parts q, q + PW, ... and
+    // some take one more than others - still far better than one wave per unit ([4096, 11008] at one row: 9.0 -> 5.6 us)
+    int pw = nparts % 4 == 0 ? 4 : (nparts % 3 == 0 ? 3 : (nparts % 2 == 0 ? 2 : 0));
+    if (pw == 0 && nparts >= 5) pw = (nparts + 3) / 4 < (nparts + 2) / 3 ? 4 : 3;
+    // LDS: the tile, then the partial sums of the workgroup's PW * 4 waves (1 KB per wave, accumulator and sub-tile)
+    if (pw == 0 || tile_bytes(MT, p.Cb) + pw * 4 * nacc * ((MT + 15) / 16) * 1024 > 160 * 1024) return -1;
     switch (kind * 10 + pw) {
         case 2: return mortar_launch_partsplit<MT, 1, false, false, 2, 4, CODE>(p, st);
         case 3: return mortar_launch_partsplit<MT, 1, false, false, 3, 4, CODE>(p, st);
@@ -155,9 +159,10 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
         int rc = -1;
         if (resident) {
             rc = t == 4 ? launch_partsplit<4, CODE>(kind, p, st) : launch_partsplit<16, CODE>(kind, p, st);
-            if (rc < 0 && t == 16 && kind != 2 && tile_bytes(16, p.Cb) + 16 * 2 * 1024 > 160 * 1024) rc = narrow_tiles();
-        } else if (fits(8, p.Cb)) {
-            rc = launch_partsplit<8, CODE>(kind, p, st);      // 8-token tiles of all K instead of K segments
+            if (rc < 0 && t == 16 && kind != 2 && tile_bytes(16, p.Cb) + 16 * 1024 > 160 * 1024) rc = narrow_tiles();
+        } else {
+            if (fits(8, p.Cb)) rc = launch_partsplit<8, CODE>(kind, p, st);      // 8-token tiles of all K instead of K segments
+            if (rc < 0) rc = narrow_tiles();
         }
         if (rc >= 0) return rc;
         // no part-split form (a plain product whose rows are one part each): above one 16-token tile the 32-token

@@ -547,6 +547,23 @@ def test_gate_up_of_wide_models_at_decode_batches(dev, d_model, rows):
         assert_close_bf16(to_np(ops.spmm(xd, Wgu)), oracle_spmm(x, spec["gate_up"]), f"gu d_model={d_model} M={M}", ulps=8)
 
 
+@pytest.mark.parametrize("Cb,rows", [(688, (1, 4, 5, 8, 9, 16, 40)), (1024, (1, 3, 5, 8, 9)), (864, (2, 7, 8, 33))])
+def test_down_of_wide_models_at_decode_batches(dev, Cb, rows):
+    """`down` with 11008 / 16384 / 13824 input features (5, 7 and 6 K segments): the waves of a row unit share its parts
+    also when their count divides by none of 4, 3, 2, and 5..8 rows run two 4-token tiles of all K; beyond that the
+    K-segmented 16-token tiles.  Plain and with the routed input mask."""
+    m = synth.synth_matrix(16 * 20, 16 * Cb, 0.25, seed=88, zipf_s=1.2)
+    W = synth.to_pack(m, dev)
+    assert W.nseg == {688: 5, 1024: 7, 864: 6}[Cb]
+    ncl = Cb
+    for M in rows:
+        x = synth.synth_x(M, 16 * Cb, 89 + M)
+        assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), oracle_spmm(x, m), f"Cb={Cb} M={M}", ulps=8)
+        act = O.remoe_gates(synth.synth_logits(M, ncl, 90), ncl // 4)[1]
+        got = ops.spmm(to_dev(x, dev), W, active=torch.from_numpy(act.astype(np.uint8)).to(dev))
+        assert_close_bf16(to_np(got), oracle_spmm(x * np.repeat(act, 16, axis=1), m), f"masked Cb={Cb} M={M}", ulps=8)
+
+
 @pytest.mark.parametrize("M", [65, 100, 128, 129])
 def test_plain_product_over_k_segments_at_65_to_128_rows(dev, M):
     """65..128 rows of a matrix with several K segments run 8-token tiles of all K (a row's parts on different waves);
