@@ -136,14 +136,18 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
     }
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
     // One matrix whose 16-token tile of all K leaves no room for the partial sums of the part-split form, or (gate_up)
-    // does not fit at all: 8-token tiles up to 32 rows, else 4-token tiles up to 8 rows - the weights are then read
+    // does not fit at all: several 8-token tiles, else 4-token tiles, while they make at most 768 workgroups - the weights are then read
     // from L2 once per tile, which beats one 2-wave workgroup per CU staging 130 KB or the 32-token prefill tiles
     // (gate_up [22016, 4096] at 12.5 %: 5.6 us at 5..8 rows, 9.6 at 16, 13.9 at 32, against 17..19 us; [43648, 8192]
     // with 4-token tiles: 16 against 22.5 us at 5..8 rows, but 34 against 23 us at 16).
     auto narrow_tiles = [&]() {
+        // one workgroup (4 row units) fills a CU's LDS: up to about three rounds of 8-token tiles, two of 4-token ones
+        // (which re-read the weights more often; a little more when there are only two tiles)
+        const int64_t per_tile = (p.n_units + 3) / 4;
         int rc = -1;
-        if (p.M <= 32) rc = launch_partsplit<8, CODE>(kind, p, st);
-        if (rc < 0 && p.M <= 8 && fits(4, p.Cb)) rc = launch_partsplit<4, CODE>(kind, p, st);
+        if ((p.M + 7) / 8 * per_tile <= 768) rc = launch_partsplit<8, CODE>(kind, p, st);
+        const int64_t t4 = (p.M + 3) / 4;
+        if (rc < 0 && (t4 * per_tile <= 512 || (t4 <= 2 && t4 * per_tile <= 704)) && fits(4, p.Cb)) rc = launch_partsplit<4, CODE>(kind, p, st);
         return rc;
     };
     if (t == 0) {
@@ -159,7 +163,7 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
         int rc = -1;
         if (resident) {
             rc = t == 4 ? launch_partsplit<4, CODE>(kind, p, st) : launch_partsplit<16, CODE>(kind, p, st);
-            if (rc < 0 && t == 16 && kind != 2 && tile_bytes(16, p.Cb) + 16 * 1024 > 160 * 1024) rc = narrow_tiles();
+            if (rc < 0 && t == 16 && kind != 2) rc = narrow_tiles();      // (fails as well where a row is one part)
         } else {
             if (fits(8, p.Cb)) rc = launch_partsplit<8, CODE>(kind, p, st);      // 8-token tiles of all K instead of K segments
             if (rc < 0) rc = narrow_tiles();
