@@ -148,6 +148,9 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
         if ((p.M + 7) / 8 * per_tile <= 768) rc = launch_partsplit<8, CODE>(kind, p, st);
         const int64_t t4 = (p.M + 3) / 4;
         if (rc < 0 && (t4 * per_tile <= 512 || (t4 <= 2 && t4 * per_tile <= 704)) && fits(4, p.Cb)) rc = launch_partsplit<4, CODE>(kind, p, st);
+        // rows of more than 19904 values: one or two 2-token tiles (down [8192, 21824] at 25 %, 12 MB of weights:
+        // 11.5 us at 1..4 rows against 18.7 us for the work-list kernel; the same time as that kernel at 8 rows)
+        if (rc < 0 && !fits(4, p.Cb) && p.M <= 4 && fits(2, p.Cb)) rc = launch_partsplit<2, CODE>(kind, p, st);
         return rc;
     };
     if (t == 0) {

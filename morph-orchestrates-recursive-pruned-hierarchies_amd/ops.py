@@ -297,9 +297,9 @@ def gemv(x: Tensor, W: MortarPack, swiglu_out: bool = False, gates: Tensor | Non
         raise ValueError(f"gemv: batch {B} outside 1..64 (use the prefill path)")
     if x.shape[1] != W.in_features:
         raise ValueError(f"gemv: x has {x.shape[1]} features, matrix expects {W.in_features}")
-    # rows so wide that not even a 4-token tile of all K fits in LDS (in_features > 19904) go to the work-list kernel,
-    # which splits K over workgroups and combines partial sums (down [8192, 21824] at b = 1: 22 us against 45 us)
-    if row_act is None and col_act is None and max_blocks is None and route_tile(W, 1) != 0:
+    # rows so wide that not even a 4-token tile of all K fits in LDS (in_features > 19904) run 2-token tiles up to 4
+    # rows; beyond that they go to the work-list kernel, which splits K over workgroups and combines partial sums
+    if row_act is None and col_act is None and max_blocks is None and (route_tile(W, 1) != 0 or (B <= 4 and not swiglu_out)):
         if swiglu_out:
             return gateup_swiglu(x, W, gates=gates.contiguous() if gates is not None else None, out=out)
         return spmm(x, W, out=out)

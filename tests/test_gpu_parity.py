@@ -515,17 +515,19 @@ def test_layer_stack_matches_single_launches(dev, B, n_layers, d_model):
                        [torch.empty((65, d_ff), dtype=torch.bfloat16, device=dev)], swiglu=True)
 
 
-@pytest.mark.parametrize("B", [1, 4, 16])
+@pytest.mark.parametrize("B", [1, 2, 3, 4, 5, 16])
 def test_decode_rows_wider_than_any_resident_tile(dev, B):
-    """in_features so wide (> 19904) that no 4-token tile of all K fits in LDS: gemv() takes the work-list kernel (K split
-    over workgroups, partial sums combined) and the plain SpMM entry point still gives the same product."""
+    """in_features so wide (> 19904) that no 4-token tile of all K fits in LDS: up to 4 rows run 2-token tiles of all K,
+    more rows the work-list kernel (K split over workgroups, partial sums combined) from gemv() and K-segmented tiles
+    from the plain SpMM entry point; with an explicit split gemv() runs the work list at any batch.  Same product."""
     m = synth.synth_matrix(16 * 6, 16 * 1300, 0.1, seed=64, zipf_s=1.2)
     W = synth.to_pack(m, dev)
     assert ops.route_tile(W, 1) == 0 and W.nseg > 8
     x = synth.synth_x(B, 16 * 1300, 65)
     ref = oracle_spmm(x, m)
-    assert_close_bf16(to_np(ops.gemv(to_dev(x, dev), W)), ref, "work-list", ulps=8)
-    assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), ref, "K-segmented SpMM", ulps=8)
+    assert_close_bf16(to_np(ops.gemv(to_dev(x, dev), W)), ref, "gemv", ulps=8)
+    assert_close_bf16(to_np(ops.gemv(to_dev(x, dev), W, max_blocks=1 << 20)), ref, "work-list", ulps=8)
+    assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), ref, "SpMM", ulps=8)
 
 
 @pytest.mark.parametrize("d_model,rows", [(4096, (5, 8, 9, 16, 24, 32, 33)), (5120, (5, 16, 32, 40)), (8192, (3, 5, 8, 9, 16))])
