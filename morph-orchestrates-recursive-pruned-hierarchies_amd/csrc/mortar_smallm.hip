@@ -38,6 +38,7 @@ int launch_kind(int kind, bool resident, SpmmParams &p, const SpmmParams *table,
     } else if (MT == 16) {
         switch (kind) {
             case 0: return mortar_launch_segmented<16, 1, false, WAVES, 1, false, CODE>(p, nullptr, 1, st);
+            case 1: if (WAVES == 8) return mortar_launch_segmented<16, 2, false, 8, 1, false, CODE>(p, nullptr, 1, st); break;
             case 3: return mortar_launch_segmented<16, 1, true, WAVES, 1, false, CODE>(p, nullptr, 1, st);
         }
     }
@@ -153,9 +154,27 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
         if (rc < 0 && !fits(4, p.Cb) && p.M <= 4 && fits(2, p.Cb)) rc = launch_partsplit<2, CODE>(kind, p, st);
         return rc;
     };
+    // gate_up over several K segments with more rows than the narrow tiles take: K-segmented 16-token tiles, 8 waves of
+    // one gate/up unit each, while they fit the chip's slots once (two workgroups per CU) - the 32-token prefill tiles
+    // leave most CUs idle at these row counts
+    auto segmented_gate_up = [&]() {
+        if (kind != 1 || p.nseg <= 1 || !fits(16, p.seg_cb)) return -1;
+        if ((p.M + 15) / 16 * (int64_t)((p.n_units + 7) / 8) > 512) return -1;
+        return launch_kind<16, 8, CODE>(1, false, p, nullptr, 1, st);
+    };
+    // gate_up: one narrow tile where the rows fit one (5.6..7 us), else the K-segmented tiles (10..12 us at 16..32 rows,
+    // where two to four 8-token tiles take 10..15 us and two 4-token tiles of d_model 8192 17 us), else narrow tiles
+    auto wide_gate_up = [&]() {
+        int rc = -1;
+        if (p.M <= 8) rc = launch_partsplit<8, CODE>(kind, p, st);
+        if (rc < 0 && p.M <= 4 && fits(4, p.Cb)) rc = launch_partsplit<4, CODE>(kind, p, st);
+        if (rc < 0) rc = segmented_gate_up();
+        if (rc < 0) rc = narrow_tiles();
+        return rc;
+    };
     if (t == 0) {
         if (!table && layers == 1 && kind == 1 && p.M <= MORTAR_SMALLM_MAX) {
-            const int rc = narrow_tiles();
+            const int rc = wide_gate_up();
             if (rc >= 0) return rc;
         }
         return -1;
@@ -166,6 +185,7 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
         int rc = -1;
         if (resident) {
             rc = t == 4 ? launch_partsplit<4, CODE>(kind, p, st) : launch_partsplit<16, CODE>(kind, p, st);
+            if (rc < 0 && t == 16 && kind == 1) rc = wide_gate_up();
             if (rc < 0 && t == 16 && kind != 2) rc = narrow_tiles();      // (fails as well where a row is one part)
         } else {
             if (fits(8, p.Cb)) rc = launch_partsplit<8, CODE>(kind, p, st);      // 8-token tiles of all K instead of K segments

@@ -530,11 +530,12 @@ def test_decode_rows_wider_than_any_resident_tile(dev, B):
     assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), ref, "SpMM", ulps=8)
 
 
-@pytest.mark.parametrize("d_model,rows", [(4096, (5, 8, 9, 16, 24, 32, 33)), (5120, (5, 16, 32, 40)), (8192, (3, 5, 8, 9, 16))])
+@pytest.mark.parametrize("d_model,rows", [(4096, (5, 8, 9, 16, 24, 32, 33, 64)), (5120, (5, 16, 32, 40, 64)), (8192, (3, 5, 8, 9, 16, 50))])
 def test_gate_up_of_wide_models_at_decode_batches(dev, d_model, rows):
-    """gate_up + SwiGLU for d_model 4096 / 5120 / 8192 at 3..40 rows: a 16-token tile of all K leaves no room for the
-    part-split form's partial sums (or does not fit at all), so 8-token tiles (up to 32 rows) or 4-token tiles (up to 8
-    rows) run, several per launch; beyond those the wider tiles.  Plain, gated, and the plain gate_up product."""
+    """gate_up + SwiGLU for d_model 4096 / 5120 / 8192 at 3..64 rows: a 16-token tile of all K leaves no room for the
+    part-split form's partial sums (or does not fit at all), so one 8- or 4-token tile of all K runs where the rows fit
+    one, and K-segmented 16-token tiles (8 waves, one gate/up unit each) beyond.  Plain, gated, and the plain gate_up
+    product (which takes several narrow tiles)."""
     d_ff, ncl = 16 * 24, 24
     spec = synth.synth_mlp(d_model, d_ff, 0.25, seed=77, zipf_s=1.2)
     Wgu = synth.to_pack(spec["gate_up"], dev)
