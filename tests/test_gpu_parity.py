@@ -530,6 +530,26 @@ def test_decode_rows_wider_than_any_resident_tile(dev, B):
     assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), ref, "SpMM", ulps=8)
 
 
+@pytest.mark.parametrize("seg_cb", [None, 8])
+def test_gate_up_many_units_over_several_16_token_tiles(dev, seg_cb):
+    """gate_up with 352 row units at 40 and 64 rows: three or four 16-token tiles of 88 four-unit workgroups each exceed
+    one round, so 8 units of two waves share a workgroup; one K segment (two parts per unit) and two (four parts)."""
+    from mortar_amd.pack import MortarPack
+    d_model, d_ff, ncl = 256, 16 * 352, 352
+    spec = synth.synth_mlp(d_model, d_ff, 0.5, seed=83, zipf_s=1.2)
+    m = spec["gate_up"]
+    Wgu = MortarPack(synth.flat_pack(m["codes"]), m["scales"], m["col_idx"], m["offsets"], m["shape"][0], m["shape"][1], dev,
+                     seg_cb=seg_cb)
+    assert Wgu.nseg == (1 if seg_cb is None else 2)
+    for M in (40, 64):
+        x = synth.synth_x(M, d_model, 84 + M)
+        g_ref = O.remoe_gates(synth.synth_logits(M, ncl, 85), 88)[0]
+        ref, refg = O.swiglu_mlp(x, spec["gate_up"], spec["down"]), O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=g_ref)
+        assert_close_bf16(to_np(ops.gateup_swiglu(to_dev(x, dev), Wgu)), ref["h"], f"h M={M}", ulps=8)
+        hg = ops.gateup_swiglu(to_dev(x, dev), Wgu, gates=torch.from_numpy(g_ref).to(dev))
+        assert_close_bf16(to_np(hg), refg["h"], f"gated h M={M}", ulps=8)
+
+
 @pytest.mark.parametrize("d_model,rows", [(4096, (5, 8, 9, 16, 24, 32, 33, 64)), (5120, (5, 16, 32, 40, 64)), (8192, (3, 5, 8, 9, 16, 50))])
 def test_gate_up_of_wide_models_at_decode_batches(dev, d_model, rows):
     """gate_up + SwiGLU for d_model 4096 / 5120 / 8192 at 3..64 rows: a 16-token tile of all K leaves no room for the
