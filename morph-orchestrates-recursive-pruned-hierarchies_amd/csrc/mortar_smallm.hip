@@ -79,11 +79,16 @@ static int launch_partsplit(int kind, SpmmParams &p, hipStream_t st) {
     if (pw == 0 && nparts >= 5) pw = (nparts + 3) / 4 < (nparts + 2) / 3 ? 4 : 3;
     // LDS: the tile, then the partial sums of the workgroup's PW * 4 waves (1 KB per wave, accumulator and sub-tile)
     if (pw == 0 || tile_bytes(MT, p.Cb) + pw * 4 * nacc * ((MT + 15) / 16) * 1024 > 160 * 1024) return -1;
-    // gate_up over more 16-token tiles than one round of 4-unit workgroups holds: 8 units per workgroup, two waves each
-    // (d_model 2048 at 33..64 rows: 8.3 -> 6.1 us)
-    if (MT == 16 && kind == 1 && nparts % 2 == 0 && (p.M + 15) / 16 * (int64_t)((p.n_units + 3) / 4) > 256 &&
-        tile_bytes(16, p.Cb) + 16 * 2 * 1024 <= 160 * 1024)
-        return mortar_launch_partsplit<16, 2, false, false, 2, 8, CODE>(p, st);
+    // more tiles x 4-unit workgroups than one round holds (one workgroup fills a CU): 8 units per workgroup, two waves
+    // each (gate_up of d_model 2048 at 33..64 rows: 8.3 -> 6.1 us)
+    if (kind != 2 && nparts >= 2 && (p.M + MT - 1) / MT * (int64_t)((p.n_units + 3) / 4) > 256 &&
+        tile_bytes(MT, p.Cb) + 16 * nacc * ((MT + 15) / 16) * 1024 <= 160 * 1024) {
+        switch (kind) {
+            case 0: return mortar_launch_partsplit<MT, 1, false, false, 2, 8, CODE>(p, st);
+            case 1: return mortar_launch_partsplit<MT, 2, false, false, 2, 8, CODE>(p, st);
+            case 3: return mortar_launch_partsplit<MT, 1, false, true, 2, 8, CODE>(p, st);
+        }
+    }
     switch (kind * 10 + pw) {
         case 2: return mortar_launch_partsplit<MT, 1, false, false, 2, 4, CODE>(p, st);
         case 3: return mortar_launch_partsplit<MT, 1, false, false, 3, 4, CODE>(p, st);
@@ -147,8 +152,9 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
     // (gate_up [22016, 4096] at 12.5 %: 5.6 us at 5..8 rows, 9.6 at 16, 13.9 at 32, against 17..19 us; [43648, 8192]
     // with 4-token tiles: 16 against 22.5 us at 5..8 rows, but 34 against 23 us at 16).
     auto narrow_tiles = [&]() {
-        // one workgroup (4 row units) fills a CU's LDS: up to about three rounds of 8-token tiles, two of 4-token ones
-        // (which re-read the weights more often; a little more when there are only two tiles)
+        // limits in 4-unit workgroups, one of which fills a CU's LDS (the launcher packs 8 units into one beyond 256):
+        // 768 for 8-token tiles, 512 for 4-token ones, which re-read the weights more often (704 when there are only
+        // two tiles); twice these limits measured slower than the K-segmented tiles that follow
         const int64_t per_tile = (p.n_units + 3) / 4;
         int rc = -1;
         if ((p.M + 7) / 8 * per_tile <= 768) rc = launch_partsplit<8, CODE>(kind, p, st);
