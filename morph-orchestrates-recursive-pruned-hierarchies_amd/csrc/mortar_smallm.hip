@@ -119,6 +119,10 @@ static int stack_tile32(int kind, const SpmmParams &p) {
     return 0;
 }
 
+static bool wide_gate_up_table(int kind, const SpmmParams &p) {
+    return kind == 1 && p.M <= MORTAR_SMALLM_MAX && p.nseg > 1 && !fits(16, p.Cb) && fits(16, p.seg_cb) && !(p.M <= 4 && fits(4, p.Cb));
+}
+
 template <int CODE>
 static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     if (table) {
@@ -188,6 +192,12 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
             const int rc = wide_gate_up();
             if (rc >= 0) return rc;
         }
+        // layer-batched gate_up whose rows fit no 16-token tile of all K: K-segmented 16-token tiles, one gate/up unit
+        // per wave
+        if (table && wide_gate_up_table(kind, p)) {
+            if (pick_waves(-16, p, layers) == 16) return mortar_launch_segmented<16, 2, false, 16, 1, true, CODE>(p, table, layers, st);
+            return mortar_launch_segmented<16, 2, false, 8, 1, true, CODE>(p, table, layers, st);
+        }
         return -1;
     }
     const bool resident = t > 0;
@@ -229,6 +239,11 @@ int mortar_smallm_shape(int kind, SpmmParams &p, int layers) {
     switch (stack_tile32(kind, p)) {       // table launches only: the choice of smallm_launch_code
         case 1: mortar_resident_shape<32, 16>(p, layers); return MORTAR_OK;
         case 2: mortar_segmented_shape<32, 16, 4>(p, layers); return MORTAR_OK;
+    }
+    if (wide_gate_up_table(kind, p)) {
+        if (pick_waves(-16, p, layers) == 16) mortar_segmented_shape<16, 16, 1>(p, layers);
+        else mortar_segmented_shape<16, 8, 1>(p, layers);
+        return MORTAR_OK;
     }
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
     if (t == 0) return mortar_fail(MORTAR_ERR_LIMIT, "shape has no small-M kernel");

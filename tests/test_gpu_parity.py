@@ -530,6 +530,20 @@ def test_decode_rows_wider_than_any_resident_tile(dev, B):
     assert_close_bf16(to_np(ops.spmm(to_dev(x, dev), W)), ref, "SpMM", ulps=8)
 
 
+@pytest.mark.parametrize("B", [3, 8, 16, 40])
+def test_layer_stack_gate_up_of_a_wide_model(dev, B):
+    """Layer-batched gate_up + SwiGLU for d_model 5120 (no 16-token tile of all K fits): 4-token tiles up to 4 rows,
+    K-segmented 16-token tiles beyond; every layer against the oracle."""
+    d_model, d_ff, n = 5120, 16 * 24, 3
+    specs = [synth.synth_mlp(d_model, d_ff, 0.25, seed=91 + i, zipf_s=1.2) for i in range(n)]
+    packs = [synth.to_pack(sp["gate_up"], dev) for sp in specs]
+    xs = [synth.synth_x(B, d_model, 95 + i) for i in range(n)]
+    hs = [torch.full((B, d_ff), float("nan"), dtype=torch.bfloat16, device=dev) for _ in range(n)]
+    ops.LayerStack(packs, [to_dev(x, dev) for x in xs], hs, swiglu=True).run()
+    for i in range(n):
+        assert_close_bf16(to_np(hs[i]), O.swiglu_mlp(xs[i], specs[i]["gate_up"], specs[i]["down"])["h"], f"layer {i} B={B}", ulps=8)
+
+
 @pytest.mark.parametrize("seg_cb", [None, 8])
 def test_gate_up_many_units_over_several_16_token_tiles(dev, seg_cb):
     """gate_up with 352 row units at 40 and 64 rows: three or four 16-token tiles of 88 four-unit workgroups each exceed
