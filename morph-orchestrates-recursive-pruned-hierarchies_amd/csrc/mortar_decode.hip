@@ -466,9 +466,23 @@ int launch_gemv_f32(const GemvF32Params &p, hipStream_t st) {
 // work-list kernel above up to the order of the fp32 additions.
 
 // thread = 8 consecutive features of one row: x (or silu(g) * u of a gate_up output) -> 16 bytes of each term row
+// Behind the split, threads of further blocks reduce the row flags: unit_on[r] = any stream has row_act[b, r] set (the
+// work-list kernel skips a unit only when all B streams are inactive, and writes zeros).  A chunk whose input column is
+// inactive for all B streams is written as zeros, which is what skipping its blocks amounts to.
 __global__ void __launch_bounds__(256) gemv_f32_split_kernel(const float *x, int B, int K, int64_t ldx, int swiglu_x,
-                                                             uint16_t *xs) {
+                                                             uint16_t *xs, const int32_t *col_act, int64_t ldc,
+                                                             const int32_t *row_act, int64_t ldr, int n_flags,
+                                                             int32_t *unit_on, int split_blocks) {
     const int nch = K / 8;
+    if ((int)blockIdx.x >= split_blocks) {
+        const int r = ((int)blockIdx.x - split_blocks) * 256 + threadIdx.x;
+        if (r < n_flags) {
+            int f = 0;
+            for (int b = 0; b < B; ++b) f |= row_act[(int64_t)b * ldr + r] != 0;
+            unit_on[r] = f;
+        }
+        return;
+    }
     const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (it >= (int64_t)B * nch) return;
     const int tok = (int)(it / nch), ch = (int)(it % nch);
@@ -492,6 +506,14 @@ __global__ void __launch_bounds__(256) gemv_f32_split_kernel(const float *x, int
         const float s0 = r0 - bf16_to_f32(m2 & 0xffffu), s1 = r1 - bf16_to_f32(m2 >> 16);
         hi[k / 2] = h2; mid[k / 2] = m2; lo[k / 2] = bf16_pack2(s0, s1);
     }
+    if (col_act) {
+        int f = 0;
+        for (int b = 0; b < B; ++b) f |= col_act[(int64_t)b * ldc + (ch >> 1)] != 0;
+        if (!f) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) hi[k] = mid[k] = lo[k] = 0u;
+        }
+    }
     uint4 *dst = reinterpret_cast<uint4 *>(xs + (int64_t)tok * K + ch * 8);
     const int64_t plane = (int64_t)B * K / 8;                    // 16-byte units per term
     dst[0] = uint4{hi[0], hi[1], hi[2], hi[3]};
@@ -502,11 +524,15 @@ __global__ void __launch_bounds__(256) gemv_f32_split_kernel(const float *x, int
 // y3 [3B, N]: the sums of the hi, mid and lo rows.  y = scale * ((hi + mid) + lo), then the epilogue of the mode.
 __global__ void __launch_bounds__(256) gemv_f32_combine3_kernel(const float *y3, const float *scale, int B, int N, int mode,
                                                                 const float *gates, int cluster_size, int64_t ldg,
-                                                                float *y, int64_t ldy) {
+                                                                const int32_t *unit_on, float *y, int64_t ldy) {
     const int nout = mode == 0 ? N : N / 2;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (int64_t)B * nout) return;
     const int tok = (int)(i / nout), o = (int)(i % nout);
+    if (unit_on && unit_on[o >> 4] == 0) {                       // the unit is off for every stream: zeros
+        y[(int64_t)tok * ldy + o] = 0.f;
+        return;
+    }
     const float s = scale[0];
     const float *r0 = y3 + (int64_t)tok * N, *r1 = r0 + (int64_t)B * N, *r2 = r1 + (int64_t)B * N;
     const float a = s * ((r0[o] + r1[o]) + r2[o]);
@@ -520,7 +546,7 @@ __global__ void __launch_bounds__(256) gemv_f32_combine3_kernel(const float *y3,
 }
 
 int64_t gemv_f32_fast_bytes(const mortar_bcsr_t *W, int B) {
-    return (int64_t)3 * B * ((int64_t)W->Rb * 16 * 4 + (int64_t)W->Cb * 16 * 2);
+    return (int64_t)3 * B * ((int64_t)W->Rb * 16 * 4 + (int64_t)W->Cb * 16 * 2) + (((int64_t)W->Rb * 4 + 15) & ~(int64_t)15);
 }
 
 // Returns MORTAR_NO_KERNEL when the SpMM kernels cannot serve the shape (the caller then runs the work-list kernel).
@@ -528,14 +554,17 @@ int gemv_f32_fast(const mortar_bcsr_t *W, const int32_t *sched, const GemvF32Par
     const int K = W->Cb * 16, N = W->Rb * 16;
     float *y3 = reinterpret_cast<float *>(ws);
     uint16_t *xs = reinterpret_cast<uint16_t *>(y3 + (int64_t)3 * p.B * N);
+    int32_t *unit_on = reinterpret_cast<int32_t *>(xs + (int64_t)3 * p.B * K);
     const int64_t nsplit = (int64_t)p.B * (K / 8);
-    hipLaunchKernelGGL(gemv_f32_split_kernel, dim3((unsigned)((nsplit + 255) / 256)), dim3(256), 0, st, p.x, p.B, K, p.ldx,
-                       p.swiglu_x, xs);
+    const int split_blocks = (int)((nsplit + 255) / 256);
+    const int n_flags = p.row_act ? (p.mode == 0 ? W->Rb : W->Rb / 2) : 0;       // gate and up rows share the gate row's flag
+    hipLaunchKernelGGL(gemv_f32_split_kernel, dim3((unsigned)(split_blocks + (n_flags + 255) / 256)), dim3(256), 0, st, p.x, p.B,
+                       K, p.ldx, p.swiglu_x, xs, p.col_act, p.ldc, p.row_act, p.ldr, n_flags, unit_on, split_blocks);
     const int rc = mortar_spmm_codes_f32(W, sched, xs, 3 * p.B, K, y3, N, st);
     if (rc) return rc;
     const int64_t total = (int64_t)p.B * (p.mode == 0 ? N : N / 2);
     hipLaunchKernelGGL(gemv_f32_combine3_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, y3, p.scale, p.B, N,
-                       p.mode, p.gates, p.cluster_size, p.ldg, p.y, p.ldy);
+                       p.mode, p.gates, p.cluster_size, p.ldg, p.row_act ? unit_on : nullptr, p.y, p.ldy);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "gemv_f32 launch: %s", hipGetErrorString(e));
     return MORTAR_OK;
@@ -583,7 +612,7 @@ extern "C" int mortar_gemv_f32(const mortar_bcsr_t *W, const float *scale, int64
     if (nslots > 1 && part_bytes < (int64_t)nslots * B * W->Rb * 16 * 4)
         return mortar_fail(MORTAR_ERR_ARG, "gemv_f32: the partial workspace holds %lld bytes, need %lld", (long long)part_bytes,
                            (long long)nslots * B * W->Rb * 16 * 4);
-    if (scale_count == 1 && sched && !row_act && !col_act && W->codes_o && part && !(reinterpret_cast<uintptr_t>(part) & 15) &&
+    if (scale_count == 1 && sched && W->codes_o && part && !(reinterpret_cast<uintptr_t>(part) & 15) &&
         part_bytes >= gemv_f32_fast_bytes(W, B) && ldx % 4 == 0 && !(reinterpret_cast<uintptr_t>(x) & 15)) {
         const int rc = gemv_f32_fast(W, sched, p, part, st);
         if (rc != MORTAR_NO_KERNEL) return rc;

@@ -360,8 +360,8 @@ def gemv_f32(x: Tensor, W: MortarPack, swiglu_x: bool = False, swiglu_out: bool 
     sc = W.scales_f32
     sc_one = sc.numel() == 1
     L = _lib.lib()
-    # one scale, no flags, no explicit split: the SpMM kernels run the product
-    fast = sc_one and row_act is None and col_act is None and max_blocks is None
+    # one scale, no explicit split: the SpMM kernels run the product (flags zero what the work list would skip)
+    fast = sc_one and max_blocks is None
     ws = _lib.check(L.mortar_gemv_f32_workspace_bytes(W.ref, B, nslots), "mortar_gemv_f32_workspace_bytes")
     part = torch.empty(ws // 4, dtype=torch.float32, device=x.device) if (nslots > 1 or fast) else None
     if fast and ((B > 1 and x.stride(0) % 4) or x.data_ptr() % 16):       # the split kernel reads 16-byte words

@@ -752,6 +752,21 @@ def test_mortar_gemv_fp32_one_scale_runs_on_the_spmm_kernels(dev, B):
         assert np.abs(y.cpu().numpy() - y_ref).max() <= _gemv_f32_tolerance(y_ref)
     y2 = ops.gemv_f32(torch.from_numpy(fast).to(dev), Wdn, swiglu_x=True)
     assert np.abs(y2.cpu().numpy() - y_ref).max() <= 4 * _gemv_f32_tolerance(y_ref)
+    # flags without gates, both forms: a unit that is off for EVERY stream gives zeros, a column that is off for every
+    # stream contributes nothing; anything a single stream has switched on is computed for all of them
+    ract = torch.from_numpy((rng.random((B, d_ff // 16)) < 0.3 / B).astype(np.int32)).to(dev)
+    cact = torch.from_numpy((rng.random((B, d_ff // 16)) < 0.5 / B).astype(np.int32)).to(dev)
+    unit_on = ract.cpu().numpy().any(axis=0)
+    want = (g * u * 0 + h_ref) * np.repeat(unit_on, 16)[None, :]
+    for kw in ({}, {"max_blocks": 1 << 20}):
+        got = ops.gemv_f32(xt, Wgu, swiglu_out=True, row_act=ract, **kw).cpu().numpy()
+        assert np.abs(got - want).max() <= _gemv_f32_tolerance(h_ref) and (got[:, ~np.repeat(unit_on, 16)] == 0).all()
+    col_on = np.repeat(cact.cpu().numpy().any(axis=0), 16)
+    hm = h.cpu().numpy() * col_on[None, :]
+    ym_ref = O.mortar_gemv(hm, dn_m["codes"], dn_m["scales"], dn_m["col_idx"], dn_m["offsets"]).astype(np.float64)
+    for kw in ({}, {"max_blocks": 1 << 20}):
+        got = ops.gemv_f32(h, Wdn, col_act=cact, **kw).cpu().numpy()
+        assert np.abs(got - ym_ref).max() <= _gemv_f32_tolerance(y_ref)
 
 
 @pytest.mark.parametrize("B,n,f32", [(1, 4, True), (3, 4, False), (16, 2, True), (40, 4, False), (5, 1, True), (7, 3, False)])
