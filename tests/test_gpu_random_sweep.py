@@ -173,3 +173,56 @@ def test_random_fp32_decode_products(dev, seed):
         ref = O.mortar_gemv(x, m["codes"], m["scales"], m["col_idx"], m["offsets"]).astype(np.float64)
         got = ops.gemv_f32(torch.from_numpy(x).to(dev), W).cpu().numpy()
         assert np.abs(got - ref).max() <= 3e-6 * max(np.abs(ref).max(), 1e-30), what
+
+
+@pytest.mark.parametrize("seed", [501])
+def test_random_wide_k_shapes(dev, seed):
+    """Rows of 2048 to 21824 values (d_model / d_ff of larger models) at 1 to 300 rows: the narrow tiles of all K (2, 4,
+    8 tokens, one or several per launch, 4 or 8 units per workgroup, parts shared unevenly), K-segmented 16-token tiles,
+    the prefill tiles, and layer-batched launches; plain, masked and gate_up + SwiGLU with gates."""
+    rng = np.random.default_rng(seed)
+    for it in range(60):
+        Cb = int(rng.choice([128, 192, 256, 300, 305, 320, 400, 512, 609, 610, 688, 864, 1024, 1244, 1245, 1364]))
+        units = int(rng.choice([4, 8, 24, 64, 128, 256, 352, 700, 1364]))
+        dens = float(rng.choice([0.03, 0.06, 0.125, 0.25]))
+        if units * Cb * dens > 40000:
+            dens = 40000 / (units * Cb)
+        cfg = dict(it=it, Cb=Cb, units=units, dens=round(dens, 4), zipf=None if rng.random() < 0.5 else 1.2,
+                   M=int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 48, 63, 64, 65, 100, 128, 129, 200, 256, 257, 300])),
+                   uniform=bool(rng.random() < 0.3), stream4=bool(rng.random() < 0.6), kind=int(rng.choice([0, 1, 3])),
+                   stack=bool(rng.random() < 0.5), seed=int(rng.integers(1, 10000)))
+        what = f"seed {seed} case {cfg}"
+        M = cfg["M"]
+        if cfg["kind"] == 1:
+            spec = synth.synth_mlp(Cb * 16, units * 16, dens, seed=cfg["seed"], zipf_s=cfg["zipf"])
+            m = spec["gate_up"]
+        else:
+            m = synth.synth_matrix(units * 16, Cb * 16, dens, seed=cfg["seed"], zipf_s=cfg["zipf"])
+        if cfg["uniform"]:
+            m["scales"] = np.float32(0.04)
+        W = _pack(m, dev, prefill_stream=cfg["stream4"])
+        x = synth.synth_x(M, Cb * 16, cfg["seed"] + 1)
+        xd = to_dev(x, dev)
+        if cfg["kind"] == 0:
+            ref = oracle_spmm(x, m)
+            assert_close_bf16(to_np(ops.spmm(xd, W)), ref, what + " spmm", ulps=8)
+            if M <= 64:
+                assert_close_bf16(to_np(ops.gemv(xd, W)), ref, what + " gemv", ulps=8)
+                if cfg["stack"]:
+                    ys = [torch.full((M, units * 16), float("nan"), dtype=torch.bfloat16, device=dev) for _ in range(2)]
+                    ops.LayerStack([W, W], [xd, xd], ys, swiglu=False).run()
+                    assert_close_bf16(to_np(ys[1]), ref, what + " stack", ulps=8)
+        elif cfg["kind"] == 3:
+            act = O.remoe_gates(synth.synth_logits(M, Cb, cfg["seed"] + 2), max(1, Cb // 4))[1]
+            got = ops.spmm(xd, W, active=torch.from_numpy(act.astype(np.uint8)).to(dev))
+            assert_close_bf16(to_np(got), oracle_spmm(x * np.repeat(act, 16, axis=1), m), what + " masked", ulps=8)
+        else:
+            g_ref = O.remoe_gates(synth.synth_logits(M, units, cfg["seed"] + 2), max(1, units // 3))[0]
+            ref = O.swiglu_mlp(x, spec["gate_up"], spec["down"])
+            refg = O.swiglu_mlp(x, spec["gate_up"], spec["down"], gates=g_ref)
+            assert_close_bf16(to_np(ops.gateup_swiglu(xd, W)), ref["h"], what + " h", ulps=8)
+            assert_close_bf16(to_np(ops.gateup_swiglu(xd, W, gates=torch.from_numpy(g_ref).to(dev))), refg["h"], what + " gated", ulps=8)
+            if M <= 64 and cfg["stack"]:
+                hs = [torch.full((M, units * 16), float("nan"), dtype=torch.bfloat16, device=dev) for _ in range(2)]
+                ops.LayerStack([W, W], [xd, xd], hs, swiglu=True).run()
+                assert_close_bf16(to_np(hs[1]), ref["h"], what + " stack h", ulps=8)
