@@ -299,7 +299,10 @@ def gemv(x: Tensor, W: MortarPack, swiglu_out: bool = False, gates: Tensor | Non
         raise ValueError(f"gemv: x has {x.shape[1]} features, matrix expects {W.in_features}")
     # rows so wide that not even a 4-token tile of all K fits in LDS (in_features > 19904) run 2-token tiles up to 4
     # rows; beyond that they go to the work-list kernel, which splits K over workgroups and combines partial sums
-    if row_act is None and col_act is None and max_blocks is None and (route_tile(W, 1) != 0 or (B <= 4 and not swiglu_out)):
+    rt1 = getattr(W, "_route_tile_1", None)
+    if rt1 is None:
+        rt1 = W._route_tile_1 = route_tile(W, 1)
+    if row_act is None and col_act is None and max_blocks is None and (rt1 != 0 or (B <= 4 and not swiglu_out)):
         if swiglu_out:
             return gateup_swiglu(x, W, gates=gates.contiguous() if gates is not None else None, out=out)
         return spmm(x, W, out=out)
