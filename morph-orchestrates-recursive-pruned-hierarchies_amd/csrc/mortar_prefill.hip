@@ -114,9 +114,9 @@ int dispatch_prefill(int kind, SpmmParams &p, hipStream_t st) {
 // A matrix with one scale (uniform_scale != 0) runs the kernels that multiply +-2 / 0 blocks and scale the
 // accumulators once (decode-sized launches always, prefill-sized ones through the 4-bit stream).
 int dispatch(int kind, SpmmParams &p, const mortar_bcsr_t *W, hipStream_t st) {
-    // a plain product over several K segments has small-tile forms beyond the decode sizes as well (the launcher
-    // returns -1 once they would need more than one round of workgroups)
-    if (p.M <= MORTAR_SMALLM_MAX || ((kind == 0 || kind == 3) && p.nseg > 1)) {
+    // products over several K segments have small-tile forms beyond the decode sizes as well (the launcher returns -1
+    // once they would need more than one round of workgroups)
+    if (p.M <= MORTAR_SMALLM_MAX || ((kind == 0 || kind == 1 || kind == 3) && p.nseg > 1)) {
         const int rc = mortar_smallm_launch(kind, p, nullptr, 1, st);
         if (rc >= 0) return rc;
     }

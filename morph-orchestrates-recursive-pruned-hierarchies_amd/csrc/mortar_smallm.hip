@@ -134,11 +134,17 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
         }
     }
     if (!table && p.M > MORTAR_SMALLM_MAX) {
-        // 65 rows and more: only a plain product over several K segments, whose 32-token prefill tiles walk the segments
+        // 65 rows and more: a plain product over several K segments, whose 32-token prefill tiles walk the segments
         // one after another in few workgroups, has faster small-tile forms, as long as these fit one round of
         // workgroups: 8-token tiles of all K with a row's parts on different waves up to 128 rows (`down`: 10.7 against
         // 13.3 us), else 16-token K-segmented tiles with 8 waves (256 rows: 11.1 against 13.7 us) or 16 waves (384 rows:
         // 12.8 against 14.0 us).
+        // gate_up over several K segments: the 16-token tiles with 8 waves of one gate/up unit each, while they fit the
+        // chip's slots once (d_model 3072 at 65..128 rows: 12.2..13.2 against 20..21 us for the 32-token tiles)
+        if (kind == 1 && p.nseg > 1 && fits(16, p.seg_cb)) {
+            if ((p.M + 15) / 16 * (int64_t)((p.n_units + 7) / 8) <= 512) return launch_kind<16, 8, CODE>(1, false, p, nullptr, 1, st);
+            return -1;
+        }
         if ((kind != 0 && kind != 3) || p.nseg <= 1) return -1;
         if (p.M <= MORTAR_PARTSPLIT_MAX && fits(8, p.Cb)) {
             const int rc = launch_partsplit<8, CODE>(kind, p, st);
