@@ -157,10 +157,10 @@ static int smallm_launch_code(int kind, SpmmParams &p, const SpmmParams *table, 
     }
     const int t = mortar_smallm_tile(p.Cb, p.seg_cb, p.M, kind);
     // One matrix whose 16-token tile of all K leaves no room for the partial sums of the part-split form, or (gate_up)
-    // does not fit at all: several 8-token tiles, else 4-token tiles, while they make at most 768 workgroups - the weights are then read
-    // from L2 once per tile, which beats one 2-wave workgroup per CU staging 130 KB or the 32-token prefill tiles
-    // (gate_up [22016, 4096] at 12.5 %: 5.6 us at 5..8 rows, 9.6 at 16, 13.9 at 32, against 17..19 us; [43648, 8192]
-    // with 4-token tiles: 16 against 22.5 us at 5..8 rows, but 34 against 23 us at 16).
+    // does not fit at all: several 8-token tiles, else 4-token tiles, while they make few enough workgroups - the weights
+    // are then read from L2 once per tile, which beats one 2-wave workgroup per CU staging 130 KB or the 32-token
+    // prefill tiles (gate_up [22016, 4096] at 12.5 %: 5.6 us at 5..8 rows against 17..19 us; [43648, 8192] with 4-token
+    // tiles: 16 against 22.5 us at 5..8 rows, but 34 against 23 us at 16).
     auto narrow_tiles = [&]() {
         // limits in 4-unit workgroups, one of which fills a CU's LDS (the launcher packs 8 units into one beyond 256):
         // 768 for 8-token tiles, 512 for 4-token ones, which re-read the weights more often (704 when there are only
