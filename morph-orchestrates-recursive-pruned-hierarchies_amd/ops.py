@@ -302,6 +302,10 @@ def gemv(x: Tensor, W: MortarPack, swiglu_out: bool = False, gates: Tensor | Non
     rt1 = getattr(W, "_route_tile_1", None)
     if rt1 is None:
         rt1 = W._route_tile_1 = route_tile(W, 1)
+    # gate_up with gates: the row flags add nothing there (the gated kernel leaves out the units whose cluster is off for
+    # every stream and stores their zeros; every other unit is computed and gated per stream, as the work list does)
+    if swiglu_out and gates is not None and col_act is None and max_blocks is None and rt1 != 0:
+        row_act = None
     if row_act is None and col_act is None and max_blocks is None and (rt1 != 0 or (B <= 4 and not swiglu_out)):
         if swiglu_out:
             return gateup_swiglu(x, W, gates=gates.contiguous() if gates is not None else None, out=out)
