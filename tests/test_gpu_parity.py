@@ -329,6 +329,11 @@ def test_remoe_gates_ties_and_edges(dev):
         g, a = ops.remoe_gates(torch.from_numpy(lg).to(dev), k)
         assert np.array_equal(a.cpu().numpy().astype(bool), a_ref), (n, k)
         np.testing.assert_allclose(g.cpu().numpy(), g_ref, rtol=3e-6, atol=0)
+    # the clamp of the gate sum at 1e-6 (routing.py:253): one entry one fp32 ulp above the k-th -> 2^-23 * 2e6
+    lg = np.array([[1.0 + 2.0 ** -23, 1.0, 0.0, -1.0], [1.0 + 2.0 ** -19, 1.0, 0.0, -1.0]], np.float32)
+    g, a = ops.remoe_gates(torch.from_numpy(lg).to(dev), 2)
+    np.testing.assert_allclose(g.cpu().numpy(), [[0.23841858, 0, 0, 0], [2.0, 0, 0, 0]], rtol=1e-6, atol=0)
+    assert a.cpu().numpy().astype(bool).tolist() == [[True, False, False, False]] * 2
     lg = synth.synth_logits(4096, 352, 42)                                      # benchmark config 3 router
     g_ref, a_ref = O.remoe_gates(lg, 88)
     g, a = ops.remoe_gates(torch.from_numpy(lg).to(dev), 88)

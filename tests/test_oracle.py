@@ -230,12 +230,41 @@ def test_swiglu_mlp_against_dense():
 
 def test_decode_gemv_form_equals_spmm_unrounded():
     m = make_mat(5, 8, 0.4, 40)
-    # decode applies fp32 scales exactly; make them bf16-representable so both forms agree
+    # with bf16-representable scales the decode form and the prefill form are the same sums
     m["scales"] = O.bf16_round(m["scales"])
     x = xbf(3, 128, 41)
     a = O.mortar_gemv(x, m["codes"], m["scales"], m["col_idx"], m["offsets"])
     b = O.bcsr_spmm(x, m["codes"], m["scales"], m["col_idx"], m["offsets"], round_out=False)
     assert np.allclose(a, b, rtol=1e-6, atol=1e-6)
+
+
+def test_decode_gemv_keeps_the_fp32_scale_unrounded():
+    """What separates the engine's GEMV from the prefill product (fused_decode_step.py:1335, 1441-1459): the scale is
+    fp32, is NOT rounded to bf16, and multiplies the block's sum.  Hand-computed cases with scales that bf16 cannot
+    hold (0.1 -> 0.10009765625 in bf16, 0.3 -> 0.30078125)."""
+    eye = np.eye(16, dtype=np.int8)[None]
+    x = np.arange(1, 17, dtype=np.float32)[None] / 4                      # 0.25 .. 4.0, exact in bf16
+    s01 = np.float32(0.1)
+    y = O.mortar_gemv(x, eye, np.array([s01]), np.array([0], np.int16), np.array([0, 1], np.int32))
+    want = (x.astype(np.float64) * float(s01)).astype(np.float32)          # float32(0.1) * x, correctly rounded
+    np.testing.assert_allclose(y, want, rtol=1e-7, atol=0)
+    rounded = x * O.bf16_round(np.array([s01]))[0]                         # what a bf16 scale would give: 9.8e-4 off
+    assert (np.abs(y - rounded) > 5e-4 * np.abs(y)).all()
+    # the prefill product, by contrast, does round the scale (deploy_quant.py:367-369)
+    yp = O.bcsr_spmm(x, eye, np.array([s01]), np.array([0], np.int16), np.array([0, 1], np.int32), round_out=False)
+    np.testing.assert_allclose(yp, rounded, rtol=1e-7)
+    # two blocks in one row, scales 0.1 and 0.3, codes +identity and -identity on block-columns 2 and 0:
+    # y[n] = 0.1 * x[32 + n] - 0.3 * x[n]
+    x2 = np.zeros((1, 48), np.float32); x2[0, 32:48] = 2.0; x2[0, 0:16] = np.arange(16) / 8
+    codes = np.concatenate([-eye, eye])                                   # CSR order: ascending column (0 then 2)
+    y2 = O.mortar_gemv(x2, codes, np.array([0.3, 0.1], np.float32), np.array([0, 2], np.int16), np.array([0, 2], np.int32))
+    hand = float(np.float32(0.1)) * 2.0 - float(np.float32(0.3)) * (np.arange(16) / 8)
+    np.testing.assert_allclose(y2[0], hand.astype(np.float32), rtol=2e-7, atol=1e-8)
+    # scale multiplies the SUM of the block (codes with several non-zeros per row): row n = x[n] + x[n+1 mod 16]
+    two = (np.eye(16, dtype=np.int8) + np.roll(np.eye(16, dtype=np.int8), 1, axis=1))[None]
+    y3 = O.mortar_gemv(x, two, np.array([s01]), np.array([0], np.int16), np.array([0, 1], np.int32))
+    hand3 = float(s01) * (x[0].astype(np.float64) + np.roll(x[0].astype(np.float64), -1))
+    np.testing.assert_allclose(y3[0], hand3.astype(np.float32), rtol=2e-7)
 
 
 # ---- ReMoE ---------------------------------------------------------------------------------------------
@@ -269,6 +298,27 @@ def test_remoe_brute_force_incl_ties():
         on = act.any(1)
         assert np.allclose(gates[on].sum(1), k, rtol=1e-5)                     # normalised to sum k
         assert (gates[~on] == 0).all()
+
+
+def test_remoe_gate_sum_clamp_known_answer():
+    """routing.py:253: the sum of the thresholded logits is clamped at 1e-6 before the division.  One entry sits one
+    fp32 ulp above the k-th largest: g0 = (2^-23, 0, 0, 0), sum = 1.19e-7 < 1e-6, so gates = 2^-23 * (2 / 1e-6) =
+    0.23841858 (without the clamp: 2.0; with a clamp at 1e-3: 2.38e-4)."""
+    import torch
+    lg = np.array([[1.0 + 2.0 ** -23, 1.0, 0.0, -1.0]], np.float32)
+    gates, act = O.remoe_gates(lg, 2)
+    assert act.tolist() == [[True, False, False, False]]
+    np.testing.assert_allclose(gates[0], [0.23841858, 0.0, 0.0, 0.0], rtol=1e-6, atol=0)
+    gc, ac = c_oracle.remoe_gates(lg, 2)
+    np.testing.assert_allclose(gc[0], [0.23841858, 0.0, 0.0, 0.0], rtol=1e-6, atol=0)
+    # the same steps written with the library's own ops (topk / relu / clamp), fp32
+    t = torch.from_numpy(lg)
+    g0 = torch.relu(t - torch.topk(t, 2, dim=-1).values[:, -1:])
+    want = g0 * (2.0 / g0.sum(dim=-1, keepdim=True).clamp(min=1e-6))
+    assert np.array_equal(gates, want.numpy())
+    # a sum just above the clamp is not clamped: normalised to k
+    lg2 = np.array([[1.0 + 2.0 ** -19, 1.0, 0.0, -1.0]], np.float32)        # g0 = 1.9e-6 > 1e-6
+    np.testing.assert_allclose(O.remoe_gates(lg2, 2)[0][0], [2.0, 0, 0, 0], rtol=1e-6)
 
 
 def test_router_logits_against_library_routines():
@@ -340,11 +390,16 @@ def test_rmsnorm_closed_form():
     y0 = O.rmsnorm(np.array([[3.0, 4.0]], np.float32), None, 0.0, bf16_out=False)
     np.testing.assert_allclose(y0[0], [3 / np.sqrt(12.5), 4 / np.sqrt(12.5)], rtol=1e-6)
     # the weight multiplies after the cast to the activation dtype (attention.py:139-141): bf16(bf16(x r) w)
-    xb = O.bf16_round(np.array([[1.0, 2.0, 3.0, 4.0]], np.float32)); w = np.array([1.5, 1.0, 0.5, 3.0], np.float32)
-    r = 1.0 / np.sqrt(7.5 + 1e-6)
-    want = O.bf16_round(O.bf16_round((xb * np.float32(r)).astype(np.float32)) * w)
-    assert np.array_equal(O.rmsnorm(xb, w, 1e-6), want)
-    assert O.rmsnorm(xb, w, 1e-6)[0, 3] == O.bf16_round(np.float32(O.bf16_round(np.float32(4 * r)) * 3.0))
+    # known answer: x = (1, 4), w = 1.375: x r = (0.342997, 1.371989) -> bf16 (0.34375, 1.375) -> * 1.375 =
+    # (0.47265625, 1.890625), both exact in bf16.  Rounding once, bf16(x r w), gives (0.47070312, 1.8828125) instead.
+    xb = np.array([[1.0, 4.0]], np.float32); w = np.array([1.375, 1.375], np.float32)
+    assert O.rmsnorm(xb, w, 1e-6).tolist() == [[0.47265625, 1.890625]]
+    r = np.float32(1.0 / np.sqrt(8.5 + 1e-6))
+    assert O.bf16_round(xb * r * w).tolist() == [[0.470703125, 1.8828125]]        # the mutant's numbers, for the record
+    import torch
+    tx = torch.tensor([[1.0, 4.0]], dtype=torch.bfloat16)
+    tn = (tx.float() * torch.rsqrt(tx.float().pow(2).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16) * torch.tensor(w).to(torch.bfloat16)
+    assert tn.float().tolist() == [[0.47265625, 1.890625]]                        # attention.py:139-141 in torch-CPU bf16
     x = xbf(4, 64, 60)
     y = O.rmsnorm(x, None, 1e-6, bf16_out=False)
     assert np.allclose((y.astype(np.float64) ** 2).mean(1), 1.0, atol=1e-4)
@@ -479,3 +534,57 @@ def test_training_fixture_matches_the_oracle():
     gu, dh = O.bf16_from_bits(z["gu_bits"]), O.bf16_from_bits(z["dh_bits"])
     assert np.array_equal(O.bf16_bits(O.swiglu(gu)), z["h_bits"])
     assert np.array_equal(O.bf16_bits(O.swiglu_backward(gu, dh)), z["dgu_bits"])
+
+
+def test_swiglu_family_bit_equal_to_torch_cpu_bf16():
+    """The bf16 rounding points of swiglu, swiglu_backward and the gated multiply are those of the eager graph
+    (transformer.py:403-427): checked against the library routine itself -- F.silu(gate) * up, its autograd, and
+    h.unflatten(-1, (n_clusters, cs)) * gates.to(bf16).unsqueeze(-1) -- in torch-CPU bf16, bit for bit."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(77)
+    M, d_ff, ncl = 64, 96, 6
+    gu = O.bf16_round((rng.standard_normal((M, 2 * d_ff)) * 3.0).astype(np.float32))
+    gu[0, :8] = [0.0, -0.0, 1e-30, -1e-30, 80.0, -80.0, 2.0 ** -120, -20.0]         # saturation / denormal corners
+    dh = O.bf16_round(rng.standard_normal((M, d_ff)).astype(np.float32))
+    t = torch.from_numpy(gu).to(torch.bfloat16).requires_grad_(True)
+    gate, up = t.chunk(2, dim=-1)
+    h = F.silu(gate) * up
+    assert np.array_equal(O.bf16_bits(O.swiglu(gu)), O.bf16_bits(h.detach().float().numpy()))
+    h.backward(torch.from_numpy(dh).to(torch.bfloat16))
+    got = O.swiglu_backward(gu, dh)
+    want = t.grad.float().numpy()
+    # torch's silu backward computes d_gate in fp32 from bf16 inputs with its own operation order; the oracle's
+    # float64 calculus rounded once may differ from it by one bf16 ulp in rare entries, never more
+    gb, wb = O.bf16_bits(got).astype(np.int64), O.bf16_bits(want).astype(np.int64)
+    same = gb == wb
+    assert same.mean() > 0.98, same.mean()
+    assert np.array_equal(gb[:, d_ff:], wb[:, d_ff:])                                 # d_up = dh * bf16(silu(g)): exact
+    assert (np.abs(got - want) <= 2.0 ** -7 * np.abs(want) + 1e-30).all()
+    # gated multiply: gates cast to bf16 first, product rounded to bf16
+    gates = (rng.random((M, ncl)) * 4).astype(np.float32); gates[:, 2] = 0.0
+    hb = h.detach()
+    hg = (hb.unflatten(-1, (ncl, d_ff // ncl)) * torch.from_numpy(gates).to(hb.dtype).unsqueeze(-1)).flatten(-2)
+    x = O.bf16_round(rng.standard_normal((M, 32)).astype(np.float32))
+    eye_gu = dict(codes=np.zeros((0, 16, 16), np.int8))                              # not used: call the pieces directly
+    hn = O.bf16_round(O.bf16_round(O.silu(gu[:, :d_ff])) * gu[:, d_ff:])              # as swiglu_mlp forms h
+    gbf = O.bf16_round(gates)
+    mine = O.bf16_round(hn.reshape(-1, ncl, d_ff // ncl) * gbf[:, :, None]).reshape(-1, d_ff)
+    assert np.array_equal(O.bf16_bits(mine), O.bf16_bits(hg.float().numpy()))
+    assert np.array_equal(O.bf16_bits(hn), O.bf16_bits(hb.float().numpy()))          # swiglu_mlp's fp32 silu == swiglu's
+
+
+def test_swiglu_mlp_gating_is_the_torch_expression():
+    """swiglu_mlp end to end on a tiny carved pair, against torch-CPU bf16 ops for everything after gate_up
+    (F.silu * up, cluster gates cast to bf16) and the dense float64 product for the matrices."""
+    import torch
+    import torch.nn.functional as F
+    gu, dn = make_mat(2 * 6, 4, 0.5, 33), make_mat(4, 6, 0.5, 34)
+    x = xbf(9, 64, 35)
+    gates = (np.random.default_rng(36).random((9, 3)) * 3).astype(np.float32); gates[::2, 1] = 0
+    r = O.swiglu_mlp(x, gu, dn, gates=gates)
+    t = torch.from_numpy(r["gu"]).to(torch.bfloat16)
+    g, u = t.chunk(2, dim=-1)
+    h = F.silu(g) * u
+    h = (h.unflatten(-1, (3, 32)) * torch.from_numpy(gates).to(h.dtype).unsqueeze(-1)).flatten(-2)
+    assert np.array_equal(O.bf16_bits(r["h"]), O.bf16_bits(h.float().numpy()))
