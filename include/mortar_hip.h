@@ -405,6 +405,14 @@ int mortar_requantize(const mortar_bcsr_t *W, const void *values, int32_t values
                       const float *scale_in, float *scale_out, int32_t *status, int32_t flags, float ternary_tol,
                       void *workspace, void *stream);
 
+/* Makes a result unusable when a re-pack reported an error: if status[0] | status[1] != 0 (the words of
+ * mortar_requantize, read on the device, no host synchronisation) every 4 bytes of out[0..bytes) become 0x7FC07FC0,
+ * NaN both as bf16 pairs and as fp32; otherwise out is not touched.  The stk_dds operator enqueues it behind its
+ * product, so data the reference's stk_dds (custom_ops.py:35-56) would multiply as arbitrary bf16 values never yields
+ * finite numbers of a silently re-quantised matrix, also in calls that do not wait for the status words.
+ *   out device, 4-byte aligned, bytes a multiple of 4; status device int32 [2]. */
+int mortar_poison_on_status(void *out, int64_t bytes, const int32_t *status, void *stream);
+
 /* ---- SwiGLU between the two matrices, training form ------------------------------------------------ */
 
 /* h = bf16(bf16(silu(gate)) * up) from a stored gate_up output gu [M, 2*d_ff] (gate = columns [0, d_ff), up =

@@ -34,6 +34,7 @@ _SIGS = {
     "mortar_requantize_workspace_bytes": (c_i64, []),
     "mortar_requantize": (C.c_int, [c_vp, c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_f32, c_vp, c_vp, c_vp, c_i32, c_f32,
                                   c_vp, c_vp]),
+    "mortar_poison_on_status": (C.c_int, [c_vp, c_i64, c_vp, c_vp]),
     "mortar_swiglu_bf16": (C.c_int, [c_vp, c_i64, c_i64, c_i32, c_vp, c_i64, c_vp]),
     "mortar_swiglu_backward_bf16": (C.c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_i32, c_vp, c_i64, c_vp]),
     "mortar_sdd_blocks_per_wave_host": (c_i32, [c_vp, c_vp, c_i32, c_i32, c_i64]),

@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import math
 
+import numpy as np
 import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
@@ -103,31 +104,31 @@ class CMSBlockLinear(nn.Module):
         B = self.tile_size
         if blocking % B != 0:
             raise ValueError(f"carve: blocking ({blocking}) not divisible by tile_size ({B})")
+        nR, nC = self.out_features // blocking, self.in_features // blocking
         with torch.no_grad():
-            tpb = blocking // B
-            Rb, Cb = self.out_features // blocking, self.in_features // blocking
-            w = self.weight.data
-            device = w.device
-            if self._prune_mask is not None:
-                tile_mask = self._prune_mask.to(device)
-                w = w * tile_mask.repeat_interleave(B, 0).repeat_interleave(B, 1).to(w.dtype)
+            dense = self.weight.data
+            dev = dense.device
+            if self._prune_mask is None:
+                kept = torch.ones(nR, nC, dtype=torch.bool, device=dev)
             else:
-                tile_mask = torch.ones(self.R, self.C, dtype=torch.bool, device=device)
-            m4 = tile_mask.view(Rb, tpb, Cb, tpb)
-            block_mask = m4.any(dim=3).any(dim=1)
-            if not bool(block_mask.any(dim=1).all()):
+                tiles = self._prune_mask.to(dev)
+                dense = dense * tiles.repeat_interleave(B, 0).repeat_interleave(B, 1).to(dense.dtype)
+                # a carve block survives when any of the (blocking / tile_size)^2 mask tiles inside it does
+                side = blocking // B
+                kept = tiles.unfold(0, side, side).unfold(1, side, side).reshape(nR, nC, -1).any(dim=-1)
+            per_row = kept.sum(dim=1)
+            if int(per_row.min()) == 0:
                 raise RuntimeError("carve: a block-row has zero kept blocks")
-            idx = block_mask.nonzero()
-            row_indices = idx[:, 0].to(torch.int16).contiguous()
-            column_indices = idx[:, 1].to(torch.int16).contiguous()
-            row_nnz = block_mask.sum(dim=1).to(torch.int32)
-            offsets = torch.cat([torch.zeros(1, dtype=torch.int32, device=device),
-                                 row_nnz.cumsum(0, dtype=torch.int32)]).contiguous()
-            blocks = w.reshape(Rb, blocking, Cb, blocking).permute(0, 2, 1, 3)
-            data = blocks[idx[:, 0], idx[:, 1]].contiguous()
+            rows, cols = torch.where(kept)                      # row-major order, columns ascending inside a row
+            offsets = torch.zeros(nR + 1, dtype=torch.int32, device=dev)
+            offsets[1:] = per_row.cumsum(0)
+            # [nR, nC, blocking, blocking] view of the matrix: element [r, c, i, j] = W[r*blocking + i, c*blocking + j]
+            data = dense.unfold(0, blocking, blocking).unfold(1, blocking, blocking)[rows, cols].contiguous()
+            row_indices, column_indices = rows.to(torch.int16), cols.to(torch.int16)
             ct, ot, bt = _stk_transpose((self.out_features, self.in_features), data, row_indices, column_indices, offsets)
-            self._init_mortar_storage(data.clone(), row_indices, column_indices, offsets, ct.contiguous(),
-                                      ot.contiguous(), bt.contiguous(), blocking)
+            self._init_mortar_storage(data, row_indices, column_indices, offsets, ct.contiguous(), ot.contiguous(),
+                                      bt.contiguous(), blocking)
+        Rb, Cb = nR, nC
         nnz = int(self.mortar_data.shape[0])
         self.density = nnz / (Rb * Cb)
         return nnz
@@ -175,7 +176,7 @@ class CMSBlockLinear(nn.Module):
         if not self._mortar:
             raise RuntimeError("mortar_pack() requires a carved layer")
         if self._mortar_blocking != 16:
-            raise ValueError(f"the gfx950 MORTAR runtime executes carve(blocking=16); this layer was carved at {self._mortar_blocking}")
+            return self._mortar_pack_recut()
         if "mortar_packed" in self._buffers:
             if self._pack is None:
                 self._pack = MortarPack(self.mortar_packed, self.mortar_scale, self.mortar_column_indices, self.mortar_offsets,
@@ -201,6 +202,41 @@ class CMSBlockLinear(nn.Module):
             self._pack_scale = self._pack.requantize(self._values(), threshold=self._values_threshold, sync=False)
             self._pack_key = key
             self._pack_gen += 1
+        return self._pack
+
+    def _mortar_pack_recut(self) -> MortarPack:
+        """Pack of a layer carved at a coarser blocking (the reference's checkpoints use carve(blocking=128),
+        block_sparse.py:810, pruning.py:85,248): the ternary codes are formed as the reference forms them (the packed
+        buffer as stored, or mortar_data through the per-tensor rule of block_sparse.py:909-919), then every block is
+        re-cut into 16 x 16 blocks on the host, all-zero sub-blocks dropped.  Inference only: the pack is rebuilt when
+        mortar_data changes (address, version), and the autograd path needs carve(blocking=16)."""
+        B = self._mortar_blocking
+        if B % 16:
+            raise ValueError(f"the gfx950 MORTAR runtime runs 16 x 16 blocks; a layer carved at {B} cannot be re-cut")
+        from .pack import recut_blocks
+        from .deploy_quant import unpack_ternary
+        if "mortar_packed" in self._buffers:
+            key = ("packed",)
+            if self._pack is not None and self._pack_key == key:
+                return self._pack
+            q = unpack_ternary(self.mortar_packed.cpu(), self._packed_numel, torch.int8).view(self._packed_shape)
+            scale = self.mortar_scale.detach().float().cpu()
+        else:
+            if not self._values_ternary_mode:
+                raise RuntimeError("carved layer holds non-ternary values: call pack_mortar_ternary() or "
+                                   "enable_values_ternary() first (the MORTAR runtime executes ternary blocks only)")
+            d = self.mortar_data
+            key = (d.data_ptr(), d._version)
+            if self._pack is not None and self._pack_key == key:
+                return self._pack
+            q, scale = _ternary_quantize(d.data, self._values_threshold)
+            q, scale = q.cpu(), scale.cpu()
+        c16, s16, col16, off16 = recut_blocks(q.numpy(), scale.numpy(), self.mortar_row_indices.cpu().numpy(),
+                                              self.mortar_column_indices.cpu().numpy(), self.out_features)
+        self._pack = MortarPack(pack_ternary_codes(torch.from_numpy(c16)), torch.from_numpy(np.asarray(s16, np.float32)),
+                                col16, off16, self.out_features, self.in_features, self.mortar_offsets.device,
+                                allow_empty_rows=True)
+        self._pack_key = key
         return self._pack
 
     def invalidate_pack(self) -> None:
@@ -235,7 +271,12 @@ class CMSBlockLinear(nn.Module):
         lead = x.shape[:-1]
         x2 = x.reshape(-1, self.in_features)
         xb = x2 if x2.dtype == torch.bfloat16 else x2.to(torch.bfloat16)
-        trainable = "mortar_packed" not in self._buffers and self._values_ternary_mode and xb.is_cuda
+        trainable = ("mortar_packed" not in self._buffers and self._values_ternary_mode and xb.is_cuda
+                     and self._mortar_blocking == 16)
+        if (not trainable and self._mortar_blocking != 16 and torch.is_grad_enabled()
+                and (xb.requires_grad or ("mortar_data" in self._parameters and self.mortar_data.requires_grad))):
+            raise RuntimeError(f"autograd through a layer carved at blocking {self._mortar_blocking}: the backward runs on "
+                               "carve(blocking=16) layers only (re-cut packs serve inference)")
         if trainable and self.mortar_data.requires_grad:
             self.invalidate_pack()            # trainable values may have been written through .data since the last call
         if trainable and torch.is_grad_enabled() and (xb.requires_grad or self.mortar_data.requires_grad):

@@ -153,7 +153,28 @@ __global__ __launch_bounds__(256) void requant_kernel(RequantArgs a) {
     }
 }
 
+// Overwrites out[0..ndw) with quiet-NaN patterns (0x7FC07FC0: NaN as two bf16 and as one fp32) when a status word is set.
+// Every thread reads the two words; the usual case (both 0) ends after that one load.
+__global__ __launch_bounds__(256) void poison_kernel(uint32_t *out, int64_t ndw, const int32_t *status) {
+    if ((status[0] | status[1]) == 0) return;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < ndw; i += (int64_t)gridDim.x * 256) out[i] = 0x7FC07FC0u;
+}
+
 }  // namespace
+
+extern "C" int mortar_poison_on_status(void *out, int64_t bytes, const int32_t *status, void *stream) {
+    if (!out || !status) return mortar_fail(MORTAR_ERR_ARG, "poison_on_status: null pointer");
+    if (bytes < 0 || (bytes & 3) || (reinterpret_cast<uintptr_t>(out) & 3))
+        return mortar_fail(MORTAR_ERR_ARG, "poison_on_status: out must be 4-byte aligned and a multiple of 4 bytes long");
+    if (bytes == 0) return MORTAR_OK;
+    const int64_t ndw = bytes / 4;
+    const int grid = (int)(ndw / 256 < 1 ? 1 : (ndw / 256 > 1024 ? 1024 : ndw / 256));
+    hipLaunchKernelGGL(poison_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint32_t *>(out), ndw, status);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "poison_on_status: %s", hipGetErrorString(e));
+    return MORTAR_OK;
+}
 
 extern "C" int64_t mortar_requantize_workspace_bytes(void) { return (int64_t)PARTIALS * sizeof(double); }
 

@@ -708,7 +708,7 @@ __global__ void __launch_bounds__(PW * UW * 64) mortar_partsplit_kernel(const Sp
     else mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, 0, p.Cb, tid);
     __syncthreads();
     bool idle = skip;
-    if (GATE_SKIP && valid && has_gates && p.cluster_size % 16 == 0) idle = __ballot(gsk > 0.f) == 0ull;
+    if (GATE_SKIP && valid && has_gates && p.cluster_size % 16 == 0) idle = __ballot(gsk != 0.f) == 0ull;      // NaN and negative gates multiply like any other
 
     f32x4_t acc[NACC][MSUB];
 #pragma unroll

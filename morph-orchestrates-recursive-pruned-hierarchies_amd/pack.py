@@ -100,6 +100,33 @@ def transpose_topology(offsets, col, Rb: int, Cb: int):
     return off_t, col_t, src
 
 
+def recut_blocks(codes: np.ndarray, scales, row_idx, col_idx, out_features: int, blk: int = BLK):
+    """A BCSR carved at a coarser blocking B (the reference's default is carve(blocking=128), block_sparse.py:810,
+    pruning.py:85) re-cut into the 16 x 16 blocks the kernels run: block j at (R, C) becomes its (B/16)^2 sub-blocks at
+    (R*B/16 + sr, C*B/16 + sc); sub-blocks whose codes are all zero are dropped, so that pruned 16 x 16 tiles inside a
+    kept coarse block cost nothing.  codes int8 [nnz, B, B]; scales scalar or [nnz] (a sub-block inherits its block's).
+    Returns (codes16 int8 [nnz16, 16, 16], scales16 fp32 scalar or [nnz16], col16 int16 [nnz16], offsets16 int32
+    [out_features/16 + 1]) in row-major order, columns ascending inside a row.  Rows of 16 may end up empty."""
+    codes = np.asarray(codes)
+    nnz, B, _ = codes.shape
+    if B % blk or codes.shape[2] != B:
+        raise ValueError(f"recut_blocks: blocks of {codes.shape[1:]} are not multiples of {blk}")
+    s = B // blk
+    sub = codes.reshape(nnz, s, blk, s, blk).transpose(0, 1, 3, 2, 4)                 # [nnz, sr, sc, 16, 16]
+    keep = sub.reshape(nnz, s, s, -1).any(axis=-1)
+    r16 = (np.asarray(row_idx, np.int64)[:, None, None] * s + np.arange(s)[None, :, None]) + np.zeros((1, 1, s), np.int64)
+    c16 = (np.asarray(col_idx, np.int64)[:, None, None] * s + np.arange(s)[None, None, :]) + np.zeros((1, s, 1), np.int64)
+    j, sr, sc = np.nonzero(keep)
+    rr, cc = r16[j, sr, sc], c16[j, sr, sc]
+    order = np.lexsort((cc, rr))
+    Rb16 = out_features // blk
+    offsets = np.zeros(Rb16 + 1, np.int32)
+    offsets[1:] = np.cumsum(np.bincount(rr, minlength=Rb16))
+    sc_arr = np.asarray(scales, np.float32).reshape(-1)
+    scales16 = sc_arr if sc_arr.size == 1 else sc_arr[j[order]]
+    return (np.ascontiguousarray(sub[j, sr, sc][order]), scales16, cc[order].astype(np.int16), offsets)
+
+
 def unit_order(offsets, Rb: int, rows_per_unit: int, group: int = SCHED_GROUP, snake: bool = True) -> np.ndarray:
     """Row units by schedule position (mortar_unit_order_host): ``snake`` reverses the odd groups, for the kernels
     that give wave w the positions w, w + group, ... of a window (matrices with several K segments)."""
@@ -264,6 +291,8 @@ class MortarPack:
             raise ValueError("requantize: ternary_tol needs a given scale")
         out = torch.empty(1 if mode in (0, 2) else self.nnz, dtype=torch.float32, device=self.device)
         st = torch.cuda.current_stream(self.device).cuda_stream
+        if sync and self._status_host is not None:
+            self.raise_status()          # a synchronous call clears the words: report what earlier asynchronous calls left first
         # asynchronous calls leave the status words sticky (flags bit 0) so that a later poll still sees a failure
         _lib.check(L.mortar_requantize(self.ref, values.data_ptr(), int(values.dtype == torch.float32), self._pos.data_ptr(),
                                        self.src_block.data_ptr() if self.src_block is not None else None,
@@ -325,6 +354,16 @@ class MortarPack:
             if self._status_host is not None:
                 self._status_host.zero_()
             raise ValueError("requantize: " + msg)
+
+    def poison_on_status(self, out: torch.Tensor) -> None:
+        """Enqueues the device-side check behind a product of this pack: ``out`` becomes all NaN if a re-pack of this pack
+        has reported an error that has not been raised yet (no host synchronisation).  No-op for packs never re-packed."""
+        if self._status is None:
+            return
+        if not out.is_contiguous() or (out.numel() * out.element_size()) % 4:
+            raise ValueError("poison_on_status: out must be contiguous with a multiple of 4 bytes")
+        _lib.check(_lib.lib().mortar_poison_on_status(out.data_ptr(), out.numel() * out.element_size(), self._status.data_ptr(),
+                                                      torch.cuda.current_stream(self.device).cuda_stream), "mortar_poison_on_status")
 
     def transposed(self) -> "MortarPack":
         """The pack of W^T [in, out] over the transposed topology (reference: stk matrix.py:107-125), all-zero until

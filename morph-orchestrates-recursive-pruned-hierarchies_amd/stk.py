@@ -20,6 +20,7 @@ def _topology(offsets: Tensor, column_indices: Tensor, nnz: int, out_f: int, in_
     pack = _cache.get(tkey)
     if pack is None:
         if len(_cache) > 64:
+            stk_check()                      # a pending error of a pack about to be dropped is raised, not lost
             _cache.clear()
         pack = MortarPack(None, None, column_indices, offsets, out_f, in_f, device)
         pack._keepalive = (offsets, column_indices)
@@ -38,8 +39,11 @@ def _pack_from_data(data: Tensor, offsets: Tensor, column_indices: Tensor, out_f
     place or by being replaced at the same address - is always honoured.  The MORTAR runtime multiplies ternary
     blocks only: the encode kernel checks that every value is 0 or +-s_j (s_j = the block's largest magnitude) and
     raises a flag on the device otherwise.  The first call on a topology waits for that flag; later calls read it
-    without waiting, so a violation is reported by the first call that finds the flag on the host (at the latest by
-    ``stk_check()``)."""
+    without waiting, so the ValueError comes from the first call that finds the flag on the host (at the latest from
+    ``stk_check()``) -- but the product of the offending call itself is already unusable: ``stk_dds`` enqueues
+    ``poison_on_status`` behind it, which turns the whole result into NaN on the device when the flag is set.
+    Values within 2^-7 of 0 or of +-s_j (relative to s_j) count as ternary: a bf16 cast of an fp32 +-s may land one
+    bf16 step beside bf16(s)."""
     d = data.detach()
     if d.dim() != 3 or d.shape[1] != 16 or d.shape[2] != 16:
         raise ValueError(f"stk_dds: data must be [nnz, 16, 16] (carve(blocking=16)), got {tuple(data.shape)}")
@@ -98,6 +102,7 @@ def stk_dds(lhs: Tensor, data: Tensor, offsets: Tensor, row_indices: Tensor, col
         W = _pack_from_data(data, offsets, column_indices, shape0, shape1, transposed=True)
     x = lhs if lhs.dtype == torch.bfloat16 else lhs.to(torch.bfloat16)
     y = ops.spmm(x, W)
+    W.poison_on_status(y)
     return y if y.dtype == lhs.dtype else y.to(lhs.dtype)
 
 

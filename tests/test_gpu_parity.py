@@ -166,13 +166,17 @@ def test_mlp_with_gates_and_skip(dev):
     assert torch.equal(y2, y)
 
 
-def test_routed_module_mask_follows_the_call(dev):
+@pytest.mark.parametrize("route_skip", [False, True])
+def test_routed_module_mask_follows_the_call(dev, route_skip):
     """The carved routed forward takes its tile mask from the gates of the current call: a no-grad call with 128 rows
     followed by a grad-enabled call with 32 other rows (router parameters trainable, weights packed) must route the
-    second call by its own gates, not by what the first call left in the router."""
+    second call by its own gates, not by what the first call left in the router.  Both prefill forms: gates in the
+    gate_up epilogue (the default) and token lists + routed gate_up + masked down (route_skip)."""
     d_model, d_ff, ncl = 256, 16 * 40, 40
     spec = synth.synth_mlp(d_model, d_ff, 0.3, seed=33)
     mlp = synth.mlp_module(spec, dev)
+    assert mlp.route_skip is False
+    mlp.route_skip = route_skip
     mlp.enable_routing(n_clusters=ncl, activation_ratio=0.25, n_iters=1)
     torch.manual_seed(5)
     with torch.no_grad():

@@ -337,16 +337,26 @@ def test_stk_dds_fp32_effective_data_and_non_ternary_report(dev):
     stk.stk_check()                                                   # nothing to report so far
     # same topology, later call, data that is NOT ternary: no wait in the call itself, the flag is raised on the device
     bad = eff.clone(); bad[3, 2, 1] = 0.37 * float(mags[0])
-    mortar_amd.stk_dds(to_dev(x, dev), bad, *args, lin.in_features, lin.out_features, True)
+    ybad = mortar_amd.stk_dds(to_dev(x, dev), bad, *args, lin.in_features, lin.out_features, True)
+    assert bool(torch.isnan(ybad).all())                              # ...and the product of that call is unusable: all NaN
     with pytest.raises(ValueError, match="not ternary"):
         stk.stk_check()
     stk.stk_check()                                                   # reported once, then clean again
-    mortar_amd.stk_dds(to_dev(x, dev), bad, *args, lin.in_features, lin.out_features, True)
+    ybad = mortar_amd.stk_dds(to_dev(x.astype(np.float32), dev).float(), bad, *args, lin.in_features, lin.out_features, True)
+    assert ybad.dtype == torch.float32 and bool(torch.isnan(ybad).all())
+    dxbad = mortar_amd.stk_dds(torch.ones(5, lin.out_features, dtype=torch.bfloat16, device=dev), bad, *args,
+                               lin.out_features, lin.in_features, False)         # the dX product through the W^T pack
+    assert bool(torch.isnan(dxbad).all())
     torch.cuda.synchronize()
     with pytest.raises(ValueError, match="earlier call"):             # the next call finds the flag on the host
         mortar_amd.stk_dds(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
     y2 = mortar_amd.stk_dds(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
     assert torch.equal(y2, y)
+    with pytest.raises(ValueError, match="not ternary"):              # the W^T pack keeps its own words
+        stk.stk_check()
+    dx = mortar_amd.stk_dds(torch.ones(5, lin.out_features, dtype=torch.bfloat16, device=dev), eff, *args,
+                            lin.out_features, lin.in_features, False)
+    assert bool(torch.isfinite(dx).all())
     # a fresh topology sees the error in its first call
     m = synth.synth_matrix(64, 64, 0.5, seed=88)
     t = lambda a: torch.from_numpy(a).to(dev)
@@ -516,3 +526,39 @@ def test_training_golden_fixture(dev):
     assert_close_bf16(to_np(ops.sdd(dy, x, W)), O.bf16_from_bits(z["dw_bits"]), "dW")
     assert_close_bf16(to_np(ops.swiglu(bits("gu_bits"))), O.bf16_from_bits(z["h_bits"]), "h")
     assert_close_bf16(to_np(ops.swiglu_backward(bits("gu_bits"), bits("dh_bits"))), O.bf16_from_bits(z["dgu_bits"]), "dgu", ulps=3)
+
+
+@pytest.mark.parametrize("packed", [True, False])
+def test_layer_carved_at_blocking_128_runs_through_the_recut_pack(dev, packed):
+    """The reference's default carve (blocking 128, block_sparse.py:810; pruning.py:85,248): a layer pruned on 16-tiles,
+    carved at 128 and either packed (deploy_quant.py:344-374) or left in values-ternary mode is re-cut into 16 x 16 blocks
+    at pack time; prefill and decode forwards against the dense float64 product of its effective weight."""
+    import mortar_amd
+    torch.manual_seed(21)
+    lin = mortar_amd.MortarLinear(512, 384, bias=False)
+    rng = np.random.default_rng(22)
+    tiles = rng.random((24, 32)) < 0.3
+    tiles[::8, 0] = True                                                   # every 128-row keeps a block
+    lin._cms._prune_mask = torch.from_numpy(tiles)
+    lin.carve(128)
+    cms = lin._cms
+    if packed:
+        mortar_amd.pack_mortar_ternary(cms, 0.5)
+    else:
+        cms.enable_values_ternary(0.5)
+    lin.to(dev)
+    eff = cms._mortar_effective_data().detach().float().cpu().numpy()
+    if not packed:                                                         # the kernels multiply bf16(scale) * code
+        sc = float(cms.mortar_data.detach().float().abs().mean().clamp(min=1e-8))
+        eff = np.sign(eff) * O.bf16_round(np.array([sc], np.float32))[0]
+    dense = O.to_dense(eff, cms.mortar_row_indices.cpu().numpy(), cms.mortar_column_indices.cpu().numpy(), (384, 512), 128)
+    W = cms.mortar_pack()
+    assert W.nnz < int(cms.mortar_row_indices.numel()) * 64                # pruned tiles inside kept blocks were dropped
+    for M in (200, 3):
+        x = synth.synth_x(M, 512, seed=23 + M)
+        with torch.no_grad():
+            y = lin(to_dev(x, dev))
+        assert_close_bf16(to_np(y), (O.bf16_round(x).astype(np.float64) @ dense.astype(np.float64).T).astype(np.float32), f"blocking 128, M={M}")
+    if not packed:
+        with pytest.raises(RuntimeError, match="blocking 128"):
+            lin(to_dev(x, dev).requires_grad_(True))

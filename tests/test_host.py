@@ -475,3 +475,76 @@ def test_operator_fake_implementations_trace_without_a_gpu():
         assert tuple(dx.shape) == (40, 96)
         dw = mortar_amd.stk_sdd_at_b(y, lhs, data, off, idx, idx)
         assert tuple(dw.shape) == (10, 16, 16) and dw.dtype == torch.bfloat16
+
+
+def test_module_carve_at_coarser_blocking_matches_oracle_layout():
+    """carve(blocking=64) with a 16-tile prune mask: a block is kept when any tile inside it is, pruned tiles inside
+    kept blocks hold zeros (reference block_sparse.py:859-890); same arrays as the oracle's carve at that blocking."""
+    torch.manual_seed(4)
+    lin = mortar_amd.MortarLinear(64 * 3, 64 * 2, bias=False)
+    rng = np.random.default_rng(8)
+    tiles = rng.random((8, 12)) < 0.15
+    tiles[0, 0] = tiles[4, 5] = True                                     # every 64-row keeps something
+    w = lin._cms.weight.detach().numpy().copy()
+    lin._cms._prune_mask = torch.from_numpy(tiles)
+    lin.carve(64)
+    bm = tiles.reshape(2, 4, 3, 4).any(axis=(1, 3))
+    c = O.carve(w * np.kron(tiles, np.ones((16, 16), np.float32)), bm, 64)
+    sd = lin.state_dict()
+    for k in ("mortar_data", "mortar_row_indices", "mortar_column_indices", "mortar_offsets"):
+        assert np.array_equal(sd["_cms." + k].numpy(), c[k]), k
+
+
+@pytest.mark.parametrize("B,per_block", [(128, False), (64, True), (32, False)])
+def test_recut_blocks_is_the_same_matrix(B, per_block):
+    """A BCSR carved at blocking B re-cut into 16 x 16 blocks scatters to the same dense matrix (oracle to_dense of both
+    layouts), keeps row-major order with ascending columns, drops exactly the all-zero sub-blocks and hands every
+    sub-block its block's scale."""
+    rng = np.random.default_rng(B)
+    Rb, Cb = 3, 4
+    mask = rng.random((Rb, Cb)) < 0.6
+    mask[np.arange(Rb), rng.integers(0, Cb, Rb)] = True
+    r, c = np.nonzero(mask)
+    nnz = r.size
+    codes = rng.integers(-1, 2, (nnz, B, B)).astype(np.int8)
+    zero_tiles = rng.random((nnz, B // 16, B // 16)) < 0.4               # pruned 16-tiles inside kept blocks
+    codes *= ~np.kron(zero_tiles, np.ones((16, 16), bool))
+    scales = rng.uniform(0.01, 0.1, nnz).astype(np.float32) if per_block else np.float32(0.037)
+    c16, s16, col16, off16 = P.recut_blocks(codes, scales, r, c, Rb * B)
+    assert c16.shape[0] == int((~zero_tiles).sum()) - int((codes.reshape(nnz, B // 16, 16, B // 16, 16).transpose(0, 1, 3, 2, 4)
+                                                           .reshape(nnz, B // 16, B // 16, -1).any(-1) != ~zero_tiles).sum())
+    assert off16[0] == 0 and off16[-1] == c16.shape[0] and off16.size == Rb * B // 16 + 1
+    row16 = np.repeat(np.arange(Rb * B // 16), np.diff(off16))
+    for rr in range(Rb * B // 16):
+        cols = col16[off16[rr]:off16[rr + 1]]
+        assert (np.diff(cols.astype(int)) > 0).all()
+    sc = np.broadcast_to(np.asarray(scales, np.float32).reshape(-1), (nnz,))
+    big = O.to_dense(codes.astype(np.float32) * sc[:, None, None], r, c, (Rb * B, Cb * B), B)
+    s16b = np.broadcast_to(np.asarray(s16, np.float32).reshape(-1), (c16.shape[0],))
+    small = O.to_dense(c16.astype(np.float32) * s16b[:, None, None], row16, col16, (Rb * B, Cb * B), 16)
+    assert np.array_equal(big, small)
+    assert c16.reshape(c16.shape[0], -1).any(axis=1).all()               # no all-zero block kept
+    with pytest.raises(ValueError):
+        P.recut_blocks(np.zeros((1, 24, 24), np.int8), 1.0, [0], [0], 24)
+
+
+def test_layer_carved_at_128_loads_and_packs_on_the_host():
+    """The reference's checkpoints are carved at blocking 128: such a state dict loads, and mortar_pack() re-cuts it
+    into a 16 x 16 pack whose decoded blocks scatter to the layer's effective dense weight."""
+    torch.manual_seed(5)
+    src = mortar_amd.MortarLinear(256, 384, bias=False)
+    info = mortar_amd.shrink_mlp_to_mortar_ternary(src, 0.5, 128, generator=torch.Generator().manual_seed(6))
+    assert src._cms._mortar_blocking == 128 and src._cms._packed_shape[1:] == (128, 128)
+    dst = mortar_amd.MortarLinear(256, 384, bias=False)
+    dst.load_state_dict(src.state_dict())
+    cms = dst._cms
+    assert cms._mortar_blocking == 128 and cms._packed_shape == src._cms._packed_shape
+    W = cms.mortar_pack()
+    assert W is cms.mortar_pack() and W.Rb == 24 and W.Cb == 16
+    eff = cms._mortar_effective_data().float().numpy()
+    dense = O.to_dense(eff, cms.mortar_row_indices.numpy(), cms.mortar_column_indices.numpy(), (384, 256), 128)
+    q16 = P.decode_blocks(W.codes.numpy().view(np.uint32))
+    s = float(O.bf16_round(np.array([float(cms.mortar_scale)], np.float32))[0])
+    row16 = np.repeat(np.arange(W.Rb), np.diff(W.h_offsets))
+    got = O.to_dense(q16.astype(np.float32) * s, row16, W.h_col, (384, 256), 16)
+    assert np.array_equal(got, dense)
