@@ -151,10 +151,11 @@ def main() -> None:
     x = torch.from_numpy(synth.synth_x(TOKENS, D_MODEL, seed=1)).to(torch.bfloat16).to(dev)
     h = torch.empty((TOKENS, D_FF), dtype=torch.bfloat16, device=dev)
     y = torch.empty((TOKENS, D_MODEL), dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(ops.mlp_hidden_bytes(TOKENS, D_FF), dtype=torch.uint8, device=dev)
 
     def step():
-        ops.gateup_swiglu(x, Wgu, out=h)
-        ops.spmm(h, Wdn, out=y)
+        # the MLP forward as the module runs it: gate_up + SwiGLU, then down, hidden activations in the library's layout
+        ops.mlp(x, Wgu, Wdn, out=y, hidden=ws)
 
     for _ in range(args.warmup):
         step()
@@ -175,9 +176,9 @@ def main() -> None:
     torch.cuda.synchronize()
     for e in evs:
         e[0].record()
-        ops.gateup_swiglu(x, Wgu, out=h)
+        ops.mlp(x, Wgu, Wdn, out=y, hidden=ws, phase=1)          # the same two launches, one at a time
         e[1].record()
-        ops.spmm(h, Wdn, out=y)
+        ops.mlp(x, Wgu, Wdn, out=y, hidden=ws, phase=2)
         e[2].record()
     torch.cuda.synchronize()
     ms_gu = sum(e[0].elapsed_time(e[1]) for e in evs) / it
@@ -196,7 +197,7 @@ def main() -> None:
                      "frac": flops_gu / (ms_gu * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_GATE_UP_BYTES,
                      "traffic_source": TRAFFIC_SOURCE,
                      "algorithmic_bytes": TOKENS * (D_MODEL + D_FF) * 2 + Wgu.weight_bytes, "ms": ms_gu},
-        "roofline_down": {"bound": "mfma", "kernel": "mortar_segmented_kernel<32 tokens, plain> (down)",
+        "roofline_down": {"bound": "mfma", "kernel": "mortar_segmented_kernel<32 tokens, plain> (down, K segments copied asynchronously from the tile-ordered hidden activations)",
                           "achieved": flops_dn / (ms_dn * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                           "frac": flops_dn / (ms_dn * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_DOWN_BYTES,
                           "traffic_source": TRAFFIC_SOURCE,
@@ -314,6 +315,13 @@ def main() -> None:
             del up, dn, hs, ys
         out["decode_stack"] = stack
         out["roofline_decode"] = {"bound": "hbm", "kernel": "mortar_resident_kernel<4 tokens>, gate_up + down launches of 160 layers each, b=1",
+                                  "form": "bandwidth probe: 160 independent MLP weight sets per launch (two launches), not a model's "
+                                          "decode step; one real MLP per step is `one_mlp_per_step` below",
+                                  "one_mlp_per_step": {k: {"us_per_mlp": v["us_per_mlp"], "achieved": v["algorithmic_GBps"],
+                                                           "frac": v["algorithmic_GBps"] / PEAK_HBM_GBS,
+                                                           "form": "gate_up + down launches of ONE MLP, HIP-graph replay, weights warm in cache"}
+                                                       for k, v in gdec.items()},
+                                  "traffic_over_algorithmic": TRAFFIC_DECODE_STACK_BYTES / float(n_sets * (wbytes + (2 * D_MODEL + 2 * D_FF) * 2)),
                                   "achieved": stack["b1"]["algorithmic_GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                   "frac": stack["b1"]["frac_hbm"], "traffic": TRAFFIC_DECODE_STACK_BYTES,
                                   "traffic_source": TRAFFIC_SOURCE,
@@ -323,11 +331,19 @@ def main() -> None:
         logits = torch.from_numpy(synth.synth_logits(TOKENS, N_CLUSTERS, seed=2)).to(dev)
 
         def routed():
+            # the module's default for prefill-sized calls: gates multiplied in gate_up's epilogue, plain down
+            gates, _ = ops.remoe_gates(logits, TOP_K)
+            ops.mlp(x, Wgu, Wdn, gates=gates, out=y, hidden=ws)
+
+        def routed_lists():
+            # the optional skipping form: token lists per (tile, cluster), routed gate_up, masked down
             gates, active = ops.remoe_gates(logits, TOP_K)
             route = ops.remoe_route(active, ops.route_tile(Wgu, TOKENS))
             ops.gateup_swiglu(x, Wgu, gates=gates, route=route, out=h)
             ops.spmm(h, Wdn, active=active, out=y)
         t = event_time_ms(routed, it)
+        t_lists = event_time_ms(routed_lists, it)
+        t_gates = event_time_ms(lambda: ops.remoe_gates(logits, TOP_K), it)
         act_now = ops.remoe_gates(logits, TOP_K)[1]
         n_act = int(act_now.sum())
         act_frac = n_act / (TOKENS * N_CLUSTERS)
@@ -335,23 +351,25 @@ def main() -> None:
         sub_exec = int(((cnt_now + 15) // 16).sum())             # 16-token MFMA sub-tiles the routed gate_up executes
         fl_active = (flops_gu + flops_dn) * act_frac          # products whose hidden cluster is active for the token
         out["routed_prefill"] = {"ms": t, "tokens_per_s": TOKENS / (t * 1e-3), "active_fraction": act_frac,
-                                 "vs_unrouted": t / ms,
-                                 "gather_efficiency": n_act / (16.0 * sub_exec),          # active tokens per executed MFMA column
-                                 "mfma_subtiles_executed": sub_exec / float(cnt_now.numel() * (ops.route_tile(Wgu, TOKENS) // 16)),
-                                 "roofline": {"bound": "mfma", "kernel": "remoe_gates + remoe_route + routed gate_up + masked down",
+                                 "vs_unrouted": t / ms, "gates_launch_ms": t_gates,
+                                 "form": "remoe_gates + MLP with the gates multiplied in gate_up's epilogue (module default)",
+                                 "token_list_form": {"ms": t_lists, "vs_unrouted": t_lists / ms,
+                                                     "gather_efficiency": n_act / (16.0 * sub_exec),      # active tokens per executed MFMA column
+                                                     "mfma_subtiles_executed": sub_exec / float(cnt_now.numel() * (ops.route_tile(Wgu, TOKENS) // 16)),
+                                                     "form": "remoe_gates + remoe_route + routed gate_up + masked down (route_skip=True)"},
+                                 "roofline": {"bound": "mfma", "kernel": "remoe_gates + gated gate_up + down",
                                               "achieved": fl_active / (t * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                               "frac": fl_active / (t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
                                               "note": "FLOPs of active (token, cluster) pairs only; a cluster is one 16-neuron row unit, "
                                                       "so a 32-token tile keeps about 8 active tokens per unit and the weight unpack, "
-                                                      "which bounds the kernel, is not reduced"}}
+                                                      "which bounds the kernel, does not shrink with the active share: nothing is skipped"}}
         # ---- the reference's own deploy format: ONE scale per matrix (pack_mortar_ternary), same shapes ----------
         spec_u = {k: dict(spec[k]) for k in ("gate_up", "down")}
         spec_u["gate_up"]["scales"], spec_u["down"]["scales"] = np.float32(0.05), np.float32(0.03)
         Ugu, Udn = synth.to_pack(spec_u["gate_up"], dev), synth.to_pack(spec_u["down"], dev)
 
         def ustep():
-            ops.gateup_swiglu(x, Ugu, out=h)
-            ops.spmm(h, Udn, out=y)
+            ops.mlp(x, Ugu, Udn, out=y, hidden=ws)
         t = event_time_ms(ustep, it)
         xb = x[:1].contiguous()
         upacks = [(Ugu, Udn) if i == 0 else (Ugu.clone_weights(), Udn.clone_weights()) for i in range(n_sets)]
@@ -398,12 +416,11 @@ def main() -> None:
         spec1 = synth.synth_mlp(768, 2048, DENSITY, seed=10)
         G1, D1 = synth.to_pack(spec1["gate_up"], dev), synth.to_pack(spec1["down"], dev)
         x1 = torch.from_numpy(synth.synth_x(16384, 768, seed=11)).to(torch.bfloat16).to(dev)
-        h1 = torch.empty((16384, 2048), dtype=torch.bfloat16, device=dev)
+        h1 = torch.empty(ops.mlp_hidden_bytes(16384, 2048), dtype=torch.uint8, device=dev)
         y1 = torch.empty((16384, 768), dtype=torch.bfloat16, device=dev)
 
         def step1():
-            ops.gateup_swiglu(x1, G1, out=h1)
-            ops.spmm(h1, D1, out=y1)
+            ops.mlp(x1, G1, D1, out=y1, hidden=h1)
         t = event_time_ms(step1, it)
         fl = 2.0 * 16384 * 256 * (G1.nnz + D1.nnz)
         out["base_width_prefill"] = {"ms": t, "tokens_per_s": 16384 / (t * 1e-3), "effective_tflops": fl / (t * 1e-3) / 1e12,
@@ -415,27 +432,31 @@ def main() -> None:
         fused_norm = all(ops.norm_fusable(m4.gate_up._cms.mortar_pack()) for m4 in mlps4)
         t = event_time_ms(lambda: mortar_amd.looped_core_forward(mlps4, x, 6), 3, 1)
         fl = 6 * sum(2.0 * TOKENS * 256 * (m4.gate_up._cms.mortar_pack().nnz + m4.down._cms.mortar_pack().nnz) for m4 in mlps4)
-        # static load balance of the Zipf rows: blocks per workgroup window of gate_up's schedule (units are then drawn
-        # dynamically by the 16 waves of a window) and blocks per wave of down's fixed assignment (4 units per wave)
-        def _balance(W, rpu, group):
-            from mortar_amd.pack import unit_order
-            nnz_row = np.diff(W.h_offsets).astype(np.int64)
-            per_unit = nnz_row.reshape(rpu, -1).sum(0)[unit_order(W.h_offsets, W.Rb, rpu)]
-            pad = (-per_unit.size) % group
-            work = np.concatenate([per_unit, np.zeros(pad, np.int64)]).reshape(-1, group)
-            return work
+        # static load balance of the Zipf rows, read from the schedule tables the kernels run (MortarPack.sched): gate_up's
+        # resident kernel gives a workgroup a window of consecutive positions whose units its 16 waves draw dynamically, so
+        # what counts is blocks per window; down's K-segmented kernel gives wave w of a 64-position window the positions
+        # w, w + 16, ... and ends every K segment with a barrier, so a window costs the sum over the segments of its
+        # fullest wave in that segment
+        def _sched_blocks(W, rpu):
+            sc = W.sched(rpu).cpu().numpy().reshape(-1, W.nseg, rpu, 4)           # [position, segment, row of unit, {g0, g1, nb, unit}]
+            return sc[..., 2].astype(np.int64).sum(axis=2)                            # blocks per (position, segment)
         lb_gu, lb_dn = [], []
         for m4 in mlps4:
             Wg4, Wd4 = m4.gate_up._cms.mortar_pack(), m4.down._cms.mortar_pack()
             n_split = max(1, 256 // (-(-TOKENS // 32)))
             per = -(-(Wg4.Rb // 2) // n_split)
-            wg = _balance(Wg4, 2, per).sum(1)                               # one row of `work` = one workgroup window
+            bg = _sched_blocks(Wg4, 2).sum(axis=1)
+            wg = np.array([bg[i:i + per].sum() for i in range(0, bg.size, per)])
             lb_gu.append(float(wg.sum() / (wg.size * wg.max())))
-            wv = _balance(Wd4, 1, 64).reshape(-1, 4, 16).sum(1).reshape(-1)   # wave w of a 64-unit group takes units w, w+16, ...
-            lb_dn.append(float(wv.sum() / (wv.size * wv.max())))
+            bd = _sched_blocks(Wd4, 1)                                                # [position, segment]
+            pad = (-bd.shape[0]) % 64
+            bd = np.concatenate([bd, np.zeros((pad, bd.shape[1]), np.int64)]).reshape(-1, 4, 16, bd.shape[1]).sum(axis=1)   # [window, wave, segment]
+            lb_dn.append(float(bd.sum() / (16.0 * bd.max(axis=1).sum())))             # all windows: blocks / (waves x barrier-bound blocks)
         out["looped_stack"] = {"ms": t, "mlp_calls": 48, "ms_per_mlp": t / 48, "tokens_per_s": TOKENS / (t * 1e-3),
                                "load_balance_efficiency": {"gate_up_workgroup_windows": min(lb_gu), "down_waves": min(lb_dn),
-                                                           "definition": "sum of blocks / (parts x blocks of the fullest part), worst of the 8 matrices"},
+                                                           "definition": "gate_up: blocks / (windows x blocks of the fullest workgroup window); down: blocks / (16 waves x sum over "
+                                                                         "windows and K segments of the fullest wave's blocks); from the schedule tables the kernels "
+                                                                         "read; worst of the 8 matrices"},
                                "effective_tflops": fl / (t * 1e-3) / 1e12,
                                "frac_mfma": fl / (t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
                                "norm_fused_into_gate_up": bool(fused_norm),

@@ -294,9 +294,11 @@ int mortar_stack_run(int32_t swiglu, int32_t n_layers, const mortar_bcsr_t *W0, 
  * nslots = 1: entries write the result directly.  nslots > 1: partial sums go to `part`
  * (fp32 [nslots, B, Rb*16], caller workspace) and a second kernel combines them in slot order, reading
  * row_slots (device copy of the work list's row_slots_out).
- * row_act / col_act (int32, may be NULL): ReMoE flags from mortar_route_flags; a unit all of whose B
- * streams are inactive is skipped (zeros written); a block whose input column is inactive for all B
- * streams is skipped. */
+ * row_act / col_act (int32, may be NULL): ReMoE flags (mortar_route_flags), applied per stream as the reference's
+ * kernel does (fused_decode_step.py:1378-1393): the sum of output block-row r is zero for stream b when
+ * row_act[b, r] == 0 (gate_up: r runs over gate rows then up rows, Rb entries), and the blocks of input block-column c
+ * contribute nothing to stream b when col_act[b, c] == 0.  Work is skipped where ALL B streams agree: a unit none of
+ * whose rows is active for any stream, a block whose input column is off for every stream. */
 int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_entries, int32_t nslots,
                      const int32_t *row_slots, int32_t kseg, int32_t mode, const uint16_t *x, int32_t B, int64_t ldx,
                      uint16_t *y, int64_t ldy, float *part,
@@ -322,9 +324,9 @@ int mortar_gemv_bf16(const mortar_bcsr_t *W, const int32_t *entries, int64_t n_e
  * the bandwidth-bound SpMM kernels instead of the work list: the three bf16 terms of the B rows become 3 * B bf16 rows,
  * the one-scale SpMM kernels contract them with the +-2 / 0 blocks and keep the fp32 sums unrounded, and a last pass
  * adds the three sums of a row and applies the scale and the epilogue - the same exact products and fp32 sums, in
- * another order of addition (2 to 3 times faster at the headline shapes).  Flags keep their meaning there: a chunk of x
- * whose column is inactive for all B streams enters as zeros, and a unit that is inactive for all B streams is written
- * as zeros; no weight is skipped, which is still faster than the work list with skipping (17 against 25 us per MLP at
+ * another order of addition (2 to 3 times faster at the headline shapes).  Flags keep their per-stream meaning there: a chunk of x
+ * whose column is off for its stream enters as zeros, and the sum of a row that is off for a stream is written as
+ * zero; no weight is skipped, which is still faster than the work list with skipping (17 against 25 us per MLP at
  * one row, 21 against 49 us at 16 rows). */
 int64_t mortar_gemv_f32_workspace_bytes(const mortar_bcsr_t *W, int32_t B, int32_t nslots);
 int mortar_gemv_f32(const mortar_bcsr_t *W, const float *scale, int64_t scale_count, const int32_t *sched,
@@ -365,6 +367,27 @@ int mortar_norm_gateup_swiglu_bf16(const mortar_bcsr_t *W, const int32_t *sched,
                                    const float *gates, int32_t n_clusters, const int32_t *tok_cnt,
                                    const uint8_t *tok_list, void *stream);
 int mortar_norm_fusable(int32_t Cb);
+
+/* The carved SwiGLU MLP as one call: y = down(silu(gate) * up [* gates per cluster]) with gate_up applied to x or to
+ * RMSNorm(x) -- _SwiGLUMortar.forward, morph/model/transformer.py:402-431 (called as mlp(norm_mlp(x)),
+ * morph/model/mhc.py:249-250).  Two launches (gate_up with the SwiGLU in its epilogue, then down), same arithmetic and
+ * same bits as mortar_[norm_]gateup_swiglu_bf16 followed by mortar_spmm_bf16.  What the call adds: the hidden
+ * activations between the launches live in `hidden`, a caller workspace of mortar_mlp_hidden_bytes(M, d_ff) bytes
+ * (16-byte aligned) whose layout belongs to the library.  From 513 rows up (both launches then run 32-token tiles) it is
+ * tile order -- the 32 tokens x 16 features of a (token tile, block-column) in 1 KB of contiguous memory -- so that
+ * gate_up stores whole result tiles as contiguous runs and down copies its K segments asynchronously into LDS without
+ * passing through registers; below, and for matrices without the 4-bit stream, it is row-major [M, d_ff].
+ *   norm != 0: RMS-normalise the rows of x on the way in (norm_w bf16 [in_features] or NULL, norm_eps), needs
+ *              mortar_norm_fusable(Wgu->Cb) != 0
+ *   gates      fp32 [M, n_clusters] or NULL, multiplied per cluster of d_ff / n_clusters hidden features (in bf16)
+ *   phase      0: both launches; 1: gate_up only (fills `hidden`); 2: down only (reads `hidden` as phase 1 of the same
+ *              M left it) -- for callers that time or interleave the two launches
+ * Token lists (routed skipping) and input masks keep their own entry points. */
+int64_t mortar_mlp_hidden_bytes(int64_t M, int32_t d_ff);
+int mortar_mlp_bf16(const mortar_bcsr_t *Wgu, const int32_t *sched_gu, const mortar_bcsr_t *Wdn, const int32_t *sched_dn,
+                    const uint16_t *x, int64_t M, int64_t ldx, int32_t norm, const uint16_t *norm_w, float norm_eps,
+                    const float *gates, int32_t n_clusters, void *hidden, uint16_t *y, int64_t ldy, int32_t phase,
+                    void *stream);
 
 /* y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) per row; x, y bf16 [M, d]; w bf16 [d] or NULL (= 1). */
 int mortar_rmsnorm_bf16(const uint16_t *x, int64_t M, int32_t d, int64_t ldx, const uint16_t *w, float eps,

@@ -53,6 +53,9 @@ _SIGS = {
     "mortar_norm_gateup_swiglu_bf16": (C.c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_f32, c_vp, c_i64, c_vp, c_i32,
                                                  c_vp, c_vp, c_vp]),
     "mortar_norm_fusable": (C.c_int, [c_i32]),
+    "mortar_mlp_hidden_bytes": (c_i64, [c_i64, c_i32]),
+    "mortar_mlp_bf16": (C.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_vp, c_f32, c_vp, c_i32, c_vp, c_vp, c_i64,
+                                  c_i32, c_vp]),
     "mortar_spmm_bf16_masked": (C.c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_i64, c_vp, c_i32, c_vp]),
     "mortar_route_tile": (C.c_int, [c_i32, c_i64]),
     "mortar_remoe_gates": (C.c_int, [c_vp, c_i64, c_i32, c_i32, c_vp, c_vp, c_vp]),

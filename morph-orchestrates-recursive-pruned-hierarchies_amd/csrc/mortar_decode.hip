@@ -92,9 +92,14 @@ __global__ void __launch_bounds__(256) mortar_gemv_kernel(const GemvParams p) {
     uint32_t *colflag = reinterpret_cast<uint32_t *>(smem + (size_t)2 * p.kseg * LDB * 16);
 
     // stage the activations of this K segment: unit (ch, tok) <- x[tok, c0*16 + ch*8 .. +8]
+    // (a block-column that is off for stream `tok` enters as zeros for that stream: the reference masks the block's
+    // products per stream, fused_decode_step.py:1387-1393)
     for (int tok = 0; tok < p.B; ++tok)
-        for (int ch = tid; ch < nch; ch += 256)
-            lx[ch * LDB + tok] = *reinterpret_cast<const uint4 *>(p.x + (int64_t)tok * p.ldx + (int64_t)c0 * 16 + ch * 8);
+        for (int ch = tid; ch < nch; ch += 256) {
+            uint4 v = *reinterpret_cast<const uint4 *>(p.x + (int64_t)tok * p.ldx + (int64_t)c0 * 16 + ch * 8);
+            if (p.col_act && p.col_act[(int64_t)tok * p.ldc + c0 + (ch >> 1)] == 0) v = uint4{0u, 0u, 0u, 0u};
+            lx[ch * LDB + tok] = v;
+        }
     if (p.col_act) {
         for (int c = tid; c < ncb; c += 256) {
             uint32_t f = 0;
@@ -113,9 +118,9 @@ __global__ void __launch_bounds__(256) mortar_gemv_kernel(const GemvParams p) {
     const int slot = __builtin_amdgcn_readfirstlane(ep[6]);
 
     bool unit_on = true;
-    if (p.row_act) {   // skip the unit when no stream has it active
+    if (p.row_act) {   // skip the unit when no stream has one of its rows active
         int f = 0;
-        if (lane < p.B) f = p.row_act[(int64_t)lane * p.ldr + rowA] != 0;
+        if (lane < p.B) f = p.row_act[(int64_t)lane * p.ldr + rowA] != 0 || (rowB >= 0 && p.row_act[(int64_t)lane * p.ldr + rowB] != 0);
         unit_on = __builtin_amdgcn_readfirstlane(__ballot(f) != 0ull);
     }
 
@@ -131,6 +136,10 @@ __global__ void __launch_bounds__(256) mortar_gemv_kernel(const GemvParams p) {
     for (int ms = 0; ms < MSUB; ++ms) {
         const int tok = ms * 16 + n;
         if (tok >= p.B) continue;
+        if (p.row_act && unit_on) {      // the flags are per stream: a row that is off for this stream contributes zeros
+            if (p.row_act[(int64_t)tok * p.ldr + rowA] == 0) accA[ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            if (rowB >= 0 && p.row_act[(int64_t)tok * p.ldr + rowB] == 0) accB[ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
         if (p.nslots > 1) {
             float *pp = p.part + ((int64_t)slot * p.B + tok) * p.N;
             *reinterpret_cast<f32x4_t *>(pp + rowA * 16 + 4 * g) = accA[ms];
@@ -347,6 +356,8 @@ __global__ void __launch_bounds__(256) mortar_gemv_f32_kernel(const GemvF32Param
     for (int it = tid; it < nch * p.B; it += 256) {
         const int tok = it / nch, ch = it % nch;
         const float *src = p.x + (int64_t)tok * p.ldx + (int64_t)c0 * 16 + ch * 8;
+        // a block-column that is off for this stream enters as zeros for it (per-stream flags, as the reference's kernel)
+        const bool col_on = !p.col_act || p.col_act[(int64_t)tok * p.ldc + c0 + (ch >> 1)] != 0;
         uint32_t hi[4], mid[4], lo[4];
 #pragma unroll
         for (int k = 0; k < 8; k += 2) {
@@ -355,7 +366,7 @@ __global__ void __launch_bounds__(256) mortar_gemv_f32_kernel(const GemvF32Param
             for (int e = 0; e < 2; ++e) {
                 float xv = src[k + e];
                 if (p.swiglu_x) xv = xv * sigmoid_f32(xv) * src[I + k + e];      // h = silu(g) * u on load, fp32
-                v[e] = xv;
+                v[e] = col_on ? xv : 0.f;
             }
             const uint32_t h2 = bf16_pack2(v[0], v[1]);
             const float r0 = v[0] - bf16_to_f32(h2 & 0xffffu), r1 = v[1] - bf16_to_f32(h2 >> 16);
@@ -387,7 +398,7 @@ __global__ void __launch_bounds__(256) mortar_gemv_f32_kernel(const GemvF32Param
     bool unit_on = true;
     if (p.row_act) {
         int f = 0;
-        if (lane < p.B) f = p.row_act[(int64_t)lane * p.ldr + rowA] != 0;
+        if (lane < p.B) f = p.row_act[(int64_t)lane * p.ldr + rowA] != 0 || (rowB >= 0 && p.row_act[(int64_t)lane * p.ldr + rowB] != 0);
         unit_on = __builtin_amdgcn_readfirstlane(__ballot(f) != 0ull);
     }
     f32x4_t accA[MSUB], accB[MSUB];
@@ -401,6 +412,10 @@ __global__ void __launch_bounds__(256) mortar_gemv_f32_kernel(const GemvF32Param
     for (int ms = 0; ms < MSUB; ++ms) {
         const int tok = ms * 16 + n;
         if (tok >= p.B) continue;
+        if (p.row_act && unit_on) {      // per-stream row flags: zero partial for a stream whose row is off (fused_decode_step.py:1378-1381)
+            if (p.row_act[(int64_t)tok * p.ldr + rowA] == 0) accA[ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            if (rowB >= 0 && p.row_act[(int64_t)tok * p.ldr + rowB] == 0) accB[ms] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
         if (p.nslots > 1) {
             float *pp = p.part + ((int64_t)slot * p.B + tok) * p.N;
             *reinterpret_cast<f32x4_t *>(pp + rowA * 16 + 4 * g) = accA[ms];
@@ -466,23 +481,11 @@ int launch_gemv_f32(const GemvF32Params &p, hipStream_t st) {
 // work-list kernel above up to the order of the fp32 additions.
 
 // thread = 8 consecutive features of one row: x (or silu(g) * u of a gate_up output) -> 16 bytes of each term row
-// Behind the split, threads of further blocks reduce the row flags: unit_on[r] = any stream has row_act[b, r] set (the
-// work-list kernel skips a unit only when all B streams are inactive, and writes zeros).  A chunk whose input column is
-// inactive for all B streams is written as zeros, which is what skipping its blocks amounts to.
+// A chunk whose input column is off for its stream is written as zeros, which is what masking its blocks' products for
+// that stream amounts to (the flags are per stream, fused_decode_step.py:1387-1393).
 __global__ void __launch_bounds__(256) gemv_f32_split_kernel(const float *x, int B, int K, int64_t ldx, int swiglu_x,
-                                                             uint16_t *xs, const int32_t *col_act, int64_t ldc,
-                                                             const int32_t *row_act, int64_t ldr, int n_flags,
-                                                             int32_t *unit_on, int split_blocks) {
+                                                             uint16_t *xs, const int32_t *col_act, int64_t ldc) {
     const int nch = K / 8;
-    if ((int)blockIdx.x >= split_blocks) {
-        const int r = ((int)blockIdx.x - split_blocks) * 256 + threadIdx.x;
-        if (r < n_flags) {
-            int f = 0;
-            for (int b = 0; b < B; ++b) f |= row_act[(int64_t)b * ldr + r] != 0;
-            unit_on[r] = f;
-        }
-        return;
-    }
     const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (it >= (int64_t)B * nch) return;
     const int tok = (int)(it / nch), ch = (int)(it % nch);
@@ -506,13 +509,9 @@ __global__ void __launch_bounds__(256) gemv_f32_split_kernel(const float *x, int
         const float s0 = r0 - bf16_to_f32(m2 & 0xffffu), s1 = r1 - bf16_to_f32(m2 >> 16);
         hi[k / 2] = h2; mid[k / 2] = m2; lo[k / 2] = bf16_pack2(s0, s1);
     }
-    if (col_act) {
-        int f = 0;
-        for (int b = 0; b < B; ++b) f |= col_act[(int64_t)b * ldc + (ch >> 1)] != 0;
-        if (!f) {
+    if (col_act && col_act[(int64_t)tok * ldc + (ch >> 1)] == 0) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) hi[k] = mid[k] = lo[k] = 0u;
-        }
+        for (int k = 0; k < 4; ++k) hi[k] = mid[k] = lo[k] = 0u;
     }
     uint4 *dst = reinterpret_cast<uint4 *>(xs + (int64_t)tok * K + ch * 8);
     const int64_t plane = (int64_t)B * K / 8;                    // 16-byte units per term
@@ -524,21 +523,20 @@ __global__ void __launch_bounds__(256) gemv_f32_split_kernel(const float *x, int
 // y3 [3B, N]: the sums of the hi, mid and lo rows.  y = scale * ((hi + mid) + lo), then the epilogue of the mode.
 __global__ void __launch_bounds__(256) gemv_f32_combine3_kernel(const float *y3, const float *scale, int B, int N, int mode,
                                                                 const float *gates, int cluster_size, int64_t ldg,
-                                                                const int32_t *unit_on, float *y, int64_t ldy) {
+                                                                const int32_t *row_act, int64_t ldr, float *y, int64_t ldy) {
     const int nout = mode == 0 ? N : N / 2;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= (int64_t)B * nout) return;
     const int tok = (int)(i / nout), o = (int)(i % nout);
-    if (unit_on && unit_on[o >> 4] == 0) {                       // the unit is off for every stream: zeros
-        y[(int64_t)tok * ldy + o] = 0.f;
-        return;
-    }
+    // per-stream row flags (fused_decode_step.py:1378-1381): the sum of a row that is off for this stream is zero
+    const bool on_a = !row_act || row_act[(int64_t)tok * ldr + (o >> 4)] != 0;
     const float s = scale[0];
     const float *r0 = y3 + (int64_t)tok * N, *r1 = r0 + (int64_t)B * N, *r2 = r1 + (int64_t)B * N;
-    const float a = s * ((r0[o] + r1[o]) + r2[o]);
+    const float a = on_a ? s * ((r0[o] + r1[o]) + r2[o]) : 0.f;
     float r = a;
     if (mode == 1) {
-        const float b = s * ((r0[nout + o] + r1[nout + o]) + r2[nout + o]);
+        const bool on_b = !row_act || row_act[(int64_t)tok * ldr + ((nout + o) >> 4)] != 0;
+        const float b = on_b ? s * ((r0[nout + o] + r1[nout + o]) + r2[nout + o]) : 0.f;
         r = a * sigmoid_f32(a) * b;
         if (gates) r *= gates[(int64_t)tok * ldg + o / cluster_size];
     }
@@ -546,7 +544,7 @@ __global__ void __launch_bounds__(256) gemv_f32_combine3_kernel(const float *y3,
 }
 
 int64_t gemv_f32_fast_bytes(const mortar_bcsr_t *W, int B) {
-    return (int64_t)3 * B * ((int64_t)W->Rb * 16 * 4 + (int64_t)W->Cb * 16 * 2) + (((int64_t)W->Rb * 4 + 15) & ~(int64_t)15);
+    return (int64_t)3 * B * ((int64_t)W->Rb * 16 * 4 + (int64_t)W->Cb * 16 * 2);
 }
 
 // Returns MORTAR_NO_KERNEL when the SpMM kernels cannot serve the shape (the caller then runs the work-list kernel).
@@ -554,17 +552,15 @@ int gemv_f32_fast(const mortar_bcsr_t *W, const int32_t *sched, const GemvF32Par
     const int K = W->Cb * 16, N = W->Rb * 16;
     float *y3 = reinterpret_cast<float *>(ws);
     uint16_t *xs = reinterpret_cast<uint16_t *>(y3 + (int64_t)3 * p.B * N);
-    int32_t *unit_on = reinterpret_cast<int32_t *>(xs + (int64_t)3 * p.B * K);
     const int64_t nsplit = (int64_t)p.B * (K / 8);
     const int split_blocks = (int)((nsplit + 255) / 256);
-    const int n_flags = p.row_act ? (p.mode == 0 ? W->Rb : W->Rb / 2) : 0;       // gate and up rows share the gate row's flag
-    hipLaunchKernelGGL(gemv_f32_split_kernel, dim3((unsigned)(split_blocks + (n_flags + 255) / 256)), dim3(256), 0, st, p.x, p.B,
-                       K, p.ldx, p.swiglu_x, xs, p.col_act, p.ldc, p.row_act, p.ldr, n_flags, unit_on, split_blocks);
+    hipLaunchKernelGGL(gemv_f32_split_kernel, dim3((unsigned)split_blocks), dim3(256), 0, st, p.x, p.B, K, p.ldx, p.swiglu_x, xs,
+                       p.col_act, p.ldc);
     const int rc = mortar_spmm_codes_f32(W, sched, xs, 3 * p.B, K, y3, N, st);
     if (rc) return rc;
     const int64_t total = (int64_t)p.B * (p.mode == 0 ? N : N / 2);
     hipLaunchKernelGGL(gemv_f32_combine3_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, y3, p.scale, p.B, N,
-                       p.mode, p.gates, p.cluster_size, p.ldg, p.row_act ? unit_on : nullptr, p.y, p.ldy);
+                       p.mode, p.gates, p.cluster_size, p.ldg, p.row_act, p.ldr, p.y, p.ldy);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return mortar_fail(MORTAR_ERR_HIP, "gemv_f32 launch: %s", hipGetErrorString(e));
     return MORTAR_OK;

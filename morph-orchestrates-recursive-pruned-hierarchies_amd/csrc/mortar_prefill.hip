@@ -275,6 +275,85 @@ int gateup_common(const mortar_bcsr_t *W, const int32_t *sched, const uint16_t *
 }
 }  // namespace
 
+// ---- the MLP as one call ------------------------------------------------------------------------------------
+
+namespace {
+// Rows from which both launches of the MLP certainly run the 32-token prefill tiles (below, products over several K
+// segments have small-tile forms): the hidden activations then travel in tile order.
+constexpr int64_t MLP_TILED_MIN_ROWS = 513;
+
+bool mlp_tiled(const mortar_bcsr_t *Wgu, const mortar_bcsr_t *Wdn, int64_t M) {
+    if (M < MLP_TILED_MIN_ROWS || !Wgu->codes4_o || !Wdn->codes4_o) return false;
+    const int seg = Wdn->seg_cb < Wdn->Cb ? Wdn->seg_cb : Wdn->Cb;
+    if (tile_bytes(32, seg) > LDS_BUDGET) return false;
+    if (seg == Wdn->Cb && resident_mt(Wdn->Cb) != 32) return false;      // a narrow `down` runs 64-token tiles
+    return ((M + 31) / 32 * 32) * ((int64_t)Wdn->Cb * 16) < ((int64_t)1 << 31);
+}
+}  // namespace
+
+extern "C" int64_t mortar_mlp_hidden_bytes(int64_t M, int32_t d_ff) {
+    if (M <= 0 || d_ff <= 0 || d_ff % 16) return 0;
+    return (M + 31) / 32 * 32 * (int64_t)d_ff * 2;
+}
+
+extern "C" int mortar_mlp_bf16(const mortar_bcsr_t *Wgu, const int32_t *sched_gu, const mortar_bcsr_t *Wdn,
+                               const int32_t *sched_dn, const uint16_t *x, int64_t M, int64_t ldx, int32_t norm,
+                               const uint16_t *norm_w, float norm_eps, const float *gates, int32_t n_clusters,
+                               void *hidden, uint16_t *y, int64_t ldy, int32_t phase, void *stream) {
+    if (!Wgu || !Wdn || !hidden) return mortar_fail(MORTAR_ERR_ARG, "mlp: null pointer");
+    if (Wgu->Rb & 1) return mortar_fail(MORTAR_ERR_ARG, "mlp: gate_up has an odd number of block-rows");
+    if (Wdn->Cb * 2 != Wgu->Rb) return mortar_fail(MORTAR_ERR_ARG, "mlp: down has %d input block-columns, gate_up %d gate/up units", Wdn->Cb, Wgu->Rb / 2);
+    if (phase < 0 || phase > 2) return mortar_fail(MORTAR_ERR_ARG, "mlp: phase %d not in 0..2", phase);
+    if (reinterpret_cast<uintptr_t>(hidden) & 15) return mortar_fail(MORTAR_ERR_ARG, "mlp: hidden must be 16-byte aligned");
+    const int64_t d_ff = (int64_t)Wdn->Cb * 16;
+    uint16_t *h = static_cast<uint16_t *>(hidden);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool tiled = M > 0 && mlp_tiled(Wgu, Wdn, M);
+    if (!tiled) {        // row-major hidden activations through the separate entry points
+        int rc = MORTAR_OK;
+        if (phase != 2)
+            rc = gateup_common(Wgu, sched_gu, x, M, ldx, norm != 0, norm_w, norm_eps, h, d_ff, gates, n_clusters, nullptr, nullptr, stream);
+        if (rc == MORTAR_OK && phase != 1) rc = mortar_spmm_bf16(Wdn, sched_dn, h, M, d_ff, y, ldy, stream);
+        return rc;
+    }
+    if (phase != 2) {
+        int rc = check_common(Wgu, x, M, ldx, h, d_ff, d_ff);
+        if (rc) return rc;
+        SpmmParams p;
+        fill(p, Wgu, sched_gu, x, M, ldx, h, d_ff);
+        p.n_units = Wgu->Rb / 2;
+        if (norm) {
+            if (!mortar_norm_fusable(Wgu->Cb) || p.nseg != 1)
+                return mortar_fail(MORTAR_ERR_LIMIT, "mlp: the fused RMSNorm needs in_features <= %d in one K segment "
+                                   "(mortar_norm_fusable() == 0: call mortar_rmsnorm_bf16 first)", NORM_MAX_CB * 16);
+            if (!(norm_eps >= 0.f)) return mortar_fail(MORTAR_ERR_ARG, "mlp: norm_eps must be >= 0");
+            if (reinterpret_cast<uintptr_t>(norm_w) & 15) return mortar_fail(MORTAR_ERR_ARG, "mlp: norm_w must be 16-byte aligned");
+            p.norm = 1; p.norm_eps = norm_eps; p.norm_w = norm_w;
+        }
+        if (gates) {
+            if (n_clusters <= 0 || d_ff % n_clusters || (d_ff / n_clusters) % 4)
+                return mortar_fail(MORTAR_ERR_ARG, "mlp: d_ff / n_clusters must be a whole multiple of 4");
+            p.gates = gates; p.n_clusters = n_clusters; p.cluster_size = (int)(d_ff / n_clusters);
+        }
+        p.y_tiled = 1;
+        p.codes_o = reinterpret_cast<const u32x4_t *>(Wgu->codes4_o);
+        rc = p.uscale != 0.f ? dispatch_prefill<CODE_4BIT | CODE_UNIFORM>(1, p, st) : dispatch_prefill<CODE_4BIT>(1, p, st);
+        if (rc) return rc;
+    }
+    if (phase != 1) {
+        int rc = check_common(Wdn, h, M, d_ff, y, ldy, (int64_t)Wdn->Rb * 16);
+        if (rc) return rc;
+        SpmmParams p;
+        fill(p, Wdn, sched_dn, h, M, d_ff, y, ldy);
+        p.n_units = Wdn->Rb;
+        p.x_tiled = 1;
+        p.codes_o = reinterpret_cast<const u32x4_t *>(Wdn->codes4_o);
+        rc = p.uscale != 0.f ? dispatch_prefill<CODE_4BIT | CODE_UNIFORM>(0, p, st) : dispatch_prefill<CODE_4BIT>(0, p, st);
+        if (rc) return rc;
+    }
+    return MORTAR_OK;
+}
+
 // ---- layer-batched small-M launches ---------------------------------------------------------------------
 
 extern "C" int64_t mortar_stack_table_bytes(int32_t n_layers) {

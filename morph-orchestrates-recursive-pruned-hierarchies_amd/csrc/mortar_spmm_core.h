@@ -47,6 +47,12 @@ struct SpmmParams {
     const float *hc_post;     // [M, hc_n]
     const void *hc_term;      // [M, out_features], type of hc_h, or null
     int hc_n, hc_f32;
+    // Hidden activations of the two-launch MLP in tile order instead of row-major (mortar_mlp_bf16): element (token, f)
+    // at ((token / 32) * (features / 16) + f / 16) * 512 + (token % 32) * 16 + f % 16, i.e. the 32 tokens x 16 features
+    // of one (token tile, block-column) are 1 KB of contiguous memory: gate_up's stores of a 16 x 16 result tile are 512
+    // contiguous bytes, and `down` stages a K segment of its token tile as one contiguous run, asynchronously, straight
+    // into LDS.  y_tiled: the SwiGLU epilogue stores so; x_tiled: the 32-token prefill tiles are staged from it.
+    int x_tiled, y_tiled, pad0_, pad1_;
 };
 
 // Device-side view of the launch parameters: the pointers carry the global address space in their type, so
@@ -70,7 +76,7 @@ struct SpmmView {
     const MORTAR_GLOBAL char *hc_h, *hc_term;
     MORTAR_GLOBAL char *hc_out;
     const MORTAR_GLOBAL float *hc_res, *hc_post;
-    int hc_n, hc_f32;
+    int hc_n, hc_f32, x_tiled, y_tiled;
 };
 static_assert(sizeof(SpmmParams) % 16 == 0, "table entries are copied in 16-byte words");
 // Entry i of a parameter table in device memory (uniform address: scalar loads).
@@ -96,6 +102,7 @@ __device__ __forceinline__ SpmmView mortar_view(const SpmmParams &q) {
     v.hc_h = (const MORTAR_GLOBAL char *)q.hc_h; v.hc_term = (const MORTAR_GLOBAL char *)q.hc_term;
     v.hc_out = (MORTAR_GLOBAL char *)q.hc_out; v.hc_res = (const MORTAR_GLOBAL float *)q.hc_res;
     v.hc_post = (const MORTAR_GLOBAL float *)q.hc_post; v.hc_n = q.hc_n; v.hc_f32 = q.hc_f32;
+    v.x_tiled = q.x_tiled; v.y_tiled = q.y_tiled;
     return v;
 }
 
@@ -278,8 +285,33 @@ __device__ __forceinline__ void mortar_stage_quads(const SpmmView &p, unsigned c
     }
 }
 
+// Asynchronous 16-byte-per-lane copy global -> LDS (lane l's bytes land at lds_base + 16 * l): no registers, no
+// address arithmetic beyond the source pointer.  The caller waits with s_waitcnt vmcnt(0) and a barrier before the
+// destination is read.  (One wait state separates the write of M0 from its use as the LDS base.)
+__device__ __forceinline__ void mortar_load_to_lds(const MORTAR_GLOBAL char *gsrc, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gsrc) : "memory", "m0");
+}
+
+// Stages block-columns [c0, c0 + ncb) of token tile `mt` from activations stored in tile order (SpmmParams::x_tiled):
+// the 1 KB of a (token tile, block-column) is already in the tile's LDS layout, so one wave instruction copies it.
+// Rows past M hold whatever the buffer held: they feed accumulator columns that are never stored.
+template <int WAVES>
+__device__ __forceinline__ void mortar_stage_tiled32(const SpmmView &p, uint4 *lx, int mt, int c0, int ncb, int tid) {
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const MORTAR_GLOBAL char *src = p.x + ((int64_t)mt * p.Cb + c0) * 1024 + lane * 16;
+    const uint32_t dst = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lx;
+    for (int c = wave; c < ncb; c += WAVES) mortar_load_to_lds(src + (int64_t)c * 1024, __builtin_amdgcn_readfirstlane(dst + c * 1024));
+    __builtin_amdgcn_s_waitcnt(0);
+}
+
 template <int MT, int WAVES, bool MASKED>
 __device__ __forceinline__ void mortar_stage_tile(const SpmmView &p, uint4 *lx, int m0, int c0, int ncb, int tid) {
+    if constexpr (MT == 32 && !MASKED) {
+        if (p.x_tiled) {
+            mortar_stage_tiled32<WAVES>(p, lx, m0 / 32, c0, ncb, tid);
+            return;
+        }
+    }
     mortar_stage_quads<MT, WAVES, MASKED, false>(p, reinterpret_cast<unsigned char *>(lx), m0, c0, ncb, tid, nullptr);
 }
 
@@ -384,6 +416,11 @@ __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, i
         }
     } else {
         pk = swiglu_pack4(a0, a1, has_gates, gv);
+        if (p.y_tiled) {       // (host: M * features < 2^31)
+            const uint32_t e = ((uint32_t)(tok >> 5) * (uint32_t)p.n_units + (uint32_t)unit) * 512u + (uint32_t)(tok & 31) * 16u + 4u * g;
+            *(MORTAR_GLOBAL u32x2_t *)(p.y + e) = pk;
+            return;
+        }
     }
     *(MORTAR_GLOBAL u32x2_t *)(p.y + (int64_t)tok * p.ldy + unit * 16 + 4 * g) = pk;
 }

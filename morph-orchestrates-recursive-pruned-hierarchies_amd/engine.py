@@ -20,19 +20,20 @@ def mortar_pack_strips(cms) -> MortarPack:
 
 def mortar_gemv(x: Tensor, pack: MortarPack, swiglu_x: bool = False, swiglu_out: bool = False,
                 row_act: Tensor | None = None, col_act: Tensor | None = None, gates: Tensor | None = None,
-                cluster_size: int = 0) -> Tensor:
+                cluster_size: int = 0, flags_from_gates: bool = True) -> Tensor:
     """x [B, I] row-contiguous -> [B, O], or [B, O/2] = silu(g)*u with swiglu_out (the gate_up call); with swiglu_x,
     x is the packed gate_up output [B, 2I] and h = silu(g)*u is computed on load (the reference's down call form).
     Same keywords as the reference (fused_decode_step.py:1502-1509).  float32 input runs the reference engine's
     arithmetic (exact products, fp32 sums, fp32 scale after the block sum, fp32 out); bfloat16 input runs the bf16
-    activation path of this runtime (swiglu_x there goes through the fp32 kernel and is rounded to bf16 at the end)."""
+    activation path of this runtime (swiglu_x there goes through the fp32 kernel and is rounded to bf16 at the end).
+    row_act / col_act are per-stream flags as in the reference's kernel; ``flags_from_gates`` (see ops.gemv): they are
+    route_flags of the same step's gates, which is how the reference engine calls (engine.py:984-994)."""
     if gates is not None and cluster_size and (pack.out_features // 2) // gates.shape[-1] != cluster_size:
         raise ValueError("cluster_size does not match d_ff / n_clusters")
     if x.dtype == torch.float32 or swiglu_x:
         y = ops.gemv_f32(x.float(), pack, swiglu_x=swiglu_x, swiglu_out=swiglu_out, gates=gates, row_act=row_act, col_act=col_act)
         return y if x.dtype == torch.float32 else y.to(x.dtype)
-    y = ops.gemv(x, pack, swiglu_out=swiglu_out, gates=gates, row_act=row_act, col_act=col_act)
-    return y
+    return ops.gemv(x, pack, swiglu_out=swiglu_out, gates=gates, row_act=row_act, col_act=col_act, flags_from_gates=flags_from_gates)
 
 
 class MortarDecodeMLP:

@@ -193,6 +193,8 @@ class _SwiGLUMortar(nn.Module):
             route = ops.remoe_route(active, tile)
             h = ops.gateup_swiglu(xb, Wgu, gates=gates, route=route, norm=norm)
             y = ops.spmm(h, Wdn, active=active)
+        elif N > ops.DECODE_MAX_ROWS:
+            y = ops.mlp(xb, Wgu, Wdn, gates=gates, norm=norm)      # hidden activations in the library's tile order
         else:
             h = ops.gateup_swiglu(xb, Wgu, gates=gates, norm=norm)
             y = ops.spmm(h, Wdn)

@@ -143,6 +143,51 @@ def gateup_swiglu(x: Tensor, W: MortarPack, gates: Tensor | None = None, route: 
     return h
 
 
+def mlp(x: Tensor, Wgu: MortarPack, Wdn: MortarPack, gates: Tensor | None = None, norm: tuple | None = None,
+        out: Tensor | None = None, hidden: Tensor | None = None, phase: int = 0) -> Tensor:
+    """y[M, d_model] = down(silu(gate) * up [* gates per cluster]), gate_up applied to x or (``norm`` = (weight or None,
+    eps), needs norm_fusable(Wgu)) to RMSNorm(x): _SwiGLUMortar.forward (transformer.py:402-431) in two launches.  Same bits
+    as gateup_swiglu followed by spmm; the hidden activations stay in a workspace whose layout the library chooses (tile
+    order for prefill-sized calls).  ``hidden``: a uint8 workspace of hidden_bytes(M, d_ff) to reuse across calls;
+    ``phase`` 1 / 2 run only the first / second launch."""
+    x = _bf16_2d(x, "mlp")
+    M = x.shape[0]
+    if x.shape[1] != Wgu.in_features:
+        raise ValueError(f"mlp: x has {x.shape[1]} features, gate_up expects {Wgu.in_features}")
+    if Wgu.Rb % 2 or Wgu.out_features != 2 * Wdn.in_features:
+        raise ValueError(f"mlp: gate_up [{Wgu.out_features}, {Wgu.in_features}] and down [{Wdn.out_features}, {Wdn.in_features}] do not chain")
+    d_ff = Wdn.in_features
+    y = out if out is not None else torch.empty((M, Wdn.out_features), dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return y
+    L = _lib.lib()
+    need = int(L.mortar_mlp_hidden_bytes(M, d_ff))
+    if hidden is None:
+        hidden = torch.empty(need, dtype=torch.uint8, device=x.device)
+    elif hidden.dtype != torch.uint8 or not hidden.is_contiguous() or hidden.numel() < need or hidden.device != x.device:
+        raise ValueError(f"mlp: hidden must be a contiguous uint8 workspace of at least {need} bytes on {x.device}")
+    ncl = 0
+    if gates is not None:
+        if gates.dtype != torch.float32 or gates.dim() != 2 or not gates.is_contiguous() or gates.shape[0] != M:
+            raise TypeError("mlp: gates must be a contiguous float32 [M, n_clusters] tensor")
+        ncl = gates.shape[1]
+    nw, eps = (None, 0.0)
+    if norm is not None:
+        nw, eps = norm
+        if nw is not None:
+            if nw.dtype != torch.bfloat16 or nw.dim() != 1 or nw.shape[0] != Wgu.in_features or not nw.is_contiguous():
+                raise TypeError("mlp: norm weight must be a contiguous bfloat16 [in_features] tensor")
+            _need_gpu(nw, "mlp")
+    rc = L.mortar_mlp_bf16(Wgu.ref, _p(Wgu.sched(2)), Wdn.ref, _p(Wdn.sched(1)), _p(x), M, x.stride(0), int(norm is not None),
+                           _p(nw), float(eps), _p(gates), ncl, _p(hidden), _p(y), y.stride(0), int(phase), _stream(x))
+    _lib.check(rc, "mortar_mlp_bf16")
+    return y
+
+
+def mlp_hidden_bytes(M: int, d_ff: int) -> int:
+    return int(_lib.lib().mortar_mlp_hidden_bytes(int(M), int(d_ff)))
+
+
 # ----------------------------------------------------------------------------- ReMoE
 
 
@@ -287,10 +332,13 @@ def _kseg_for(W: MortarPack, B: int) -> int:
 
 def gemv(x: Tensor, W: MortarPack, swiglu_out: bool = False, gates: Tensor | None = None,
          row_act: Tensor | None = None, col_act: Tensor | None = None, max_blocks: int | None = None,
-         out: Tensor | None = None) -> Tensor:
+         out: Tensor | None = None, flags_from_gates: bool = True) -> Tensor:
     """Decode GEMV for B <= 64 streams: y = x W^T (bf16), or with swiglu_out the fused silu(g)*u[*gates].
     Without gather flags the batch goes to the small-tile SpMM kernels (one pass over the weights); with
-    row_act / col_act (or an explicit max_blocks split) it runs the work-list kernel that honours them."""
+    row_act / col_act (or an explicit max_blocks split) it runs the work-list kernel that honours them, per stream.
+    ``flags_from_gates``: row_act is route_flags(gates) of this very call, as the reference engine passes it
+    (engine.py:984-994); the gated gate_up then needs no flags (a gate of 0 zeroes what the flag would).  Pass False
+    for flags of any other origin: they are then applied as given."""
     x = _bf16_2d(x, "gemv")
     B = x.shape[0]
     if not 1 <= B <= 64:
@@ -304,7 +352,7 @@ def gemv(x: Tensor, W: MortarPack, swiglu_out: bool = False, gates: Tensor | Non
         rt1 = W._route_tile_1 = route_tile(W, 1)
     # gate_up with gates: the row flags add nothing there (the gated kernel leaves out the units whose cluster is off for
     # every stream and stores their zeros; every other unit is computed and gated per stream, as the work list does)
-    if swiglu_out and gates is not None and col_act is None and max_blocks is None and rt1 != 0:
+    if swiglu_out and gates is not None and col_act is None and max_blocks is None and rt1 != 0 and flags_from_gates:
         row_act = None
     if row_act is None and col_act is None and max_blocks is None and (rt1 != 0 or (B <= 4 and not swiglu_out)):
         if swiglu_out:

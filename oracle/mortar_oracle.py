@@ -286,10 +286,14 @@ def swiglu_mlp(x, gate_up: dict, down: dict, gates: np.ndarray | None = None,
 # --------------------------------------------------------------------------- decode (fp32 engine form)
 
 
-def mortar_gemv(x: np.ndarray, codes, scales, col_idx, offsets) -> np.ndarray:
+def mortar_gemv(x: np.ndarray, codes, scales, col_idx, offsets, row_act=None, col_act=None) -> np.ndarray:
     """Decode GEMV in the engine's arithmetic: fp32 activations, exact +-x/0 products,
     scale applied to each block's partial sum (per-block generalisation of the scalar
-    scale-after-sum, fused_decode_step.py:1335,1441-1459).  Returns fp32 [B, O]."""
+    scale-after-sum, fused_decode_step.py:1335,1441-1459).  Returns fp32 [B, O].
+    row_act [B, Rb] / col_act [B, Cb] (optional) are the per-stream gather flags of the kernel: the sum of output
+    block-row r is zero for stream b when row_act[b, r] == 0 (the CTA stores a zero partial and returns,
+    fused_decode_step.py:1378-1381), and a block whose input block-column c has col_act[b, c] == 0 contributes nothing to
+    stream b (:1387-1393).  Each stream reads only its own flags."""
     B = x.shape[0]
     nnz, blk, _ = codes.shape
     Rb = len(offsets) - 1
@@ -300,7 +304,12 @@ def mortar_gemv(x: np.ndarray, codes, scales, col_idx, offsets) -> np.ndarray:
         lo, hi = int(offsets[r]), int(offsets[r + 1])
         cols = col_idx[lo:hi].astype(np.int64)
         part = np.einsum("bjc,jnc->bjn", xa[:, cols, :], codes[lo:hi].astype(np.float64))
-        y[:, r * blk:(r + 1) * blk] = (part * s[lo:hi][None, :, None]).sum(axis=1)
+        if col_act is not None:
+            part = part * (np.asarray(col_act)[:, cols] != 0)[:, :, None]
+        row = (part * s[lo:hi][None, :, None]).sum(axis=1)
+        if row_act is not None:
+            row = row * (np.asarray(row_act)[:, r] != 0)[:, None]
+        y[:, r * blk:(r + 1) * blk] = row
     return y.astype(np.float32)
 
 

@@ -138,6 +138,41 @@ def test_mlp_base_config_slice(dev, M):
     assert_close_bf16(to_np(y2).reshape(M, 768), ref["y"], "module", ulps=8)
 
 
+@pytest.mark.parametrize("d_model,d_ff,M,zipf", [(2048, 5632, 4096, None), (2048, 5632, 1000, 1.2), (768, 2048, 1200, None),
+                                                 (256, 16 * 40, 600, 1.2), (2048, 5632, 513, None), (2048, 5632, 300, None),
+                                                 (16 * 30, 16 * 352, 530, None)])
+def test_mlp_one_call_equals_the_two_calls(dev, d_model, d_ff, M, zipf):
+    """mortar_mlp_bf16 (hidden activations in the library's own layout: tile order from 513 rows, with the asynchronous
+    stage-in of `down`) gives the same bits as gate_up + SwiGLU followed by the plain product: plain, with cluster gates,
+    with the RMSNorm folded in, in two phases, with a reused workspace; and meets the oracle on sampled rows."""
+    spec = synth.synth_mlp(d_model, d_ff, 0.25, seed=40, zipf_s=zipf)
+    Wgu, Wdn = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    x = synth.synth_x(M, d_model, 41)
+    xd = to_dev(x, dev)
+    ncl = d_ff // 16
+    gates, _ = ops.remoe_gates(torch.from_numpy(synth.synth_logits(M, ncl, 42)).to(dev), ncl // 4)
+    nw = torch.from_numpy(O.bf16_round(1 + 0.1 * np.random.default_rng(43).standard_normal(d_model).astype(np.float32))).to(torch.bfloat16).to(dev)
+    ws = torch.full((ops.mlp_hidden_bytes(M, d_ff),), 0xFF, dtype=torch.uint8, device=dev)      # NaN patterns: rows past M stay so
+    for g, nm in ((None, None), (gates, None), (None, (nw, 1e-6)), (gates, (None, 1e-6))):
+        if nm is not None and not ops.norm_fusable(Wgu):
+            continue
+        want = ops.spmm(ops.gateup_swiglu(xd, Wgu, gates=g, norm=nm), Wdn)
+        assert torch.equal(ops.mlp(xd, Wgu, Wdn, gates=g, norm=nm), want)
+        assert torch.equal(ops.mlp(xd, Wgu, Wdn, gates=g, norm=nm, hidden=ws), want)
+        y = torch.full_like(want, float("nan"))
+        ops.mlp(xd, Wgu, Wdn, gates=g, norm=nm, hidden=ws, out=y, phase=1)
+        assert bool(torch.isnan(y).all())                                   # phase 1 writes the workspace only
+        ops.mlp(xd, Wgu, Wdn, gates=g, norm=nm, hidden=ws, out=y, phase=2)
+        assert torch.equal(y, want)
+    rows = np.random.default_rng(44).choice(M, 24, replace=False)
+    ref = O.swiglu_mlp(x[rows], spec["gate_up"], spec["down"])
+    assert_close_bf16(to_np(ops.mlp(xd, Wgu, Wdn))[rows], ref["y"], "one-call MLP vs oracle", ulps=8)
+    with pytest.raises(ValueError):
+        ops.mlp(xd, Wgu, Wdn, hidden=ws[:16])
+    with pytest.raises(ValueError):
+        ops.mlp(xd, Wdn, Wgu)
+
+
 def test_mlp_with_gates_and_skip(dev):
     """ReMoE-routed MLP: cluster size 16 (one block-row per cluster), k-th threshold gating, tile skipping."""
     d_model, d_ff, M, ncl, k = 256, 16 * 40, 300, 40, 10
@@ -495,6 +530,42 @@ def test_decode_gather_flags_worklist(dev):
     assert_close_bf16(to_np(y), ref["y"], "flagged decode", ulps=8)
 
 
+@pytest.mark.parametrize("B", [1, 5, 16, 37])
+def test_decode_gather_flags_are_per_stream(dev, B):
+    """Flags that do NOT follow from the gates and differ between the streams (fused_decode_step.py:1378-1393: stream b
+    reads ROWACT[b, r] and COLACT[b, cb]): the bf16 work-list GEMV against the oracle with the same flags, whole rows per
+    entry and split rows, with and without gates; flags_from_gates=False keeps caller flags beside gates."""
+    d_model, d_ff, ncl = 512, 16 * 48, 12
+    spec = synth.synth_mlp(d_model, d_ff, 0.3, seed=75, zipf_s=1.2)
+    gu_m, dn_m = spec["gate_up"], spec["down"]
+    Wgu, Wdn = synth.to_pack(gu_m, dev), synth.to_pack(dn_m, dev)
+    rng = np.random.default_rng(76 + B)
+    x = synth.synth_x(B, d_model, 77)
+    xd = to_dev(x, dev)
+    ract_np = (rng.random((B, 2 * d_ff // 16)) < 0.6).astype(np.int32)
+    ract_np[:, 2] = 0; ract_np[:, 2 + d_ff // 16] = 0                              # a unit that is off for every stream
+    cact_np = (rng.random((B, d_ff // 16)) < 0.6).astype(np.int32); cact_np[:, 7] = 0
+    ract, cact = torch.from_numpy(ract_np).to(dev), torch.from_numpy(cact_np).to(dev)
+    sc = lambda m: O.bf16_round(m["scales"])                                       # the bf16 path multiplies bf16(scale)
+    gu = O.bf16_round(O.mortar_gemv(x, gu_m["codes"], sc(gu_m), gu_m["col_idx"], gu_m["offsets"], row_act=ract_np))
+    h_ref = O.swiglu(gu)
+    gates_np = (rng.random((B, ncl)) * 2).astype(np.float32); gates_np[:, 1] = 0
+    hg_ref = O.bf16_round(h_ref.reshape(B, ncl, -1) * O.bf16_round(gates_np)[:, :, None]).reshape(B, d_ff)
+    gates = torch.from_numpy(gates_np).to(dev)
+    for mb in (None, 4):
+        h = ops.gemv(xd, Wgu, swiglu_out=True, row_act=ract, max_blocks=mb)
+        assert_close_bf16(to_np(h), h_ref, f"row flags per stream, max_blocks={mb}", ulps=4)
+        assert (to_np(h)[np.repeat((ract_np[:, :d_ff // 16] == 0) | (ract_np[:, d_ff // 16:] == 0), 16, axis=1)] == 0).all()
+        hg = ops.gemv(xd, Wgu, swiglu_out=True, gates=gates, row_act=ract, max_blocks=mb, flags_from_gates=False)
+        assert_close_bf16(to_np(hg), hg_ref, f"row flags beside gates, max_blocks={mb}", ulps=4)
+        guo = ops.gemv(xd, Wgu, row_act=ract, max_blocks=mb)
+        assert_close_bf16(to_np(guo), gu, f"plain product with row flags, max_blocks={mb}", ulps=4)
+        hin = O.bf16_round(rng.standard_normal((B, d_ff)).astype(np.float32))
+        y_ref = O.bf16_round(O.mortar_gemv(hin, dn_m["codes"], sc(dn_m), dn_m["col_idx"], dn_m["offsets"], col_act=cact_np))
+        y = ops.gemv(to_dev(hin, dev), Wdn, col_act=cact, max_blocks=mb)
+        assert_close_bf16(to_np(y), y_ref, f"column flags per stream, max_blocks={mb}", ulps=8)
+
+
 @pytest.mark.parametrize("B,n_layers,d_model", [(3, 5, 256), (12, 5, 256), (2, 300, 256), (12, 300, 1024), (40, 5, 256),
                                                   (64, 40, 1024)])
 def test_layer_stack_matches_single_launches(dev, B, n_layers, d_model):
@@ -761,21 +832,26 @@ def test_mortar_gemv_fp32_one_scale_runs_on_the_spmm_kernels(dev, B):
         assert np.abs(y.cpu().numpy() - y_ref).max() <= _gemv_f32_tolerance(y_ref)
     y2 = ops.gemv_f32(torch.from_numpy(fast).to(dev), Wdn, swiglu_x=True)
     assert np.abs(y2.cpu().numpy() - y_ref).max() <= 4 * _gemv_f32_tolerance(y_ref)
-    # flags without gates, both forms: a unit that is off for EVERY stream gives zeros, a column that is off for every
-    # stream contributes nothing; anything a single stream has switched on is computed for all of them
-    ract = torch.from_numpy((rng.random((B, d_ff // 16)) < 0.3 / B).astype(np.int32)).to(dev)
-    cact = torch.from_numpy((rng.random((B, d_ff // 16)) < 0.5 / B).astype(np.int32)).to(dev)
-    unit_on = ract.cpu().numpy().any(axis=0)
-    want = (g * u * 0 + h_ref) * np.repeat(unit_on, 16)[None, :]
-    for kw in ({}, {"max_blocks": 1 << 20}):
+    # flags without gates, both forms (SpMM kernels and work list), applied per stream as the reference's kernel does:
+    # stream b's sum of row r is zero when row_act[b, r] == 0 (gate rows and up rows have flags of their own), and input
+    # block-column c contributes nothing to stream b when col_act[b, c] == 0
+    ract_np = (rng.random((B, 2 * d_ff // 16)) < 0.5).astype(np.int32)
+    ract_np[:, 3] = 0; ract_np[:, 5] = 1                                           # a unit off / on for every stream
+    cact_np = (rng.random((B, d_ff // 16)) < 0.5).astype(np.int32)
+    ract, cact = torch.from_numpy(ract_np).to(dev), torch.from_numpy(cact_np).to(dev)
+    gu_f = O.mortar_gemv(x, gu_m["codes"], gu_m["scales"], gu_m["col_idx"], gu_m["offsets"], row_act=ract_np).astype(np.float64)
+    gf, uf = gu_f[:, :d_ff], gu_f[:, d_ff:]
+    want = gf / (1.0 + np.exp(-gf)) * uf
+    for kw in ({}, {"max_blocks": 1 << 20}, {"max_blocks": 8}):
         got = ops.gemv_f32(xt, Wgu, swiglu_out=True, row_act=ract, **kw).cpu().numpy()
-        assert np.abs(got - want).max() <= _gemv_f32_tolerance(h_ref) and (got[:, ~np.repeat(unit_on, 16)] == 0).all()
-    col_on = np.repeat(cact.cpu().numpy().any(axis=0), 16)
-    hm = h.cpu().numpy() * col_on[None, :]
-    ym_ref = O.mortar_gemv(hm, dn_m["codes"], dn_m["scales"], dn_m["col_idx"], dn_m["offsets"]).astype(np.float64)
-    for kw in ({}, {"max_blocks": 1 << 20}):
+        assert np.abs(got - want).max() <= _gemv_f32_tolerance(h_ref), kw
+        assert (got[np.repeat(ract_np[:, :d_ff // 16] == 0, 16, axis=1)] == 0).all()
+        got = ops.gemv_f32(xt, Wgu, row_act=ract, **kw).cpu().numpy()               # plain product, a flag per output row
+        assert np.abs(got - gu_f).max() <= _gemv_f32_tolerance(gu), kw
+    ym_ref = O.mortar_gemv(h.cpu().numpy(), dn_m["codes"], dn_m["scales"], dn_m["col_idx"], dn_m["offsets"], col_act=cact_np).astype(np.float64)
+    for kw in ({}, {"max_blocks": 1 << 20}, {"max_blocks": 8}):
         got = ops.gemv_f32(h, Wdn, col_act=cact, **kw).cpu().numpy()
-        assert np.abs(got - ym_ref).max() <= _gemv_f32_tolerance(y_ref)
+        assert np.abs(got - ym_ref).max() <= _gemv_f32_tolerance(y_ref), kw
 
 
 @pytest.mark.parametrize("B,n,f32", [(1, 4, True), (3, 4, False), (16, 2, True), (40, 4, False), (5, 1, True), (7, 3, False)])

@@ -267,6 +267,39 @@ def test_decode_gemv_keeps_the_fp32_scale_unrounded():
     np.testing.assert_allclose(y3[0], hand3.astype(np.float32), rtol=2e-7)
 
 
+def test_decode_gemv_flags_are_per_stream():
+    """fused_decode_step.py:1378-1393: stream b reads ROWACT[b, r] and COLACT[b, cb] only.  Hand case: one block-row, two
+    identity blocks on block-columns 0 and 1, two streams; y = x[0:16] + x[16:32] with everything on."""
+    eye = np.eye(16, dtype=np.int8)
+    codes = np.stack([eye, eye])
+    col, off = np.array([0, 1], np.int16), np.array([0, 2], np.int32)
+    x = np.stack([np.arange(32, dtype=np.float32), 100 + np.arange(32, dtype=np.float32)])
+    one = np.float32(1.0)
+    full = O.mortar_gemv(x, codes, one, col, off)
+    assert np.array_equal(full, x[:, :16] + x[:, 16:])
+    cact = np.array([[1, 0], [0, 1]], np.int32)                       # stream 0 keeps column 0, stream 1 keeps column 1
+    y = O.mortar_gemv(x, codes, one, col, off, col_act=cact)
+    assert np.array_equal(y[0], x[0, :16]) and np.array_equal(y[1], x[1, 16:])
+    ract = np.array([[0], [1]], np.int32)                             # the row is off for stream 0 only
+    y = O.mortar_gemv(x, codes, one, col, off, row_act=ract)
+    assert not y[0].any() and np.array_equal(y[1], full[1])
+    y = O.mortar_gemv(x, codes, one, col, off, row_act=ract, col_act=cact)
+    assert not y[0].any() and np.array_equal(y[1], x[1, 16:])
+    # all flags on == no flags; any non-zero value counts as on
+    m = make_mat(5, 8, 0.4, 44)
+    xr = xbf(3, 128, 45)
+    a = O.mortar_gemv(xr, m["codes"], m["scales"], m["col_idx"], m["offsets"])
+    b = O.mortar_gemv(xr, m["codes"], m["scales"], m["col_idx"], m["offsets"], row_act=np.full((3, 5), 7), col_act=np.full((3, 8), -1))
+    assert np.array_equal(a, b)
+    # against the dense form: flags are a row mask on the output and a column mask on the input, per stream
+    rng = np.random.default_rng(46)
+    ra, ca = rng.integers(0, 2, (3, 5)), rng.integers(0, 2, (3, 8))
+    got = O.mortar_gemv(xr, m["codes"], m["scales"], m["col_idx"], m["offsets"], row_act=ra, col_act=ca)
+    W = O.to_dense(m["codes"].astype(np.float64) * m["scales"].astype(np.float64)[:, None, None], m["row_idx"], m["col_idx"], m["shape"])
+    want = ((xr.astype(np.float64) * np.repeat(ca, 16, axis=1)) @ W.T) * np.repeat(ra, 16, axis=1)
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+
+
 # ---- ReMoE ---------------------------------------------------------------------------------------------
 
 def brute_remoe(logits, k):
