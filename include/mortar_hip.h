@@ -354,6 +354,27 @@ int mortar_gemv_bf16_noalloc(const mortar_bcsr_t *W, const int32_t *entries, int
                              const int32_t *row_act, int64_t ldr, const int32_t *col_act, int64_t ldc,
                              void *stream);
 
+/* ---- product over stored bf16 block values (the operator-level drop-in) ------------------------ */
+
+/* y = x W^T with W given by the reference's BCSR arrays as they are: stk_dds(lhs, data, offsets, row_indices,
+ * column_indices, ..., transpose_b = True), morph/sparse/stk/backend/custom_ops.py:35-56 (kernel
+ * triton_kernels.py:170-230): bf16 operands, fp32 accumulation, bf16 store, for ANY bf16 block values -- no ternary
+ * restriction, nothing is quantised.  (The ternary entry points above stream 2- / 4-bit codes and are the fast path of
+ * the modules; this one is what the stk_dds operator calls.)
+ *   row_ptr  device int32 [Rb+1] (mortar_offsets);  col device int16 [nnz] (mortar_column_indices), ascending in a row
+ *   data     device bf16 [nnz,16,16] (mortar_data, element [j, lr, c] = W[row_j*16+lr, col_j*16+c]), 16-byte aligned
+ *   seg_ptr  device int32 [Rb, nseg+1] from mortar_segment_ptr_host with seg_cb = mortar_values_seg_cb(Cb), nseg =
+ *            ceil(Cb / seg_cb); needed when nseg > 1 (in_features too wide for one 32-token LDS tile), else may be NULL
+ *   x bf16 [M, ldx] 16-byte aligned, ldx % 8 == 0;  y bf16 [M, ldy] 8-byte aligned, ldy % 4 == 0
+ * The dX product (transpose_b = False) is the same call on the transposed topology (mortar_transpose_topology_host)
+ * with the blocks gathered in that order and transposed. */
+int32_t mortar_values_seg_cb(int32_t Cb);
+int mortar_segment_ptr_host(const int32_t *row_ptr, const int16_t *col, int32_t Rb, int32_t Cb, int32_t seg_cb,
+                            int32_t *seg_ptr_out);
+int mortar_dds_values_bf16(const int32_t *row_ptr, const int16_t *col, const int32_t *seg_ptr, const uint16_t *data,
+                           int32_t Rb, int32_t Cb, int64_t nnz, const uint16_t *x, int64_t M, int64_t ldx, uint16_t *y,
+                           int64_t ldy, void *stream);
+
 /* ---- RMSNorm ---------------------------------------------------------------------------------- */
 
 /* mortar_gateup_swiglu_bf16 with the RMSNorm in front of the MLP (attention.RMSNorm, morph/model/attention.py:133-141,

@@ -53,6 +53,9 @@ _SIGS = {
     "mortar_norm_gateup_swiglu_bf16": (C.c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_f32, c_vp, c_i64, c_vp, c_i32,
                                                  c_vp, c_vp, c_vp]),
     "mortar_norm_fusable": (C.c_int, [c_i32]),
+    "mortar_values_seg_cb": (c_i32, [c_i32]),
+    "mortar_segment_ptr_host": (C.c_int, [c_vp, c_vp, c_i32, c_i32, c_i32, c_vp]),
+    "mortar_dds_values_bf16": (C.c_int, [c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i64, c_vp, c_i64, c_i64, c_vp, c_i64, c_vp]),
     "mortar_mlp_hidden_bytes": (c_i64, [c_i64, c_i32]),
     "mortar_mlp_bf16": (C.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_vp, c_f32, c_vp, c_i32, c_vp, c_vp, c_i64,
                                   c_i32, c_vp]),

@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB = os.path.join(_HERE, "libmortar_hip.so")
 SOURCES = ["mortar_host.cpp", "mortar_prefill.hip", "mortar_smallm.hip", "mortar_decode.hip", "mortar_route.hip",
-           "mortar_pack.hip", "mortar_sdd.hip", "mortar_swiglu.hip"]
+           "mortar_pack.hip", "mortar_sdd.hip", "mortar_swiglu.hip", "mortar_values.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

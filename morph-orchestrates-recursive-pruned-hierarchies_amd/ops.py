@@ -8,7 +8,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .pack import BLK, MortarPack
+from .pack import BLK, BcsrTopology, MortarPack
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -64,6 +64,27 @@ def spmm(x: Tensor, W: MortarPack, out: Tensor | None = None, active: Tensor | N
         rc = L.mortar_spmm_bf16_masked(W.ref, _p(sched), _p(x), M, x.stride(0), _p(y), y.stride(0),
                                        _p(active), active.shape[1], _stream(x))
     _lib.check(rc, "mortar_spmm_bf16")
+    return y
+
+
+def dds_values(x: Tensor, data: Tensor, T: BcsrTopology, out: Tensor | None = None) -> Tensor:
+    """y[M, out] = x[M, in] @ W^T for W given as stored bf16 block values ``data`` [nnz, 16, 16] on the topology ``T``:
+    the arithmetic of the reference's stk_dds (custom_ops.py:35-56) for any block values, nothing quantised."""
+    x = _bf16_2d(x, "dds_values")
+    _need_gpu(data, "dds_values")
+    if data.dtype != torch.bfloat16 or tuple(data.shape) != (T.nnz, BLK, BLK) or not data.is_contiguous():
+        raise TypeError(f"dds_values: data must be a contiguous bfloat16 [{T.nnz}, 16, 16] tensor")
+    if x.shape[1] != T.in_features:
+        raise ValueError(f"dds_values: x has {x.shape[1]} features, matrix expects {T.in_features}")
+    M = x.shape[0]
+    y = out if out is not None else torch.empty((M, T.out_features), dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return y
+    if T.nnz == 0:
+        return y.zero_()
+    rc = _lib.lib().mortar_dds_values_bf16(_p(T.row_ptr), _p(T.col), _p(T.seg_ptr), _p(data), T.Rb, T.Cb, T.nnz, _p(x), M,
+                                           x.stride(0), _p(y), y.stride(0), _stream(x))
+    _lib.check(rc, "mortar_dds_values_bf16")
     return y
 
 

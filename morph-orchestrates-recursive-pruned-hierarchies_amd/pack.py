@@ -170,6 +170,47 @@ def decode_worklist(offsets, col, Rb: int, Cb: int, rows_per_unit: int, kseg: in
     return ent, int(ns.value), row_slots
 
 
+class BcsrTopology:
+    """The reference's BCSR index arrays of one matrix (mortar_offsets, mortar_column_indices) on the device, with what the
+    product over stored block values needs beside them: the per-segment row pointers for wide K and the transposed topology
+    (reference: stk matrix.py:107-125) for the dX product.  No codes, no scales: the values stay where the caller has them."""
+
+    def __init__(self, offsets, col, out_features: int, in_features: int, device):
+        if out_features % BLK or in_features % BLK:
+            raise ValueError(f"[{out_features},{in_features}] not divisible by blocking {BLK}")
+        self.out_features, self.in_features = int(out_features), int(in_features)
+        self.Rb, self.Cb = out_features // BLK, in_features // BLK
+        self.h_offsets = _np(offsets, np.int32).reshape(-1)
+        self.h_col = _np(col, np.int16).reshape(-1)
+        if self.h_offsets.size != self.Rb + 1:
+            raise ValueError(f"offsets has {self.h_offsets.size} entries, expected {self.Rb + 1}")
+        self.nnz = int(self.h_offsets[-1])
+        if self.h_col.size != self.nnz:
+            raise ValueError(f"column_indices has {self.h_col.size} entries, offsets say {self.nnz}")
+        validate_bcsr(self.h_offsets, self.h_col, self.Rb, self.Cb)
+        self.device = torch.device(device)
+        self.row_ptr = torch.from_numpy(self.h_offsets).to(self.device)
+        self.col = torch.from_numpy(self.h_col).to(self.device)
+        L = _lib.lib()
+        self.seg_cb = int(L.mortar_values_seg_cb(self.Cb))
+        self.nseg = -(-self.Cb // self.seg_cb)
+        self.seg_ptr = None
+        if self.nseg > 1:
+            sp = np.empty(self.Rb * (self.nseg + 1), dtype=np.int32)
+            _lib.check(L.mortar_segment_ptr_host(_vp(self.h_offsets), _vp(self.h_col), self.Rb, self.Cb, self.seg_cb, _vp(sp)),
+                       "mortar_segment_ptr_host")
+            self.seg_ptr = torch.from_numpy(sp).to(self.device)
+        self._t = None
+
+    def transposed(self):
+        """(topology of W^T, src): block j of W^T is block src[j] of W, transposed (int64 device index)."""
+        if self._t is None:
+            off_t, col_t, src = transpose_topology(self.h_offsets, self.h_col, self.Rb, self.Cb)
+            self._t = (BcsrTopology(off_t, col_t, self.in_features, self.out_features, self.device),
+                       torch.from_numpy(src.astype(np.int64)).to(self.device))
+        return self._t
+
+
 class MortarPack:
     """One carved matrix W [out, in] resident on a device, plus its cached schedules.
 

@@ -114,8 +114,49 @@ def test_stk_dds_operator_signature(dev):
     assert_close_bf16(to_np(y), oracle_spmm(x, m))
     with pytest.raises(ValueError, match="int16"):
         mortar_amd.stk_dds(to_dev(x, dev), data, t(m["offsets"]), t(m["row_idx"]).int(), t(m["col_idx"]), z32, z16, z32, 96, 128, True)
+    # any block values, as the reference's operator: random bf16 data against the dense float64 product
+    rnd = torch.randn_like(data)
+    yr = mortar_amd.stk_dds(to_dev(x, dev), rnd, t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32, 96, 128, True)
+    dense = O.to_dense(rnd.float().cpu().numpy(), m["row_idx"], m["col_idx"], (128, 96)).astype(np.float64)
+    assert_close_bf16(to_np(yr), (O.bf16_round(x).astype(np.float64) @ dense.T).astype(np.float32), "stk_dds, arbitrary values")
+    from mortar_amd.stk import stk_dds_ternary
+    yt = stk_dds_ternary(to_dev(x, dev), data, t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32, 96, 128, True)
+    assert_close_bf16(to_np(yt), oracle_spmm(x, m), "stk_dds_ternary")
     with pytest.raises(ValueError, match="ternary"):
-        mortar_amd.stk_dds(to_dev(x, dev), torch.randn_like(data), t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32, 96, 128, True)
+        stk_dds_ternary(to_dev(x, dev), rnd, t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32, 96, 128, True)
+
+
+@pytest.mark.parametrize("out_f,in_f,M,density,zipf", [(16 * 8, 16 * 6, 70, 0.5, None), (2048, 768, 64, 0.25, None),
+                                                       (16 * 40, 2048, 333, 0.25, 1.2), (16 * 12, 16 * 352, 200, 0.25, 1.2),
+                                                       (16 * 70, 16 * 400, 37, 0.1, None), (16 * 3, 16 * 3, 1, 1.0, None)])
+def test_dds_values_any_block_values(dev, out_f, in_f, M, density, zipf):
+    """The product over stored bf16 block values (what stk_dds calls) against the dense float64 product of the scattered
+    matrix: one K segment and several (in_features > 2480), ragged rows, odd block counts, M below and above one token
+    tile, both orientations; 1e-2 / bf16 rounding bar as for the ternary kernels."""
+    m = synth.synth_matrix(out_f, in_f, density, seed=out_f + in_f, zipf_s=zipf)
+    nnz = m["col_idx"].size
+    rng = np.random.default_rng(nnz)
+    vals = O.bf16_round((rng.standard_normal((nnz, 16, 16)) * rng.uniform(0.01, 2.0, (nnz, 1, 1))).astype(np.float32))
+    dense = O.to_dense(vals, m["row_idx"], m["col_idx"], (out_f, in_f)).astype(np.float64)
+    from mortar_amd.pack import BcsrTopology
+    T = BcsrTopology(m["offsets"], m["col_idx"], out_f, in_f, dev)
+    assert (T.nseg > 1) == (in_f // 16 > 155)
+    data = torch.from_numpy(vals).to(torch.bfloat16).to(dev)
+    x = synth.synth_x(M, in_f, seed=5)
+    y = ops.dds_values(to_dev(x, dev), data, T)
+    assert_close_bf16(to_np(y), (x.astype(np.float64) @ dense.T).astype(np.float32), "values product", ulps=4)
+    Tt, src = T.transposed()
+    dy = synth.synth_x(M, out_f, seed=6)
+    dx = ops.dds_values(to_dev(dy, dev), data[src].transpose(1, 2).contiguous(), Tt)
+    assert_close_bf16(to_np(dx), (dy.astype(np.float64) @ dense).astype(np.float32), "values product, W^T", ulps=4)
+    z16, z32 = torch.zeros(1, dtype=torch.int16, device=dev), torch.zeros(1, dtype=torch.int32, device=dev)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    y2 = mortar_amd.stk_dds(to_dev(x, dev), data, t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32, in_f, out_f, True)
+    assert torch.equal(y2, y)
+    dx2 = mortar_amd.stk_dds(to_dev(dy, dev), data, t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32, out_f, in_f, False)
+    assert torch.equal(dx2, dx)
+    with pytest.raises(TypeError):
+        ops.dds_values(to_dev(x, dev), data.float(), T)
 
 
 # ---------------------------------------------------------------------------------------------- SwiGLU MLP

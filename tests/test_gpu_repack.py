@@ -316,12 +316,15 @@ def test_qat_pack_follows_writes_through_data(dev):
         assert torch.equal(lin(xt.detach()), y0)
 
 
-def test_stk_dds_fp32_effective_data_and_non_ternary_report(dev):
+def test_stk_dds_fp32_effective_data_and_the_ternary_form(dev):
     """The reference's own caller in fp32: _mortar_effective_data() = d + (scale*q - d).detach() is +-s only to within an
-    fp32 ulp (several distinct magnitudes) and must be accepted; data that is not ternary is reported, by the first
-    call on a topology synchronously and by later calls through the device flag (stk_check waits for it)."""
+    fp32 ulp (several distinct magnitudes).  stk_dds multiplies it as it is (cast to bf16); stk_dds_ternary runs it on the
+    ternary kernels and must accept it; data that is NOT ternary makes stk_dds_ternary's result NaN in the same call and
+    raises -- synchronously in the first call on a topology, through the device flag later (stk_check waits for it) --
+    while stk_dds just multiplies it."""
     import mortar_amd
     from mortar_amd import stk
+    from mortar_amd.stk import stk_dds_ternary
     lin = _qat_layer(16 * 8, 16 * 6, 0.5, 86, dev)
     eff = lin._mortar_effective_data().detach()
     assert eff.dtype == torch.float32
@@ -330,41 +333,47 @@ def test_stk_dds_fp32_effective_data_and_non_ternary_report(dev):
     z32, z16 = torch.zeros(1, dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int16, device=dev)
     args = (lin.mortar_offsets, lin.mortar_row_indices, lin.mortar_column_indices, z32, z16, z32)
     x = synth.synth_x(30, lin.in_features, seed=87)
-    y = mortar_amd.stk_dds(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
-    assert_close_bf16(to_np(y), (O.bf16_round(x).astype(np.float64) @ _effective_dense(lin).T).astype(np.float32), "fp32 effective data")
-    yb = mortar_amd.stk_dds(to_dev(x, dev), eff.to(torch.bfloat16), *args, lin.in_features, lin.out_features, True)
-    assert torch.equal(y, yb)
-    dx0 = mortar_amd.stk_dds(torch.ones(5, lin.out_features, dtype=torch.bfloat16, device=dev), eff, *args,
-                             lin.out_features, lin.in_features, False)          # first call on the W^T pack (waits)
+    want = (O.bf16_round(x).astype(np.float64) @ _effective_dense(lin).T).astype(np.float32)
+    for op in (mortar_amd.stk_dds, stk_dds_ternary):
+        y = op(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
+        assert_close_bf16(to_np(y), want, "fp32 effective data")
+        yb = op(to_dev(x, dev), eff.to(torch.bfloat16), *args, lin.in_features, lin.out_features, True)
+        assert torch.equal(y, yb)
+    ones = torch.ones(5, lin.out_features, dtype=torch.bfloat16, device=dev)
+    dx0 = stk_dds_ternary(ones, eff, *args, lin.out_features, lin.in_features, False)             # first call on the W^T pack (waits)
+    assert_close_bf16(to_np(dx0), to_np(mortar_amd.stk_dds(ones, eff, *args, lin.out_features, lin.in_features, False)), "dX both forms", ulps=4)
     stk.stk_check()                                                   # nothing to report so far
     # same topology, later call, data that is NOT ternary: no wait in the call itself, the flag is raised on the device
     bad = eff.clone(); bad[3, 2, 1] = 0.37 * float(mags[0])
-    ybad = mortar_amd.stk_dds(to_dev(x, dev), bad, *args, lin.in_features, lin.out_features, True)
+    ybad = stk_dds_ternary(to_dev(x, dev), bad, *args, lin.in_features, lin.out_features, True)
     assert bool(torch.isnan(ybad).all())                              # ...and the product of that call is unusable: all NaN
     with pytest.raises(ValueError, match="not ternary"):
         stk.stk_check()
     stk.stk_check()                                                   # reported once, then clean again
-    ybad = mortar_amd.stk_dds(to_dev(x.astype(np.float32), dev).float(), bad, *args, lin.in_features, lin.out_features, True)
+    ybad = stk_dds_ternary(to_dev(x.astype(np.float32), dev).float(), bad, *args, lin.in_features, lin.out_features, True)
     assert ybad.dtype == torch.float32 and bool(torch.isnan(ybad).all())
-    dxbad = mortar_amd.stk_dds(torch.ones(5, lin.out_features, dtype=torch.bfloat16, device=dev), bad, *args,
-                               lin.out_features, lin.in_features, False)         # the dX product through the W^T pack
+    dxbad = stk_dds_ternary(ones, bad, *args, lin.out_features, lin.in_features, False)           # the dX product through the W^T pack
     assert bool(torch.isnan(dxbad).all())
     torch.cuda.synchronize()
     with pytest.raises(ValueError, match="earlier call"):             # the next call finds the flag on the host
-        mortar_amd.stk_dds(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
-    y2 = mortar_amd.stk_dds(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
-    assert torch.equal(y2, y)
+        stk_dds_ternary(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
+    y2 = stk_dds_ternary(to_dev(x, dev), eff, *args, lin.in_features, lin.out_features, True)
+    assert_close_bf16(to_np(y2), want, "after the report")
     with pytest.raises(ValueError, match="not ternary"):              # the W^T pack keeps its own words
         stk.stk_check()
-    dx = mortar_amd.stk_dds(torch.ones(5, lin.out_features, dtype=torch.bfloat16, device=dev), eff, *args,
-                            lin.out_features, lin.in_features, False)
+    dx = stk_dds_ternary(ones, eff, *args, lin.out_features, lin.in_features, False)
     assert torch.equal(dx, dx0)
+    # the general operator multiplies the non-ternary data as the reference does
+    yg = mortar_amd.stk_dds(to_dev(x, dev), bad, *args, lin.in_features, lin.out_features, True)
+    bad_dense = O.to_dense(O.bf16_round(bad.cpu().numpy()), lin.mortar_row_indices.cpu().numpy(), lin.mortar_column_indices.cpu().numpy(),
+                           (lin.out_features, lin.in_features)).astype(np.float64)
+    assert_close_bf16(to_np(yg), (O.bf16_round(x).astype(np.float64) @ bad_dense.T).astype(np.float32), "non-ternary data, general operator")
     # a fresh topology sees the error in its first call
     m = synth.synth_matrix(64, 64, 0.5, seed=88)
     t = lambda a: torch.from_numpy(a).to(dev)
     with pytest.raises(ValueError, match="not ternary"):
-        mortar_amd.stk_dds(torch.zeros(4, 64, dtype=torch.bfloat16, device=dev), torch.randn(m["col_idx"].size, 16, 16, device=dev),
-                           t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32, 64, 64, True)
+        stk_dds_ternary(torch.zeros(4, 64, dtype=torch.bfloat16, device=dev), torch.randn(m["col_idx"].size, 16, 16, device=dev),
+                        t(m["offsets"]), t(m["row_idx"]), t(m["col_idx"]), z32, z16, z32, 64, 64, True)
 
 
 def test_qat_mlp_trains_layer_by_layer(dev):
