@@ -135,6 +135,8 @@ def main() -> None:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="prefill only (for profiling one kernel)")
     ap.add_argument("--cpu-tokens", type=int, default=TOKENS)
+    ap.add_argument("--precondition-ms", type=float, default=300.0,
+                    help="untimed run of the step before the warm-up steps, so that the clocks have settled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the path shards by tokens with replicated weights; "
@@ -157,6 +159,14 @@ def main() -> None:
         # the MLP forward as the module runs it: gate_up + SwiGLU, then down, hidden activations in the library's layout
         ops.mlp(x, Wgu, Wdn, out=y, hidden=ws)
 
+    # Preconditioning (untimed, before the W warm-up steps): the first ~0.1 s of work on an idle GPU runs 15-25 % slower
+    # than the steady state (measured: 130 against 107 us per step inside one process) while the clocks settle, so a timed
+    # region that starts 5 steps after idle measures the ramp, not the kernels.  The same step runs for about 0.3 s first.
+    t_pre = time.perf_counter()
+    while time.perf_counter() - t_pre < args.precondition_ms * 1e-3:
+        for _ in range(50):
+            step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -187,7 +197,7 @@ def main() -> None:
         "metric": "sparse-MLP prefill tokens/s @ d_model=2048, d_ff=5632, 25% block density, 4096 tokens",
         "value": TOKENS / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic",
+        "data": "synthetic", "precondition_ms": args.precondition_ms,
         "config": {"workload": "carved SwiGLU MLP prefill, d_model 2048 / d_ff 5632, 16x16 BCSR 25 % uniform, "
                                "ternary + per-block scale, 4096 tokens bf16 (benchmark configs 2/3 shapes)",
                    "tokens": TOKENS, "nnz_blocks": [Wgu.nnz, Wdn.nnz]},
