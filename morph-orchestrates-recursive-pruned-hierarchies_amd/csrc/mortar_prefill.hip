@@ -58,11 +58,11 @@ int resident_mt(int Cb) {
 // prefill tiles: 16 wavefronts (4 per SIMD) for both tiles (the 64-token tile with 8 wavefronts was measured 18 % slower
 // on the base-width gate_up, although the 16-wave gate_up form spills six registers; a 96-token tile of a narrow
 // matrix leaves only two waves per SIMD and is slower still)
-template <int NACC, bool ROUTED, int CODE>
+template <int NACC, bool ROUTED, int CODE, bool TL = false>
 int launch_resident_any(SpmmParams &p, hipStream_t st) {
     switch (resident_mt(p.Cb)) {
-        case 64: return mortar_launch_resident<64, NACC, ROUTED, 16, false, CODE>(p, nullptr, 1, st);
-        default: return mortar_launch_resident<32, NACC, ROUTED, 16, false, CODE>(p, nullptr, 1, st);
+        case 64: return mortar_launch_resident<64, NACC, ROUTED, 16, false, CODE, TL>(p, nullptr, 1, st);
+        default: return mortar_launch_resident<32, NACC, ROUTED, 16, false, CODE, TL>(p, nullptr, 1, st);
     }
 }
 
@@ -82,6 +82,24 @@ int segmented_upw(const SpmmParams &p) {
         if (upw == SEG_UPW || cost < best_cost) { best = upw; best_cost = cost; }
     }
     return best;
+}
+
+// Plain product of a `down` whose input is stored in tile order (mortar_mlp_bf16): the instantiations that copy their
+// token tiles straight into LDS.  The caller has checked that the matrix runs 32-token tiles.
+template <int CODE>
+int dispatch_gateup_tiled(SpmmParams &p, hipStream_t st) {     // gate_up + SwiGLU storing tile-ordered hidden activations
+    if (p.nseg == 1) return launch_resident_any<2, false, CODE, true>(p, st);
+    return mortar_launch_segmented<32, 2, false, SEG_WAVES, 2, false, CODE, true>(p, nullptr, 1, st);
+}
+
+template <int CODE>
+int dispatch_prefill_tiled(SpmmParams &p, hipStream_t st) {
+    if (p.nseg == 1) return mortar_launch_resident<32, 1, false, 16, false, CODE, true>(p, nullptr, 1, st);
+    switch (segmented_upw(p)) {
+        case 1: return mortar_launch_segmented<32, 1, false, SEG_WAVES, 1, false, CODE, true>(p, nullptr, 1, st);
+        case 2: return mortar_launch_segmented<32, 1, false, SEG_WAVES, 2, false, CODE, true>(p, nullptr, 1, st);
+    }
+    return mortar_launch_segmented<32, 1, false, SEG_WAVES, SEG_UPW, false, CODE, true>(p, nullptr, 1, st);
 }
 
 template <int CODE>
@@ -337,7 +355,7 @@ extern "C" int mortar_mlp_bf16(const mortar_bcsr_t *Wgu, const int32_t *sched_gu
         }
         p.y_tiled = 1;
         p.codes_o = reinterpret_cast<const u32x4_t *>(Wgu->codes4_o);
-        rc = p.uscale != 0.f ? dispatch_prefill<CODE_4BIT | CODE_UNIFORM>(1, p, st) : dispatch_prefill<CODE_4BIT>(1, p, st);
+        rc = p.uscale != 0.f ? dispatch_gateup_tiled<CODE_4BIT | CODE_UNIFORM>(p, st) : dispatch_gateup_tiled<CODE_4BIT>(p, st);
         if (rc) return rc;
     }
     if (phase != 1) {
@@ -348,7 +366,7 @@ extern "C" int mortar_mlp_bf16(const mortar_bcsr_t *Wgu, const int32_t *sched_gu
         p.n_units = Wdn->Rb;
         p.x_tiled = 1;
         p.codes_o = reinterpret_cast<const u32x4_t *>(Wdn->codes4_o);
-        rc = p.uscale != 0.f ? dispatch_prefill<CODE_4BIT | CODE_UNIFORM>(0, p, st) : dispatch_prefill<CODE_4BIT>(0, p, st);
+        rc = p.uscale != 0.f ? dispatch_prefill_tiled<CODE_4BIT | CODE_UNIFORM>(p, st) : dispatch_prefill_tiled<CODE_4BIT>(p, st);
         if (rc) return rc;
     }
     return MORTAR_OK;

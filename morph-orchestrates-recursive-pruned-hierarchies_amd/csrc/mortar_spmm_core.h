@@ -304,15 +304,17 @@ __device__ __forceinline__ void mortar_stage_tiled32(const SpmmView &p, uint4 *l
     __builtin_amdgcn_s_waitcnt(0);
 }
 
-template <int MT, int WAVES, bool MASKED>
+// XT: the activations are stored in tile order (SpmmParams::x_tiled, set by the host for exactly these instantiations).
+// A compile-time choice: the register-staged path holds up to eight 16-byte loads per lane, which the kernels that
+// copy straight into LDS should not pay for in their register budget.
+template <int MT, int WAVES, bool MASKED, bool XT = false>
 __device__ __forceinline__ void mortar_stage_tile(const SpmmView &p, uint4 *lx, int m0, int c0, int ncb, int tid) {
-    if constexpr (MT == 32 && !MASKED) {
-        if (p.x_tiled) {
-            mortar_stage_tiled32<WAVES>(p, lx, m0 / 32, c0, ncb, tid);
-            return;
-        }
+    if constexpr (XT) {
+        static_assert(MT == 32 && !MASKED, "tile-ordered activations are staged by the 32-token plain kernels");
+        mortar_stage_tiled32<WAVES>(p, lx, m0 / 32, c0, ncb, tid);
+    } else {
+        mortar_stage_quads<MT, WAVES, MASKED, false>(p, reinterpret_cast<unsigned char *>(lx), m0, c0, ncb, tid, nullptr);
     }
-    mortar_stage_quads<MT, WAVES, MASKED, false>(p, reinterpret_cast<unsigned char *>(lx), m0, c0, ncb, tid, nullptr);
 }
 
 // The same staging with the rows RMS-normalised on the way (gate_up with the block's norm folded in).  First every
@@ -390,7 +392,7 @@ __device__ __forceinline__ void mortar_hc_post(const SpmmView &p, int tok, int f
 
 // Epilogue of one row unit for the 16 tokens of sub-tile `ms`: the lane holds D[4g+v][token].
 // `gv` is the router gate of the lane's four features for this token (read when has_gates).
-template <int NACC, int CODE = 0, bool HC = false>
+template <int NACC, int CODE = 0, bool HC = false, bool YT = false>
 __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, int tok, int g, bool has_gates, float gv,
                                                   f32x4_t a0, f32x4_t a1) {
     if (CODE & CODE_UNIFORM) {      // the blocks were multiplied as +-2: p.uscale is half the matrix's scale
@@ -416,7 +418,7 @@ __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, i
         }
     } else {
         pk = swiglu_pack4(a0, a1, has_gates, gv);
-        if (p.y_tiled) {       // (host: M * features < 2^31)
+        if constexpr (YT) {    // tile-ordered hidden activations (SpmmParams::y_tiled; host: M * features < 2^31)
             const uint32_t e = ((uint32_t)(tok >> 5) * (uint32_t)p.n_units + (uint32_t)unit) * 512u + (uint32_t)(tok & 31) * 16u + 4u * g;
             *(MORTAR_GLOBAL u32x2_t *)(p.y + e) = pk;
             return;
@@ -428,7 +430,7 @@ __device__ __forceinline__ void mortar_store_unit(const SpmmView &p, int unit, i
 // Epilogue of one row unit for all sub-tiles of the token tile.  tl[ms] is the tile row of the lane's token in
 // sub-tile ms, `cnt` the number of live rows per 16-row sub-tile set (MT, or the routed list length).  The cluster of
 // the lane's features is found once per unit and the gates of all sub-tiles are requested before the first SwiGLU.
-template <int MSUB, int NACC, int CODE, bool HC>
+template <int MSUB, int NACC, int CODE, bool HC, bool YT = false>
 __device__ __forceinline__ void mortar_store_tile(const SpmmView &p, int unit, int m0, const uint32_t (&tl)[MSUB], int cnt,
                                                   int n, int g, bool has_gates, const f32x4_t (&a0)[MSUB],
                                                   const f32x4_t (&a1)[MSUB]) {
@@ -447,7 +449,7 @@ __device__ __forceinline__ void mortar_store_tile(const SpmmView &p, int unit, i
     }
 #pragma unroll
     for (int ms = 0; ms < MSUB; ++ms)
-        if (ok[ms]) mortar_store_unit<NACC, CODE, HC>(p, unit, m0 + (int)tl[ms], g, has_gates, gv[ms], a0[ms], a1[ms]);
+        if (ok[ms]) mortar_store_unit<NACC, CODE, HC, YT>(p, unit, m0 + (int)tl[ms], g, has_gates, gv[ms], a0[ms], a1[ms]);
 }
 
 // Part descriptor of schedule position `pos`, segment `sg`, row `a` of the unit: {g0, g1, nb, unit}.
@@ -471,9 +473,12 @@ __device__ __forceinline__ u32x4_t mortar_part_desc(const SpmmView &p, int pos, 
 // No barrier after the first one.  A wave's work is a chain of row parts (unit, segment, row of the unit) whose
 // descriptors come from the schedule table one part ahead; latency is hidden by the waves that share a SIMD.
 // ---------------------------------------------------------------------------------------------------------
-template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE, int CODE>
+// TL: the hidden activations of the two-launch MLP are in tile order: a plain product (NACC = 1) stages its input from
+// them (SpmmParams::x_tiled), a gate_up (NACC = 2) stores its result so (SpmmParams::y_tiled).
+template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE, int CODE, bool TL = false>
 __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmParams p0, const SpmmParams *table) {
     constexpr int MSUB = (MT + 15) / 16;
+    constexpr bool XT = TL && NACC == 1, YT = TL && NACC == 2;
     const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint4 *lx = reinterpret_cast<uint4 *>(smem);
@@ -503,7 +508,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
     u32x4_t d0 = mortar_part_desc<NACC>(p, pos, 0, 0);
 
     if (NACC == 2 && p.norm) mortar_stage_tile_norm<MT, WAVES>(p, lx, m0, p.Cb, tid, reinterpret_cast<float *>(next_unit + 4));      // gate_up may carry the norm
-    else mortar_stage_tile<MT, WAVES, false>(p, lx, m0, 0, p.Cb, tid);
+    else mortar_stage_tile<MT, WAVES, false, XT>(p, lx, m0, 0, p.Cb, tid);
     __syncthreads();
 
     while (pos < u_end) {
@@ -560,8 +565,8 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
         pos = npos;
         if (skip) continue;
 
-        mortar_store_tile<MSUB, NACC, CODE, (MT <= 16 && NACC == 1 && !TABLE)>(p, unit, m0, tk, ROUTED ? cnt : MT, n, g, has_gates,
-                                                                               acc[0], acc[NACC - 1]);
+        mortar_store_tile<MSUB, NACC, CODE, (MT <= 16 && NACC == 1 && !TABLE), YT>(p, unit, m0, tk, ROUTED ? cnt : MT, n, g, has_gates,
+                                                                                   acc[0], acc[NACC - 1]);
     }
 }
 
@@ -572,9 +577,10 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_resident_kernel(const SpmmP
 // The descriptors of the next segment are fetched before the barrier pair, so their latency hides behind the
 // staging.
 // ---------------------------------------------------------------------------------------------------------
-template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE, int CODE>
+template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE, int CODE, bool TL = false>
 __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const SpmmParams p0, const SpmmParams *table) {
     constexpr int MSUB = (MT + 15) / 16, NP = UPW * NACC;
+    constexpr bool XT = TL && NACC == 1, YT = TL && NACC == 2;
     const SpmmView p = mortar_view(TABLE ? mortar_table_entry(table, blockIdx.y) : p0);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint4 *lx = reinterpret_cast<uint4 *>(smem);
@@ -638,7 +644,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
         MortarBatch bq;
         if (BATCH_AHEAD) first_batch(bq, 0);
         if (sg > 0) __syncthreads();
-        mortar_stage_tile<MT, WAVES, MASKED>(p, lx, m0, c0, ncb, tid);
+        mortar_stage_tile<MT, WAVES, MASKED, XT>(p, lx, m0, c0, ncb, tid);
         __syncthreads();
         if (!BATCH_AHEAD) {
 #pragma unroll
@@ -675,8 +681,8 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
 #pragma unroll
     for (int k = 0; k < UPW; ++k) {
         if (units[k] < 0) continue;
-        mortar_store_tile<MSUB, NACC, CODE, (MT <= 16 && NACC == 1 && !TABLE)>(p, units[k], m0, tl, MT, n, g, has_gates, acc[k][0],
-                                                                               acc[k][NACC - 1]);
+        mortar_store_tile<MSUB, NACC, CODE, (MT <= 16 && NACC == 1 && !TABLE), YT>(p, units[k], m0, tl, MT, n, g, has_gates, acc[k][0],
+                                                                                   acc[k][NACC - 1]);
     }
 }
 
@@ -849,13 +855,14 @@ inline int64_t mortar_resident_shape(SpmmParams &p, int layers) {
     return mortar_grid_width(p, layers);
 }
 
-template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE = false, int CODE = 0>
+template <int MT, int NACC, bool ROUTED, int WAVES, bool TABLE = false, int CODE = 0, bool TL = false>
 int mortar_launch_resident(SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     if (TABLE != (table != nullptr)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: parameter table mismatch");
     const int smem = tile_bytes(MT, p.Cb) + LDS_EXTRA;
     if (smem > LDS_BUDGET + LDS_PAD * 16 + LDS_EXTRA) return mortar_fail(MORTAR_ERR_LIMIT, "resident tile of %d bytes does not fit LDS", smem);
     static bool attr_done = false;
-    auto kern = mortar_resident_kernel<MT, NACC, ROUTED, WAVES, TABLE, CODE>;
+    if (TL != ((NACC == 1 ? p.x_tiled : p.y_tiled) != 0)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: activation layout mismatch");
+    auto kern = mortar_resident_kernel<MT, NACC, ROUTED, WAVES, TABLE, CODE, TL>;
     int rc = mortar_allow_big_lds(kern, attr_done);
     if (rc) return rc;
     const int64_t grid = mortar_resident_shape<MT, WAVES>(p, layers);
@@ -873,13 +880,14 @@ inline int64_t mortar_segmented_shape(SpmmParams &p, int layers) {
     return mortar_grid_width(p, layers);
 }
 
-template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE = false, int CODE = 0>
+template <int MT, int NACC, bool MASKED, int WAVES, int UPW, bool TABLE = false, int CODE = 0, bool TL = false>
 int mortar_launch_segmented(SpmmParams &p, const SpmmParams *table, int layers, hipStream_t st) {
     if (TABLE != (table != nullptr)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: parameter table mismatch");
     const int smem = tile_bytes(MT, p.seg_cb);
     if (smem > LDS_BUDGET + LDS_PAD * 16) return mortar_fail(MORTAR_ERR_LIMIT, "segment tile of %d bytes does not fit LDS", smem);
     static bool attr_done = false;
-    auto kern = mortar_segmented_kernel<MT, NACC, MASKED, WAVES, UPW, TABLE, CODE>;
+    if (TL != ((NACC == 1 ? p.x_tiled : p.y_tiled) != 0)) return mortar_fail(MORTAR_ERR_ARG, "spmm launch: activation layout mismatch");
+    auto kern = mortar_segmented_kernel<MT, NACC, MASKED, WAVES, UPW, TABLE, CODE, TL>;
     int rc = mortar_allow_big_lds(kern, attr_done);
     if (rc) return rc;
     const int64_t grid = mortar_segmented_shape<MT, WAVES, UPW>(p, layers);
