@@ -55,15 +55,31 @@ __device__ __forceinline__ void remoe_gates_wave(const float *lp, int n, int k, 
     float kth = 0.f;
     const bool thresh = k < n;
     if (thresh) {
+        // [prefix, prefix + 2^(bit+1)) is the bucket that holds the k-th largest key: c_lo keys are >= its lower end, c_hi keys
+        // >= its upper end.  Once the bucket holds ONE key that key is the answer and the remaining bits need no counting
+        // (distinct logits get there after about log2(n) + the exponent bits they share; exact ties walk all 32 bits).
         uint32_t prefix = 0;
-        for (int bit = 31; bit >= 0; --bit) {
+        int c_lo = 64 * MAXPL, c_hi = 0, bit = 31;
+        for (; bit >= 0 && c_lo - c_hi > 1; --bit) {
             const uint32_t cand = prefix | (1u << bit);
             // counted on the vector ALU: a ballot + scalar popcount per key would queue on the one scalar ALU that the
             // sixteen waves of a CU share
             uint32_t own = 0;
 #pragma unroll
             for (int i = 0; i < MAXPL; ++i) own += key[i] >= cand ? 1u : 0u;             // padding keys are 0 < cand
-            if (wave_count_total(own) >= k) prefix = cand;
+            const int c = wave_count_total(own);
+            if (c >= k) { prefix = cand; c_lo = c; } else { c_hi = c; }
+        }
+        if (bit >= 0) {                       // left early: the bucket's one key (bits 0..bit of it were never looked at)
+            uint32_t m = 0;
+#pragma unroll
+            for (int i = 0; i < MAXPL; ++i) m = (key[i] >> (bit + 1)) == (prefix >> (bit + 1)) && key[i] > m ? key[i] : m;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const uint32_t t = (uint32_t)__shfl_xor((int)m, o, 64);
+                m = t > m ? t : m;
+            }
+            prefix = m;
         }
         kth = key_to_float(prefix);
     }
