@@ -25,9 +25,9 @@ PEAK_BF16_TFLOPS, PEAK_HBM_GBS = 2500.0, 8000.0
 # HBM-side bytes per launch (read + written) measured with `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` on this
 # workload and calibrated on a plain copy; the runs and factors are in profiles/bench_prefill_step_hbm_traffic_pmc.md
 # and profiles/bench_all_legs_hbm_traffic_pmc.md.  Not measured live: counters need the profiler.
-TRAFFIC_GATE_UP_BYTES = 41.60e6 + 51.03e6
-TRAFFIC_DOWN_BYTES = 60.43e6 + 17.64e6
-TRAFFIC_DECODE_STACK_BYTES = (263.04e6 + 4.54e6) + (169.04e6 + 1.96e6)   # gate_up + down launches, 160 layers, b = 1
+TRAFFIC_GATE_UP_BYTES = 41.57e6 + 46.14e6
+TRAFFIC_DOWN_BYTES = 60.41e6 + 17.68e6
+TRAFFIC_DECODE_STACK_BYTES = (263.02e6 + 4.54e6) + (169.01e6 + 1.96e6)   # gate_up + down launches, 160 layers, b = 1
 TRAFFIC_SOURCE = ("constant from profiles/bench_prefill_step_hbm_traffic_pmc.md and profiles/bench_all_legs_hbm_traffic_pmc.md "
                   "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command); not measured in this run")
 

@@ -226,3 +226,66 @@ def test_random_wide_k_shapes(dev, seed):
                 hs = [torch.full((M, units * 16), float("nan"), dtype=torch.bfloat16, device=dev) for _ in range(2)]
                 ops.LayerStack([W, W], [xd, xd], hs, swiglu=True).run()
                 assert_close_bf16(to_np(hs[1]), ref["h"], what + " stack h", ulps=8)
+
+
+@pytest.mark.parametrize("seed", [601, 602])
+def test_random_one_call_mlp_and_values_product(dev, seed):
+    """The MLP as one call (tile-ordered hidden activations from 513 rows, row-major below) against the two separate calls
+    (bit-equal) and the oracle on sampled rows, with gates and the fused RMSNorm drawn at random; and the product over
+    stored bf16 block values (any values, ragged and empty rows, one or several K segments) against a dense float64
+    product of the scattered matrix."""
+    from mortar_amd.pack import BcsrTopology
+    rng = np.random.default_rng(seed)
+    for it in range(14):
+        dm_b = int(rng.choice([2, 5, 16, 30, 48, 78, 128]))
+        dff_b = int(rng.choice([4, 7, 22, 40, 130, 352]))
+        cfg = dict(it=it, d_model=dm_b * 16, d_ff=dff_b * 16, dens=float(rng.choice([0.1, 0.25, 0.5])),
+                   zipf=None if rng.random() < 0.5 else 1.2, M=int(rng.choice([1, 33, 200, 512, 513, 544, 777, 1025, 1500])),
+                   seg=None if rng.random() < 0.6 else int(rng.integers(8, 80)), stream4=bool(rng.random() < 0.8),
+                   gated=bool(rng.random() < 0.5), norm=bool(rng.random() < 0.5), seed=int(rng.integers(1, 10000)))
+        what = f"seed {seed} case {cfg}"
+        spec = synth.synth_mlp(cfg["d_model"], cfg["d_ff"], cfg["dens"], seed=cfg["seed"], zipf_s=cfg["zipf"])
+        M = cfg["M"]
+        x = synth.synth_x(M, cfg["d_model"], cfg["seed"] + 1)
+        xd = to_dev(x, dev)
+        Wgu = _pack(spec["gate_up"], dev, seg_cb=cfg["seg"], prefill_stream=cfg["stream4"])
+        Wdn = _pack(spec["down"], dev, seg_cb=cfg["seg"], prefill_stream=cfg["stream4"])
+        gates = g_ref = None
+        if cfg["gated"]:
+            logits = synth.synth_logits(M, dff_b, cfg["seed"] + 2)
+            g_ref, _ = O.remoe_gates(logits, max(1, dff_b // 3))
+            gates, _ = ops.remoe_gates(torch.from_numpy(logits).to(dev), max(1, dff_b // 3))
+        nm = None
+        if cfg["norm"] and ops.norm_fusable(Wgu):
+            nw = O.bf16_round(1 + 0.1 * rng.standard_normal(cfg["d_model"]).astype(np.float32))
+            nm = (torch.from_numpy(nw).to(torch.bfloat16).to(dev), 1e-6)
+        want = ops.spmm(ops.gateup_swiglu(xd, Wgu, gates=gates, norm=nm), Wdn)
+        got = ops.mlp(xd, Wgu, Wdn, gates=gates, norm=nm)
+        assert torch.equal(got, want), what + " one call vs two"
+        rows = rng.choice(M, min(M, 12), replace=False)
+        xin = x[rows] if nm is None else O.rmsnorm(x[rows], nw, 1e-6)
+        ref = O.swiglu_mlp(xin, spec["gate_up"], spec["down"], gates=None if g_ref is None else g_ref[rows])
+        assert_close_bf16(to_np(got)[rows], ref["y"], what + " one call vs oracle", ulps=16)
+
+        # any block values on the same topologies (rows emptied at random)
+        for name in ("gate_up", "down"):
+            m = spec[name]
+            off = np.asarray(m["offsets"]).astype(np.int64)
+            col = np.asarray(m["col_idx"]).astype(np.int64)
+            keep = np.ones(off[-1], dtype=bool)
+            for r in rng.choice(off.size - 1, max(1, (off.size - 1) // 7), replace=False):
+                keep[off[r]:off[r + 1]] = False
+            nb = np.array([keep[off[r]:off[r + 1]].sum() for r in range(off.size - 1)])
+            off2 = np.concatenate([[0], np.cumsum(nb)]).astype(np.int32)
+            col2 = col[keep].astype(np.int16)
+            if off2[-1] == 0:
+                continue
+            vals = O.bf16_round(rng.standard_normal((int(off2[-1]), 16, 16)).astype(np.float32))
+            T = BcsrTopology(off2, col2, m["shape"][0], m["shape"][1], dev)
+            dense = np.zeros(m["shape"], dtype=np.float64)
+            for r in range(off2.size - 1):
+                for j in range(off2[r], off2[r + 1]):
+                    dense[r * 16:(r + 1) * 16, col2[j] * 16:(col2[j] + 1) * 16] = vals[j]
+            xv = synth.synth_x(M, m["shape"][1], cfg["seed"] + 3)
+            y = ops.dds_values(to_dev(xv, dev), torch.from_numpy(vals).to(torch.bfloat16).to(dev), T)
+            assert_close_bf16(to_np(y), (O.bf16_round(xv).astype(np.float64) @ dense.T).astype(np.float32), what + f" values {name}", ulps=8)
