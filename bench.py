@@ -62,9 +62,6 @@ def _dense_twin(spec, tokens: int, dtype, budget_s: float) -> dict:
     """The reference's CPU-expressible form of the carved MLP (scatter the kept blocks into dense matrices, as
     morph/sparse/stk/ops/matrix_ops.py:37-49 / morph/inference/engine.py:74-84 do, then torch.nn.functional.linear and
     silu * up) timed through PyTorch on the host cores."""
-    global SETTLE_MS
-    SETTLE_MS = min(100.0, args.precondition_ms)
-
     import numpy as np
     import torch
     import torch.nn.functional as F
@@ -152,6 +149,8 @@ def main() -> None:
     ap.add_argument("--precondition-ms", type=float, default=300.0,
                     help="untimed run of the step before the warm-up steps, so that the clocks have settled")
     args = ap.parse_args()
+    global SETTLE_MS
+    SETTLE_MS = min(100.0, args.precondition_ms)
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the path shards by tokens with replicated weights; "
                  "no multi-GPU code is part of it). Use --gpus 1.")
