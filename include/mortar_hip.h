@@ -263,6 +263,20 @@ int mortar_router_bf16(const void *x, int32_t x_is_f32, int64_t B, int32_t d, in
                        const float *kb, int32_t nsk, const float *bias, int32_t n, int32_t k, float *qv,
                        float *logits_out, float *gates, uint8_t *active, void *stream);
 
+/* The router behind a library GEMM, for prefill-sized calls: TileRouter.forward steps 2-8 (morph/model/routing.py:188-284)
+ * on the projected query qv = x Wq^T (fp32 [N, d], row stride ldq; the dense projection of step 1, routing.py:181-186,
+ * is a plain GEMM and stays with the caller's BLAS).  q = LayerNorm(qv + iter_vec), sub-key scores, product-key logits
+ * (direct, wrapped or ranked exactly as in mortar_router_bf16), gating tail as mortar_remoe_gates: one launch instead
+ * of the reference's layer_norm, two matmuls, broadcast add, topk, bias add, topk, relu, sum, divide.
+ * iter_vec fp32 [d] or NULL; ln_w, ln_b fp32 [d]; ka, kb fp32 [nsk, d/2]; bias fp32 [n]; all 16-byte aligned.
+ * logits_out fp32 [N, n] or NULL; gates fp32 [N, n]; active uint8 [N, n] or NULL.  d a multiple of 8 up to 8192,
+ * n <= 1024; the ranked branch (nsk^2 > n) takes up to 1024 product keys (sorted in a wavefront's registers).  Sums are ordered differently from the library routines, so gates agree with the eager path
+ * to fp32 rounding (the active set exactly, away from logits within rounding of the threshold). */
+int mortar_router_tail_f32(const float *qv, int64_t N, int32_t d, int64_t ldq, const float *iter_vec, const float *ln_w,
+                           const float *ln_b, float ln_eps, const float *ka, const float *kb, int32_t nsk,
+                           const float *bias, int32_t n, int32_t k, float *logits_out, float *gates, uint8_t *active,
+                           void *stream);
+
 /* ---- decode (M <= 64) ------------------------------------------------------------------------ */
 
 /* mortar_spmm_bf16 / mortar_gateup_swiglu_bf16 / mortar_spmm_bf16_masked serve decode batches directly: for

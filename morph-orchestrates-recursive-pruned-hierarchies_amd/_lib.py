@@ -65,6 +65,8 @@ _SIGS = {
     "mortar_remoe_route": (C.c_int, [c_vp, c_i64, c_i32, c_i32, c_vp, c_vp, c_vp]),
     "mortar_router_bf16": (C.c_int, [c_vp, c_i32, c_i64, c_i32, c_i64, c_vp, c_vp, c_vp, c_vp, c_f32, c_vp, c_vp, c_i32,
                                      c_vp, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp]),
+    "mortar_router_tail_f32": (C.c_int, [c_vp, c_i64, c_i32, c_i64, c_vp, c_vp, c_vp, c_f32, c_vp, c_vp, c_i32, c_vp, c_i32,
+                                         c_i32, c_vp, c_vp, c_vp, c_vp]),
     "mortar_route_flags": (C.c_int, [c_vp, c_i64, c_i32, c_i64, c_i32, c_vp, c_i64, c_vp, c_i64, c_vp]),
     "mortar_stack_table_bytes": (c_i64, [c_i32]),
     "mortar_stack_prepare": (C.c_int, [c_i32, c_i32, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),

@@ -27,6 +27,23 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// Sum over the wavefront with DPP adds only (no LDS crossbar): quads, half rows, rows, then the row broadcasts; the total
+// arrives in the last row and is read from lane 63.  Adds in another order than wave_sum, so not for results that have
+// to match a kernel built on wave_sum bit for bit.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f32(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += dpp_f32<0xB1, 0xf>(v);     // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E, 0xf>(v);     // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141, 0xf>(v);    // row_half_mirror
+    v += dpp_f32<0x140, 0xf>(v);    // row_mirror
+    v += dpp_f32<0x142, 0xa>(v);    // row_bcast:15 into rows 1 and 3
+    v += dpp_f32<0x143, 0xc>(v);    // row_bcast:31 into rows 2 and 3
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
 // Sum of a per-lane count over the wavefront with DPP adds only (quads, half rows, rows, then the row broadcasts): the
 // total arrives in the lanes of the last row and is read from lane 63.
 __device__ __forceinline__ int wave_count_total(uint32_t v) {
@@ -314,6 +331,238 @@ __global__ void __launch_bounds__(256) router_tail_kernel(const float *qv, int d
         remoe_gates_wave<MAXPL>(lg, n, k, gates + (int64_t)b * n, active ? active + (int64_t)b * n : nullptr, lane);
 }
 
+// ---- router tail for prefill-sized calls (TileRouter.forward steps 2-8 behind a library GEMM for the projection) ----
+
+// Descending bitonic sort of 64 * KPL keys held KPL per lane (element lane * KPL + r in register r): steps between
+// elements of one lane are register compare-exchanges, steps between lanes one shuffle per register.  No LDS, no barrier.
+template <int KPL>
+__device__ __forceinline__ void wave_sort_desc(uint32_t (&key)[KPL], int lane) {
+    for (int k2 = 2; k2 <= 64 * KPL; k2 <<= 1) {
+        const bool lane_desc = ((lane * KPL) & k2) == 0;       // direction of this lane's elements once k2 >= KPL
+        for (int lj = k2 / (2 * KPL); lj >= 1; lj >>= 1) {       // partners in other lanes (distance j = lj * KPL)
+            const bool keep_max = ((lane & lj) == 0) == lane_desc;
+#pragma unroll
+            for (int r = 0; r < KPL; ++r) {
+                const uint32_t a = key[r], o = (uint32_t)__shfl_xor((int)a, lj, 64);
+                key[r] = keep_max ? (a > o ? a : o) : (a > o ? o : a);
+            }
+        }
+#pragma unroll
+        for (int j = KPL / 2; j > 0; j >>= 1) {                  // partners in this lane's registers (distance j < k2)
+            if (j < k2) {
+#pragma unroll
+                for (int r = 0; r < KPL; ++r) {
+                    if ((r & j) == 0) {
+                        const bool desc = k2 < KPL ? (r & k2) == 0 : lane_desc;
+                        const uint32_t a = key[r], c = key[r | j];
+                        const uint32_t hi = a > c ? a : c, lo = a > c ? c : a;
+                        key[r] = desc ? hi : lo;
+                        key[r | j] = desc ? lo : hi;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// The n largest of the P = nsk * nsk product scores of one token in descending order (+ bias) -> lgt[0 .. n), on one wave.
+template <int KPL>
+__device__ __forceinline__ void ranked_logits(const float *sct, int nsk, int P, const float *bias, int n, uint32_t *sk,
+                                              float *lgt, float *logits_row, int lane) {
+    uint32_t key[KPL];
+#pragma unroll
+    for (int r = 0; r < KPL; ++r) {
+        const int i = lane * KPL + r;
+        uint32_t kk = 0u;                                    // padding: the smallest key
+        if (i < P) {
+            const uint32_t u = __float_as_uint(sct[i / nsk] + sct[nsk + i % nsk]);
+            kk = (u & 0x80000000u) ? ~u : (u | 0x80000000u);   // NaN ranks above +inf, as torch.topk has it
+        }
+        key[r] = kk;
+    }
+    wave_sort_desc<KPL>(key, lane);
+#pragma unroll
+    for (int r = 0; r < KPL; ++r) {
+        const int g = lane * KPL + r;
+        if (g < n) {
+            const float l = __uint_as_float((key[r] & 0x80000000u) ? (key[r] & 0x7fffffffu) : ~key[r]) + bias[g];
+            lgt[g] = l;
+            if (logits_row) logits_row[g] = l;
+        }
+    }
+    (void)sk;
+}
+
+// A workgroup of four waves takes groups of up to TT = 4 tokens (a loop over its share of the groups), so the sub-key
+// rows are read from L2 once per group instead of once per token.
+//   1. LayerNorm by the whole workgroup: every thread holds its float4 pieces of all rows of the group, the iteration
+//      vector and the LayerNorm parameters from ONE round of loads; the sums meet through LDS; normalised rows -> LDS.
+//   2. the 2 * nsk sub-key dot products, one key row per wave at a time against all tokens of the group; the next row's
+//      piece is requested before the current one is multiplied.
+//   3. per token (one wave each): product-key logits (+ bias) -> LDS, ranked first when nsk^2 > n (a bitonic network
+//      in the wave's registers), then the gating tail.
+// Same arithmetic as router_tail_kernel; the sums are ordered differently.  A group is a chain of latencies (about 3 us of
+// loads, 2 us of LayerNorm, 1.3 us per key row and wave, 2-10 us of logits and gating), so throughput comes from the
+// groups in flight: two workgroups per CU at this register count.
+constexpr int TAIL_TT = 4;
+
+template <int MAXPL, int J>      // J: float4 pieces of a row per thread (d <= 1024 * J); tokens per group tt = min(4, 8 / J)
+__global__ void __launch_bounds__(256, 2) router_tail_group_kernel(const float *qv, int64_t N, int d, int64_t ldq, const float *iter_vec,
+                                                                 const float *ln_w, const float *ln_b, float ln_eps,
+                                                                 const float *ka, const float *kb, int nsk, const float *bias,
+                                                                 int n, int k, int tt, float *logits_out, float *gates,
+                                                                 uint8_t *active) {
+    extern __shared__ __attribute__((aligned(16))) float sm[];       // qn[tt][d] | sc[tt][2 nsk] | lg[tt][n] | red[16]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int d2 = d / 2, d4 = d / 4, n4 = d2 / 4;
+    const int P = nsk * nsk;
+    float *qn = sm, *sc = qn + (size_t)tt * d, *lg = sc + tt * 2 * nsk, *red = lg + (size_t)tt * n;
+    const float4 *iv4 = reinterpret_cast<const float4 *>(iter_vec);
+    const float4 *lw4 = reinterpret_cast<const float4 *>(ln_w), *lb4 = reinterpret_cast<const float4 *>(ln_b);
+    const float4 zero4 = float4{0.f, 0.f, 0.f, 0.f};
+    for (int64_t g0 = (int64_t)blockIdx.x * tt; g0 < N; g0 += (int64_t)gridDim.x * tt) {
+        const int nt = N - g0 < tt ? (int)(N - g0) : tt;
+        {
+            // LayerNorm of the group's tokens by the whole workgroup: thread tid holds the float4 pieces tid + 256 * j of every
+            // token (tt * pieces <= 8), so all rows, the iteration vector and the LayerNorm parameters are one round of
+            // loads; sums meet through LDS (red: [4 waves][4 tokens]).
+            constexpr int TT = 8 / J < TAIL_TT ? 8 / J : TAIL_TT, E = TT * J;
+            float4 v[E], w[J], b[J];
+#pragma unroll
+            for (int jj = 0; jj < J; ++jj) {
+                const int i = tid + 256 * jj, ic = i < d4 ? i : d4 - 1;
+                w[jj] = lw4[ic];
+                b[jj] = lb4[ic];
+#pragma unroll
+                for (int t = 0; t < TT; ++t) {
+                    const bool on = t < nt && i < d4;
+                    float4 a = reinterpret_cast<const float4 *>(qv + (g0 + (t < nt ? t : 0)) * ldq)[ic];
+                    if (iter_vec) { const float4 c = iv4[ic]; a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w; }
+                    v[t * J + jj] = on ? a : zero4;
+                }
+            }
+            float s[TT], mean[TT], rstd[TT];
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+                s[t] = 0.f;
+#pragma unroll
+                for (int jj = 0; jj < J; ++jj) { const float4 a = v[t * J + jj]; s[t] += (a.x + a.y) + (a.z + a.w); }
+                const float a = wave_sum_dpp(s[t]);
+                if (lane == 0) red[wave * TAIL_TT + t] = a;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int t = 0; t < TT; ++t) mean[t] = (red[t] + red[TAIL_TT + t] + red[2 * TAIL_TT + t] + red[3 * TAIL_TT + t]) / (float)d;
+            __syncthreads();
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+                s[t] = 0.f;
+#pragma unroll
+                for (int jj = 0; jj < J; ++jj) {
+                    if (tid + 256 * jj < d4) {
+                        const float4 q = v[t * J + jj];
+                        const float a = q.x - mean[t], c = q.y - mean[t], f = q.z - mean[t], h = q.w - mean[t];
+                        s[t] = __builtin_fmaf(h, h, __builtin_fmaf(f, f, __builtin_fmaf(c, c, __builtin_fmaf(a, a, s[t]))));
+                    }
+                }
+                const float a = wave_sum_dpp(s[t]);
+                if (lane == 0) red[wave * TAIL_TT + t] = a;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+                rstd[t] = 1.0f / sqrtf((red[t] + red[TAIL_TT + t] + red[2 * TAIL_TT + t] + red[3 * TAIL_TT + t]) / (float)d + ln_eps);
+#pragma unroll
+                for (int jj = 0; jj < J; ++jj) {
+                    const int i = tid + 256 * jj;
+                    if (t < nt && i < d4) {
+                        const float4 q = v[t * J + jj];
+                        const float m = mean[t], r = rstd[t];
+                        reinterpret_cast<float4 *>(qn + (size_t)t * d)[i] =
+                            float4{(q.x - m) * r * w[jj].x + b[jj].x, (q.y - m) * r * w[jj].y + b[jj].y,
+                                   (q.z - m) * r * w[jj].z + b[jj].z, (q.w - m) * r * w[jj].w + b[jj].w};
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        {
+            // items of this wave: (key row c = wave + 4 * row, piece of 256 float4); the next item's piece is loaded first
+            const int chunks = (n4 + 255) / 256;
+            const int rows = (2 * nsk - wave + 3) / 4;
+            const int items = rows * chunks;
+            auto load_item = [&](int it, float4 (&kv)[4]) {
+                const int itc = it < items ? it : items - 1;
+                const int c = wave + 4 * (itc / chunks), i0 = lane + 256 * (itc % chunks);
+                const float4 *kr = reinterpret_cast<const float4 *>(c < nsk ? ka + (int64_t)c * d2 : kb + (int64_t)(c - nsk) * d2);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) kv[u] = kr[i0 + 64 * u < n4 ? i0 + 64 * u : n4 - 1];
+            };
+            float4 kv[4];
+            if (items > 0) load_item(0, kv);
+            float acc[TAIL_TT];
+#pragma unroll
+            for (int t = 0; t < TAIL_TT; ++t) acc[t] = 0.f;
+            for (int it = 0; it < items; ++it) {
+                float4 kn[4];
+                load_item(it + 1, kn);
+                const int c = wave + 4 * (it / chunks), i0 = lane + 256 * (it % chunks);
+                const int off4 = c < nsk ? 0 : n4;
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (i0 + 64 * u >= n4) kv[u] = zero4;
+#pragma unroll
+                for (int t = 0; t < TAIL_TT; ++t) {
+                    if (t < nt) {
+                        const float4 *qh = reinterpret_cast<const float4 *>(qn + (size_t)t * d) + off4;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const float4 qq = qh[i0 + 64 * u < n4 ? i0 + 64 * u : n4 - 1];
+                            acc[t] = __builtin_fmaf(qq.w, kv[u].w, __builtin_fmaf(qq.z, kv[u].z, __builtin_fmaf(qq.y, kv[u].y, __builtin_fmaf(qq.x, kv[u].x, acc[t]))));
+                        }
+                    }
+                }
+                if (it % chunks == chunks - 1) {
+#pragma unroll
+                    for (int t = 0; t < TAIL_TT; ++t) {
+                        const float a = wave_sum_dpp(acc[t]);
+                        if (lane == 0 && t < nt) sc[t * 2 * nsk + c] = a;
+                        acc[t] = 0.f;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) kv[u] = kn[u];
+            }
+        }
+        __syncthreads();
+        if (wave < nt) {                             // tt <= 4: one token per wave, nothing shared between waves from here on
+            const int t = wave;
+            const float *sct = sc + t * 2 * nsk;
+            float *lgt = lg + (size_t)t * n;
+            float *lrow = logits_out ? logits_out + (g0 + t) * n : nullptr;
+            if (P > n) {
+                // more product keys than groups: the n largest product scores in descending order (routing.py:212-222)
+                if (P <= 512) ranked_logits<8>(sct, nsk, P, bias, n, nullptr, lgt, lrow, lane);
+                else ranked_logits<16>(sct, nsk, P, bias, n, nullptr, lgt, lrow, lane);        // the host admits P <= 1024
+            } else {
+                for (int g = lane; g < n; g += 64) {
+                    const int pr = g % P;
+                    const float l = (sct[pr / nsk] + sct[nsk + pr % nsk]) + bias[g];
+                    lgt[g] = l;
+                    if (lrow) lrow[g] = l;
+                }
+            }
+            // the wave reads logits that other lanes of it wrote: LDS serves a wave's accesses in order, the fence keeps
+            // the compiler from moving the reads up
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            remoe_gates_wave<MAXPL>(lgt, n, k, gates + (g0 + t) * n, active ? active + (g0 + t) * n : nullptr, lane);
+        }
+        __syncthreads();
+    }
+}
+
 // Workgroup = (token tile, chunk of 64 clusters).  The tile's active bytes for the chunk are staged in LDS
 // with coalesced reads; then every wave compacts whole clusters: lanes = tokens, ballot -> prefix popcount.
 __global__ void __launch_bounds__(256) remoe_route_kernel(const uint8_t *active, int64_t M, int n, int tile,
@@ -468,6 +717,42 @@ extern "C" int mortar_router_bf16(const void *x, int32_t x_is_f32, int64_t B, in
     else if (npl <= 8) MORTAR_TAIL(8);
     else MORTAR_TAIL(16);
 #undef MORTAR_TAIL
+    return check_launch("router tail");
+}
+
+extern "C" int mortar_router_tail_f32(const float *qv, int64_t N, int32_t d, int64_t ldq, const float *iter_vec,
+                                      const float *ln_w, const float *ln_b, float ln_eps, const float *ka, const float *kb,
+                                      int32_t nsk, const float *bias, int32_t n, int32_t k, float *logits_out, float *gates,
+                                      uint8_t *active, void *stream) {
+    if (!qv || !ln_w || !ln_b || !ka || !kb || !bias || !gates) return mortar_fail(MORTAR_ERR_ARG, "router tail: null pointer");
+    if (N <= 0 || N > ((int64_t)1 << 31) / (n > 0 ? n : 1)) return mortar_fail(MORTAR_ERR_ARG, "router tail: N=%lld out of range", (long long)N);
+    if (d <= 0 || d % 8 || d > 8192 || ldq < d || ldq % 4)
+        return mortar_fail(MORTAR_ERR_ARG, "router tail: d must be a multiple of 8 up to 8192 and ldq >= d, 16-byte aligned rows");
+    if ((reinterpret_cast<uintptr_t>(qv) | reinterpret_cast<uintptr_t>(iter_vec) | reinterpret_cast<uintptr_t>(ln_w) |
+         reinterpret_cast<uintptr_t>(ln_b) | reinterpret_cast<uintptr_t>(ka) | reinterpret_cast<uintptr_t>(kb)) & 15)
+        return mortar_fail(MORTAR_ERR_ARG, "router tail: qv, iter_vec, ln_w, ln_b, ka and kb must be 16-byte aligned");
+    if (n <= 0 || k <= 0 || nsk <= 0) return mortar_fail(MORTAR_ERR_ARG, "router tail: n, k, nsk must be positive");
+    if (n > 64 * MAXPL_LIMIT) return mortar_fail(MORTAR_ERR_LIMIT, "router tail: n=%d exceeds %d clusters", n, 64 * MAXPL_LIMIT);
+    if ((int64_t)nsk * nsk > n && (int64_t)nsk * nsk > 1024)
+        return mortar_fail(MORTAR_ERR_LIMIT, "router tail: %d x %d product keys for %d groups exceed the 1024 the kernel ranks", nsk, nsk, n);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // a thread holds J float4 pieces of every row of its group (J = 1, 2, 4 or 8 for d <= 1024 J) and tt = min(4, 8 / J)
+    // tokens share a group, so the normalised rows take at most 32 KB of LDS
+    const int J = d <= 1024 ? 1 : d <= 2048 ? 2 : d <= 4096 ? 4 : 8;
+    const int tt = 8 / J < TAIL_TT ? 8 / J : TAIL_TT;
+    const size_t smem = ((size_t)tt * d + (size_t)tt * 2 * nsk + (size_t)tt * n + 16) * sizeof(float);
+    const int64_t groups = (N + tt - 1) / tt;
+    const dim3 grid((unsigned)(groups < 3072 ? groups : 3072)), blk(256);
+    const int npl = (n + 63) / 64;
+#define MORTAR_TAILG(PL, JJ) hipLaunchKernelGGL((router_tail_group_kernel<PL, JJ>), grid, blk, smem, st, qv, N, d, ldq, iter_vec, ln_w, \
+                                               ln_b, ln_eps, ka, kb, nsk, bias, n, k, tt, logits_out, gates, active)
+#define MORTAR_TAILJ(PL) do { if (J == 1) MORTAR_TAILG(PL, 1); else if (J == 2) MORTAR_TAILG(PL, 2); else if (J == 4) MORTAR_TAILG(PL, 4); \
+                              else MORTAR_TAILG(PL, 8); } while (0)
+    if (npl <= 2) MORTAR_TAILJ(2);
+    else if (npl <= 6) MORTAR_TAILJ(6);
+    else MORTAR_TAILJ(16);
+#undef MORTAR_TAILJ
+#undef MORTAR_TAILG
     return check_launch("router tail");
 }
 

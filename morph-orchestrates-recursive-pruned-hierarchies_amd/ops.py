@@ -258,6 +258,33 @@ def router_fused(x: Tensor, wq: Tensor, iter_vec: Tensor | None, ln_w: Tensor, l
     return (gates, active, logits) if want_logits else (gates, active)
 
 
+def router_tail(qv: Tensor, iter_vec: Tensor | None, ln_w: Tensor, ln_b: Tensor, ln_eps: float, ka: Tensor, kb: Tensor,
+                bias: Tensor, k: int, want_logits: bool = False):
+    """TileRouter.forward steps 2-8 in one launch on the projected query qv = x Wq^T (fp32 [N, d], any N): LayerNorm of
+    qv + iter_vec, sub-key scores, product-key logits, gating tail.  The projection itself is a dense GEMM and stays with
+    the library.  -> (gates fp32 [N, n], active uint8 [N, n][, logits])."""
+    _need_gpu(qv, "router_tail")
+    if qv.dim() != 2 or qv.dtype != torch.float32:
+        raise TypeError("router_tail: qv must be a 2-D float32 tensor")
+    if qv.stride(1) != 1 or qv.stride(0) % 4 or qv.data_ptr() % 16:
+        qv = qv.contiguous()
+    N, d = qv.shape
+    n, nsk = bias.numel(), ka.shape[0]
+    for name, t, shp in (("ln_w", ln_w, (d,)), ("ln_b", ln_b, (d,)), ("ka", ka, (nsk, d // 2)), ("kb", kb, (nsk, d // 2)),
+                         ("bias", bias, (n,))) + ((("iter_vec", iter_vec, (d,)),) if iter_vec is not None else ()):
+        if t.dtype != torch.float32 or tuple(t.shape) != shp or not t.is_contiguous() or t.device != qv.device:
+            raise TypeError(f"router_tail: {name} must be a contiguous float32 {shp} tensor on {qv.device}")
+    gates = torch.empty((N, n), dtype=torch.float32, device=qv.device)
+    active = torch.empty((N, n), dtype=torch.uint8, device=qv.device)
+    logits = torch.empty((N, n), dtype=torch.float32, device=qv.device) if want_logits else None
+    if N:
+        rc = _lib.lib().mortar_router_tail_f32(_p(qv), N, d, qv.stride(0), _p(iter_vec), _p(ln_w), _p(ln_b), float(ln_eps),
+                                               _p(ka), _p(kb), nsk, _p(bias), n, int(k), _p(logits), _p(gates), _p(active),
+                                               _stream(qv))
+        _lib.check(rc, "mortar_router_tail_f32")
+    return (gates, active, logits) if want_logits else (gates, active)
+
+
 def route_tile(W: MortarPack, M: int = 0) -> int:
     """Token tile of the routed gate_up kernels for M rows against this matrix (the tile remoe_route must use);
     0 when the matrix is too wide for routed skipping (use the dense gated call)."""

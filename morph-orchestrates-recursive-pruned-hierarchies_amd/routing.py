@@ -3,7 +3,8 @@
 Interface mirror of the reference's morph/model/routing.py (same parameters, forward signature, outputs).
 The gating tail (steps 5-8: k-th largest threshold, ReLU, normalise to sum k, active mask) runs in the HIP
 kernel for inference.  For decode-sized calls (up to 64 rows) the front end (query projection, LayerNorm, sub-key
-scores, product-key logits) runs in HIP as well, two launches in all; larger calls use library GEMMs through torch.
+scores, product-key logits) runs in HIP as well, two launches in all; larger calls run the dense query projection as
+a library GEMM through torch and everything behind it (LayerNorm to gates) in one HIP launch.
 With autograd enabled the tail stays in differentiable torch ops.
 """
 from __future__ import annotations
@@ -71,24 +72,37 @@ class TileRouter(nn.Module):
                 and self.n_sub_keys * self.n_sub_keys <= 2048 and self.d_model % 8 == 0
                 and self.n_tile_groups <= 1024)
 
+    def _tail_ok(self, x_flat: Tensor) -> bool:
+        """Inference calls of any size on the GPU with fp32 router parameters: library GEMM for the projection, then the
+        one-launch tail."""
+        return (x_flat.is_cuda and x_flat.shape[0] > 0 and not torch.is_grad_enabled()
+                and x_flat.dtype in (torch.bfloat16, torch.float32) and self.query_proj.weight.dtype == torch.float32
+                and self.n_sub_keys * self.n_sub_keys <= max(1024, self.n_tile_groups) and self.d_model % 8 == 0
+                and self.d_model <= 8192 and self.n_tile_groups <= 1024)
+
     @torch.no_grad()
     def route(self, x_flat: Tensor, iter_idx: int = 0) -> Tuple[Tensor, Tensor]:
         """Inference-only routing of [N, d_model] rows: (gates fp32 [N, n], active uint8 [N, n]) and nothing else (no
         load statistics, no auxiliary loss), as the reference's decode engine calls its fused router
-        (morph/kernels/triton/fused_router.py:100-140).  Two launches for decode-sized N, torch GEMMs + the gating
-        kernel otherwise."""
+        (morph/kernels/triton/fused_router.py:100-140).  Two launches for decode-sized N; a library GEMM for the query
+        projection plus one launch for everything behind it otherwise."""
         if self._fused_ok(x_flat):
             it = max(0, min(int(iter_idx), self.n_iters - 1))
             return ops.router_fused(x_flat, self.query_proj.weight, self.iter_embed[it], self.query_norm.weight,
                                     self.query_norm.bias, self.query_norm.eps, self.sub_keys_a, self.sub_keys_b,
                                     self.group_bias, self.activation_k)
+        if self._tail_ok(x_flat):
+            it = max(0, min(int(iter_idx), self.n_iters - 1))
+            qv = F.linear(x_flat.float(), self.query_proj.weight)
+            return ops.router_tail(qv, self.iter_embed[it], self.query_norm.weight, self.query_norm.bias,
+                                   self.query_norm.eps, self.sub_keys_a, self.sub_keys_b, self.group_bias, self.activation_k)
         return gates_from_logits(self.group_logits(x_flat, iter_idx), self.activation_k)
 
     def forward(self, x: Tensor, iter_idx: int = 0) -> Tuple[Tensor, Tensor]:
         orig_shape = x.shape
         x_flat = x.reshape(-1, orig_shape[-1])
         k = self.activation_k
-        if self._fused_ok(x_flat):
+        if self._fused_ok(x_flat) or self._tail_ok(x_flat):
             gates, active = self.route(x_flat, iter_idx)
             self.last_active = active
             logits = None

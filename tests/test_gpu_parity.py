@@ -463,6 +463,62 @@ def test_fused_router_front_end(dev, B, d, nsk, n, xdt):
     np.testing.assert_allclose(lt.cpu().numpy(), ref, rtol=0, atol=2e-5 * max(1.0, np.abs(ref).max()))
 
 
+@pytest.mark.parametrize("N,d,nsk,n", [(65, 256, 4, 16), (200, 768, 4, 16), (513, 2048, 19, 352), (300, 2048, 8, 64),
+                                       (130, 264, 3, 20), (70, 512, 32, 1000), (100, 4096, 4, 16), (33, 8192, 5, 25), (3, 512, 4, 16),
+                                       (66, 256, 23, 500)])
+def test_router_tail_behind_a_library_projection(dev, N, d, nsk, n):
+    """Prefill-sized router: the dense query projection through the library, then ONE launch for LayerNorm, sub-key
+    scores, product-key logits (direct, wrapped and ranked branches) and the gating tail, against the float64 oracle (same
+    bars as the two-launch decode router) and against the module's eager torch ops."""
+    rng = np.random.default_rng(170 + N)
+    k = max(1, n // 4)
+    x = O.bf16_round(rng.standard_normal((N, d)).astype(np.float32))
+    wq = (rng.standard_normal((d, d)) / np.sqrt(d)).astype(np.float32); it = (0.1 * rng.standard_normal(d)).astype(np.float32)
+    lw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32); lb = (0.1 * rng.standard_normal(d)).astype(np.float32)
+    ka = (rng.standard_normal((nsk, d // 2)) / np.sqrt(d // 2)).astype(np.float32)
+    kb = (rng.standard_normal((nsk, d // 2)) / np.sqrt(d // 2)).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(n)).astype(np.float32)
+    T = lambda a: torch.from_numpy(a).to(dev)
+    xd = to_dev(x, dev)
+    qv = torch.nn.functional.linear(xd.float(), T(wq))
+    gates, active, logits = ops.router_tail(qv, T(it), T(lw), T(lb), 1e-5, T(ka), T(kb), T(bias), k, want_logits=True)
+    ref = O.router_logits(x, wq, it, lw, lb, 1e-5, ka, kb, bias)
+    np.testing.assert_allclose(logits.cpu().numpy(), ref, rtol=0, atol=2e-5 * max(1.0, np.abs(ref).max()))
+    g_ref, a_ref = O.remoe_gates(ref.astype(np.float32), k)
+    kth = O.kth_largest(ref.astype(np.float32), k)[:, None] if k < n else np.full((N, 1), -np.inf)
+    clear = np.abs(ref - kth) > 1e-4                       # logits not within rounding of the threshold
+    assert np.array_equal(active.cpu().numpy().astype(bool)[clear], a_ref[clear])
+    rows = clear.all(axis=1)                                # a token with a logit at the threshold may normalise differently
+    np.testing.assert_allclose(gates.cpu().numpy()[rows], g_ref[rows], rtol=0, atol=2e-4)
+    g2, a2 = ops.remoe_gates(logits, k)                     # the fused tail is the stand-alone gates kernel on its own logits
+    assert torch.equal(g2, gates) and torch.equal(a2, active)
+    # a strided qv (rows of a wider buffer) and no iteration vector
+    wide = torch.zeros((N, d + 8), dtype=torch.float32, device=dev)
+    wide[:, :d] = qv + T(it)
+    g3, a3 = ops.router_tail(wide[:, :d], None, T(lw), T(lb), 1e-5, T(ka), T(kb), T(bias), k)
+    assert torch.equal(g3, gates) and torch.equal(a3, active)
+    from mortar_amd.routing import TileRouter
+    rt = TileRouter(n, d, activation_ratio=k / n, n_sub_keys=nsk, n_iters=2).to(dev)
+    with torch.no_grad():
+        rt.query_proj.weight.copy_(T(wq)); rt.iter_embed[1].copy_(T(it)); rt.query_norm.weight.copy_(T(lw))
+        rt.query_norm.bias.copy_(T(lb)); rt.sub_keys_a.copy_(T(ka)); rt.sub_keys_b.copy_(T(kb)); rt.group_bias.copy_(T(bias))
+        assert rt.activation_k == k and rt._tail_ok(xd)
+        if N > ops.ROUTER_MAX_TOKENS:
+            gm, am = rt.route(xd, iter_idx=1)
+            assert torch.equal(gm, gates) and torch.equal(am, active)
+            gf, _ = rt(xd, iter_idx=1)
+            assert torch.equal(gf, gates) and torch.equal(rt.last_active, active)
+        lt = rt.group_logits(xd, 1)                       # eager torch ops
+    np.testing.assert_allclose(lt.cpu().numpy(), ref, rtol=0, atol=2e-5 * max(1.0, np.abs(ref).max()))
+    with pytest.raises(TypeError):
+        ops.router_tail(qv.double(), None, T(lw), T(lb), 1e-5, T(ka), T(kb), T(bias), k)
+    if N == 3:      # more than 1024 product keys to rank: refused, the module keeps its eager path for such a router
+        k33 = T((rng.standard_normal((33, d // 2))).astype(np.float32))
+        with pytest.raises(ValueError):
+            ops.router_tail(qv, None, T(lw), T(lb), 1e-5, k33, k33, T(np.zeros(1024, dtype=np.float32)), 5)
+        assert not TileRouter(1024, d, n_sub_keys=33).to(dev)._tail_ok(xd)
+
+
 def test_decode_mlp_module_routes_with_its_own_router(dev):
     """MortarDecodeMLP with a router attached (no token lists: the gated gate_up kernel leaves out inactive units
     itself) equals the step-by-step composition rmsnorm -> route -> gated gate_up -> down, and the oracle."""
