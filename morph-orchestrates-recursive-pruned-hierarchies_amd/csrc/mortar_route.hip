@@ -192,6 +192,66 @@ __device__ __forceinline__ float block_sum256(float v, float *red) {      // red
     return red[0] + red[1] + red[2] + red[3];
 }
 
+// Descending bitonic sort of 64 * KPL keys held KPL per lane (element lane * KPL + r in register r): steps between
+// elements of one lane are register compare-exchanges, steps between lanes one shuffle per register.  No LDS, no barrier.
+template <int KPL>
+__device__ __forceinline__ void wave_sort_desc(uint32_t (&key)[KPL], int lane) {
+    for (int k2 = 2; k2 <= 64 * KPL; k2 <<= 1) {
+        const bool lane_desc = ((lane * KPL) & k2) == 0;       // direction of this lane's elements once k2 >= KPL
+        for (int lj = k2 / (2 * KPL); lj >= 1; lj >>= 1) {       // partners in other lanes (distance j = lj * KPL)
+            const bool keep_max = ((lane & lj) == 0) == lane_desc;
+#pragma unroll
+            for (int r = 0; r < KPL; ++r) {
+                const uint32_t a = key[r], o = (uint32_t)__shfl_xor((int)a, lj, 64);
+                key[r] = keep_max ? (a > o ? a : o) : (a > o ? o : a);
+            }
+        }
+#pragma unroll
+        for (int j = KPL / 2; j > 0; j >>= 1) {                  // partners in this lane's registers (distance j < k2)
+            if (j < k2) {
+#pragma unroll
+                for (int r = 0; r < KPL; ++r) {
+                    if ((r & j) == 0) {
+                        const bool desc = k2 < KPL ? (r & k2) == 0 : lane_desc;
+                        const uint32_t a = key[r], c = key[r | j];
+                        const uint32_t hi = a > c ? a : c, lo = a > c ? c : a;
+                        key[r] = desc ? hi : lo;
+                        key[r | j] = desc ? lo : hi;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// The n largest of the P = nsk * nsk product scores of one token in descending order (+ bias) -> lgt[0 .. n), on one wave.
+template <int KPL>
+__device__ __forceinline__ void ranked_logits(const float *sct, int nsk, int P, const float *bias, int n, uint32_t *sk,
+                                              float *lgt, float *logits_row, int lane) {
+    uint32_t key[KPL];
+#pragma unroll
+    for (int r = 0; r < KPL; ++r) {
+        const int i = lane * KPL + r;
+        uint32_t kk = 0u;                                    // padding: the smallest key
+        if (i < P) {
+            const uint32_t u = __float_as_uint(sct[i / nsk] + sct[nsk + i % nsk]);
+            kk = (u & 0x80000000u) ? ~u : (u | 0x80000000u);   // NaN ranks above +inf, as torch.topk has it
+        }
+        key[r] = kk;
+    }
+    wave_sort_desc<KPL>(key, lane);
+#pragma unroll
+    for (int r = 0; r < KPL; ++r) {
+        const int g = lane * KPL + r;
+        if (g < n) {
+            const float l = __uint_as_float((key[r] & 0x80000000u) ? (key[r] & 0x7fffffffu) : ~key[r]) + bias[g];
+            lgt[g] = l;
+            if (logits_row) logits_row[g] = l;
+        }
+    }
+    (void)sk;
+}
+
 // Launch 2, one workgroup per token: LayerNorm(qv) -> sub-key scores of the two query halves -> product-key logits
 // (+ group bias) -> gating tail.  P = nsk * nsk products map to the n groups one to one (P == n), wrap (P < n), or are
 // ranked and the n largest kept (P > n).
@@ -288,35 +348,44 @@ __global__ void __launch_bounds__(256) router_tail_kernel(const float *qv, int d
     if (P > n) {
         // more product keys than groups: the group logits are the n largest product scores in descending order
         // (torch.topk(product_scores, n).values, morph/model/routing.py:212-222).  Bitonic sort of order-preserving
-        // integer keys (NaN ranks above +inf, as torch.topk has it), padded with the smallest key.
-        uint32_t *sk = reinterpret_cast<uint32_t *>(red + 4);
-        int P2 = 1;
-        while (P2 < P) P2 <<= 1;
-        for (int i = tid; i < P2; i += 256) {
-            uint32_t key = 0u;
-            if (i < P) {
-                const uint32_t u = __float_as_uint(sc[i / nsk] + sc[nsk + i % nsk]);
-                key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+        // integer keys (NaN ranks above +inf, as torch.topk has it), padded with the smallest key: in one wave's registers
+        // up to 1024 products, through LDS by the whole workgroup beyond.
+        if (P <= 1024) {           // one wave ranks them in its registers (no LDS traffic, no barrier per step)
+            float *lrow = logits_out ? logits_out + (int64_t)b * n : nullptr;
+            if (wave == 0) {
+                if (P <= 512) ranked_logits<8>(sc, nsk, P, bias, n, nullptr, lg, lrow, lane);
+                else ranked_logits<16>(sc, nsk, P, bias, n, nullptr, lg, lrow, lane);
             }
-            sk[i] = key;
-        }
-        __syncthreads();
-        for (int k2 = 2; k2 <= P2; k2 <<= 1) {
-            for (int j = k2 >> 1; j > 0; j >>= 1) {
-                for (int t = tid; t < P2 / 2; t += 256) {
-                    const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1)), l = i | j;
-                    const uint32_t a = sk[i], c = sk[l];
-                    const bool desc = (i & k2) == 0;
-                    if (desc ? a < c : a > c) { sk[i] = c; sk[l] = a; }
+        } else {
+            uint32_t *sk = reinterpret_cast<uint32_t *>(red + 4);
+            int P2 = 1;
+            while (P2 < P) P2 <<= 1;
+            for (int i = tid; i < P2; i += 256) {
+                uint32_t key = 0u;
+                if (i < P) {
+                    const uint32_t u = __float_as_uint(sc[i / nsk] + sc[nsk + i % nsk]);
+                    key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
                 }
-                __syncthreads();
+                sk[i] = key;
             }
-        }
-        for (int g = tid; g < n; g += 256) {
-            const uint32_t key = sk[g];
-            const float l = __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key) + bias[g];
-            lg[g] = l;
-            if (logits_out) logits_out[(int64_t)b * n + g] = l;
+            __syncthreads();
+            for (int k2 = 2; k2 <= P2; k2 <<= 1) {
+                for (int j = k2 >> 1; j > 0; j >>= 1) {
+                    for (int t = tid; t < P2 / 2; t += 256) {
+                        const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1)), l = i | j;
+                        const uint32_t a = sk[i], c = sk[l];
+                        const bool desc = (i & k2) == 0;
+                        if (desc ? a < c : a > c) { sk[i] = c; sk[l] = a; }
+                    }
+                    __syncthreads();
+                }
+            }
+            for (int g = tid; g < n; g += 256) {
+                const uint32_t key = sk[g];
+                const float l = __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key) + bias[g];
+                lg[g] = l;
+                if (logits_out) logits_out[(int64_t)b * n + g] = l;
+            }
         }
     } else {
         for (int g = tid; g < n; g += 256) {
@@ -332,66 +401,6 @@ __global__ void __launch_bounds__(256) router_tail_kernel(const float *qv, int d
 }
 
 // ---- router tail for prefill-sized calls (TileRouter.forward steps 2-8 behind a library GEMM for the projection) ----
-
-// Descending bitonic sort of 64 * KPL keys held KPL per lane (element lane * KPL + r in register r): steps between
-// elements of one lane are register compare-exchanges, steps between lanes one shuffle per register.  No LDS, no barrier.
-template <int KPL>
-__device__ __forceinline__ void wave_sort_desc(uint32_t (&key)[KPL], int lane) {
-    for (int k2 = 2; k2 <= 64 * KPL; k2 <<= 1) {
-        const bool lane_desc = ((lane * KPL) & k2) == 0;       // direction of this lane's elements once k2 >= KPL
-        for (int lj = k2 / (2 * KPL); lj >= 1; lj >>= 1) {       // partners in other lanes (distance j = lj * KPL)
-            const bool keep_max = ((lane & lj) == 0) == lane_desc;
-#pragma unroll
-            for (int r = 0; r < KPL; ++r) {
-                const uint32_t a = key[r], o = (uint32_t)__shfl_xor((int)a, lj, 64);
-                key[r] = keep_max ? (a > o ? a : o) : (a > o ? o : a);
-            }
-        }
-#pragma unroll
-        for (int j = KPL / 2; j > 0; j >>= 1) {                  // partners in this lane's registers (distance j < k2)
-            if (j < k2) {
-#pragma unroll
-                for (int r = 0; r < KPL; ++r) {
-                    if ((r & j) == 0) {
-                        const bool desc = k2 < KPL ? (r & k2) == 0 : lane_desc;
-                        const uint32_t a = key[r], c = key[r | j];
-                        const uint32_t hi = a > c ? a : c, lo = a > c ? c : a;
-                        key[r] = desc ? hi : lo;
-                        key[r | j] = desc ? lo : hi;
-                    }
-                }
-            }
-        }
-    }
-}
-
-// The n largest of the P = nsk * nsk product scores of one token in descending order (+ bias) -> lgt[0 .. n), on one wave.
-template <int KPL>
-__device__ __forceinline__ void ranked_logits(const float *sct, int nsk, int P, const float *bias, int n, uint32_t *sk,
-                                              float *lgt, float *logits_row, int lane) {
-    uint32_t key[KPL];
-#pragma unroll
-    for (int r = 0; r < KPL; ++r) {
-        const int i = lane * KPL + r;
-        uint32_t kk = 0u;                                    // padding: the smallest key
-        if (i < P) {
-            const uint32_t u = __float_as_uint(sct[i / nsk] + sct[nsk + i % nsk]);
-            kk = (u & 0x80000000u) ? ~u : (u | 0x80000000u);   // NaN ranks above +inf, as torch.topk has it
-        }
-        key[r] = kk;
-    }
-    wave_sort_desc<KPL>(key, lane);
-#pragma unroll
-    for (int r = 0; r < KPL; ++r) {
-        const int g = lane * KPL + r;
-        if (g < n) {
-            const float l = __uint_as_float((key[r] & 0x80000000u) ? (key[r] & 0x7fffffffu) : ~key[r]) + bias[g];
-            lgt[g] = l;
-            if (logits_row) logits_row[g] = l;
-        }
-    }
-    (void)sk;
-}
 
 // A workgroup of four waves takes groups of up to TT = 4 tokens (a loop over its share of the groups), so the sub-key
 // rows are read from L2 once per group instead of once per token.
