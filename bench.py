@@ -392,6 +392,22 @@ def main() -> None:
                                               "note": "FLOPs of active (token, cluster) pairs only; a cluster is one 16-neuron row unit, "
                                                       "so a 32-token tile keeps about 8 active tokens per unit and the weight unpack, "
                                                       "which bounds the kernel, does not shrink with the active share: nothing is skipped"}}
+        # ---- the router that produces those logits in a model (TileRouter over 352 clusters, 19 x 19 product keys): the dense
+        # query projection through the library, everything behind it in one launch; beside it the eager torch ops
+        from mortar_amd.routing import TileRouter
+        torch.manual_seed(3)
+        rt352 = TileRouter(N_CLUSTERS, D_MODEL, activation_ratio=TOP_K / N_CLUSTERS).to(dev).eval()
+        with torch.no_grad():
+            qv = torch.nn.functional.linear(x.float(), rt352.query_proj.weight)
+            t_route = event_time_ms(lambda: rt352.route(x), 10, 2, settle=True)
+            t_tail = event_time_ms(lambda: ops.router_tail(qv, rt352.iter_embed[0], rt352.query_norm.weight, rt352.query_norm.bias,
+                                                           rt352.query_norm.eps, rt352.sub_keys_a, rt352.sub_keys_b,
+                                                           rt352.group_bias, rt352.activation_k), 10, 2)
+            t_torch = event_time_ms(lambda: ops.remoe_gates(rt352.group_logits(x, 0), rt352.activation_k), 10, 2)
+        out["router_prefill"] = {"route_ms": t_route, "tail_kernel_ms": t_tail, "eager_torch_ops_ms": t_torch,
+                                 "form": "TileRouter.route at 4096 tokens: fp32 query projection (library GEMM, 34 GFLOP) + one launch for "
+                                         "LayerNorm, sub-key scores, ranked product-key logits and gates; eager = the module's torch ops + gates kernel"}
+        del qv, rt352
         # ---- the reference's own deploy format: ONE scale per matrix (pack_mortar_ternary), same shapes ----------
         spec_u = {k: dict(spec[k]) for k in ("gate_up", "down")}
         spec_u["gate_up"]["scales"], spec_u["down"]["scales"] = np.float32(0.05), np.float32(0.03)
