@@ -255,10 +255,10 @@ __device__ __forceinline__ void ranked_logits(const float *sct, int nsk, int P, 
 // Launch 2, one workgroup per token: LayerNorm(qv) -> sub-key scores of the two query halves -> product-key logits
 // (+ group bias) -> gating tail.  P = nsk * nsk products map to the n groups one to one (P == n), wrap (P < n), or are
 // ranked and the n largest kept (P > n).
-// PRE (d <= 2048, nsk <= 4): every parameter a thread needs (LayerNorm weights, its slices of the sub-keys, its
-// bias) is fetched into registers before the first reduction, so the kernel pays one memory round trip instead of
-// one per phase.
-template <int MAXPL, bool PRE>
+// PRE > 0 (d <= 2048; PRE = sub-key rows per wave: 2 for nsk <= 4, 10 for nsk <= 20): every parameter a thread needs
+// (LayerNorm weights, its slices of the sub-key rows of its wave) is fetched into registers before the first reduction,
+// so the kernel pays one memory round trip instead of one per phase and key row.
+template <int MAXPL, int PRE>
 __global__ void __launch_bounds__(256) router_tail_kernel(const float *qv, int d, const float *ln_w, const float *ln_b,
                                                            float ln_eps, const float *ka, const float *kb, int nsk,
                                                            const float *bias, int n, int k, float *logits_out,
@@ -268,7 +268,7 @@ __global__ void __launch_bounds__(256) router_tail_kernel(const float *qv, int d
     const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const float *q = qv + (int64_t)b * d;
     const int d2 = d / 2, n4 = d2 / 4;          // d % 8 == 0: both halves are whole float4 runs
-    constexpr int QE = 8, DPW = 2, KU = 4;      // PRE: entries per thread, sub-key dots per wave, float4 per lane and dot
+    constexpr int QE = 8, DPW = PRE > 0 ? PRE : 1, KU = 4;      // PRE: entries per thread, sub-key dots per wave, float4 per lane and dot
     float qe[QE], lw[QE], lbv[QE];
     float4 kreg[DPW][KU];
     if (PRE) {
@@ -714,17 +714,17 @@ extern "C" int mortar_router_bf16(const void *x, int32_t x_is_f32, int64_t B, in
     const size_t smem = (size_t)(d + 2 * nsk + n + 4 + sort_keys) * sizeof(float);
     const dim3 tg((unsigned)B);
     const int npl = (n + 63) / 64;
-    const bool pre = d <= 2048 && nsk <= 4;
-#define MORTAR_TAIL(PL) do { if (pre) hipLaunchKernelGGL((router_tail_kernel<PL, true>), tg, blk, smem, st, qv, d, ln_w, ln_b, ln_eps, \
-                                      ka, kb, nsk, bias, n, k, logits_out, gates, active); \
-        else hipLaunchKernelGGL((router_tail_kernel<PL, false>), tg, blk, smem, st, qv, d, ln_w, ln_b, ln_eps, ka, kb, nsk, \
-                                bias, n, k, logits_out, gates, active); } while (0)
+    const int pre = d > 2048 ? 0 : nsk <= 4 ? 2 : nsk <= 20 ? 10 : 0;      // sub-key dots per wave with their rows in registers
+#define MORTAR_TAILP(PL, PR) hipLaunchKernelGGL((router_tail_kernel<PL, PR>), tg, blk, smem, st, qv, d, ln_w, ln_b, ln_eps, \
+                                               ka, kb, nsk, bias, n, k, logits_out, gates, active)
+#define MORTAR_TAIL(PL) do { if (pre == 2) MORTAR_TAILP(PL, 2); else if (pre == 10) MORTAR_TAILP(PL, 10); else MORTAR_TAILP(PL, 0); } while (0)
     if (npl <= 1) MORTAR_TAIL(1);
     else if (npl <= 2) MORTAR_TAIL(2);
     else if (npl <= 4) MORTAR_TAIL(4);
     else if (npl <= 6) MORTAR_TAIL(6);
     else if (npl <= 8) MORTAR_TAIL(8);
     else MORTAR_TAIL(16);
+#undef MORTAR_TAILP
 #undef MORTAR_TAIL
     return check_launch("router tail");
 }
