@@ -519,6 +519,30 @@ def test_router_tail_behind_a_library_projection(dev, N, d, nsk, n):
         assert not TileRouter(1024, d, n_sub_keys=33).to(dev)._tail_ok(xd)
 
 
+def test_empty_batches_launch_nothing(dev):
+    """Zero rows through every operator and module of the path: empty results of the right shape, no launch, no error."""
+    from mortar_amd.pack import BcsrTopology
+    from mortar_amd.routing import TileRouter
+    spec = synth.synth_mlp(256, 640, 0.25, seed=3)
+    G, D = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    e = lambda *shape, dt=torch.bfloat16: torch.empty(shape, dtype=dt, device=dev)
+    assert ops.mlp(e(0, 256), G, D).shape == (0, 256) and ops.mlp_hidden_bytes(0, 640) == 0
+    assert ops.gateup_swiglu(e(0, 256), G).shape == (0, 640) and ops.spmm(e(0, 640), D).shape == (0, 256)
+    m = spec["down"]
+    T = BcsrTopology(m["offsets"], m["col_idx"], m["shape"][0], m["shape"][1], dev)
+    assert ops.dds_values(e(0, 640), torch.zeros((T.nnz, 16, 16), dtype=torch.bfloat16, device=dev), T).shape == (0, 256)
+    g, a = ops.remoe_gates(e(0, 40, dt=torch.float32), 3)
+    assert g.shape == (0, 40) and a.shape == (0, 40)
+    z = lambda *shape: torch.zeros(shape, device=dev)
+    g, a = ops.router_tail(e(0, 256, dt=torch.float32), None, z(256), z(256), 1e-5, z(4, 128), z(4, 128), z(16), 4)
+    assert g.shape == (0, 16) and a.shape == (0, 16)
+    rt = TileRouter(16, 256).to(dev).eval()
+    with torch.no_grad():
+        assert rt(e(0, 256))[0].shape == (0, 16) and rt(torch.randn(2, 70, 256, device=dev).to(torch.bfloat16))[0].shape == (2, 70, 16)
+    mlp = synth.mlp_module(spec, dev)
+    assert mlp(e(0, 256)).shape == (0, 256) and mlp(e(2, 0, 256)).shape == (2, 0, 256)
+
+
 def test_decode_mlp_module_routes_with_its_own_router(dev):
     """MortarDecodeMLP with a router attached (no token lists: the gated gate_up kernel leaves out inactive units
     itself) equals the step-by-step composition rmsnorm -> route -> gated gate_up -> down, and the oracle."""
