@@ -226,8 +226,8 @@ __device__ __forceinline__ void wave_sort_desc(uint32_t (&key)[KPL], int lane) {
 
 // The n largest of the P = nsk * nsk product scores of one token in descending order (+ bias) -> lgt[0 .. n), on one wave.
 template <int KPL>
-__device__ __forceinline__ void ranked_logits(const float *sct, int nsk, int P, const float *bias, int n, uint32_t *sk,
-                                              float *lgt, float *logits_row, int lane) {
+__device__ __forceinline__ void ranked_logits(const float *sct, int nsk, int P, const float *bias, int n, float *lgt,
+                                              float *logits_row, int lane) {
     uint32_t key[KPL];
 #pragma unroll
     for (int r = 0; r < KPL; ++r) {
@@ -249,7 +249,6 @@ __device__ __forceinline__ void ranked_logits(const float *sct, int nsk, int P, 
             if (logits_row) logits_row[g] = l;
         }
     }
-    (void)sk;
 }
 
 // Launch 2, one workgroup per token: LayerNorm(qv) -> sub-key scores of the two query halves -> product-key logits
@@ -353,8 +352,8 @@ __global__ void __launch_bounds__(256) router_tail_kernel(const float *qv, int d
         if (P <= 1024) {           // one wave ranks them in its registers (no LDS traffic, no barrier per step)
             float *lrow = logits_out ? logits_out + (int64_t)b * n : nullptr;
             if (wave == 0) {
-                if (P <= 512) ranked_logits<8>(sc, nsk, P, bias, n, nullptr, lg, lrow, lane);
-                else ranked_logits<16>(sc, nsk, P, bias, n, nullptr, lg, lrow, lane);
+                if (P <= 512) ranked_logits<8>(sc, nsk, P, bias, n, lg, lrow, lane);
+                else ranked_logits<16>(sc, nsk, P, bias, n, lg, lrow, lane);
             }
         } else {
             uint32_t *sk = reinterpret_cast<uint32_t *>(red + 4);
@@ -551,8 +550,8 @@ __global__ void __launch_bounds__(256, 2) router_tail_group_kernel(const float *
             float *lrow = logits_out ? logits_out + (g0 + t) * n : nullptr;
             if (P > n) {
                 // more product keys than groups: the n largest product scores in descending order (routing.py:212-222)
-                if (P <= 512) ranked_logits<8>(sct, nsk, P, bias, n, nullptr, lgt, lrow, lane);
-                else ranked_logits<16>(sct, nsk, P, bias, n, nullptr, lgt, lrow, lane);        // the host admits P <= 1024
+                if (P <= 512) ranked_logits<8>(sct, nsk, P, bias, n, lgt, lrow, lane);
+                else ranked_logits<16>(sct, nsk, P, bias, n, lgt, lrow, lane);        // the host admits P <= 1024
             } else {
                 for (int g = lane; g < n; g += 64) {
                     const int pr = g % P;
