@@ -27,7 +27,7 @@ PEAK_BF16_TFLOPS, PEAK_HBM_GBS = 2500.0, 8000.0
 # and profiles/bench_all_legs_hbm_traffic_pmc.md.  Not measured live: counters need the profiler.
 TRAFFIC_GATE_UP_BYTES = 41.57e6 + 46.14e6
 TRAFFIC_DOWN_BYTES = 60.41e6 + 17.68e6
-TRAFFIC_DECODE_STACK_BYTES = (263.02e6 + 4.54e6) + (169.01e6 + 1.96e6)   # gate_up + down launches, 160 layers, b = 1
+TRAFFIC_DECODE_STACK_BYTES = (263.05e6 + 4.54e6) + (145.54e6 + 1.83e6)   # gate_up + down launches, 160 layers, b = 1
 TRAFFIC_SOURCE = ("constant from profiles/bench_prefill_step_hbm_traffic_pmc.md and profiles/bench_all_legs_hbm_traffic_pmc.md "
                   "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command); not measured in this run")
 

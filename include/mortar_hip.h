@@ -133,6 +133,12 @@ int mortar_transpose_topology_host(const int32_t *row_ptr, const int16_t *col, i
  * Cb <= this runs the single-segment prefill kernel.  Use seg_cb = ceil(Cb / ceil(Cb / max)). */
 int mortar_prefill_max_seg_cb(void);
 
+/* Largest K segment whose 4-token tile fits in LDS.  A second stream of a matrix laid out with ONE segment of Cb <= this
+ * (same codes, rows padded to octets once per row instead of once per (segment, row)) serves calls of up to 4 rows only:
+ * the layer-batched decode launches read about 8 % fewer bytes from it for a `down` whose prefill stream has three
+ * segments.  Calls with more rows on such a stream are refused.  No counterpart in the reference. */
+int mortar_decode_max_seg_cb(void);
+
 /* Row-unit order for uneven nnz: units sorted by descending block count and dealt into groups of `group`
  * consecutive positions with similar totals (longest-processing-time first); use group = 16, the number of
  * wavefronts of a prefill workgroup.  rows_per_unit = 1 (plain) or 2 (gate row u and up row u + Rb/2).

@@ -17,8 +17,13 @@ int check_common(const mortar_bcsr_t *W, const uint16_t *x, int64_t M, int64_t l
     if (!W || !W->row_desc || !W->codes_o || !W->sd_o || !W->col_o || !x || !y)
         return mortar_fail(MORTAR_ERR_ARG, "spmm: null pointer");
     if (W->Rb <= 0 || W->Cb <= 0 || W->nnz <= 0) return mortar_fail(MORTAR_ERR_ARG, "spmm: empty matrix");
-    if (W->seg_cb <= 0 || tile_bytes(32, W->seg_cb < W->Cb ? W->seg_cb : W->Cb) > LDS_BUDGET)
-        return mortar_fail(MORTAR_ERR_ARG, "spmm: seg_cb=%d does not fit LDS (max %d)", W->seg_cb, mortar_prefill_max_seg_cb());
+    {   // K segments as wide as a 32-token tile allows serve every row count; a decode-only stream (one segment as wide as a
+        // 4-token tile allows, mortar_decode_max_seg_cb) serves calls of up to 4 rows
+        const int seg = W->seg_cb < W->Cb ? W->seg_cb : W->Cb;
+        if (W->seg_cb <= 0 || tile_bytes(M <= 4 ? 4 : 32, seg) > LDS_BUDGET)
+            return mortar_fail(MORTAR_ERR_ARG, "spmm: K segments of %d block-columns do not fit LDS for %lld rows (max %d; %d for up to 4 rows)",
+                               W->seg_cb, (long long)M, mortar_prefill_max_seg_cb(), mortar_decode_max_seg_cb());
+    }
     {   // the kernels address the octet stream with 32-bit byte offsets (1 KiB of 4-bit codes per octet)
         const int64_t nseg = (W->Cb + W->seg_cb - 1) / W->seg_cb;
         if ((int64_t)W->nnz / 8 + (int64_t)W->Rb * nseg >= ((int64_t)1 << 22))
@@ -150,6 +155,7 @@ int dispatch(int kind, SpmmParams &p, const mortar_bcsr_t *W, hipStream_t st) {
 }  // namespace
 
 extern "C" int mortar_prefill_max_seg_cb(void) { return (LDS_BUDGET - LDS_PAD * 16) / (32 * 32); }
+extern "C" int mortar_decode_max_seg_cb(void) { return (LDS_BUDGET - LDS_PAD * 16) / (4 * 32); }
 
 extern "C" int mortar_route_tile(int32_t Cb, int64_t M) {
     if (M > 0 && M <= MORTAR_SMALLM_MAX) {
