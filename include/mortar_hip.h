@@ -133,11 +133,12 @@ int mortar_transpose_topology_host(const int32_t *row_ptr, const int16_t *col, i
  * Cb <= this runs the single-segment prefill kernel.  Use seg_cb = ceil(Cb / ceil(Cb / max)). */
 int mortar_prefill_max_seg_cb(void);
 
-/* Largest K segment whose 4-token tile fits in LDS.  A second stream of a matrix laid out with ONE segment of Cb <= this
- * (same codes, rows padded to octets once per row instead of once per (segment, row)) serves calls of up to 4 rows only:
- * the layer-batched decode launches read about 8 % fewer bytes from it for a `down` whose prefill stream has three
- * segments.  Calls with more rows on such a stream are refused.  No counterpart in the reference. */
-int mortar_decode_max_seg_cb(void);
+/* Largest K segment whose 4-token (rows <= 4) or 16-token (rows <= 16) tile fits in LDS.  A second stream of a matrix laid
+ * out with segments that wide (same codes; fewer, longer row parts, so less padding to octets and fewer barrier pairs:
+ * one segment instead of three for a `down` of 5632 inputs at up to 4 rows, two at up to 16) serves calls of up to that
+ * many rows only: the layer-batched decode launches run 9 % faster on it.  Calls with more rows on such a stream are
+ * refused.  No counterpart in the reference. */
+int mortar_decode_max_seg_cb(int32_t rows);
 
 /* Row-unit order for uneven nnz: units sorted by descending block count and dealt into groups of `group`
  * consecutive positions with similar totals (longest-processing-time first); use group = 16, the number of

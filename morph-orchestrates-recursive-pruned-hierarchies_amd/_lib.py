@@ -42,7 +42,7 @@ _SIGS = {
     "mortar_sdd_workspace_bytes": (c_i64, [c_i32, c_i32, c_i32, c_i64]),
     "mortar_sdd_bf16": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_i64, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp]),
     "mortar_prefill_max_seg_cb": (C.c_int, []),
-    "mortar_decode_max_seg_cb": (C.c_int, []),
+    "mortar_decode_max_seg_cb": (C.c_int, [c_i32]),
     "mortar_validate_bcsr_host": (C.c_int, [c_vp, c_vp, c_i32, c_i32]),
     "mortar_schedule_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp]),
     "mortar_unit_order_host": (C.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp]),

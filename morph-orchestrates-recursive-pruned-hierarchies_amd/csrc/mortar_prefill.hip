@@ -17,12 +17,12 @@ int check_common(const mortar_bcsr_t *W, const uint16_t *x, int64_t M, int64_t l
     if (!W || !W->row_desc || !W->codes_o || !W->sd_o || !W->col_o || !x || !y)
         return mortar_fail(MORTAR_ERR_ARG, "spmm: null pointer");
     if (W->Rb <= 0 || W->Cb <= 0 || W->nnz <= 0) return mortar_fail(MORTAR_ERR_ARG, "spmm: empty matrix");
-    {   // K segments as wide as a 32-token tile allows serve every row count; a decode-only stream (one segment as wide as a
-        // 4-token tile allows, mortar_decode_max_seg_cb) serves calls of up to 4 rows
+    {   // K segments as wide as a 32-token tile allows serve every row count; a decode stream laid out with wider segments
+        // (as wide as a 4- or 16-token tile allows, mortar_decode_max_seg_cb) serves calls of up to 4 or 16 rows
         const int seg = W->seg_cb < W->Cb ? W->seg_cb : W->Cb;
-        if (W->seg_cb <= 0 || tile_bytes(M <= 4 ? 4 : 32, seg) > LDS_BUDGET)
-            return mortar_fail(MORTAR_ERR_ARG, "spmm: K segments of %d block-columns do not fit LDS for %lld rows (max %d; %d for up to 4 rows)",
-                               W->seg_cb, (long long)M, mortar_prefill_max_seg_cb(), mortar_decode_max_seg_cb());
+        if (W->seg_cb <= 0 || tile_bytes(M <= 4 ? 4 : M <= 16 ? 16 : 32, seg) > LDS_BUDGET)
+            return mortar_fail(MORTAR_ERR_ARG, "spmm: K segments of %d block-columns do not fit LDS for %lld rows (max %d; %d up to 16 rows, %d up to 4)",
+                               W->seg_cb, (long long)M, mortar_prefill_max_seg_cb(), mortar_decode_max_seg_cb(16), mortar_decode_max_seg_cb(4));
     }
     {   // the kernels address the octet stream with 32-bit byte offsets (1 KiB of 4-bit codes per octet)
         const int64_t nseg = (W->Cb + W->seg_cb - 1) / W->seg_cb;
@@ -155,7 +155,9 @@ int dispatch(int kind, SpmmParams &p, const mortar_bcsr_t *W, hipStream_t st) {
 }  // namespace
 
 extern "C" int mortar_prefill_max_seg_cb(void) { return (LDS_BUDGET - LDS_PAD * 16) / (32 * 32); }
-extern "C" int mortar_decode_max_seg_cb(void) { return (LDS_BUDGET - LDS_PAD * 16) / (4 * 32); }
+extern "C" int mortar_decode_max_seg_cb(int32_t rows) {
+    return (LDS_BUDGET - LDS_PAD * 16) / ((rows <= 4 ? 4 : rows <= 16 ? 16 : 32) * 32);
+}
 
 extern "C" int mortar_route_tile(int32_t Cb, int64_t M) {
     if (M > 0 && M <= MORTAR_SMALLM_MAX) {

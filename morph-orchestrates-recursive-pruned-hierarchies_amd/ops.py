@@ -505,9 +505,9 @@ class LayerStack:
                 raise TypeError("LayerStack: outputs must be bfloat16 device tensors")
         L = _lib.lib()
         if M <= 4 and not swiglu:
-            # products over several K segments (`down`) read their one-segment decode streams: rows padded to octets once
-            # per row and one part per row (all layers or none: a launch takes one segment width)
-            views = [p.decode_view() for p in packs]
+            # products over several K segments (`down`) read their one-segment decode streams: one part and one padding to
+            # octets per row (all layers or none: a launch takes one segment width)
+            views = [p.decode_view(M) for p in packs]
             if all(v is not None for v in views):
                 packs = views
         self.packs, self.xs, self.ys, self.swiglu, self.M, self.n = packs, xs, ys, int(bool(swiglu)), M, n

@@ -232,7 +232,7 @@ class MortarPack:
 
     def __init__(self, packed, scale, col, offsets, out_features: int, in_features: int, device,
                  prefill_stream: bool = True, scale_after_sum: bool = True, allow_empty_rows: bool = False,
-                 seg_cb: int | None = None, decode_only: bool = False):
+                 seg_cb: int | None = None, decode_rows: int = 0):
         if out_features % BLK or in_features % BLK:
             raise ValueError(f"[{out_features},{in_features}] not divisible by blocking {BLK}")
         self.out_features, self.in_features = int(out_features), int(in_features)
@@ -265,8 +265,8 @@ class MortarPack:
         self.sdup = torch.from_numpy(sdup.view(np.int32)).to(dev)
         self.col = torch.from_numpy(self.h_col).to(dev)
         self.row_ptr = torch.from_numpy(self.h_offsets).to(dev)
-        max_seg = int(_lib.lib().mortar_decode_max_seg_cb() if decode_only else _lib.lib().mortar_prefill_max_seg_cb())
-        self.decode_only = bool(decode_only)          # K segments wider than a 32-token tile: calls of up to 4 rows only
+        max_seg = int(_lib.lib().mortar_decode_max_seg_cb(decode_rows) if decode_rows else _lib.lib().mortar_prefill_max_seg_cb())
+        self.decode_rows = int(decode_rows)     # > 0: K segments wider than a 32-token tile allows; calls of up to that many rows
         if seg_cb is not None:
             if not 0 < seg_cb <= max_seg:
                 raise ValueError(f"seg_cb={seg_cb} outside 1..{max_seg}")
@@ -286,7 +286,7 @@ class MortarPack:
         self._scheds: dict[int, torch.Tensor] = {}
         self._worklists: dict[tuple, tuple] = {}
         # what decode_view() rebuilds the stream from; dropped once the values are rewritten on the device
-        self._h_codes, self._h_sdup, self._dview = (codes, sdup, None) if packed is not None else (None, None, None)
+        self._h_codes, self._h_sdup, self._dview = (codes, sdup, {}) if packed is not None else (None, None, {})
         self._pos = self._ws = self._status = self.src_block = self._sdd = None
         self._status_host = self._status_event = None
         self._transposed: "MortarPack | None" = None
@@ -300,30 +300,35 @@ class MortarPack:
                                self.codes4_o.data_ptr() if self.codes4_o is not None else None,
                                self.Rb, self.Cb, self.nnz, self.seg_cb, self.uniform_scale, 0)
 
-    def decode_view(self) -> "MortarPack | None":
-        """A second stream of this matrix for calls of up to 4 rows: ONE K segment (a 4-token tile of all K fits LDS), so a
-        row's blocks are padded to octets once, not once per segment, and a row is one part.  Shares the topology and code
-        arrays; costs 72 bytes per block.  None when the pack already has one segment, the rows are too wide, or the values
-        were rewritten on the device (the view is built from the host copy of the codes)."""
-        if self.nseg == 1 or self.decode_only or self._h_codes is None or self.Cb > int(_lib.lib().mortar_decode_max_seg_cb()):
+    def decode_view(self, rows: int) -> "MortarPack | None":
+        """A second stream of this matrix for calls of up to 4 rows: K segments as wide as a 4-token tile allows (one
+        segment for rows of up to 19840 values), so a row is one part and is padded to octets once.  Shares the topology and
+        code arrays; costs 72 bytes per block.  None for more rows (a two-segment stream for 16-token tiles was measured
+        slower than the three-segment one: its 90 KB tile leaves one workgroup per CU), when it would not reduce the number
+        of segments, or when the values were rewritten on the device (the view is built from the host copy of the codes)."""
+        if rows > 4 or self.decode_rows or self._h_codes is None:
             return None
-        if self._dview is None:
+        tile = 4
+        nseg = -(-self.Cb // int(_lib.lib().mortar_decode_max_seg_cb(tile)))
+        if nseg >= self.nseg:
+            return None
+        if tile not in self._dview:
             v = object.__new__(MortarPack)
             v.__dict__.update(self.__dict__)
-            v.decode_only, v.seg_cb, v.nseg = True, self.Cb, 1
-            grp, codes_o, sd_o, col_o = octet_layout(self.h_offsets, self.Rb, self.Cb, self.Cb, self._h_codes, self._h_sdup, self.h_col)
+            v.decode_rows, v.seg_cb, v.nseg = tile, -(-self.Cb // nseg), nseg
+            grp, codes_o, sd_o, col_o = octet_layout(self.h_offsets, self.Rb, self.Cb, v.seg_cb, self._h_codes, self._h_sdup, self.h_col)
             v.h_row_desc = grp
             v.row_desc = torch.from_numpy(grp).to(self.device)
             v.codes_o = torch.from_numpy(codes_o.view(np.int32)).to(self.device)
             v.sd_o = torch.from_numpy(sd_o.view(np.int32)).to(self.device)
             v.col_o = torch.from_numpy(col_o).to(self.device)
             v.codes4_o = None
-            v._scheds, v._worklists, v._transposed, v._dview = {}, {}, None, None
+            v._scheds, v._worklists, v._transposed, v._dview = {}, {}, None, {}
             v._h_codes = v._h_sdup = None
             v.struct = v._make_struct()
             v.ref = C.byref(v.struct)
-            self._dview = v
-        return self._dview
+            self._dview[tile] = v
+        return self._dview[tile]
 
     # ---- device-side re-pack ----------------------------------------------------------------------------------
 
@@ -344,7 +349,7 @@ class MortarPack:
             raise ValueError("requantize: values must be bf16 or fp32 on the pack's device")
         if tuple(values.shape) != (self.nnz, BLK, BLK) or not values.is_contiguous():
             raise ValueError(f"requantize: values must be contiguous [{self.nnz}, 16, 16], got {tuple(values.shape)}")
-        self._h_codes = self._h_sdup = self._dview = None      # the host copy of the codes is stale from here on
+        self._h_codes, self._h_sdup, self._dview = None, None, {}      # the host copy of the codes is stale from here on
         L = _lib.lib()
         if self._pos is None:
             self._pos = torch.from_numpy(octet_positions(self.h_offsets, self.Rb, self.Cb, self.seg_cb, self.h_col)).to(self.device)
@@ -502,7 +507,7 @@ class MortarPack:
                 setattr(c, name, getattr(self, name).clone())
         c._scheds = {k: v.clone() for k, v in self._scheds.items()}
         c._worklists = {k: (v[0].clone(), v[1], v[2].clone(), v[3]) for k, v in self._worklists.items()}
-        c._transposed = c._dview = None      # the clone builds its own views
+        c._transposed, c._dview = None, {}      # the clone builds its own views
         c.struct = c._make_struct()
         c.ref = C.byref(c.struct)
         return c

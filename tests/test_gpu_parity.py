@@ -520,34 +520,35 @@ def test_router_tail_behind_a_library_projection(dev, N, d, nsk, n):
 
 
 def test_decode_view_of_a_segmented_matrix(dev):
-    """A matrix whose prefill stream has several K segments (`down`) carries a second, one-segment stream for calls of up to
-    4 rows: the layer-batched launch picks it by itself and gives the bits of the segmented stream; more rows on it are
-    refused; a matrix with one segment, too wide rows or device-rewritten values has none."""
+    """A matrix whose prefill stream has several K segments (`down`) carries a one-segment decode stream for calls of up to
+    4 rows.  The layer-batched launch picks it by itself (same results to the usual bar: the pairing of blocks into MFMAs
+    follows the segments); more rows on it are refused; a matrix with one segment or device-rewritten values has none."""
     spec = synth.synth_mlp(512, 16 * 352, 0.25, seed=91, zipf_s=1.2)
     m = spec["down"]
     W = synth.to_pack(m, dev)
-    assert W.nseg == 3 and synth.to_pack(spec["gate_up"], dev).decode_view() is None
-    V = W.decode_view()
-    assert V is not None and V.nseg == 1 and V.decode_only and V is W.decode_view()
-    assert V.codes_o.numel() <= W.codes_o.numel()                      # rows padded to octets once, not once per segment
-    for B in (1, 3, 4):
+    assert W.nseg == 3 and synth.to_pack(spec["gate_up"], dev).decode_view(1) is None and W.decode_view(5) is None
+    V = W.decode_view(3)
+    assert V.nseg == 1 and V.decode_rows == 4 and V is W.decode_view(1)
+    assert V.codes_o.numel() <= W.codes_o.numel()                      # one part per row: padded to octets once
+    for B in (1, 3, 4, 5):
         x = synth.synth_x(B, 16 * 352, 92 + B)
         xd = to_dev(x, dev)
         ref = oracle_spmm(x, m)
         ys = [torch.empty((B, 512), dtype=torch.bfloat16, device=dev) for _ in range(3)]
         st = ops.LayerStack([W, W.clone_weights(), W], [xd] * 3, ys, swiglu=False)
-        assert all(p.decode_only for p in st.packs)
+        assert all(p.decode_rows == (4 if B <= 4 else 0) for p in st.packs)
         st.run()
         for y in ys:
             assert_close_bf16(to_np(y), ref, f"decode view B={B}", ulps=8)
-        assert torch.equal(ops.spmm(xd, V), ys[0]) and torch.equal(ops.spmm(xd, W), ys[0])
+        if B <= 4:
+            assert_close_bf16(to_np(ops.spmm(xd, V)), ref, f"single launch on the decode view B={B}", ulps=8)
     with pytest.raises(ValueError):
         ops.spmm(to_dev(synth.synth_x(5, 16 * 352, 99), dev), V)            # more than 4 rows: not on this stream
     W.requantize(torch.from_numpy(O.effective_blocks(m["codes"], m["scales"])).to(dev), per_block=True)
-    assert W.decode_view() is None                                          # the host copy of the codes is stale now
+    assert W.decode_view(1) is None                                          # the host copy of the codes is stale now
     ys = [torch.empty((2, 512), dtype=torch.bfloat16, device=dev)]
     st = ops.LayerStack([W], [to_dev(synth.synth_x(2, 16 * 352, 98), dev)], ys, swiglu=False)
-    assert not st.packs[0].decode_only
+    assert st.packs[0].decode_rows == 0
 
 
 def test_empty_batches_launch_nothing(dev):
