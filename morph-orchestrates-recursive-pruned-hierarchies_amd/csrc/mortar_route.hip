@@ -226,7 +226,7 @@ __device__ __forceinline__ void wave_sort_desc(uint32_t (&key)[KPL], int lane) {
 
 // The n largest of the P = nsk * nsk product scores of one token in descending order (+ bias) -> lgt[0 .. n), on one wave.
 template <int KPL>
-__device__ __forceinline__ void ranked_logits(const float *sct, int nsk, int P, const float *bias, int n, float *lgt,
+__device__ __attribute__((noinline)) void ranked_logits(const float *sct, int nsk, int P, const float *bias, int n, float *lgt,
                                               float *logits_row, int lane) {
     uint32_t key[KPL];
 #pragma unroll
@@ -411,11 +411,12 @@ __global__ void __launch_bounds__(256) router_tail_kernel(const float *qv, int d
 //      in the wave's registers), then the gating tail.
 // Same arithmetic as router_tail_kernel; the sums are ordered differently.  A group is a chain of latencies (about 3 us of
 // loads, 2 us of LayerNorm, 1.3 us per key row and wave, 2-10 us of logits and gating), so throughput comes from the
-// groups in flight: two workgroups per CU at this register count.
+// groups in flight: three workgroups per CU (two for rows wider than 4096 values) at this register count, with the
+// sort kept out of line (inlined, its registers add to the whole kernel's).
 constexpr int TAIL_TT = 4;
 
 template <int MAXPL, int J>      // J: float4 pieces of a row per thread (d <= 1024 * J); tokens per group tt = min(4, 8 / J)
-__global__ void __launch_bounds__(256, 2) router_tail_group_kernel(const float *qv, int64_t N, int d, int64_t ldq, const float *iter_vec,
+__global__ void __launch_bounds__(256, J == 8 ? 2 : 3) router_tail_group_kernel(const float *qv, int64_t N, int d, int64_t ldq, const float *iter_vec,
                                                                  const float *ln_w, const float *ln_b, float ln_eps,
                                                                  const float *ka, const float *kb, int nsk, const float *bias,
                                                                  int n, int k, int tt, float *logits_out, float *gates,
@@ -439,8 +440,10 @@ __global__ void __launch_bounds__(256, 2) router_tail_group_kernel(const float *
 #pragma unroll
             for (int jj = 0; jj < J; ++jj) {
                 const int i = tid + 256 * jj, ic = i < d4 ? i : d4 - 1;
-                w[jj] = lw4[ic];
-                b[jj] = lb4[ic];
+                if (J < 4) {              // wide rows fetch the LayerNorm parameters when they are used (registers)
+                    w[jj] = lw4[ic];
+                    b[jj] = lb4[ic];
+                }
 #pragma unroll
                 for (int t = 0; t < TT; ++t) {
                     const bool on = t < nt && i < d4;
@@ -483,6 +486,10 @@ __global__ void __launch_bounds__(256, 2) router_tail_group_kernel(const float *
 #pragma unroll
                 for (int jj = 0; jj < J; ++jj) {
                     const int i = tid + 256 * jj;
+                    if (J >= 4) {
+                        w[jj] = lw4[i < d4 ? i : d4 - 1];
+                        b[jj] = lb4[i < d4 ? i : d4 - 1];
+                    }
                     if (t < nt && i < d4) {
                         const float4 q = v[t * J + jj];
                         const float m = mean[t], r = rstd[t];
