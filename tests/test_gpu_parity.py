@@ -1234,3 +1234,52 @@ def test_argument_errors_are_raised_before_launch(dev):
     assert ops.spmm(x[:0], W).shape == (0, 64)                                    # empty batch: no launch, empty result
     y = ops.spmm(x, W)                                                            # and the good call still works
     assert_close_bf16(to_np(y), oracle_spmm(to_np(x), m), "after errors")
+
+
+def test_raw_c_abi_refuses_bad_calls_of_the_newer_entry_points(dev):
+    """mortar_mlp_bf16, mortar_dds_values_bf16 and mortar_router_tail_f32 called through ctypes with bad arguments return a
+    negative code and a message, launch nothing, and leave the outputs untouched."""
+    import ctypes as C
+    from mortar_amd import _lib
+    from mortar_amd.pack import BcsrTopology
+    L = _lib.lib()
+    err = lambda: C.c_char_p(L.mortar_last_error()).value.decode()
+    spec = synth.synth_mlp(256, 640, 0.25, seed=7)
+    G, D = synth.to_pack(spec["gate_up"], dev), synth.to_pack(spec["down"], dev)
+    x = to_dev(synth.synth_x(40, 256, 8), dev)
+    y = torch.full((40, 256), 7.0, dtype=torch.bfloat16, device=dev)
+    ws = torch.zeros(ops.mlp_hidden_bytes(40, 640), dtype=torch.uint8, device=dev)
+    p = lambda t: C.c_void_p(t.data_ptr())
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    call = lambda Wg, Wd, hidden, phase: L.mortar_mlp_bf16(Wg.ref, p(Wg.sched(2)), Wd.ref, p(Wd.sched(1)), p(x), 40, 256, 0, None, 0.0,
+                                                             None, 0, hidden, p(y), 256, phase, st)
+    assert call(G, D, None, 0) < 0 and "null" in err()
+    assert call(D, G, p(ws), 0) < 0                                     # matrices swapped: shapes do not chain
+    assert call(G, D, p(ws), 3) < 0 and "phase" in err()
+    assert call(G, D, C.c_void_p(ws.data_ptr() + 2), 0) < 0 and "aligned" in err()
+    torch.cuda.synchronize()
+    assert bool((y == 7.0).all())
+    assert call(G, D, p(ws), 0) == 0                                    # and the good call runs
+    torch.cuda.synchronize()
+    assert_close_bf16(to_np(y), O.swiglu_mlp(to_np(x), spec["gate_up"], spec["down"])["y"], "mlp after refused calls", ulps=8)
+
+    m = spec["down"]
+    T = BcsrTopology(m["offsets"], m["col_idx"], m["shape"][0], m["shape"][1], dev)
+    data = torch.zeros((T.nnz, 16, 16), dtype=torch.bfloat16, device=dev)
+    h = to_dev(synth.synth_x(40, 640, 9), dev)
+    y.fill_(7.0)
+    dds = lambda xp, M, ldx: L.mortar_dds_values_bf16(p(T.row_ptr), p(T.col), None, p(data), T.Rb, T.Cb, T.nnz, xp, M, ldx, p(y), 256, st)
+    assert dds(None, 40, 640) < 0 and dds(p(h), -1, 640) < 0 and dds(p(h), 40, 100) < 0
+    assert dds(C.c_void_p(h.data_ptr() + 2), 40, 640) < 0
+    torch.cuda.synchronize()
+    assert bool((y == 7.0).all())
+
+    z = lambda *shape: torch.zeros(shape, device=dev)
+    qv, g = z(8, 256), torch.full((8, 16), 7.0, device=dev)
+    tail = lambda d, ldq, nsk, n, k: L.mortar_router_tail_f32(p(qv), 8, d, ldq, None, p(z(256)), p(z(256)), 1e-5, p(z(4, 128)), p(z(4, 128)), nsk, p(z(16)),
+                                                               n, k, None, p(g), None, st)
+    assert tail(250, 256, 4, 16, 4) < 0 and tail(256, 100, 4, 16, 4) < 0 and tail(256, 256, 0, 16, 4) < 0 and tail(256, 256, 4, 16, 0) < 0
+    assert tail(256, 256, 40, 16, 4) < 0 and "product keys" in err()
+    torch.cuda.synchronize()
+    assert bool((g == 7.0).all())
+
