@@ -143,6 +143,16 @@ __device__ __forceinline__ uint32_t mortar_row_bcast(uint32_t v, int k) {
     }
 }
 
+// s_setprio with a value that folds to a constant after unrolling (the instruction takes an immediate 0..3).
+__device__ __forceinline__ void mortar_setprio(int p) {
+    switch (p) {
+        case 0: __builtin_amdgcn_s_setprio(0); break;
+        case 1: __builtin_amdgcn_s_setprio(1); break;
+        case 2: __builtin_amdgcn_s_setprio(2); break;
+        default: __builtin_amdgcn_s_setprio(3); break;
+    }
+}
+
 // One batch of the octet stream in registers: RES_GROUPS octets (8 blocks = 4 pairs each) = 16 block pairs.
 // A lane holds its code dwords of the 16 pairs (one 16-byte load per octet) and, as lane k of its 16-lane row,
 // the scale pattern and block-column of pair k (one dword each); pair u's metadata reaches the row by a DPP
@@ -660,6 +670,11 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
         }
 #pragma unroll
         for (int q = 0; q < NP; ++q) {
+            // A wave lowers its priority with every part of the segment it has finished: the arbiter serves the oldest wave of
+            // a SIMD first, so without this the four waves finish a segment one after another (4.8 / 6.3 / 8.0 / 9.4 us measured)
+            // and the SIMD runs the end of it on one or two waves.  Tile-ordered form only: with the register-staged forms the
+            // same priorities cost time (the staging of the next segment then starts from uneven waves).
+            if constexpr (XT) mortar_setprio(NP - 1 - q);
             MortarBatch bn;
             if (q + 1 < NP) first_batch(bn, q + 1);
             const int nbq = g0[q] < g1[q] ? nb[q] : 0;
@@ -673,6 +688,7 @@ __global__ void __launch_bounds__(WAVES * 64) mortar_segmented_kernel(const Spmm
             }
             if (q + 1 < NP) bq = bn;
         }
+        if constexpr (XT) mortar_setprio(0);
     }
 
     uint32_t tl[MSUB];
