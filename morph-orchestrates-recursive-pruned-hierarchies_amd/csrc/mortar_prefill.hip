@@ -61,8 +61,8 @@ int resident_mt(int Cb) {
 }
 
 // prefill tiles: 16 wavefronts (4 per SIMD) for both tiles (the 64-token tile with 8 wavefronts was measured 18 % slower
-// on the base-width gate_up, although the 16-wave gate_up form spills six registers; a 96-token tile of a narrow
-// matrix leaves only two waves per SIMD and is slower still)
+// on the base-width gate_up; the 16-wave form fits its 128 registers with the LDS operands fetched one pair ahead
+// instead of two; a 96-token tile of a narrow matrix leaves only two waves per SIMD and is slower still)
 template <int NACC, bool ROUTED, int CODE, bool TL = false>
 int launch_resident_any(SpmmParams &p, hipStream_t st) {
     switch (resident_mt(p.Cb)) {

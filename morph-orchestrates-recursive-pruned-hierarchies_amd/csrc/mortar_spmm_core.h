@@ -204,9 +204,10 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
         // per octet (a whole octet past the end of the part is skipped) and, for prefill tiles, per half octet;
         // otherwise the pairs run straight, pairs past the end being the all-zero padding blocks of the stream.
         constexpr int NP = 4 * RES_GROUPS;
-        uint4 Bq[3][MSUB];
+        constexpr int PD = MT == 64 ? 1 : 2;      // pairs ahead (the distance makes no difference in time; the 64-token tile has no registers to spare)
+        uint4 Bq[PD + 1][MSUB];
 #pragma unroll
-        for (int d = 0; d < 2; ++d) {
+        for (int d = 0; d < PD; ++d) {
             const uint32_t xo = mortar_row_bcast(ccs, d) + xo_base;
 #pragma unroll
             for (int ms = 0; ms < MSUB; ++ms) Bq[d][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 32u : ms * 512u));
@@ -220,16 +221,16 @@ __device__ __forceinline__ void mortar_row_part(const SpmmView &p, const uint4 *
                     if (t == 2 && u >= pairs) break;                  // the padded half of the last octet
                     const uint32_t nib = (CODE & CODE_4BIT) ? b.cw[k][t] : ((b.cw[k][t] << (2 * hsel)) & 0xCCCCCCCCu);
                     const u32x4_t A = (CODE & CODE_UNIFORM) ? mortar_nib4(nib) : mortar_scale4(nib, mortar_row_bcast(b.sdv, u));
-                    if (u + 2 < NP) {
-                        const uint32_t xo = mortar_row_bcast(ccs, u + 2) + xo_base;
+                    if (u + PD < NP) {
+                        const uint32_t xo = mortar_row_bcast(ccs, u + PD) + xo_base;
 #pragma unroll
                         for (int ms = 0; ms < MSUB; ++ms)
-                            Bq[(u + 2) % 3][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 32u : ms * 512u));
+                            Bq[(u + PD) % (PD + 1)][ms] = *reinterpret_cast<const uint4 *>(lb + xo + (ROUTED ? tk[ms] * 32u : ms * 512u));
                     }
 #pragma unroll
                     for (int ms = 0; ms < MSUB; ++ms) {
                         if (!ROUTED || ms < nsub) {
-                            const uint4 bq = Bq[u % 3][ms];
+                            const uint4 bq = Bq[u % (PD + 1)][ms];
                             const u32x4_t Bv = {bq.x, bq.y, bq.z, bq.w};
                             acc[ms] = mortar_mfma(A, Bv, acc[ms]);
                         }
